@@ -1,0 +1,279 @@
+/*
+ * zenu_hip.h -- C ABI of the MI355X (gfx950) device tensor-kernel layer for ZeNu.
+ *
+ * This is the boundary a `Hip` device of zenu-matrix binds to, in place of the
+ * bindgen output over zenu-cuda-kernel-sys/kernel/kernel.h and of the cudart
+ * wrappers in zenu-cuda/src/runtime/mod.rs.  Plain pointers and sizes only.
+ *
+ * Conventions
+ *   - every pointer named *_dev / inside a zenu_tensor_t is DEVICE memory;
+ *   - strides are in ELEMENTS; a tensor's ptr already includes its offset
+ *     (Matrix::as_ptr, zenu-matrix/src/matrix.rs:288-290);
+ *   - at most 6 dimensions (zenu-matrix/src/dim/dim_dyn.rs:10-13,75);
+ *   - `stream` is a hipStream_t passed as void*; NULL = the HIP null stream;
+ *     all launches are asynchronous on that stream unless stated otherwise;
+ *   - every function returns ZENU_OK (0) or an error code; nothing aborts.  Where the
+ *     reference panics (shape / rank / axis mismatch) the code is ZENU_ERR_SHAPE,
+ *     ZENU_ERR_RANK or ZENU_ERR_AXIS and nothing is launched.
+ *   - exactly aliased input/output (the *_assign forms) is supported; partially
+ *     overlapping operands are not.
+ */
+#ifndef ZENU_HIP_H
+#define ZENU_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ZENU_MAX_DIM 6
+
+typedef enum {
+    ZENU_OK = 0,
+    ZENU_ERR_RANK = 1,        /* "The rank of the matrix is different."      */
+    ZENU_ERR_SHAPE = 2,       /* shapes not broadcast-compatible / mismatch  */
+    ZENU_ERR_AXIS = 3,        /* "Invalid axis" / "Axis out of bounds"       */
+    ZENU_ERR_ARG = 4,         /* null pointer, bad enum, ndim > 6, negative size */
+    ZENU_ERR_HIP = 5,         /* a HIP runtime call failed: see zenu_hip_last_hip_error */
+    ZENU_ERR_OOM = 6,         /* device allocation failed even after trimming the cache */
+    ZENU_ERR_UNSUPPORTED = 7, /* valid request this build has no kernel for  */
+    ZENU_ERR_NOT_OWNED = 8    /* zenu_hip_free: pointer unknown to the pool (MemPoolFreeError) */
+} zenu_status_t;
+
+typedef enum { ZENU_F32 = 0, ZENU_F64 = 1 } zenu_dtype_t;
+
+typedef enum { ZENU_ADD = 0, ZENU_SUB = 1, ZENU_MUL = 2, ZENU_DIV = 3 } zenu_binop_t;
+
+typedef enum {
+    ZENU_EXP = 0, ZENU_LOG = 1, ZENU_TANH = 2, ZENU_SQRT = 3, ZENU_ABS = 4,
+    ZENU_SIN = 5, ZENU_COS = 6, ZENU_TAN = 7, ZENU_ASIN = 8, ZENU_ACOS = 9, ZENU_ATAN = 10,
+    ZENU_SINH = 11, ZENU_COSH = 12,
+    ZENU_SIGMOID = 13 /* 0.5 + 0.5*tanh(0.5*x), zenu-autograd/src/activation/sigmoid.rs:7-15 */
+} zenu_unop_t;
+
+/* A strided view: Matrix<_, DimDyn, D> flattened (zenu-matrix/src/matrix.rs:224-233). */
+typedef struct zenu_tensor {
+    void   *ptr;
+    int32_t ndim;
+    int32_t reserved;
+    int64_t shape[ZENU_MAX_DIM];
+    int64_t stride[ZENU_MAX_DIM];
+} zenu_tensor_t;
+
+typedef void *zenu_stream_t;
+
+/* ------------------------------------------------------------------------- */
+/* Runtime: replaces zenu-cuda/src/runtime/mod.rs and zenu-cuda/src/lib.rs    */
+/* ------------------------------------------------------------------------- */
+
+/* Select the device and create the library state (allocator, default stream).
+ * Idempotent.  zenu-cuda/src/lib.rs:18-25,60-72. */
+int zenu_hip_init(int device);
+/* Release every cached block and the library state. */
+int zenu_hip_shutdown(void);
+const char *zenu_hip_status_string(int status);
+/* hipError_t of the last failed runtime call on this thread, and its text. */
+int zenu_hip_last_hip_error(void);
+const char *zenu_hip_last_hip_error_string(void);
+
+int zenu_hip_stream_create(zenu_stream_t *stream);   /* runtime/mod.rs:113-121; default priority */
+int zenu_hip_stream_destroy(zenu_stream_t stream);
+int zenu_hip_stream_synchronize(zenu_stream_t stream);
+int zenu_hip_device_synchronize(void);
+
+/* Stream-ordered caching allocator: replaces zenu-matrix/src/memory_pool/mod.rs:79-145 and
+ * cuda_malloc_bytes / cuda_free (runtime/mod.rs:30-60, which synchronise the stream on every
+ * call).  zenu_hip_malloc never synchronises on a cache hit.  A block freed on stream S is
+ * reusable at once by allocations on S, and by other streams only after an event recorded at
+ * the free has completed.  On out-of-memory the cache is trimmed and the request retried once
+ * (the flow zenu-matrix/src/memory_pool/mod.rs:9-20 documents).  Thread-safe.
+ * Honours ZENU_USE_MEMPOOL=0 (zenu-matrix/src/lib.rs:36): every call goes to hipMalloc/hipFree. */
+int zenu_hip_malloc(void **ptr_dev, size_t bytes, zenu_stream_t stream);
+int zenu_hip_free(void *ptr_dev, zenu_stream_t stream);
+/* Return all cached (free) blocks to the driver. */
+int zenu_hip_mempool_trim(void);
+typedef struct zenu_mempool_stats {
+    uint64_t bytes_in_use;      /* handed out and not yet freed              */
+    uint64_t bytes_cached;      /* free blocks held by the pool              */
+    uint64_t bytes_reserved;    /* total obtained from the driver            */
+    uint64_t n_alloc_calls;     /* zenu_hip_malloc calls                     */
+    uint64_t n_cache_hits;      /* of which served from the cache            */
+    uint64_t n_driver_allocs;   /* hipMalloc calls                           */
+    uint64_t n_driver_frees;    /* hipFree calls                             */
+    uint64_t n_oom_retries;     /* allocation retried after a trim           */
+} zenu_mempool_stats_t;
+int zenu_hip_mempool_stats(zenu_mempool_stats_t *out);
+
+/* Raw driver allocation, bypassing the pool (DeviceBase::raw_alloc / raw_drop_ptr,
+ * zenu-matrix/src/device/nvidia/mod.rs:8-16). */
+int zenu_hip_raw_malloc(void **ptr_dev, size_t bytes);
+int zenu_hip_raw_free(void *ptr_dev);
+
+/* Copies (runtime/mod.rs:83-97).  h2d / d2h return after the host buffer may be reused / read. */
+int zenu_hip_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes, zenu_stream_t stream);
+int zenu_hip_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes, zenu_stream_t stream);
+int zenu_hip_memcpy_d2d(void *dst_dev, const void *src_dev, size_t bytes, zenu_stream_t stream);
+/* Matrix::zeros: a fill kernel, not BLAS scal-by-0 on uninitialised memory
+ * (zenu-matrix/src/device/nvidia/mod.rs:53-58). */
+int zenu_hip_memset_zero(void *dst_dev, size_t bytes, zenu_stream_t stream);
+
+/* ------------------------------------------------------------------------- */
+/* N-d elementwise ops: one launch per Matrix-level call                       */
+/* ------------------------------------------------------------------------- */
+
+/* to = lhs op rhs with ZeNu's broadcasting (add_array / sub_array / mul_array / div_array,
+ * zenu-matrix/src/operation/basic_operations.rs:336-374; legality:
+ * zenu-matrix/src/with_clousers.rs:155-178, zenu-matrix/src/dim/dim_dyn.rs:24-58,119-148).
+ * `to` must have the larger operand's shape. */
+int zenu_hip_binary(int op, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *lhs,
+                    const zenu_tensor_t *rhs, zenu_stream_t stream);
+/* to op= rhs (add_assign ..., basic_operations.rs:318-334; with_clousers.rs:87-153). */
+int zenu_hip_binary_assign(int op, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *rhs,
+                           zenu_stream_t stream);
+/* to = other op scalar (add_scalar ..., basic_operations.rs:291-309); scalar is converted to dtype. */
+int zenu_hip_binary_scalar(int op, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other,
+                           double scalar, zenu_stream_t stream);
+/* to op= scalar (add_scalar_assign ..., basic_operations.rs:310-316). */
+int zenu_hip_binary_scalar_assign(int op, int dtype, const zenu_tensor_t *to, double scalar,
+                                  zenu_stream_t stream);
+/* Same with the scalar read from device memory (the 0-d tensor operand; trait methods
+ * scalar_ptr / scalar_assign_ptr, basic_operations.rs:74-88).  No host synchronisation. */
+int zenu_hip_binary_scalar_ptr(int op, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other,
+                               const void *scalar_dev, zenu_stream_t stream);
+int zenu_hip_binary_scalar_assign_ptr(int op, int dtype, const zenu_tensor_t *to,
+                                      const void *scalar_dev, zenu_stream_t stream);
+
+/* to = f(other), same shapes (exp_array / log_array / tanh_array / sqrt_array / abs_array ...,
+ * basic_operations.rs:512-575); ZENU_SIGMOID is the fused composite. */
+int zenu_hip_unary(int fn, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other,
+                   zenu_stream_t stream);
+int zenu_hip_unary_assign(int fn, int dtype, const zenu_tensor_t *to, zenu_stream_t stream);
+/* to = powf(other, scalar) (basic_operations.rs:577-611). */
+int zenu_hip_powf(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other, double scalar,
+                  zenu_stream_t stream);
+
+/* to = other > 0 ? other : alpha*other ; mask = other > 0 ? 1 : alpha*(-1)
+ * (zenu-matrix/src/operation/relu.rs:169-242). */
+int zenu_hip_relu(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other, double alpha,
+                  zenu_stream_t stream);
+int zenu_hip_relu_backward_mask(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other,
+                                double alpha, zenu_stream_t stream);
+
+/* Strided copy, same shapes (copy_from, zenu-matrix/src/operation/copy_from.rs:211-267;
+ * to_default_stride, to_default_stride.rs:7-15). */
+int zenu_hip_copy(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *src, zenu_stream_t stream);
+
+/* ------------------------------------------------------------------------- */
+/* Reductions (deterministic: fixed tree, no atomics on data)                  */
+/* ------------------------------------------------------------------------- */
+
+/* out = src.sum(axis): out has src's shape without `axis`, or with it kept as size 1
+ * (zenu-matrix/src/operation/sum.rs:9-32).  out may be strided. */
+int zenu_hip_sum_axis(int dtype, const zenu_tensor_t *out, const zenu_tensor_t *src, int axis,
+                      zenu_stream_t stream);
+/* *out_dev = sum of every element (sum_to(x, []), sum.rs:35-94). */
+int zenu_hip_sum_all(int dtype, void *out_dev, const zenu_tensor_t *src, zenu_stream_t stream);
+/* target = sum_to(src) for any legal target shape (sum.rs:35-94). */
+int zenu_hip_sum_to(int dtype, const zenu_tensor_t *target, const zenu_tensor_t *src,
+                    zenu_stream_t stream);
+/* out = src.max_axis(axis) (zenu-matrix/src/operation/max.rs:67-99). */
+int zenu_hip_max_axis(int dtype, const zenu_tensor_t *out, const zenu_tensor_t *src, int axis,
+                      zenu_stream_t stream);
+/* out_idx_dev[j] = position along `axis` of the FIRST maximum, row-major over the remaining dims
+ * (max_axis_idx_ravel, max.rs:103-134); int64 on the ABI, usize in ZeNu. */
+int zenu_hip_max_axis_idx(int dtype, int64_t *out_idx_dev, const zenu_tensor_t *src, int axis,
+                          zenu_stream_t stream);
+/* *out_flat_idx_dev = row-major flat index of the first maximum of the whole view; if
+ * out_val_dev is not NULL the maximum itself is stored there (Matrix::max_idx / max_item,
+ * max.rs:45-62).  Stays on the device: no host synchronisation. */
+int zenu_hip_max_idx(int dtype, int64_t *out_flat_idx_dev, void *out_val_dev,
+                     const zenu_tensor_t *src, zenu_stream_t stream);
+/* *out_dev = sum |x| (Asum, zenu-matrix/src/operation/asum.rs:14-68). */
+int zenu_hip_asum(int dtype, void *out_dev, const zenu_tensor_t *src, zenu_stream_t stream);
+
+/* ------------------------------------------------------------------------- */
+/* Fused optimizer updates (one launch, 4 loads + 3 stores per element)        */
+/* ------------------------------------------------------------------------- */
+
+/* p -= g*lr (zenu-optimizer/src/sgd.rs:20-31). */
+int zenu_hip_sgd_step(int dtype, void *p_dev, const void *g_dev, int64_t n, double lr,
+                      zenu_stream_t stream);
+/* Adam (zenu-optimizer/src/adam.rs:19-59).  `step` is the counter AFTER the increment;
+ * 1-beta, beta^step and 1-beta^step are formed on the host in dtype, as the reference does. */
+int zenu_hip_adam_step(int dtype, void *p_dev, const void *g_dev, void *m_dev, void *v_dev,
+                       int64_t n, double lr, double beta1, double beta2, double eps, double step,
+                       zenu_stream_t stream);
+/* AdamW (zenu-optimizer/src/adamw.rs:20-70): apply_decay != 0 for keys in weights() only. */
+int zenu_hip_adamw_step(int dtype, void *p_dev, const void *g_dev, void *m_dev, void *v_dev,
+                        int64_t n, double lr, double beta1, double beta2, double eps,
+                        double weight_decay, int apply_decay, double step, zenu_stream_t stream);
+/* Multi-tensor form: one launch over a model's parameter tensors.  The pointer / size tables are
+ * HOST arrays of length n_tensors; apply_decay may be NULL (no decay) or per-tensor flags. */
+int zenu_hip_adam_step_multi(int dtype, int n_tensors, void *const *p_dev, const void *const *g_dev,
+                             void *const *m_dev, void *const *v_dev, const int64_t *sizes, double lr,
+                             double beta1, double beta2, double eps, double weight_decay,
+                             const int32_t *apply_decay, double step, zenu_stream_t stream);
+
+/* ------------------------------------------------------------------------- */
+/* Entry points with the reference's own names and argument order              */
+/* (the headers under zenu-cuda-kernel-sys/kernel/): 1-D, int sizes/strides, null stream. */
+/* They let the unchanged zenu-cuda/src/kernel/mod.rs wrappers link.            */
+/* ------------------------------------------------------------------------- */
+
+#define ZENU_DECL_1D(T, S)                                                                         \
+    /* array_array.h:7-28 */                                                                       \
+    void array_array_add_##S(T *a, int stride_a, T *b, int stride_b, T *c, int stride_c, int n);  \
+    void array_array_sub_##S(T *a, int stride_a, T *b, int stride_b, T *c, int stride_c, int n);  \
+    void array_array_mul_##S(T *a, int stride_a, T *b, int stride_b, T *c, int stride_c, int n);  \
+    void array_array_div_##S(T *a, int stride_a, T *b, int stride_b, T *c, int stride_c, int n);  \
+    void array_array_add_assign_##S(T *a, int stride_a, T *b, int stride_b, int n);               \
+    void array_array_sub_assign_##S(T *a, int stride_a, T *b, int stride_b, int n);               \
+    void array_array_mul_assign_##S(T *a, int stride_a, T *b, int stride_b, int n);               \
+    void array_array_div_assign_##S(T *a, int stride_a, T *b, int stride_b, int n);               \
+    /* array_scalar.h:7-44 */                                                                      \
+    void array_scalar_add_##S(T *a, int size, int stride_a, T scalar, T *out, int stride_out);    \
+    void array_scalar_sub_##S(T *a, int size, int stride_a, T scalar, T *out, int stride_out);    \
+    void array_scalar_mul_##S(T *a, int size, int stride_a, T scalar, T *out, int stride_out);    \
+    void array_scalar_div_##S(T *a, int size, int stride_a, T scalar, T *out, int stride_out);    \
+    void array_scalar_add_assign_##S(T *a, int size, int stride, T scalar);                       \
+    void array_scalar_sub_assign_##S(T *a, int size, int stride, T scalar);                       \
+    void array_scalar_mul_assign_##S(T *a, int size, int stride, T scalar);                       \
+    void array_scalar_div_assign_##S(T *a, int size, int stride, T scalar);                       \
+    void array_scalar_pointer_add_##S(T *a, int size, int stride_a, T *scalar, T *out, int stride_out); \
+    void array_scalar_pointer_sub_##S(T *a, int size, int stride_a, T *scalar, T *out, int stride_out); \
+    void array_scalar_pointer_mul_##S(T *a, int size, int stride_a, T *scalar, T *out, int stride_out); \
+    void array_scalar_pointer_div_##S(T *a, int size, int stride_a, T *scalar, T *out, int stride_out); \
+    void array_scalar_pointer_add_assign_##S(T *a, int size, int stride, T *scalar);              \
+    void array_scalar_pointer_sub_assign_##S(T *a, int size, int stride, T *scalar);              \
+    void array_scalar_pointer_mul_assign_##S(T *a, int size, int stride, T *scalar);              \
+    void array_scalar_pointer_div_assign_##S(T *a, int size, int stride, T *scalar);              \
+    /* array_scalar.h:46-112 (unary) */                                                            \
+    void array_exp_##S(T *a, int size, int stride_in, T *out, int stride_out);                    \
+    void array_log_##S(T *a, int size, int stride_in, T *out, int stride_out);                    \
+    void array_tanh_##S(T *a, int size, int stride_in, T *out, int stride_out);                   \
+    void array_sqrt_##S(T *a, int size, int stride_in, T *out, int stride_out);                   \
+    void array_abs_##S(T *a, int size, int stride_in, T *out, int stride_out);                    \
+    void array_exp_assign_##S(T *a, int size, int stride);                                        \
+    void array_log_assign_##S(T *a, int size, int stride);                                        \
+    void array_tanh_assign_##S(T *a, int size, int stride);                                       \
+    void array_sqrt_assign_##S(T *a, int size, int stride);                                       \
+    void array_abs_assign_##S(T *a, int size, int stride);                                        \
+    /* activations.h:7-11 */                                                                       \
+    void relu_##S(T *input, T *output, T alpha, int size, int input_stride, int output_stride);   \
+    void relu_backward_mask_##S(T *input, T *mask, T alpha, int size, int input_stride,           \
+                                int mask_stride);                                                  \
+    /* element_wise.h:7-9: `out` is a HOST int (zenu-cuda/src/kernel/mod.rs:570-588); blocking */ \
+    void array_max_idx_##S(T *a, int size, int stride, int *out);                                 \
+    /* memory_access.h:7-11: blocking single-element copies */                                    \
+    void memory_access_##S(T *array, int offset, T *result);                                      \
+    void memory_set_##S(T *array, int offset, T value);
+
+ZENU_DECL_1D(float, float)
+ZENU_DECL_1D(double, double)
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ZENU_HIP_H */

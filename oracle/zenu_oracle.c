@@ -1,0 +1,190 @@
+/*
+ * zenu_oracle.c -- CPU restatement of ZeNu's Cpu device path.
+ * TEST INFRASTRUCTURE ONLY: the checker for the HIP kernels and the CPU baseline of the
+ * benchmark.  See zenu_oracle.h for the reference files each part follows.
+ *
+ * Build: gcc -O2 -fno-fast-math -ffp-contract=off (no FMA fusion, IEEE semantics), one thread.
+ *
+ * Pinning status of each function group (how the restatement is checked without running the
+ * reference, which is Rust and cannot be built in this environment):
+ *   binary / scalar / broadcast / strided ops : reference test vectors
+ *       (basic_operations.rs:649-1335, with_clousers.rs:356-508) + brute-force N-d loops
+ *   unary exp/log/tanh/sqrt/abs/sin..cosh, pow : reference literal tables
+ *       (zenu-cuda/src/kernel/mod.rs:1015-1241, basic_operations.rs:1341-1451) + same libm symbols
+ *   relu / relu_backward_mask : relu.rs:255-296, zenu-cuda/src/kernel/activation.rs:88-147
+ *   sigmoid : zenu-autograd/src/activation/sigmoid.rs:26-66
+ *   sum / sum_to : sum.rs:109-245 + f64 brute force
+ *   max_idx / max_axis / max_axis_idx_ravel : max.rs:157-844 + brute force incl. ties / NaN
+ *   copy_from : copy_from.rs:285-398, to_default_stride.rs:28-89
+ *   SGD / Adam / AdamW : zenu-optimizer/tests/net_test.rs:107-232 (via a tiny Linear+MSE net
+ *       restated in the test) + closed-form invariants
+ *   asum : asum.rs:78-120 for small exact integers; accumulation order of OpenBLAS
+ *       s/dasum is PARITY UNPINNED (compared with a tolerance)
+ */
+#include "zenu_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+static uint64_t g_leaf_calls = 0;
+
+uint64_t zo_leaf_calls(void) { return g_leaf_calls; }
+void zo_reset_leaf_calls(void) { g_leaf_calls = 0; }
+
+/* dim/mod.rs:70-92 */
+void zo_default_stride(int ndim, const int64_t *shape, int64_t *stride)
+{
+    if (ndim == 0) return;
+    stride[ndim - 1] = 1;
+    for (int i = ndim - 2; i >= 0; i--) stride[i] = stride[i + 1] * shape[i + 1];
+}
+
+static int64_t zo_num_elm(const zo_view *v)
+{
+    int64_t n = 1;
+    for (int i = 0; i < v->ndim; i++) n *= v->shape[i];
+    return n;
+}
+
+/* dim/mod.rs:40-42 */
+static int zo_is_scalar(const zo_view *v) { return v->ndim == 0 || zo_num_elm(v) == 1; }
+
+static int64_t zo_last_stride(const zo_view *v) { return v->ndim ? v->stride[v->ndim - 1] : 1; }
+
+static int zo_is_strict_default_stride(const zo_view *v)
+{
+    int64_t d[ZO_MAX_DIM];
+    zo_default_stride(v->ndim, v->shape, d);
+    for (int i = 0; i < v->ndim; i++)
+        if (d[i] != v->stride[i]) return 0;
+    return 1;
+}
+
+/* shape_stride.rs:116-121: every 1-D view counts as default stride whatever its stride */
+int zo_is_default_stride(const zo_view *v)
+{
+    if (v->ndim == 1) return 1;
+    return zo_is_strict_default_stride(v);
+}
+
+/* shape_stride.rs:65-83 */
+int zo_is_contiguous(const zo_view *v)
+{
+    int nd = v->ndim;
+    if (nd == 0) return 1;
+    int order[ZO_MAX_DIM];
+    for (int i = 0; i < nd; i++) order[i] = i;
+    /* stable sort by stride, descending */
+    for (int i = 1; i < nd; i++) {
+        int o = order[i], j = i - 1;
+        while (j >= 0 && v->stride[order[j]] < v->stride[o]) { order[j + 1] = order[j]; j--; }
+        order[j + 1] = o;
+    }
+    int64_t sshape[ZO_MAX_DIM], sstride[ZO_MAX_DIM], d[ZO_MAX_DIM];
+    for (int i = 0; i < nd; i++) { sshape[i] = v->shape[order[i]]; sstride[i] = v->stride[order[i]]; }
+    zo_default_stride(nd, sshape, d);
+    if (sstride[0] == 0) return 0; /* the reference divides by zero here */
+    int64_t n = d[0] / sstride[0];
+    if (d[0] % sstride[0] != 0) return 0;
+    for (int i = 0; i < nd; i++)
+        if (d[i] * n != sstride[i]) return 0;
+    return 1;
+}
+
+static int zo_dims_equal(int na, const int64_t *a, int nb, const int64_t *b)
+{
+    if (na != nb) return 0;
+    for (int i = 0; i < na; i++)
+        if (a[i] != b[i]) return 0;
+    return 1;
+}
+
+static int zo_same_shape(const zo_view *a, const zo_view *b)
+{
+    return zo_dims_equal(a->ndim, a->shape, b->ndim, b->shape);
+}
+
+/* dim_dyn.rs:119-130 */
+static int zo_dim_is_include(int ns, const int64_t *s, int no, const int64_t *o)
+{
+    if (ns < no) return zo_dim_is_include(no, o, ns, s);
+    for (int i = 0; i < no; i++)
+        if (s[ns - 1 - i] != o[no - 1 - i]) return 0;
+    return 1;
+}
+
+/* dim_dyn.rs:137-148 (the caller guarantees ns >= no; the reference asserts it) */
+static int zo_dim_is_include_broadcast(int ns, const int64_t *s, int no, const int64_t *o)
+{
+    if (ns < no) return 0;
+    for (int i = 0; i < no; i++) {
+        if (s[ns - 1 - i] == o[no - 1 - i] || o[no - 1 - i] == 1) continue;
+        return 0;
+    }
+    return 1;
+}
+
+/* dim_dyn.rs:24-47 */
+int zo_larger_shape(int nx, const int64_t *x, int ny, const int64_t *y)
+{
+    if (nx < ny) return zo_dim_is_include(ny, y, nx, x) ? 1 : -ZO_ERR_SHAPE;
+    if (nx > ny) return zo_dim_is_include(nx, x, ny, y) ? 0 : -ZO_ERR_SHAPE;
+    if (zo_dim_is_include_broadcast(nx, x, ny, y)) return 0;
+    if (zo_dim_is_include_broadcast(ny, y, nx, x)) return 1;
+    return -ZO_ERR_SHAPE;
+}
+
+/* ---- float instance ---- */
+#define T float
+#define S f32
+#define ZO_EXP_FN expf
+#define ZO_LOG_FN logf
+#define ZO_TANH_FN tanhf
+#define ZO_SQRT_FN sqrtf
+#define ZO_FABS_FN fabsf
+#define ZO_SIN_FN sinf
+#define ZO_COS_FN cosf
+#define ZO_TAN_FN tanf
+#define ZO_ASIN_FN asinf
+#define ZO_ACOS_FN acosf
+#define ZO_ATAN_FN atanf
+#define ZO_SINH_FN sinhf
+#define ZO_COSH_FN coshf
+#define ZO_POW_FN powf
+#include "zenu_oracle_impl.inc"
+#undef T
+#undef S
+#undef ZO_EXP_FN
+#undef ZO_LOG_FN
+#undef ZO_TANH_FN
+#undef ZO_SQRT_FN
+#undef ZO_FABS_FN
+#undef ZO_SIN_FN
+#undef ZO_COS_FN
+#undef ZO_TAN_FN
+#undef ZO_ASIN_FN
+#undef ZO_ACOS_FN
+#undef ZO_ATAN_FN
+#undef ZO_SINH_FN
+#undef ZO_COSH_FN
+#undef ZO_POW_FN
+
+/* ---- double instance ---- */
+#define T double
+#define S f64
+#define ZO_EXP_FN exp
+#define ZO_LOG_FN log
+#define ZO_TANH_FN tanh
+#define ZO_SQRT_FN sqrt
+#define ZO_FABS_FN fabs
+#define ZO_SIN_FN sin
+#define ZO_COS_FN cos
+#define ZO_TAN_FN tan
+#define ZO_ASIN_FN asin
+#define ZO_ACOS_FN acos
+#define ZO_ATAN_FN atan
+#define ZO_SINH_FN sinh
+#define ZO_COSH_FN cosh
+#define ZO_POW_FN pow
+#include "zenu_oracle_impl.inc"

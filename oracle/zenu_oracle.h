@@ -1,0 +1,135 @@
+/*
+ * zenu_oracle.h -- CPU restatement of ZeNu's Cpu device path (TEST INFRASTRUCTURE ONLY).
+ *
+ * This library is the checker for the HIP kernels: tests, the smoke check and the
+ * cpu_baseline leg of the benchmark may link or load it.  Nothing in the product
+ * (the HIP library or the host layer above it) may call into it.
+ *
+ * It restates, single-threaded and in the reference's evaluation order, the
+ * algorithms of the reference's CPU path:
+ *   - the 1-D strided leaf loops of the device traits
+ *       zenu-matrix/src/operation/basic_operations.rs:91-182,397-421
+ *       zenu-matrix/src/operation/relu.rs:31-91
+ *       zenu-matrix/src/operation/max.rs:19-34
+ *   - the host-side N-d -> 1-D decomposition (one leaf call per row / slice)
+ *       zenu-matrix/src/with_clousers.rs:9-242
+ *       zenu-matrix/src/operation/basic_operations.rs:278-381,512-575
+ *       zenu-matrix/src/operation/relu.rs:169-242
+ *   - sum / sum_to               zenu-matrix/src/operation/sum.rs:9-94
+ *   - max_idx / max_axis / max_axis_idx_ravel
+ *                                zenu-matrix/src/operation/max.rs:43-135
+ *   - asum (plain loop; the reference calls OpenBLAS sasum/dasum whose
+ *     accumulation order is not specified -> "parity unpinned", compared with
+ *     a tolerance)               zenu-matrix/src/operation/asum.rs:49-68
+ *   - copy_from / to_default_stride
+ *                                zenu-matrix/src/operation/copy_from.rs:211-267
+ *   - sigmoid composite          zenu-autograd/src/activation/sigmoid.rs:7-15
+ *   - SGD / Adam / AdamW         zenu-optimizer/src/{sgd.rs:20-31,adam.rs:19-59,adamw.rs:20-70}
+ *
+ * exp/log/tanh/pow call the host libm (expf/logf/tanhf/powf, exp/log/tanh/pow):
+ * the same symbols Rust's f32::exp/ln/tanh/powf lower to.
+ *
+ * Every entry exists for float (suffix _f32) and double (suffix _f64).
+ * Strides are in ELEMENTS.  A view's ptr already includes its offset.
+ * Functions returning int return 0 on success and a ZO_ERR_* code where the
+ * reference would panic (shape / rank / axis errors).
+ */
+#ifndef ZENU_ORACLE_H
+#define ZENU_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ZO_MAX_DIM 6
+
+typedef struct zo_view {
+    void   *ptr;                 /* base pointer + offset, element type given by the suffix */
+    int32_t ndim;                /* 0..6 (0 = scalar) */
+    int32_t reserved;
+    int64_t shape[ZO_MAX_DIM];
+    int64_t stride[ZO_MAX_DIM];  /* in elements */
+} zo_view;
+
+enum { ZO_OK = 0, ZO_ERR_RANK = 1, ZO_ERR_SHAPE = 2, ZO_ERR_AXIS = 3, ZO_ERR_ARG = 4 };
+enum { ZO_ADD = 0, ZO_SUB = 1, ZO_MUL = 2, ZO_DIV = 3 };
+enum {
+    ZO_EXP = 0, ZO_LOG = 1, ZO_TANH = 2, ZO_SQRT = 3, ZO_ABS = 4,
+    ZO_SIN = 5, ZO_COS = 6, ZO_TAN = 7, ZO_ASIN = 8, ZO_ACOS = 9, ZO_ATAN = 10,
+    ZO_SINH = 11, ZO_COSH = 12
+};
+
+/* number of leaf (device-trait) calls issued since the last reset: mirrors the
+ * call-counting tests of zenu-matrix/src/with_clousers.rs:356-379 */
+uint64_t zo_leaf_calls(void);
+void     zo_reset_leaf_calls(void);
+
+/* shape helpers shared by both dtypes */
+void zo_default_stride(int ndim, const int64_t *shape, int64_t *stride);
+int  zo_is_default_stride(const zo_view *v);
+int  zo_is_contiguous(const zo_view *v);
+/* larger_shape (dim_dyn.rs:24-58): writes the broadcast result shape; returns
+ * 0 if x is the larger, 1 if y is, <0 (-ZO_ERR_SHAPE) where the reference panics */
+int  zo_larger_shape(int nx, const int64_t *x, int ny, const int64_t *y);
+
+#define ZO_DECLARE(T, S)                                                                           \
+    /* ---- device-trait leaves (1-D strided loops) ---- */                                        \
+    void zo_array_array_##S(int op, T *to, const T *lhs, const T *rhs, size_t n, size_t st,       \
+                            size_t sl, size_t sr);                                                 \
+    void zo_array_assign_##S(int op, T *to, const T *rhs, size_t n, size_t st, size_t sr);        \
+    void zo_scalar_##S(int op, T *to, const T *lhs, T rhs, size_t n, size_t st, size_t sl);       \
+    void zo_scalar_assign_##S(int op, T *to, T rhs, size_t n, size_t st);                         \
+    void zo_scalar_ptr_##S(int op, T *to, const T *lhs, const T *scalar, size_t st, size_t sl,    \
+                           size_t n);                                                              \
+    void zo_scalar_assign_ptr_##S(int op, T *to, const T *scalar, size_t n, size_t st);           \
+    void zo_unary_leaf_##S(int fn, T *to, const T *other, size_t n, size_t st, size_t so);        \
+    void zo_unary_assign_leaf_##S(int fn, T *to, size_t n, size_t st);                            \
+    void zo_pow_leaf_##S(T *to, const T *other, T scalar, size_t n, size_t st, size_t so);        \
+    void zo_relu_leaf_##S(const T *input, T *output, T alpha, size_t n, size_t si, size_t so);    \
+    void zo_relu_backward_mask_leaf_##S(const T *input, T *mask, T alpha, size_t n, size_t si,    \
+                                        size_t sm);                                                \
+    size_t zo_max_idx_leaf_##S(const T *input, size_t size, size_t stride);                       \
+    T    zo_asum_leaf_##S(size_t n, const T *x, size_t incx);                                     \
+    /* ---- Matrix-level ops (reference-shaped decomposition) ---- */                              \
+    int zo_binary_array_##S(int op, const zo_view *to, const zo_view *lhs, const zo_view *rhs);   \
+    int zo_binary_assign_##S(int op, const zo_view *to, const zo_view *rhs);                      \
+    int zo_binary_scalar_##S(int op, const zo_view *to, const zo_view *other, T scalar);          \
+    int zo_binary_scalar_assign_##S(int op, const zo_view *to, T scalar);                         \
+    int zo_unary_##S(int fn, const zo_view *to, const zo_view *other);                            \
+    int zo_unary_assign_##S(int fn, const zo_view *to);                                           \
+    int zo_powf_##S(const zo_view *to, const zo_view *other, T scalar);                           \
+    int zo_relu_##S(const zo_view *to, const zo_view *other, T alpha);                            \
+    int zo_relu_backward_mask_##S(const zo_view *to, const zo_view *other, T alpha);              \
+    int zo_sigmoid_##S(const zo_view *to, const zo_view *x);                                      \
+    int zo_copy_from_##S(const zo_view *to, const zo_view *src);                                  \
+    /* out: caller-allocated default-stride buffer with shape = src.shape minus axis */           \
+    int zo_sum_##S(const zo_view *src, int axis, T *out);                                         \
+    int zo_sum_to_##S(const zo_view *src, const zo_view *target);                                 \
+    /* idx_out: N-d index (src.ndim entries) of the first maximum in row-major order */           \
+    int zo_max_idx_##S(const zo_view *src, int64_t *idx_out);                                     \
+    int zo_max_item_##S(const zo_view *src, T *out);                                              \
+    int zo_max_axis_##S(const zo_view *src, int axis, T *out);                                    \
+    int zo_max_axis_idx_ravel_##S(const zo_view *src, int axis, int64_t *out);                    \
+    T   zo_asum_##S(const zo_view *src);                                                          \
+    /* ---- optimizers on one parameter tensor (flat, n elements) ---- */                          \
+    void zo_sgd_update_##S(T *p, const T *g, size_t n, T lr);                                     \
+    /* step = value of the step counter AFTER the increment (adam.rs:21-22) */                    \
+    void zo_adam_update_##S(T *p, const T *g, T *m, T *v, size_t n, T lr, T beta1, T beta2,       \
+                            T eps, T step);                                                        \
+    void zo_adamw_update_##S(T *p, const T *g, T *m, T *v, size_t n, T lr, T beta1, T beta2,      \
+                             T eps, T weight_decay, int is_weight, T step);                        \
+    /* fused single-pass loops with identical per-element arithmetic (plain-loop CPU figure) */   \
+    void zo_adam_update_fused_##S(T *p, const T *g, T *m, T *v, size_t n, T lr, T beta1,          \
+                                  T beta2, T eps, T weight_decay, int is_weight, int adamw,       \
+                                  T step);
+
+ZO_DECLARE(float, f32)
+ZO_DECLARE(double, f64)
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ZENU_ORACLE_H */

@@ -1,0 +1,169 @@
+"""CpuMatrix: the oracle behind the same method names as zenu_amd.Matrix.
+
+This is the `Cpu` leg of the reference's run_mat_test! pattern (zenu-test/src/lib.rs:62-91): one
+generic test body, instantiated once with the CPU oracle and once with the HIP device.
+"""
+import numpy as np
+
+import zenu_oracle as zo
+
+
+class CpuMatrix:
+    Error = zo.OracleError
+
+    def __init__(self, arr):
+        self.a = arr  # a numpy view; strides carry the Matrix view
+
+    # constructors
+    @staticmethod
+    def alloc(shape, dtype=np.float32):
+        return CpuMatrix(np.empty(tuple(shape), dtype=dtype))
+
+    @staticmethod
+    def zeros(shape, dtype=np.float32):
+        return CpuMatrix(np.zeros(tuple(shape), dtype=dtype))
+
+    @staticmethod
+    def from_numpy(arr):
+        return CpuMatrix(np.array(arr, copy=True, order="C"))
+
+    @staticmethod
+    def from_vec(vec, shape, dtype=np.float32):
+        return CpuMatrix(np.asarray(vec, dtype=dtype).reshape(tuple(shape)).copy())
+
+    def alloc_like(self):
+        return CpuMatrix.alloc(self.a.shape, self.a.dtype)
+
+    @property
+    def shape(self):
+        return tuple(self.a.shape)
+
+    @property
+    def dtype(self):
+        return self.a.dtype
+
+    @property
+    def ndim(self):
+        return self.a.ndim
+
+    def to_numpy(self):
+        return np.array(self.a, copy=True, order="C")
+
+    def index_item(self, index):
+        return self.a[tuple(index)]
+
+    # views
+    def index_axis(self, axis, index):
+        return CpuMatrix(self.a[(slice(None),) * axis + (index,)])
+
+    def slice(self, *slices):
+        return CpuMatrix(self.a[tuple(slices)])
+
+    def transpose(self):
+        return CpuMatrix(np.swapaxes(self.a, -1, -2))
+
+    def transpose_by_index(self, index):
+        return CpuMatrix(np.transpose(self.a, index))
+
+    def add_axis(self, axis):
+        return CpuMatrix(np.expand_dims(self.a, axis))
+
+    def reshape(self, new_shape):
+        assert self.a.flags["C_CONTIGUOUS"]
+        return CpuMatrix(self.a.reshape(tuple(new_shape)))
+
+    # copies
+    def copy_from(self, src):
+        zo.copy_from(self.a, src.a)
+
+    def to_default_stride(self):
+        out = self.alloc_like()
+        out.copy_from(self)
+        return out
+
+    # operators (impl_ops.rs)
+    def _operator(self, op, rhs):
+        if isinstance(rhs, CpuMatrix):
+            from zenu_amd.matrix import larger_shape  # pure shape arithmetic, no device call
+            out = CpuMatrix.alloc(larger_shape(self.shape, rhs.shape), self.dtype)
+            zo.binary_array(op, out.a, self.a, rhs.a)
+            return out
+        out = self.alloc_like()
+        zo.binary_scalar(op, out.a, self.a, rhs)
+        return out
+
+    def _ioperator(self, op, rhs):
+        if isinstance(rhs, CpuMatrix):
+            zo.binary_assign(op, self.a, rhs.a)
+        else:
+            zo.binary_scalar_assign(op, self.a, rhs)
+        return self
+
+    def __add__(self, r): return self._operator(zo.ADD, r)
+    def __sub__(self, r): return self._operator(zo.SUB, r)
+    def __mul__(self, r): return self._operator(zo.MUL, r)
+    def __truediv__(self, r): return self._operator(zo.DIV, r)
+    def __iadd__(self, r): return self._ioperator(zo.ADD, r)
+    def __isub__(self, r): return self._ioperator(zo.SUB, r)
+    def __imul__(self, r): return self._ioperator(zo.MUL, r)
+    def __itruediv__(self, r): return self._ioperator(zo.DIV, r)
+
+    def powf(self, other, scalar): zo.powf(self.a, other.a, scalar)
+
+    def powf_array(self, scalar):
+        out = self.alloc_like()
+        out.powf(self, scalar)
+        return out
+
+    def sigmoid(self):
+        out = self.alloc_like()
+        zo.sigmoid(out.a, self.a)
+        return out
+
+    def relu(self, other, alpha): zo.relu(self.a, other.a, alpha)
+    def relu_backward_mask(self, other, alpha): zo.relu_backward_mask(self.a, other.a, alpha)
+
+    # reductions
+    def sum(self, axis, keep_dim=False): return CpuMatrix(zo.sum_axis(self.a, axis, keep_dim))
+
+    def sum_all(self):
+        out = CpuMatrix.zeros((), self.dtype)
+        zo.sum_to(self.a, out.a)
+        return out
+
+    def max_idx(self): return zo.max_idx(self.a)
+    def max_item(self): return zo.max_item(self.a)
+    def max_axis(self, axis, keep_dim=False): return CpuMatrix(zo.max_axis(self.a, axis, keep_dim))
+    def max_axis_idx_ravel(self, axis): return [int(i) for i in zo.max_axis_idx_ravel(self.a, axis)]
+    def asum(self): return zo.asum(self.a)
+
+
+def _named(name, op):
+    setattr(CpuMatrix, f"{name}_array", lambda self, l, r: zo.binary_array(op, self.a, l.a, r.a))
+    setattr(CpuMatrix, f"{name}_assign", lambda self, r: zo.binary_assign(op, self.a, r.a))
+    setattr(CpuMatrix, f"{name}_scalar", lambda self, o, s: zo.binary_scalar(op, self.a, o.a, s))
+    setattr(CpuMatrix, f"{name}_scalar_assign", lambda self, s: zo.binary_scalar_assign(op, self.a, s))
+
+
+for _n, _o in (("add", zo.ADD), ("sub", zo.SUB), ("mul", zo.MUL), ("div", zo.DIV)):
+    _named(_n, _o)
+
+
+def _unary(name, fn):
+    def out(self):
+        r = self.alloc_like()
+        zo.unary(fn, r.a, self.a)
+        return r
+    setattr(CpuMatrix, name, out)
+    setattr(CpuMatrix, f"{name}_array", lambda self, o: zo.unary(fn, self.a, o.a))
+    setattr(CpuMatrix, f"{name}_assign", lambda self: zo.unary_assign(fn, self.a))
+
+
+for _n, _f in (("exp", zo.EXP), ("log", zo.LOG), ("tanh", zo.TANH), ("sqrt", zo.SQRT), ("abs", zo.ABS),
+               ("sin", zo.SIN), ("cos", zo.COS), ("tan", zo.TAN), ("asin", zo.ASIN), ("acos", zo.ACOS),
+               ("atan", zo.ATAN), ("sinh", zo.SINH), ("cosh", zo.COSH)):
+    _unary(_n, _f)
+
+
+def sum_to(source, target):
+    zo.sum_to(source.a, target.a)

@@ -1,0 +1,651 @@
+"""Parity of the HIP kernels with the CPU oracle on identical seeded inputs, at the BASELINE
+configurations (full size) and on edge cases.  Everything goes through the C ABI.
+
+Bars (written where they are used):
+  add/sub/mul/div, relu, max, arg-max, copy, SGD/Adam/AdamW .......... bit-exact
+  exp/log (device math library) ....................................... <= 2 ulp
+  tanh, sigmoid (f32: same algorithm as the host libm) ................. bit-exact (bar: <= 2 ulp)
+  sums ................................................................ |gpu - cpu| <= 1e-5 (f32) /
+      1e-12 (f64) times max(|cpu|, sum|x| / sqrt(n)); the second term is the typical magnitude
+      of a sum of n such terms, so a result that cancels to ~0 is not held to a relative bar
+      the sequential CPU sum itself cannot meet.
+"""
+import numpy as np
+import pytest
+
+import zenu_oracle as zo
+
+pytestmark = pytest.mark.gpu
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def ordered(a):
+    """Map floats to integers so that the integer difference is the distance in ulps."""
+    if a.dtype == np.float32:
+        i = a.view(np.int32).astype(np.int64)
+        return np.where(i < 0, np.int64(-2**31) - i, i)
+    i = a.view(np.int64)
+    return np.where(i < 0, np.int64(-2**63) - i, i)
+
+
+def max_ulp(a, b):
+    nan_a, nan_b = np.isnan(a), np.isnan(b)
+    assert np.array_equal(nan_a, nan_b)
+    ok = ~nan_a
+    if not ok.any():
+        return 0
+    return int(np.max(np.abs(ordered(a[ok]) - ordered(b[ok]))))
+
+
+def bits_equal(a, b):
+    return a.shape == b.shape and np.array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
+def assert_bits(got, exp, what):
+    if not bits_equal(got, exp):
+        bad = np.flatnonzero(got.reshape(-1).view(f"u{got.itemsize}") != exp.reshape(-1).view(f"u{exp.itemsize}"))
+        raise AssertionError(f"{what}: {bad.size} of {got.size} elements differ, first at {bad[0]}: "
+                             f"got {got.reshape(-1)[bad[0]]!r} exp {exp.reshape(-1)[bad[0]]!r}")
+
+
+def sum_tol(dtype):
+    return 1e-5 if np.dtype(dtype) == np.float32 else 1e-12
+
+
+def assert_sum_close(got, cpu, x, axis, what):
+    n = x.size if axis is None else x.shape[axis]
+    scale = np.abs(x.astype(np.float64)).sum(axis=axis) / np.sqrt(n)
+    denom = np.maximum(np.abs(cpu.astype(np.float64)), scale)
+    err = np.abs(got.astype(np.float64) - cpu.astype(np.float64)) / denom
+    assert err.max() <= sum_tol(x.dtype), f"{what}: rel err {err.max():.3e}"
+    exact = x.astype(np.float64).sum(axis=axis)
+    err64 = np.abs(got.astype(np.float64) - exact) / np.maximum(np.abs(exact), scale)
+    assert err64.max() <= sum_tol(x.dtype), f"{what}: rel err vs f64 sum {err64.max():.3e}"
+
+
+# ---- config[0]: contiguous f32 [2^24], uniform[-1,1), seed 0 -------------------------------------------
+
+@pytest.mark.parametrize("n", [1, 3, 1023, 4096, 4097, 1 << 20, (1 << 24)])
+def test_c0_contiguous(hip, n):
+    print(f"[c0] n={n}", flush=True)
+    r = rng(0)
+    a = r.uniform(-1, 1, n).astype(np.float32)
+    b = r.uniform(-1, 1, n).astype(np.float32)
+    A, B = hip.Matrix.from_numpy(a), hip.Matrix.from_numpy(b)
+    for name, op in (("add", zo.ADD), ("mul", zo.MUL), ("sub", zo.SUB), ("div", zo.DIV)):
+        exp = np.empty_like(a)
+        zo.binary_array(op, exp, a, b)
+        out = hip.Matrix.alloc([n])
+        getattr(out, f"{name}_array")(A, B)
+        assert_bits(out.to_numpy(), exp, f"{name} n={n}")          # bit-exact
+    exp = np.empty_like(a)
+    zo.relu(exp, a, 0.0)
+    out = hip.Matrix.alloc([n])
+    out.relu(A, 0.0)
+    assert_bits(out.to_numpy(), exp, f"relu n={n}")                # bit-exact incl. -0.0
+    zo.relu_backward_mask(exp, a, 0.0)
+    out.relu_backward_mask(A, 0.0)
+    assert_bits(out.to_numpy(), exp, f"relu_mask n={n}")
+
+
+def test_relu_edge_values(hip):
+    x = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 3e38], dtype=np.float32)
+    for alpha in (0.0, 0.2, -1.5):
+        exp = np.empty_like(x)
+        zo.relu(exp, x, alpha)
+        out = hip.Matrix.alloc(x.shape)
+        out.relu(hip.Matrix.from_numpy(x), alpha)
+        got = out.to_numpy()
+        nan = np.isnan(exp)
+        assert np.array_equal(np.isnan(got), nan)
+        assert_bits(got[~nan], exp[~nan], f"relu alpha={alpha}")
+        zo.relu_backward_mask(exp, x, alpha)
+        out.relu_backward_mask(hip.Matrix.from_numpy(x), alpha)
+        assert_bits(out.to_numpy(), exp, f"relu mask alpha={alpha}")
+
+
+def test_unaligned_and_inplace(hip):
+    """views whose base is not 16-byte aligned, and the *_assign forms (exact aliasing)"""
+    r = rng(10)
+    a = r.standard_normal(10007).astype(np.float32)
+    b = r.standard_normal(10007).astype(np.float32)
+    A, B = hip.Matrix.from_numpy(a), hip.Matrix.from_numpy(b)
+    out = hip.Matrix.zeros([10007])
+    out.slice(slice(1, None)).add_array(A.slice(slice(1, None)), B.slice(slice(0, 10006)))
+    exp = np.zeros_like(a)
+    zo.binary_array(zo.ADD, exp[1:], a[1:], b[:10006])
+    assert_bits(out.to_numpy(), exp, "unaligned add")
+    A.mul_assign(B)
+    zo.binary_assign(zo.MUL, a, b)
+    assert_bits(A.to_numpy(), a, "mul_assign")
+    A.div_scalar_assign(3.0)
+    zo.binary_scalar_assign(zo.DIV, a, 3.0)
+    assert_bits(A.to_numpy(), a, "div_scalar_assign")
+    A.exp_assign()
+    zo.unary_assign(zo.EXP, a)
+    assert max_ulp(A.to_numpy(), a) <= 2
+
+
+# ---- config[1]: [4096,4096] f32, normal(0,1), seed 1 ----------------------------------------------------
+
+@pytest.fixture(scope="module")
+def c1(hip):
+    r = rng(1)
+    a = r.standard_normal((4096, 4096)).astype(np.float32)
+    b = r.standard_normal((4096, 4096)).astype(np.float32)
+    row = r.standard_normal((1, 4096)).astype(np.float32)
+    return dict(a=a, b=b, row=row, A=hip.Matrix.from_numpy(a), B=hip.Matrix.from_numpy(b),
+                ROW=hip.Matrix.from_numpy(row))
+
+
+def test_c1_row_broadcast(hip, c1):
+    exp = np.empty_like(c1["a"])
+    zo.binary_array(zo.ADD, exp, c1["a"], c1["row"])      # 4096 leaf calls in the reference
+    out = hip.Matrix.alloc([4096, 4096])
+    out.add_array(c1["A"], c1["ROW"])                     # one launch
+    assert_bits(out.to_numpy(), exp, "a + b[1,4096]")
+    out2 = c1["A"] + c1["ROW"]
+    assert_bits(out2.to_numpy(), exp, "operator +")
+
+
+def test_c1_transposed(hip, c1):
+    exp = np.empty_like(c1["a"])
+    zo.binary_array(zo.ADD, exp, c1["a"], c1["b"].T)
+    out = hip.Matrix.alloc([4096, 4096])
+    out.add_array(c1["A"], c1["B"].transpose())
+    assert_bits(out.to_numpy(), exp, "a + b^T")
+    zo.binary_array(zo.SUB, exp, c1["b"].T, c1["a"])      # transposed operand on the left
+    out.sub_array(c1["B"].transpose(), c1["A"])
+    assert_bits(out.to_numpy(), exp, "b^T - a")
+
+
+def test_c1_scalar(hip, c1):
+    exp = np.empty_like(c1["a"])
+    zo.binary_scalar(zo.MUL, exp, c1["a"], 0.5)
+    assert_bits((c1["A"] * 0.5).to_numpy(), exp, "a * 0.5")
+    half = hip.Matrix.from_vec([0.5], [])                 # 0-d device operand: scalar_ptr path
+    out = hip.Matrix.alloc([4096, 4096])
+    out.mul_array(c1["A"], half)
+    assert_bits(out.to_numpy(), exp, "a * Variable(0.5)")
+    out.scalar_ptr(zo.MUL, c1["A"], half)
+    assert_bits(out.to_numpy(), exp, "scalar_ptr")
+
+
+@pytest.mark.parametrize("name,fn,bar", [("exp", zo.EXP, 2), ("tanh", zo.TANH, 0), ("log", zo.LOG, 2),
+                                         ("sqrt", zo.SQRT, 0), ("abs", zo.ABS, 0)])
+def test_c1_unary(hip, c1, name, fn, bar):
+    x = np.abs(c1["a"]) + np.float32(1e-3) if name in ("log", "sqrt") else c1["a"]
+    X = hip.Matrix.from_numpy(x)
+    exp = np.empty_like(x)
+    zo.unary(fn, exp, x)                                  # 4096 leaf calls in the reference
+    got = getattr(X, name)().to_numpy()                   # one launch
+    u = max_ulp(got, exp)
+    print(f"[c1] {name}: max ulp vs libm = {u}", flush=True)
+    assert u <= bar, f"{name}: {u} ulp"                   # <= 2 ulp (0 = bit-exact where attainable)
+
+
+def test_c1_sigmoid(hip, c1):
+    exp = np.empty_like(c1["a"])
+    zo.sigmoid(exp, c1["a"])                              # mul, tanh, mul, add on the CPU
+    got = c1["A"].sigmoid().to_numpy()                    # fused
+    u = max_ulp(got, exp)
+    print(f"[c1] sigmoid: max ulp = {u}", flush=True)
+    assert u <= 2                                          # bar <= 2 ulp; f32 is bit-exact
+    assert u == 0
+
+
+def test_transcendental_special_values(hip):
+    x = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-30, -1e-30, 1e-45, 88.7, 88.8, -87.4, -103.9, -104.0,
+                  21.9, 22.0, -22.5, 0.99999994, 1.0, 1.0000001, 0.346, 0.347, 1.039, 1.04, 9.01, 9.011,
+                  3e38, -3e38, 1.1754944e-38, 5e-39], dtype=np.float32)
+    X = hip.Matrix.from_numpy(x)
+    for name, fn in (("exp", zo.EXP), ("tanh", zo.TANH), ("log", zo.LOG), ("sqrt", zo.SQRT)):
+        exp = np.empty_like(x)
+        with np.errstate(all="ignore"):
+            zo.unary(fn, exp, x)
+        got = getattr(X, name)().to_numpy()
+        assert np.array_equal(np.isnan(got), np.isnan(exp)), name
+        assert max_ulp(got, exp) <= 2, (name, got, exp)
+    exp = np.empty_like(x)
+    zo.sigmoid(exp, x)
+    assert max_ulp(X.sigmoid().to_numpy(), exp) == 0
+
+
+def test_tanh_sigmoid_dense_sweep(hip):
+    """every 64th f32 bit pattern: tanh and sigmoid are the host libm's bits"""
+    bits = np.arange(0, 1 << 32, 64, dtype=np.uint64).astype(np.uint32)
+    x = bits.view(np.float32)
+    X = hip.Matrix.from_numpy(x)
+    exp = np.empty_like(x)
+    with np.errstate(all="ignore"):
+        zo.unary(zo.TANH, exp, x)
+    assert max_ulp(X.tanh().to_numpy(), exp) == 0
+    with np.errstate(all="ignore"):
+        zo.sigmoid(exp, x)
+    assert max_ulp(X.sigmoid().to_numpy(), exp) == 0
+    fin = np.isfinite(x)
+    with np.errstate(all="ignore"):
+        zo.unary(zo.EXP, exp, x)
+    got = X.exp().to_numpy()
+    assert max_ulp(got[fin], exp[fin]) <= 2
+    pos = fin & (x > 0)
+    with np.errstate(all="ignore"):
+        zo.unary(zo.LOG, exp, x)
+    got = X.log().to_numpy()
+    assert max_ulp(got[pos], exp[pos]) <= 2
+
+
+def test_unary_f64(hip):
+    r = rng(11)
+    x = r.standard_normal((257, 129))
+    X = hip.Matrix.from_numpy(x)
+    for name, fn, bar in (("exp", zo.EXP, 2), ("tanh", zo.TANH, 4), ("sqrt", zo.SQRT, 0), ("abs", zo.ABS, 0)):
+        xx = np.abs(x) if name == "sqrt" else x
+        exp = np.empty_like(xx)
+        zo.unary(fn, exp, xx)
+        got = getattr(hip.Matrix.from_numpy(xx), name)().to_numpy()
+        u = max_ulp(got, exp)
+        print(f"[f64] {name}: {u} ulp", flush=True)
+        # f64 tanh comes from the device math library: parity unpinned beyond a few ulp
+        assert u <= bar, (name, u)
+    del X
+
+
+# ---- strided / broadcast engine: randomized shapes vs brute force and oracle ------------------------------
+
+SHAPES = [
+    # (out shape, lhs view builder, rhs view builder) expressed on numpy arrays
+    ((7, 5), lambda r: r((7, 5)), lambda r: r((1, 5))),
+    ((7, 5), lambda r: r((7, 5)), lambda r: r((7, 1))),
+    ((7, 5), lambda r: r((7, 1)), lambda r: r((7, 5))),
+    ((70, 130), lambda r: r((70, 130)), lambda r: r((130, 70)).T),
+    ((64, 64), lambda r: r((64, 64)).T, lambda r: r((64, 64)).T),
+    ((3, 70, 130), lambda r: r((3, 70, 130)), lambda r: np.swapaxes(r((3, 130, 70)), -1, -2)),
+    ((3, 70, 130), lambda r: r((3, 70, 130)), lambda r: r((70, 130))),
+    ((2, 3, 4, 5, 6, 7), lambda r: r((2, 3, 4, 5, 6, 7)), lambda r: r((2, 1, 4, 1, 6, 1))),
+    ((2, 3, 4, 5, 6, 7), lambda r: r((2, 3, 4, 5, 6, 7)), lambda r: r((5, 6, 7))),
+    ((33, 65), lambda r: r((66, 130))[::2, ::2], lambda r: r((33, 65))),
+    ((33, 65), lambda r: r((33, 130))[:, 1::2], lambda r: r((65,))),
+    ((128, 256), lambda r: r((128, 512))[:, :256], lambda r: r((256, 128)).T),
+    ((5, 1, 9), lambda r: r((5, 1, 9)), lambda r: r((5, 1, 1))),
+    ((1,), lambda r: r((1,)), lambda r: r(())),
+    ((), lambda r: r(()), lambda r: r(())),
+    ((300, 4), lambda r: r((300, 4)), lambda r: r((4, 300)).T),
+]
+
+
+def dev_view(hip, base, view):
+    """Upload `base` and return the Matrix view with the geometry of numpy view `view` of base."""
+    m = hip.Matrix.from_numpy(base)
+    off = (view.__array_interface__["data"][0] - base.__array_interface__["data"][0]) // base.itemsize
+    stride = tuple(s // base.itemsize for s in view.strides)
+    return hip.Matrix(m.buf, off, view.shape, stride, base.dtype)
+
+
+def root_of(v):
+    while v.base is not None:
+        v = v.base
+    return v
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("idx", range(len(SHAPES)))
+def test_strided_broadcast_binary(hip, idx, dt):
+    shape, fl, fr = SHAPES[idx]
+    print(f"[strided] case {idx} {shape} {np.dtype(dt).name}", flush=True)
+    r = rng(100 + idx)
+    gen = lambda s: r.standard_normal(s).astype(dt)
+    lhs, rhs = fl(gen), fr(gen)
+    L, R = dev_view(hip, root_of(lhs), lhs), dev_view(hip, root_of(rhs), rhs)
+    for name, op in (("add", zo.ADD), ("sub", zo.SUB), ("mul", zo.MUL), ("div", zo.DIV)):
+        exp = np.empty(shape, dtype=dt)
+        zo.binary_array(op, exp, lhs, rhs)
+        brute = {"add": np.add, "sub": np.subtract, "mul": np.multiply, "div": np.divide}[name](lhs, rhs)
+        assert_bits(exp, np.ascontiguousarray(np.broadcast_to(brute, shape)), "oracle vs brute force")
+        out = hip.Matrix.alloc(shape, dt)
+        getattr(out, f"{name}_array")(L, R)
+        assert_bits(out.to_numpy(), exp, f"{name} case {idx}")
+    # strided destination: write into every other row / the transposed view of a larger buffer
+    if len(shape) == 2:
+        big = np.zeros((shape[1], shape[0] * 2), dtype=dt)
+        dst_np = big[:, ::2].T                              # transposed and strided destination
+        BIG = hip.Matrix.from_numpy(big)
+        dev_view_on(hip, BIG, big, dst_np).add_array(L, R)
+        zo.binary_array(zo.ADD, dst_np, lhs, rhs)
+        assert_bits(BIG.to_numpy(), big, f"strided destination case {idx}")
+
+
+def test_copy_transpose_large(hip):
+    r = rng(12)
+    a = r.standard_normal((1000, 777)).astype(np.float32)
+    A = hip.Matrix.from_numpy(a)
+    assert_bits(A.transpose().to_default_stride().to_numpy(), np.ascontiguousarray(a.T), "transpose copy")
+    dst = hip.Matrix.zeros([777, 1000])
+    dst.transpose().copy_from(A)                           # write through a transposed destination
+    assert_bits(dst.to_numpy(), np.ascontiguousarray(a.T), "copy into transposed")
+
+
+# ---- config[2]: [8192,4096] reductions, normal(0,1), seed 2, ~1% duplicate maxima ---------------------------
+
+def make_c2(dt):
+    r = rng(2)
+    x = r.standard_normal((8192, 4096)).astype(dt)
+    rows = r.choice(8192, size=82, replace=False)
+    for k, row in enumerate(rows):                         # exact duplicates of the row maximum
+        j = int(np.argmax(x[row]))
+        others = [c for c in r.choice(4096, size=3, replace=False) if c != j]
+        if k % 2 == 0:
+            x[row, others[0]] = x[row, j]                   # one duplicate (earlier or later)
+        else:
+            x[row, others[0]] = x[row, j]
+            x[row, others[1]] = x[row, j]                   # two duplicates
+    return x, rows
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_c2_reductions(hip, dt):
+    print(f"[c2] {np.dtype(dt).name}", flush=True)
+    x, tie_rows = make_c2(dt)
+    X = hip.Matrix.from_numpy(x)
+    # sums
+    assert_sum_close(X.sum(0).to_numpy(), zo.sum_axis(x, 0), x, 0, "sum axis 0")
+    assert_sum_close(X.sum(1).to_numpy(), zo.sum_axis(x, 1), x, 1, "sum axis 1")
+    assert X.sum(1, True).shape == (8192, 1)
+    cpu_all = np.zeros((), dtype=dt)
+    zo.sum_to(x, cpu_all)
+    assert_sum_close(X.sum_all().to_numpy(), cpu_all, x, None, "full sum")
+    tgt = hip.Matrix.zeros([], dt)
+    hip.sum_to(X, tgt)
+    assert_sum_close(tgt.to_numpy(), cpu_all, x, None, "sum_to []")
+    # max / arg-max along axis 1: bit-exact, first index wins ties
+    exp_idx = zo.max_axis_idx_ravel(x, 1)
+    brute = np.argmax(x, axis=1)                           # numpy also returns the first maximum
+    assert np.array_equal(exp_idx, brute)
+    got_idx = np.array(X.max_axis_idx_ravel(1))
+    assert np.array_equal(got_idx, exp_idx)
+    for row in tie_rows:                                    # the injected ties really are ties
+        assert (x[row] == x[row].max()).sum() >= 2
+    assert_bits(X.max_axis(1).to_numpy(), zo.max_axis(x, 1), "max axis 1")
+    # axis 0 as well (column reduce with (value, index) pairs)
+    xs = x[:2048]
+    XS = hip.Matrix.from_numpy(xs)
+    assert np.array_equal(np.array(XS.max_axis_idx_ravel(0)), np.argmax(xs, axis=0))
+    assert_bits(XS.max_axis(0).to_numpy(), xs.max(axis=0), "max axis 0")
+    # whole-tensor arg-max
+    assert X.max_idx() == tuple(int(i) for i in np.unravel_index(np.argmax(x), x.shape))
+    assert X.max_item() == x.max()
+
+
+def test_sum_determinism(hip):
+    x = rng(13).standard_normal((8192, 4096)).astype(np.float32)
+    X = hip.Matrix.from_numpy(x)
+    a0, a1, al = X.sum(0).to_numpy(), X.sum(1).to_numpy(), X.sum_all().to_numpy()
+    for _ in range(3):
+        assert_bits(X.sum(0).to_numpy(), a0, "sum axis 0 repeat")
+        assert_bits(X.sum(1).to_numpy(), a1, "sum axis 1 repeat")
+        assert_bits(X.sum_all().to_numpy(), al, "sum all repeat")
+
+
+RED_SHAPES = [(1,), (5,), (1000,), (100000,), (3, 4), (4, 3), (1, 7), (7, 1), (2, 3, 4, 5), (17, 1, 33),
+              (64, 1025), (1025, 64), (3, 1000, 7), (300, 17, 40), (2, 2, 2, 2, 2, 3), (4096, 10), (10, 4096),
+              (256, 10), (9, 100003)]
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("shape", RED_SHAPES, ids=str)
+def test_reduction_shapes(hip, shape, dt):
+    print(f"[red] {shape} {np.dtype(dt).name}", flush=True)
+    r = rng(hash(shape) % 1000)
+    x = r.integers(-8, 9, size=shape).astype(dt)           # small integers: sums are exact, ties common
+    X = hip.Matrix.from_numpy(x)
+    for axis in range(len(shape)):
+        assert_bits(X.sum(axis).to_numpy(), zo.sum_axis(x, axis), f"sum {shape} axis {axis}")
+        assert_bits(X.sum(axis, True).to_numpy(), zo.sum_axis(x, axis, True), f"sum keep {shape} axis {axis}")
+        assert np.array_equal(np.array(X.max_axis_idx_ravel(axis)), zo.max_axis_idx_ravel(x, axis)), (shape, axis)
+        assert_bits(X.max_axis(axis).to_numpy(), zo.max_axis(x, axis), f"max {shape} axis {axis}")
+    assert tuple(X.max_idx()) == tuple(zo.max_idx(x))
+    assert X.asum() == zo.asum(x)
+    y = r.standard_normal(shape).astype(dt)
+    Y = hip.Matrix.from_numpy(y)
+    for axis in range(len(shape)):
+        assert_sum_close(Y.sum(axis).to_numpy(), zo.sum_axis(y, axis), y, axis, f"sum {shape} axis {axis}")
+    a = float(Y.asum())
+    assert abs(a - float(zo.asum(y))) <= sum_tol(dt) * np.abs(y).sum()   # order unpinned: tolerance
+
+
+def test_reduction_strided_views(hip):
+    r = rng(14)
+    x = r.integers(-5, 6, size=(40, 50, 30)).astype(np.float32)
+    views = [x[::2, :, ::3], np.swapaxes(x, 0, 2), x[:, 10:20, :], np.swapaxes(x, 1, 2)[3:, ::2]]
+    for v in views:
+        V = dev_view(hip, x, v)
+        for axis in range(v.ndim):
+            assert_bits(V.sum(axis).to_numpy(), zo.sum_axis(v, axis), "strided sum")
+            assert np.array_equal(np.array(V.max_axis_idx_ravel(axis)), zo.max_axis_idx_ravel(v, axis))
+        assert tuple(V.max_idx()) == tuple(zo.max_idx(v))
+    # strided destination through sum_to
+    t = np.zeros((50, 60), dtype=np.float32)
+    T = hip.Matrix.from_numpy(t)
+    tv = t[:, ::2]
+    hip.sum_to(hip.Matrix.from_numpy(x), dev_view_on(hip, T, t, tv))
+    zo.sum_to(x, tv)
+    assert_bits(T.to_numpy(), t, "sum_to strided target")
+
+
+def dev_view_on(hip, M, base, view):
+    off = (view.__array_interface__["data"][0] - base.__array_interface__["data"][0]) // base.itemsize
+    return hip.Matrix(M.buf, off, view.shape, tuple(s // base.itemsize for s in view.strides), base.dtype)
+
+
+def test_argmax_nan_zero_ties(hip):
+    """strict '>' from element 0 (max.rs:23-31): NaN at 0 is sticky, NaN elsewhere is ignored,
+    +0/-0 compare equal so the first is kept, all-equal rows give 0"""
+    nan, inf = np.nan, np.inf
+    rows = np.array([
+        [nan, 1, 2, 3, 4, 5, 6, 7],
+        [1, nan, 2, 9, nan, 9, 0, 1],
+        [-inf, nan, -inf, nan, -inf, -inf, nan, -inf],
+        [0.0, -0.0, 0.0, -0.0, -1, -2, -3, -4],
+        [-0.0, 0.0, -0.0, 0.0, -1, -2, -3, -4],
+        [5, 5, 5, 5, 5, 5, 5, 5],
+        [nan, inf, inf, 1, 2, 3, 4, 5],
+        [1, 2, inf, inf, 3, nan, 4, 5],
+        [nan] * 8,
+    ], dtype=np.float32)
+    exp_idx = zo.max_axis_idx_ravel(rows, 1)
+    assert list(exp_idx) == [0, 3, 0, 0, 0, 0, 0, 2, 0]
+    X = hip.Matrix.from_numpy(rows)
+    assert X.max_axis_idx_ravel(1) == list(exp_idx)
+    got, exp = X.max_axis(1).to_numpy(), zo.max_axis(rows, 1)
+    assert np.array_equal(np.isnan(got), np.isnan(exp))
+    assert_bits(got[~np.isnan(exp)], exp[~np.isnan(exp)], "max values incl. signed zeros")
+    # long rows so that the tree (DPP + LDS + two-pass) is exercised with the same rules
+    big = np.full((4, 100000), -1.0, dtype=np.float32)
+    big[0, 0] = nan
+    big[1, 77777] = 3.0; big[1, 99999] = 3.0; big[1, 5] = nan
+    big[2, :] = 7.0
+    big[3, 50000] = 0.0; big[3, 50001] = -0.0; big[3, 40000] = -0.0
+    B = hip.Matrix.from_numpy(big)
+    assert B.max_axis_idx_ravel(1) == list(zo.max_axis_idx_ravel(big, 1)) == [0, 77777, 0, 40000]
+    assert np.signbit(B.max_axis(1).to_numpy()[3])
+    T = hip.Matrix.from_numpy(np.ascontiguousarray(big.T))
+    assert T.max_axis_idx_ravel(0) == [0, 77777, 0, 40000]
+
+
+# ---- config[3]: fused Adam / AdamW, 25M f32, seed 3 -------------------------------------------------------------
+
+def adam_inputs(n, dt, seed=3):
+    r = rng(seed)
+    p = (r.standard_normal(n) * 0.02).astype(dt)
+    g = (r.standard_normal(n) * 1e-3).astype(dt)
+    m = (r.standard_normal(n) * 1e-4).astype(dt)
+    v = np.abs(r.standard_normal(n) * 1e-6).astype(dt)
+    return p, g, m, v
+
+
+HP = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.01, step=10)
+
+
+@pytest.mark.parametrize("n,dt", [(25_000_000, np.float32), (1_000_003, np.float32), (1_000_003, np.float64), (5, np.float32)])
+def test_c3_adamw(hip, n, dt):
+    from zenu_amd import _lib
+    from zenu_amd._lib import check
+    print(f"[c3] n={n} {np.dtype(dt).name}", flush=True)
+    p, g, m, v = adam_inputs(n, dt)
+    f = np.dtype(dt).type
+    for adamw in (True, False):
+        P, G, M, V = (hip.Matrix.from_numpy(t) for t in (p, g, m, v))
+        pe, me, ve = p.copy(), m.copy(), v.copy()
+        if adamw:
+            zo.adamw_update(pe, g, me, ve, f(HP["lr"]), f(HP["beta1"]), f(HP["beta2"]), f(HP["eps"]), f(HP["wd"]), True, f(HP["step"]))
+            check(hip.lib().zenu_hip_adamw_step(_lib.F32 if dt == np.float32 else _lib.F64, P.as_ptr(), G.as_ptr(),
+                                                M.as_ptr(), V.as_ptr(), n, float(f(HP["lr"])), float(f(HP["beta1"])),
+                                                float(f(HP["beta2"])), float(f(HP["eps"])), float(f(HP["wd"])), 1,
+                                                float(HP["step"]), None), "adamw")
+        else:
+            zo.adam_update(pe, g, me, ve, f(HP["lr"]), f(HP["beta1"]), f(HP["beta2"]), f(HP["eps"]), f(HP["step"]))
+            check(hip.lib().zenu_hip_adam_step(_lib.F32 if dt == np.float32 else _lib.F64, P.as_ptr(), G.as_ptr(),
+                                               M.as_ptr(), V.as_ptr(), n, float(f(HP["lr"])), float(f(HP["beta1"])),
+                                               float(f(HP["beta2"])), float(f(HP["eps"])), float(HP["step"]), None),
+                  "adam")
+        # bar: rel <= 1e-5 (f32) / 1e-12 (f64); with contraction off the update is bit-exact
+        assert_bits(P.to_numpy(), pe, f"adam{'w' if adamw else ''} p")
+        assert_bits(M.to_numpy(), me, "m")
+        assert_bits(V.to_numpy(), ve, "v")
+        assert_bits(G.to_numpy(), g, "g untouched")
+
+
+def test_sgd(hip):
+    from zenu_amd import _lib
+    from zenu_amd._lib import check
+    for dt in (np.float32, np.float64):
+        p, g, _, _ = adam_inputs(1_000_003, dt, seed=5)
+        P, G = hip.Matrix.from_numpy(p), hip.Matrix.from_numpy(g)
+        zo.sgd_update(p, g, np.dtype(dt).type(0.9))
+        check(hip.lib().zenu_hip_sgd_step(_lib.F32 if dt == np.float32 else _lib.F64, P.as_ptr(), G.as_ptr(), p.size,
+                                          float(np.dtype(dt).type(0.9)), None), "sgd")
+        assert_bits(P.to_numpy(), p, "sgd")
+
+
+def test_optimizer_classes_multi_tensor(hip):
+    """Optimizer::update over a model-like set of tensors: the multi-tensor launch equals the
+    per-tensor launches and the oracle; AdamW decays weights only (adamw.rs:61-65)"""
+    r = rng(6)
+    shapes = {"l1.weight": (512, 784), "l1.bias": (512,), "l2.weight": (512, 512), "l2.bias": (512,),
+              "l3.weight": (10, 512), "l3.bias": (10,), "odd": (3, 7, 11)}
+    host = {k: ((r.standard_normal(s) * 0.05).astype(np.float32), (r.standard_normal(s) * 0.01).astype(np.float32))
+            for k, s in shapes.items()}
+    weights = [k for k in shapes if k.endswith("weight")]
+
+    def device_params():
+        return {k: (hip.Matrix.from_numpy(p), hip.Matrix.from_numpy(g)) for k, (p, g) in host.items()}
+
+    for multi in (True, False):
+        params = device_params()
+        opt = hip.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, params, weights)
+        ref = {k: (p.copy(), np.zeros_like(p), np.zeros_like(p)) for k, (p, _) in host.items()}
+        for step in (1, 2, 3):
+            opt.update(params, multi_tensor=multi)
+            for k, (pe, me, ve) in ref.items():
+                zo.adamw_update(pe.reshape(-1), host[k][1].reshape(-1), me.reshape(-1), ve.reshape(-1),
+                                np.float32(1e-3), np.float32(0.9), np.float32(0.999), np.float32(1e-8),
+                                np.float32(0.01), k in weights, np.float32(step))
+        for k in shapes:
+            assert_bits(params[k][0].to_numpy(), ref[k][0], f"{k} multi={multi}")
+            assert_bits(opt.m[k].to_numpy(), ref[k][1], f"m {k}")
+            assert_bits(opt.v[k].to_numpy(), ref[k][2], f"v {k}")
+
+
+# ---- the reference's own 1-D entry points -----------------------------------------------------------------------
+
+def test_reference_named_entry_points(hip):
+    import ctypes as C
+    l = hip.lib()
+    r = rng(7)
+    n = 1000
+    a = r.standard_normal(3 * n).astype(np.float32)
+    b = r.standard_normal(2 * n).astype(np.float32)
+    A, B, OUT = hip.Matrix.from_numpy(a), hip.Matrix.from_numpy(b), hip.Matrix.zeros([n])
+    vp = C.c_void_p
+    l.array_array_add_float.argtypes = [vp, C.c_int, vp, C.c_int, vp, C.c_int, C.c_int]
+    l.array_array_add_float.restype = None
+    l.array_array_add_float(A.as_ptr(), 3, B.as_ptr(), 2, OUT.as_ptr(), 1, n)      # strides 3, 2, 1
+    exp = np.empty(n, dtype=np.float32)
+    zo.lib().zo_array_array_f32(zo.ADD, vp(exp.ctypes.data), vp(a.ctypes.data), vp(b.ctypes.data),
+                                C.c_size_t(n), C.c_size_t(1), C.c_size_t(3), C.c_size_t(2))
+    hip.synchronize()
+    assert_bits(OUT.to_numpy(), exp, "array_array_add_float")
+    l.array_scalar_mul_float.argtypes = [vp, C.c_int, C.c_int, C.c_float, vp, C.c_int]
+    l.array_scalar_mul_float.restype = None
+    l.array_scalar_mul_float(A.as_ptr(), n, 3, C.c_float(0.5), OUT.as_ptr(), 1)
+    assert_bits(OUT.to_numpy(), a[::3] * np.float32(0.5), "array_scalar_mul_float")
+    l.relu_float.argtypes = [vp, vp, C.c_float, C.c_int, C.c_int, C.c_int]
+    l.relu_float.restype = None
+    l.relu_float(A.as_ptr(), OUT.as_ptr(), C.c_float(0.2), n, 3, 1)
+    exp = np.empty(n, dtype=np.float32)
+    zo.relu(exp, a[::3], 0.2)
+    assert_bits(OUT.to_numpy(), exp, "relu_float")
+    out_idx = C.c_int(-1)
+    l.array_max_idx_float.argtypes = [vp, C.c_int, C.c_int, C.POINTER(C.c_int)]
+    l.array_max_idx_float.restype = None
+    l.array_max_idx_float(A.as_ptr(), n, 3, C.byref(out_idx))
+    assert out_idx.value == int(np.argmax(a[::3]))
+    res = C.c_float()
+    l.memory_access_float.argtypes = [vp, C.c_int, C.POINTER(C.c_float)]
+    l.memory_access_float.restype = None
+    l.memory_access_float(A.as_ptr(), 17, C.byref(res))
+    assert res.value == a[17]
+    l.memory_set_float.argtypes = [vp, C.c_int, C.c_float]
+    l.memory_set_float.restype = None
+    l.memory_set_float(A.as_ptr(), 17, C.c_float(42.5))
+    assert A.to_numpy()[17] == np.float32(42.5)
+
+
+# ---- allocator on the device ------------------------------------------------------------------------------------
+
+def test_allocator_device(hip):
+    import ctypes as C
+    from zenu_amd import _lib
+    l = hip.lib()
+    st = _lib.MempoolStats()
+    hip.synchronize()
+    l.zenu_hip_mempool_trim()
+    l.zenu_hip_mempool_stats(C.byref(st))
+    base_allocs, base_hits = st.n_driver_allocs, st.n_cache_hits
+    ptrs = []
+    for _ in range(3):
+        p = C.c_void_p()
+        _lib.check(l.zenu_hip_malloc(C.byref(p), 100 << 20, None), "malloc")
+        ptrs.append(p.value)
+    for p in ptrs:
+        _lib.check(l.zenu_hip_free(p, None), "free")
+    p = C.c_void_p()
+    _lib.check(l.zenu_hip_malloc(C.byref(p), 100 << 20, None), "malloc")      # served from the cache
+    l.zenu_hip_mempool_stats(C.byref(st))
+    assert st.n_driver_allocs == base_allocs + 3
+    assert st.n_cache_hits >= base_hits + 1
+    assert p.value in ptrs
+    _lib.check(l.zenu_hip_free(p.value, None), "free")
+    assert l.zenu_hip_free(C.c_void_p(0xdead000), None) == _lib.ERR_NOT_OWNED  # foreign pointer
+    # cross-stream reuse goes through an event; results stay correct
+    s1, s2 = C.c_void_p(), C.c_void_p()
+    _lib.check(l.zenu_hip_stream_create(C.byref(s1)), "stream")
+    _lib.check(l.zenu_hip_stream_create(C.byref(s2)), "stream")
+    q = C.c_void_p()
+    _lib.check(l.zenu_hip_malloc(C.byref(q), 64 << 20, s1), "malloc s1")
+    _lib.check(l.zenu_hip_memset_zero(q, 64 << 20, s1), "zero")
+    _lib.check(l.zenu_hip_free(q, s1), "free s1")
+    q2 = C.c_void_p()
+    _lib.check(l.zenu_hip_malloc(C.byref(q2), 64 << 20, s2), "malloc s2")
+    assert q2.value == q.value
+    _lib.check(l.zenu_hip_free(q2, s2), "free s2")
+    _lib.check(l.zenu_hip_stream_synchronize(s1), "sync")
+    _lib.check(l.zenu_hip_stream_synchronize(s2), "sync")
+    _lib.check(l.zenu_hip_stream_destroy(s1), "destroy")
+    _lib.check(l.zenu_hip_stream_destroy(s2), "destroy")
+    _lib.check(l.zenu_hip_mempool_trim(), "trim")
+    l.zenu_hip_mempool_stats(C.byref(st))
+    assert st.bytes_reserved == st.bytes_in_use + st.bytes_cached

@@ -1,0 +1,307 @@
+// allocator.hpp -- stream-ordered caching device allocator.
+//
+// Replaces ZeNu's host-side memory pool (zenu-matrix/src/memory_pool/mod.rs:79-145: three size
+// classes, bump pointers inside slabs, not stream aware) together with cuda_malloc_bytes /
+// cuda_free (zenu-cuda/src/runtime/mod.rs:30-60), which synchronise the stream on every call.
+//
+// Design
+//   * Two pools.  Requests <= 1 MiB are carved out of 2 MiB segments; larger requests come from
+//     segments of 20 MiB (requests < 10 MiB) or of the request rounded up to 2 MiB.  The
+//     segment sizes are the reference's slab sizes (memory_pool/mod.rs:70-84); unlike its
+//     bump-pointer slabs, blocks are split on allocation and merged with free neighbours on
+//     release, so holes in the middle of a segment are reusable.
+//   * Stream ordered.  Every free block belongs to the stream it was freed on.  An allocation
+//     on the same stream reuses it immediately: the kernels already queued on that stream run
+//     before anything the new owner enqueues.  An allocation on another stream may take the
+//     block only through an event: record on the owner stream, make the new stream wait.  No
+//     host synchronisation on any hit.
+//   * Out of memory: wait for the device, release every completely free segment, retry once
+//     (the flow memory_pool/mod.rs:9-20 describes), then report ZENU_ERR_OOM.
+//   * free() of a pointer the pool does not know returns ZENU_ERR_NOT_OWNED so the caller can
+//     fall back to a raw free (device/mod.rs:34-45).
+//
+// The device is reached only through `Backend`, so the bookkeeping is testable on the host
+// with a fake backend (as memory_pool/test.rs:18-49 does with MockDeviceBase).
+#pragma once
+
+#include <stdint.h>
+
+#include <map>
+#include <mutex>
+#include <set>
+#include <unordered_map>
+#include <vector>
+
+namespace zenu {
+
+struct AllocBackend {
+    virtual ~AllocBackend() {}
+    virtual int raw_alloc(void **p, size_t bytes) = 0;  // 0 = ok, else out of memory / error
+    virtual int raw_free(void *p) = 0;
+    // order `waiter` after everything queued on `owner` so far; 0 = ok
+    virtual int order_after(void *owner_stream, void *waiter_stream) = 0;
+    virtual int device_synchronize() = 0;
+};
+
+struct AllocStats {
+    uint64_t bytes_in_use = 0, bytes_cached = 0, bytes_reserved = 0;
+    uint64_t n_alloc_calls = 0, n_cache_hits = 0, n_driver_allocs = 0, n_driver_frees = 0,
+             n_oom_retries = 0;
+};
+
+class CachingAllocator {
+public:
+    static constexpr size_t kMinBlock = 512;               // rounding of every request
+    static constexpr size_t kSmallLimit = 1u << 20;        // <= 1 MiB -> small pool
+    static constexpr size_t kSmallSegment = 2u << 20;      // 2 MiB
+    static constexpr size_t kLargeSegment = 20u << 20;     // 20 MiB
+    static constexpr size_t kLargeSplitLimit = 10u << 20;  // < 10 MiB share a 20 MiB segment
+    static constexpr size_t kRoundLarge = 2u << 20;
+
+    // status codes mirror zenu_status_t: 0 ok, 4 arg, 6 oom, 8 not owned, 5 backend failure
+    enum { kOk = 0, kErrArg = 4, kErrBackend = 5, kErrOom = 6, kErrNotOwned = 8 };
+
+    explicit CachingAllocator(AllocBackend *backend) : be_(backend) {}
+    ~CachingAllocator() { release_all(); }
+
+    int malloc(void **out, size_t bytes, void *stream)
+    {
+        if (!out) return kErrArg;
+        *out = nullptr;
+        std::lock_guard<std::mutex> g(mu_);
+        stats_.n_alloc_calls++;
+        if (bytes == 0) bytes = 1;
+        const size_t size = round_size(bytes);
+        const bool small = size <= kSmallLimit;
+
+        Block *b = take_free_block(size, small, stream, /*other_streams=*/false);
+        if (!b) b = take_free_block(size, small, stream, /*other_streams=*/true);
+        if (b) {
+            stats_.n_cache_hits++;
+        } else {
+            size_t seg = segment_size(size);
+            void *p = nullptr;
+            int rc = be_->raw_alloc(&p, seg);
+            if (rc != 0 || !p) {
+                // out of memory: drop the cache and retry once
+                stats_.n_oom_retries++;
+                be_->device_synchronize();
+                release_free_segments();
+                rc = be_->raw_alloc(&p, seg);
+                if (rc != 0 || !p) return kErrOom;
+            }
+            stats_.n_driver_allocs++;
+            stats_.bytes_reserved += seg;
+            b = new Block();
+            b->ptr = static_cast<char *>(p);
+            b->size = seg;
+            b->small = small;
+            b->stream = stream;
+            b->segment_head = true;
+        }
+        // split when the remainder is worth keeping
+        const size_t min_rem = small ? kMinBlock : kSmallLimit + kMinBlock;
+        if (b->size - size >= min_rem) {
+            Block *r = new Block();
+            r->ptr = b->ptr + size;
+            r->size = b->size - size;
+            r->small = b->small;
+            r->stream = stream;
+            r->prev = b;
+            r->next = b->next;
+            if (b->next) b->next->prev = r;
+            b->next = r;
+            b->size = size;
+            insert_free(r);
+        }
+        b->allocated = true;
+        b->stream = stream;
+        live_[b->ptr] = b;
+        stats_.bytes_in_use += b->size;
+        *out = b->ptr;
+        return kOk;
+    }
+
+    int free(void *p, void *stream)
+    {
+        if (!p) return kOk;
+        std::lock_guard<std::mutex> g(mu_);
+        auto it = live_.find(static_cast<char *>(p));
+        if (it == live_.end()) return kErrNotOwned;
+        Block *b = it->second;
+        live_.erase(it);
+        stats_.bytes_in_use -= b->size;
+        b->allocated = false;
+        b->stream = stream;  // the last stream to use the block: stream-ordered free
+        // merge with free neighbours that belong to the same stream
+        b = try_merge(b, b->prev);
+        b = try_merge(b, b->next);
+        insert_free(b);
+        return kOk;
+    }
+
+    // hand every completely free segment back to the driver
+    int trim()
+    {
+        std::lock_guard<std::mutex> g(mu_);
+        be_->device_synchronize();
+        release_free_segments();
+        return kOk;
+    }
+
+    AllocStats stats()
+    {
+        std::lock_guard<std::mutex> g(mu_);
+        return stats_;
+    }
+
+    bool owns(void *p)
+    {
+        std::lock_guard<std::mutex> g(mu_);
+        return live_.count(static_cast<char *>(p)) != 0;
+    }
+
+    static size_t round_size(size_t bytes)
+    {
+        if (bytes <= kSmallLimit) return (bytes + kMinBlock - 1) / kMinBlock * kMinBlock;
+        return (bytes + kRoundLarge - 1) / kRoundLarge * kRoundLarge;
+    }
+
+    static size_t segment_size(size_t rounded)
+    {
+        if (rounded <= kSmallLimit) return kSmallSegment;
+        if (rounded < kLargeSplitLimit) return kLargeSegment;
+        return rounded;
+    }
+
+private:
+    struct Block {
+        char *ptr = nullptr;
+        size_t size = 0;
+        bool small = false;
+        bool allocated = false;
+        bool segment_head = false;  // first block of a driver allocation
+        void *stream = nullptr;
+        Block *prev = nullptr, *next = nullptr;  // neighbours inside the segment
+    };
+    struct BlockLess {
+        bool operator()(const Block *a, const Block *b) const
+        {
+            if (a->size != b->size) return a->size < b->size;
+            return a->ptr < b->ptr;
+        }
+    };
+    typedef std::set<Block *, BlockLess> FreeSet;
+    struct PoolKey {
+        void *stream;
+        bool small;
+        bool operator<(const PoolKey &o) const
+        {
+            if (stream != o.stream) return stream < o.stream;
+            return small < o.small;
+        }
+    };
+
+    void insert_free(Block *b)
+    {
+        free_[PoolKey{b->stream, b->small}].insert(b);
+        stats_.bytes_cached += b->size;
+    }
+    void erase_free(Block *b)
+    {
+        auto it = free_.find(PoolKey{b->stream, b->small});
+        if (it != free_.end()) it->second.erase(b);
+        stats_.bytes_cached -= b->size;
+    }
+
+    // best fit in one stream's list (other_streams=false) or any other stream's (true)
+    Block *take_free_block(size_t size, bool small, void *stream, bool other_streams)
+    {
+        Block key;
+        key.size = size;
+        key.ptr = nullptr;
+        for (auto &kv : free_) {
+            if (kv.first.small != small) continue;
+            if ((kv.first.stream == stream) == other_streams) continue;
+            FreeSet &fs = kv.second;
+            auto it = fs.lower_bound(&key);
+            if (it == fs.end()) continue;
+            Block *b = *it;
+            // do not burn a huge block on a much smaller large-pool request
+            if (!small && size >= kLargeSplitLimit && b->size >= size + kLargeSegment) continue;
+            if (other_streams) {
+                if (be_->order_after(b->stream, stream) != 0) continue;
+            }
+            fs.erase(it);
+            stats_.bytes_cached -= b->size;
+            return b;
+        }
+        return nullptr;
+    }
+
+    Block *try_merge(Block *b, Block *nb)
+    {
+        if (!nb || nb->allocated || nb->stream != b->stream) return b;
+        erase_free(nb);
+        if (nb == b->prev) {
+            nb->size += b->size;
+            nb->next = b->next;
+            if (b->next) b->next->prev = nb;
+            delete b;
+            return nb;
+        }
+        b->size += nb->size;
+        b->next = nb->next;
+        if (nb->next) nb->next->prev = b;
+        delete nb;
+        return b;
+    }
+
+    void release_free_segments()
+    {
+        for (auto &kv : free_) {
+            FreeSet &fs = kv.second;
+            for (auto it = fs.begin(); it != fs.end();) {
+                Block *b = *it;
+                if (b->segment_head && !b->prev && !b->next) {
+                    it = fs.erase(it);
+                    stats_.bytes_cached -= b->size;
+                    stats_.bytes_reserved -= b->size;
+                    stats_.n_driver_frees++;
+                    be_->raw_free(b->ptr);
+                    delete b;
+                } else {
+                    ++it;
+                }
+            }
+        }
+    }
+
+    void release_all()
+    {
+        std::lock_guard<std::mutex> g(mu_);
+        release_free_segments();
+        // blocks still live or fragmented at shutdown: free their segments through the heads
+        std::vector<Block *> rest;
+        for (auto &kv : free_)
+            for (Block *b : kv.second) rest.push_back(b);
+        for (auto &kv : live_) rest.push_back(kv.second);
+        free_.clear();
+        live_.clear();
+        for (Block *b : rest)
+            if (b->segment_head) {
+                be_->raw_free(b->ptr);
+                stats_.n_driver_frees++;
+            }
+        for (Block *b : rest) delete b;
+        stats_.bytes_cached = stats_.bytes_in_use = stats_.bytes_reserved = 0;
+    }
+
+    AllocBackend *be_;
+    std::mutex mu_;
+    std::map<PoolKey, FreeSet> free_;
+    std::unordered_map<char *, Block *> live_;
+    AllocStats stats_;
+};
+
+}  // namespace zenu

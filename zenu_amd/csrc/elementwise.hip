@@ -1,0 +1,840 @@
+// elementwise.hip -- N-d elementwise engine for gfx950 (binary, scalar, unary, relu, copy).
+//
+// One Matrix-level call of the reference (add_array, mul_scalar, exp_array, relu, copy_from ...,
+// zenu-matrix/src/operation/basic_operations.rs:278-381,512-611, relu.rs:169-242,
+// copy_from.rs:211-267) becomes ONE launch here instead of one 1-D launch per row
+// (zenu-matrix/src/with_clousers.rs:180-223).  After the host has folded the operands into a
+// common iteration space (shape.cpp) one of four kernels runs:
+//
+//   contig : every operand is one contiguous run.  128-bit loads/stores, 4 vectors in flight
+//            per thread, block tile = 256 threads x 4 x 16 B.                        [HBM bound]
+//   rows   : the innermost dim is contiguous (stride 1) or broadcast (stride 0) in every operand;
+//            outer dims are arbitrary.  Covers row / column broadcast and row-sliced views.  The
+//            outer index is decomposed once per thread, the inner dim is walked with 128-bit
+//            accesses; a broadcast row stays in L2.                                   [HBM bound]
+//   tile   : some input is contiguous along a different dim than the output (a transposed
+//            operand).  64x64 tiles: the transposed input is read along ITS contiguous dim with
+//            128-bit loads, turned through LDS (pitch 65 words: conflict-free both ways on the
+//            64-lane wavefront), and every HBM access stays coalesced.               [HBM bound]
+//   generic: anything else (strided output, gathers): one element per thread, index arithmetic
+//            per element.
+//
+// Arithmetic is plain IEEE with contraction off; + - * / sqrt are correctly rounded on gfx950,
+// so results are bit-identical to the CPU loops of basic_operations.rs:93-181.
+#include <math.h>
+
+#include "common.hpp"
+#include "zmath.hpp"
+
+namespace zenu {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kUnroll = 4;
+
+template <typename T> struct VecOf;
+template <> struct VecOf<float> { typedef float4 type; static constexpr int N = 4; };
+template <> struct VecOf<double> { typedef double2 type; static constexpr int N = 2; };
+
+template <typename T, int N> struct Pack { T v[N]; };
+
+template <typename T, int N> __device__ __forceinline__ Pack<T, N> load_pack(const T *p)
+{
+    Pack<T, N> r;
+    if constexpr (N == 1) {
+        r.v[0] = *p;
+    } else {
+        typedef typename VecOf<T>::type V;
+        V x = *reinterpret_cast<const V *>(p);
+        __builtin_memcpy(&r, &x, sizeof(V));
+    }
+    return r;
+}
+template <typename T, int N> __device__ __forceinline__ void store_pack(T *p, const Pack<T, N> &r)
+{
+    if constexpr (N == 1) {
+        *p = r.v[0];
+    } else {
+        typedef typename VecOf<T>::type V;
+        V x;
+        __builtin_memcpy(&x, &r, sizeof(V));
+        *reinterpret_cast<V *>(p) = x;
+    }
+}
+template <typename T, int N> __device__ __forceinline__ Pack<T, N> splat(T s)
+{
+    Pack<T, N> r;
+#pragma unroll
+    for (int i = 0; i < N; i++) r.v[i] = s;
+    return r;
+}
+
+// ---- functors -----------------------------------------------------------------------------------
+
+template <typename T, int OP> __device__ __forceinline__ T bin_apply(T a, T b)
+{
+    if constexpr (OP == ZENU_ADD) return a + b;
+    else if constexpr (OP == ZENU_SUB) return a - b;
+    else if constexpr (OP == ZENU_MUL) return a * b;
+    else return a / b;
+}
+
+template <typename T, int OP> struct BinF {
+    static constexpr int NIN = 2;
+    __device__ __forceinline__ void init() {}
+    __device__ __forceinline__ T operator()(T a, T b) const { return bin_apply<T, OP>(a, b); }
+};
+
+// a op s; the scalar comes by value or from device memory (0-d tensor operand)
+template <typename T, int OP> struct ScalarF {
+    static constexpr int NIN = 1;
+    T s;
+    const T *sp;
+    __device__ __forceinline__ void init() { if (sp) s = *sp; }
+    __device__ __forceinline__ T operator()(T a, T) const { return bin_apply<T, OP>(a, s); }
+};
+
+__device__ __forceinline__ float dev_tanh(float x) { return zmath::tanhf_fdlibm(x); }
+__device__ __forceinline__ double dev_tanh(double x) { return tanh(x); }
+__device__ __forceinline__ float dev_sigmoid(float x) { return zmath::sigmoidf_zenu(x); }
+__device__ __forceinline__ double dev_sigmoid(double x)
+{
+    double xh = x * 0.5;
+    double th = tanh(xh);
+    double ht = 0.5 * th;
+    return 0.5 + ht;
+}
+
+template <typename T, int FN> struct UnaryF {
+    static constexpr int NIN = 1;
+    __device__ __forceinline__ void init() {}
+    __device__ __forceinline__ T operator()(T a, T) const
+    {
+        if constexpr (FN == ZENU_EXP) return exp(a);
+        else if constexpr (FN == ZENU_LOG) return log(a);
+        else if constexpr (FN == ZENU_TANH) return dev_tanh(a);
+        else if constexpr (FN == ZENU_SQRT) return sqrt(a);
+        else if constexpr (FN == ZENU_ABS) return fabs(a);
+        else if constexpr (FN == ZENU_SIN) return sin(a);
+        else if constexpr (FN == ZENU_COS) return cos(a);
+        else if constexpr (FN == ZENU_TAN) return tan(a);
+        else if constexpr (FN == ZENU_ASIN) return asin(a);
+        else if constexpr (FN == ZENU_ACOS) return acos(a);
+        else if constexpr (FN == ZENU_ATAN) return atan(a);
+        else if constexpr (FN == ZENU_SINH) return sinh(a);
+        else if constexpr (FN == ZENU_COSH) return cosh(a);
+        else return dev_sigmoid(a);
+    }
+};
+
+template <typename T> struct PowF {
+    static constexpr int NIN = 1;
+    T s;
+    __device__ __forceinline__ void init() {}
+    __device__ __forceinline__ T operator()(T a, T) const { return pow(a, s); }
+};
+
+// relu.rs:44-48: the non-positive branch returns the PRODUCT alpha*x (-0.0 for alpha = 0)
+template <typename T> struct ReluF {
+    static constexpr int NIN = 1;
+    T alpha;
+    __device__ __forceinline__ void init() {}
+    __device__ __forceinline__ T operator()(T a, T) const { return (a > (T)0) ? a : alpha * a; }
+};
+// relu.rs:74-78
+template <typename T> struct ReluMaskF {
+    static constexpr int NIN = 1;
+    T alpha;
+    __device__ __forceinline__ void init() {}
+    __device__ __forceinline__ T operator()(T a, T) const { return (a > (T)0) ? (T)1 : alpha * (T)-1; }
+};
+template <typename T> struct CopyF {
+    static constexpr int NIN = 1;
+    __device__ __forceinline__ void init() {}
+    __device__ __forceinline__ T operator()(T a, T) const { return a; }
+};
+
+template <typename T, int N, typename F>
+__device__ __forceinline__ Pack<T, N> apply_pack(const F &f, const Pack<T, N> &a, const Pack<T, N> &b)
+{
+    Pack<T, N> r;
+#pragma unroll
+    for (int i = 0; i < N; i++) r.v[i] = f(a.v[i], b.v[i]);
+    return r;
+}
+
+// ---- kernel 1: contiguous ------------------------------------------------------------------------
+
+template <typename T, int VEC, typename F>
+__global__ __launch_bounds__(kBlock) void ew_contig_kernel(T *out, const T *a, const T *b,
+                                                           int64_t n, F f)
+{
+    f.init();
+    constexpr int64_t kTile = (int64_t)kBlock * VEC * kUnroll;
+    const int64_t base = (int64_t)blockIdx.x * kTile;
+    const int tid = threadIdx.x;
+    if (base + kTile <= n) {
+        Pack<T, VEC> va[kUnroll], vb[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            int64_t i = base + ((int64_t)u * kBlock + tid) * VEC;
+            va[u] = load_pack<T, VEC>(a + i);
+            if constexpr (F::NIN == 2) vb[u] = load_pack<T, VEC>(b + i);
+            else vb[u] = va[u];
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            int64_t i = base + ((int64_t)u * kBlock + tid) * VEC;
+            store_pack<T, VEC>(out + i, apply_pack<T, VEC, F>(f, va[u], vb[u]));
+        }
+    } else {
+        for (int u = 0; u < kUnroll; u++) {
+            int64_t i = base + ((int64_t)u * kBlock + tid) * VEC;
+#pragma unroll
+            for (int j = 0; j < VEC; j++) {
+                if (i + j < n) {
+                    T x = a[i + j];
+                    T y = (F::NIN == 2) ? b[i + j] : x;
+                    out[i + j] = f(x, y);
+                }
+            }
+        }
+    }
+}
+
+// ---- shared index descriptor ---------------------------------------------------------------------
+
+struct OuterDesc {
+    int nouter;                          // number of outer dims (0..5)
+    int64_t shape[kMaxDim];              // outer dims, slowest first
+    int64_t stride[kMaxOperands][kMaxDim];
+};
+
+__device__ __forceinline__ void decompose(const OuterDesc &d, int64_t lin, int64_t &o0, int64_t &o1,
+                                          int64_t &o2)
+{
+    o0 = o1 = o2 = 0;
+    for (int k = d.nouter - 1; k >= 0; k--) {
+        int64_t q, r;
+        if (lin < 0x7fffffffLL && d.shape[k] < 0x7fffffffLL) {
+            uint32_t l32 = (uint32_t)lin, s32 = (uint32_t)d.shape[k];
+            q = l32 / s32;
+            r = l32 - (uint32_t)q * s32;
+        } else {
+            q = lin / d.shape[k];
+            r = lin - q * d.shape[k];
+        }
+        o0 += r * d.stride[0][k];
+        o1 += r * d.stride[1][k];
+        o2 += r * d.stride[2][k];
+        lin = q;
+    }
+}
+
+// ---- kernel 2: rows (inner dim contiguous or broadcast) -------------------------------------------
+
+struct RowsParams {
+    OuterDesc outer;
+    int64_t nrows;     // product of outer dims
+    int64_t ncols;     // inner length
+    int inner_a;       // inner stride of input a: 1 or 0
+    int inner_b;       // inner stride of input b: 1 or 0
+    int tx_shift;      // threads along the row = 1 << tx_shift (<= 256)
+    int64_t col_tiles; // column tiles per row
+};
+
+template <typename T, int VEC, typename F>
+__global__ __launch_bounds__(kBlock) void ew_rows_kernel(T *out, const T *a, const T *b,
+                                                         RowsParams p, F f)
+{
+    f.init();
+    const int tx_n = 1 << p.tx_shift;
+    const int ty_n = kBlock >> p.tx_shift;
+    const int tx = threadIdx.x & (tx_n - 1);
+    const int ty = threadIdx.x >> p.tx_shift;
+    const int64_t blk = blockIdx.x;
+    const int64_t row_blk = blk / p.col_tiles;
+    const int64_t col_tile = blk - row_blk * p.col_tiles;
+    const int64_t row = row_blk * ty_n + ty;
+    if (row >= p.nrows) return;
+    int64_t oo, oa, ob;
+    decompose(p.outer, row, oo, oa, ob);
+    T *orow = out + oo;
+    const T *arow = a + oa;
+    const T *brow = (F::NIN == 2) ? b + ob : arow;
+
+    const int64_t cols_per_tile = (int64_t)tx_n * VEC * kUnroll;
+    const int64_t c0 = col_tile * cols_per_tile;
+    Pack<T, VEC> sa, sb;
+    if (p.inner_a == 0) sa = splat<T, VEC>(arow[0]);
+    if (F::NIN == 2 && p.inner_b == 0) sb = splat<T, VEC>(brow[0]);
+
+    if (c0 + cols_per_tile <= p.ncols) {
+        Pack<T, VEC> va[kUnroll], vb[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            int64_t c = c0 + ((int64_t)u * tx_n + tx) * VEC;
+            va[u] = p.inner_a ? load_pack<T, VEC>(arow + c) : sa;
+            if constexpr (F::NIN == 2) vb[u] = p.inner_b ? load_pack<T, VEC>(brow + c) : sb;
+            else vb[u] = va[u];
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            int64_t c = c0 + ((int64_t)u * tx_n + tx) * VEC;
+            store_pack<T, VEC>(orow + c, apply_pack<T, VEC, F>(f, va[u], vb[u]));
+        }
+    } else {
+        for (int u = 0; u < kUnroll; u++) {
+            int64_t c = c0 + ((int64_t)u * tx_n + tx) * VEC;
+            if (c + VEC <= p.ncols) {
+                Pack<T, VEC> x = p.inner_a ? load_pack<T, VEC>(arow + c) : sa;
+                Pack<T, VEC> y = x;
+                if constexpr (F::NIN == 2) y = p.inner_b ? load_pack<T, VEC>(brow + c) : sb;
+                store_pack<T, VEC>(orow + c, apply_pack<T, VEC, F>(f, x, y));
+            } else {
+                for (int j = 0; j < VEC; j++) {
+                    if (c + j < p.ncols) {
+                        T x = p.inner_a ? arow[c + j] : sa.v[0];
+                        T y = x;
+                        if constexpr (F::NIN == 2) y = p.inner_b ? brow[c + j] : sb.v[0];
+                        orow[c + j] = f(x, y);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---- kernel 3: 64x64 tiles with an LDS turn for transposed inputs ----------------------------------
+
+// 64x64 tiles for f32 (16.6 KB of LDS per staged input), 32x32 for f64 (8.4 KB).
+template <typename T> struct TileOf { static constexpr int N = sizeof(T) == 4 ? 64 : 32; };
+
+struct TileParams {
+    OuterDesc outer;      // batch dims (everything except the two tile dims)
+    int64_t nbatch;
+    int64_t R, C;         // tile dims: R = dim where transposed inputs are contiguous, C = output inner dim
+    int64_t ldr[kMaxOperands];  // stride along R per operand
+    int64_t ldc[kMaxOperands];  // stride along C per operand (1 for out; 0/1 direct; ld for transposed)
+    int trans_a, trans_b;       // input goes through LDS
+    int vec_ok;                 // alignment allows 128-bit accesses on full tiles
+    int64_t tiles_r, tiles_c;
+};
+
+template <typename T, typename F>
+__global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, const T *b,
+                                                         TileParams p, F f)
+{
+    constexpr int VEC = VecOf<T>::N;
+    constexpr int kTile = TileOf<T>::N;
+    constexpr int kPitch = kTile + 1;
+    constexpr int VPR = kTile / VEC;        // vectors per tile row
+    constexpr int RPP = kBlock / VPR;       // tile rows per pass
+    __shared__ T lds_a[kTile * kPitch];
+    __shared__ T lds_b[(F::NIN == 2) ? kTile * kPitch : 1];
+    f.init();
+
+    int64_t blk = blockIdx.x;
+    const int64_t tc = blk % p.tiles_c;
+    blk /= p.tiles_c;
+    const int64_t tr = blk % p.tiles_r;
+    const int64_t batch = blk / p.tiles_r;
+    int64_t oo, oa, ob;
+    decompose(p.outer, batch, oo, oa, ob);
+    const int64_t r0 = tr * kTile, c0 = tc * kTile;
+    const int64_t nr = (p.R - r0 < kTile) ? p.R - r0 : kTile;
+    const int64_t nc = (p.C - c0 < kTile) ? p.C - c0 : kTile;
+    const bool full = (nr == kTile) && (nc == kTile) && p.vec_ok;
+    const int tid = threadIdx.x;
+
+    T *obase = out + oo + r0 * p.ldr[0] + c0;
+    const T *abase = a + oa + r0 * p.ldr[1] + c0 * p.ldc[1];
+    const T *bbase = (F::NIN == 2) ? b + ob + r0 * p.ldr[2] + c0 * p.ldc[2] : abase;
+
+    // phase 1: transposed inputs -> LDS, reading along R (their contiguous dim)
+    if (p.trans_a || (F::NIN == 2 && p.trans_b)) {
+        if (full) {
+            const int rv = (tid % VPR) * VEC;
+#pragma unroll
+            for (int k = 0; k < kTile / RPP; k++) {
+                const int c = tid / VPR + k * RPP;
+                if (p.trans_a) {
+                    Pack<T, VEC> x = load_pack<T, VEC>(abase + rv + (int64_t)c * p.ldc[1]);
+#pragma unroll
+                    for (int j = 0; j < VEC; j++) lds_a[(rv + j) * kPitch + c] = x.v[j];
+                }
+                if constexpr (F::NIN == 2) {
+                    if (p.trans_b) {
+                        Pack<T, VEC> x = load_pack<T, VEC>(bbase + rv + (int64_t)c * p.ldc[2]);
+#pragma unroll
+                        for (int j = 0; j < VEC; j++) lds_b[(rv + j) * kPitch + c] = x.v[j];
+                    }
+                }
+            }
+        } else {
+            for (int e = tid; e < kTile * kTile; e += kBlock) {
+                const int r = e % kTile, c = e / kTile;
+                if (r < nr && c < nc) {
+                    if (p.trans_a) lds_a[r * kPitch + c] = abase[r + (int64_t)c * p.ldc[1]];
+                    if constexpr (F::NIN == 2) {
+                        if (p.trans_b) lds_b[r * kPitch + c] = bbase[r + (int64_t)c * p.ldc[2]];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    // phase 2: walk the tile along C (the output's contiguous dim)
+    if (full) {
+        const int cv = (tid % VPR) * VEC;
+#pragma unroll
+        for (int k = 0; k < kTile / RPP; k++) {
+            const int r = tid / VPR + k * RPP;
+            Pack<T, VEC> x, y;
+            if (p.trans_a) {
+#pragma unroll
+                for (int j = 0; j < VEC; j++) x.v[j] = lds_a[r * kPitch + cv + j];
+            } else if (p.ldc[1] == 0) {
+                x = splat<T, VEC>(abase[(int64_t)r * p.ldr[1]]);
+            } else {
+                x = load_pack<T, VEC>(abase + (int64_t)r * p.ldr[1] + cv);
+            }
+            if constexpr (F::NIN == 2) {
+                if (p.trans_b) {
+#pragma unroll
+                    for (int j = 0; j < VEC; j++) y.v[j] = lds_b[r * kPitch + cv + j];
+                } else if (p.ldc[2] == 0) {
+                    y = splat<T, VEC>(bbase[(int64_t)r * p.ldr[2]]);
+                } else {
+                    y = load_pack<T, VEC>(bbase + (int64_t)r * p.ldr[2] + cv);
+                }
+            } else {
+                y = x;
+            }
+            store_pack<T, VEC>(obase + (int64_t)r * p.ldr[0] + cv, apply_pack<T, VEC, F>(f, x, y));
+        }
+    } else {
+        for (int e = tid; e < kTile * kTile; e += kBlock) {
+            const int c = e % kTile, r = e / kTile;
+            if (r < nr && c < nc) {
+                T x = p.trans_a ? lds_a[r * kPitch + c] : abase[(int64_t)r * p.ldr[1] + (int64_t)c * p.ldc[1]];
+                T y = x;
+                if constexpr (F::NIN == 2)
+                    y = p.trans_b ? lds_b[r * kPitch + c]
+                                  : bbase[(int64_t)r * p.ldr[2] + (int64_t)c * p.ldc[2]];
+                obase[(int64_t)r * p.ldr[0] + c] = f(x, y);
+            }
+        }
+    }
+}
+
+// ---- kernel 4: generic -----------------------------------------------------------------------------
+
+struct GenericParams {
+    OuterDesc dims;  // all collapsed dims
+    int64_t numel;
+};
+
+template <typename T, typename F>
+__global__ __launch_bounds__(kBlock) void ew_generic_kernel(T *out, const T *a, const T *b,
+                                                            GenericParams p, F f)
+{
+    f.init();
+    const int64_t step = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < p.numel; i += step) {
+        int64_t oo, oa, ob;
+        decompose(p.dims, i, oo, oa, ob);
+        T x = a[oa];
+        T y = (F::NIN == 2) ? b[ob] : x;
+        out[oo] = f(x, y);
+    }
+}
+
+// ---- host dispatch ---------------------------------------------------------------------------------
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t stream)
+{
+    constexpr int VEC = VecOf<T>::N;
+    ew_collapse(p);
+    if (p.numel == 0) return ZENU_OK;
+    T *out = static_cast<T *>(p.ptr[0]);
+    const T *a = static_cast<const T *>(p.ptr[1]);
+    const T *b = (F::NIN == 2) ? static_cast<const T *>(p.ptr[2]) : a;
+    const int nin = F::NIN;
+    if (p.ndim == 0) {  // a single element
+        p.ndim = 1;
+        p.shape[0] = 1;
+        for (int o = 0; o < p.nops; o++) p.stride[o][0] = 1;
+    }
+    const int last = p.ndim - 1;
+
+    // contig
+    bool all_unit = p.ndim == 1;
+    for (int o = 0; o <= nin && all_unit; o++)
+        if (p.stride[o][0] != 1) all_unit = false;
+    if (all_unit) {
+        const int64_t n = p.numel;
+        bool vec = aligned16(out) && aligned16(a) && aligned16(b);
+        if (vec) {
+            int64_t tile = (int64_t)kBlock * VEC * kUnroll;
+            int64_t grid = (n + tile - 1) / tile;
+            if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
+            ew_contig_kernel<T, VEC, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, n, f);
+        } else {
+            int64_t tile = (int64_t)kBlock * kUnroll;
+            int64_t grid = (n + tile - 1) / tile;
+            if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
+            ew_contig_kernel<T, 1, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, n, f);
+        }
+        ZENU_LAUNCH_CHECK();
+        return ZENU_OK;
+    }
+
+    const bool out_inner_unit = p.stride[0][last] == 1;
+    bool inner_01 = out_inner_unit;
+    for (int o = 1; o <= nin && inner_01; o++)
+        if (p.stride[o][last] != 0 && p.stride[o][last] != 1) inner_01 = false;
+
+    if (inner_01) {
+        RowsParams rp;
+        rp.outer.nouter = p.ndim - 1;
+        for (int d = 0; d < kMaxDim; d++) {
+            rp.outer.shape[d] = d < p.ndim - 1 ? p.shape[d] : 1;
+            for (int o = 0; o < kMaxOperands; o++)
+                rp.outer.stride[o][d] = (d < p.ndim - 1 && o < p.nops) ? p.stride[o][d] : 0;
+        }
+        rp.ncols = p.shape[last];
+        rp.nrows = p.numel / rp.ncols;
+        rp.inner_a = (int)p.stride[1][last];
+        rp.inner_b = nin == 2 ? (int)p.stride[2][last] : 1;
+        bool vec = aligned16(out) && (rp.ncols % VEC == 0);
+        for (int o = 1; o <= nin && vec; o++)
+            if (p.stride[o][last] == 1 && !aligned16(p.ptr[o])) vec = false;
+        for (int d = 0; d < p.ndim - 1 && vec; d++) {
+            if (p.stride[0][d] % VEC) vec = false;
+            for (int o = 1; o <= nin; o++)
+                if (p.stride[o][last] == 1 && p.stride[o][d] % VEC) vec = false;
+        }
+        const int v = vec ? VEC : 1;
+        int64_t vcols = (rp.ncols + v - 1) / v;
+        int shift = 0;
+        while ((1 << shift) < kBlock && ((int64_t)1 << shift) < vcols) shift++;
+        rp.tx_shift = shift;
+        int64_t cols_per_tile = ((int64_t)1 << shift) * v * kUnroll;
+        rp.col_tiles = (rp.ncols + cols_per_tile - 1) / cols_per_tile;
+        int64_t rows_per_blk = kBlock >> shift;
+        int64_t grid = ((rp.nrows + rows_per_blk - 1) / rows_per_blk) * rp.col_tiles;
+        if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
+        if (vec) ew_rows_kernel<T, VEC, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, rp, f);
+        else     ew_rows_kernel<T, 1, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, rp, f);
+        ZENU_LAUNCH_CHECK();
+        return ZENU_OK;
+    }
+
+    // tile: every input is either inner-{0,1} or unit-stride along one common other dim `ri`
+    if (out_inner_unit && p.ndim >= 2) {
+        int ri = -1;
+        bool ok = true;
+        int trans[kMaxOperands] = {0, 0, 0};
+        for (int o = 1; o <= nin && ok; o++) {
+            int64_t s = p.stride[o][last];
+            if (s == 0 || s == 1) continue;
+            int found = -1;
+            for (int d = 0; d < last; d++)
+                if (p.stride[o][d] == 1) { found = d; break; }
+            if (found < 0 || (ri >= 0 && ri != found)) ok = false;
+            else { ri = found; trans[o] = 1; }
+        }
+        if (ok && ri >= 0) {
+            TileParams tp;
+            int k = 0;
+            for (int d = 0; d < kMaxDim; d++) {
+                tp.outer.shape[d] = 1;
+                for (int o = 0; o < kMaxOperands; o++) tp.outer.stride[o][d] = 0;
+            }
+            for (int d = 0; d < last; d++) {
+                if (d == ri) continue;
+                tp.outer.shape[k] = p.shape[d];
+                for (int o = 0; o < p.nops; o++) tp.outer.stride[o][k] = p.stride[o][d];
+                k++;
+            }
+            tp.outer.nouter = k;
+            tp.R = p.shape[ri];
+            tp.C = p.shape[last];
+            tp.nbatch = p.numel / (tp.R * tp.C);
+            for (int o = 0; o < kMaxOperands; o++) {
+                tp.ldr[o] = o < p.nops ? p.stride[o][ri] : 0;
+                tp.ldc[o] = o < p.nops ? p.stride[o][last] : 0;
+            }
+            tp.trans_a = trans[1];
+            tp.trans_b = nin == 2 ? trans[2] : 0;
+            bool vec = true;
+            for (int o = 0; o <= nin && vec; o++) {
+                if (!aligned16(p.ptr[o])) vec = false;
+                // every stride that moves a vector's base address must keep 16 B alignment
+                for (int d = 0; d < p.ndim && vec; d++) {
+                    int64_t s = p.stride[o][d];
+                    if (s == 1 || s == 0) continue;
+                    if (s % VEC) vec = false;
+                }
+            }
+            tp.vec_ok = vec ? 1 : 0;
+            constexpr int kTile = TileOf<T>::N;
+            tp.tiles_r = (tp.R + kTile - 1) / kTile;
+            tp.tiles_c = (tp.C + kTile - 1) / kTile;
+            int64_t grid = tp.nbatch * tp.tiles_r * tp.tiles_c;
+            if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
+            ew_tile_kernel<T, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, tp, f);
+            ZENU_LAUNCH_CHECK();
+            return ZENU_OK;
+        }
+    }
+
+    // generic
+    GenericParams gp;
+    gp.dims.nouter = p.ndim;
+    for (int d = 0; d < kMaxDim; d++) {
+        gp.dims.shape[d] = d < p.ndim ? p.shape[d] : 1;
+        for (int o = 0; o < kMaxOperands; o++)
+            gp.dims.stride[o][d] = (d < p.ndim && o < p.nops) ? p.stride[o][d] : 0;
+    }
+    gp.numel = p.numel;
+    int64_t grid = (p.numel + kBlock - 1) / kBlock;
+    int64_t cap = (int64_t)device_info().num_cus * 32;
+    if (grid > cap) grid = cap;
+    ew_generic_kernel<T, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, gp, f);
+    ZENU_LAUNCH_CHECK();
+    return ZENU_OK;
+}
+
+// problem builders -----------------------------------------------------------------------------------
+
+void init_problem(EwProblem &p, const zenu_tensor_t &to, int nops)
+{
+    p.nops = nops;
+    p.ndim = to.ndim;
+    for (int d = 0; d < to.ndim; d++) p.shape[d] = to.shape[d];
+    for (int d = to.ndim; d < kMaxDim; d++) p.shape[d] = 1;
+    for (int o = 0; o < kMaxOperands; o++) {
+        p.ptr[o] = nullptr;
+        for (int d = 0; d < kMaxDim; d++) p.stride[o][d] = 0;
+    }
+    ew_set_operand(p, 0, to, to.ndim, to.shape);
+    // the output is never broadcast: keep its own strides even on size-1 dims
+    for (int d = 0; d < to.ndim; d++) p.stride[0][d] = to.stride[d];
+}
+
+template <typename T, typename F>
+int run1(const zenu_tensor_t &to, const zenu_tensor_t &in, F f, hipStream_t s)
+{
+    EwProblem p;
+    init_problem(p, to, 2);
+    ew_set_operand(p, 1, in, to.ndim, to.shape);
+    return launch_ew<T, F>(p, f, s);
+}
+
+template <typename T, typename F>
+int run2(const zenu_tensor_t &to, const zenu_tensor_t &x, const zenu_tensor_t &y, F f, hipStream_t s)
+{
+    EwProblem p;
+    init_problem(p, to, 3);
+    ew_set_operand(p, 1, x, to.ndim, to.shape);
+    ew_set_operand(p, 2, y, to.ndim, to.shape);
+    return launch_ew<T, F>(p, f, s);
+}
+
+template <typename T> int binary_t(int op, const zenu_tensor_t &to, const zenu_tensor_t &l,
+                                   const zenu_tensor_t &r, hipStream_t s)
+{
+    switch (op) {
+    case ZENU_ADD: return run2<T>(to, l, r, BinF<T, ZENU_ADD>(), s);
+    case ZENU_SUB: return run2<T>(to, l, r, BinF<T, ZENU_SUB>(), s);
+    case ZENU_MUL: return run2<T>(to, l, r, BinF<T, ZENU_MUL>(), s);
+    case ZENU_DIV: return run2<T>(to, l, r, BinF<T, ZENU_DIV>(), s);
+    default: return ZENU_ERR_ARG;
+    }
+}
+
+template <typename T> int scalar_t(int op, const zenu_tensor_t &to, const zenu_tensor_t &in, T sv,
+                                   const T *sp, hipStream_t s)
+{
+    switch (op) {
+    case ZENU_ADD: { ScalarF<T, ZENU_ADD> f; f.s = sv; f.sp = sp; return run1<T>(to, in, f, s); }
+    case ZENU_SUB: { ScalarF<T, ZENU_SUB> f; f.s = sv; f.sp = sp; return run1<T>(to, in, f, s); }
+    case ZENU_MUL: { ScalarF<T, ZENU_MUL> f; f.s = sv; f.sp = sp; return run1<T>(to, in, f, s); }
+    case ZENU_DIV: { ScalarF<T, ZENU_DIV> f; f.s = sv; f.sp = sp; return run1<T>(to, in, f, s); }
+    default: return ZENU_ERR_ARG;
+    }
+}
+
+template <typename T> int unary_t(int fn, const zenu_tensor_t &to, const zenu_tensor_t &in, hipStream_t s)
+{
+    switch (fn) {
+    case ZENU_EXP: return run1<T>(to, in, UnaryF<T, ZENU_EXP>(), s);
+    case ZENU_LOG: return run1<T>(to, in, UnaryF<T, ZENU_LOG>(), s);
+    case ZENU_TANH: return run1<T>(to, in, UnaryF<T, ZENU_TANH>(), s);
+    case ZENU_SQRT: return run1<T>(to, in, UnaryF<T, ZENU_SQRT>(), s);
+    case ZENU_ABS: return run1<T>(to, in, UnaryF<T, ZENU_ABS>(), s);
+    case ZENU_SIN: return run1<T>(to, in, UnaryF<T, ZENU_SIN>(), s);
+    case ZENU_COS: return run1<T>(to, in, UnaryF<T, ZENU_COS>(), s);
+    case ZENU_TAN: return run1<T>(to, in, UnaryF<T, ZENU_TAN>(), s);
+    case ZENU_ASIN: return run1<T>(to, in, UnaryF<T, ZENU_ASIN>(), s);
+    case ZENU_ACOS: return run1<T>(to, in, UnaryF<T, ZENU_ACOS>(), s);
+    case ZENU_ATAN: return run1<T>(to, in, UnaryF<T, ZENU_ATAN>(), s);
+    case ZENU_SINH: return run1<T>(to, in, UnaryF<T, ZENU_SINH>(), s);
+    case ZENU_COSH: return run1<T>(to, in, UnaryF<T, ZENU_COSH>(), s);
+    case ZENU_SIGMOID: return run1<T>(to, in, UnaryF<T, ZENU_SIGMOID>(), s);
+    default: return ZENU_ERR_ARG;
+    }
+}
+
+int check2(const zenu_tensor_t *a, const zenu_tensor_t *b)
+{
+    int rc = validate_tensor(a);
+    if (rc) return rc;
+    return validate_tensor(b);
+}
+
+}  // namespace
+}  // namespace zenu
+
+using namespace zenu;
+
+extern "C" {
+
+int zenu_hip_binary(int op, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *lhs,
+                    const zenu_tensor_t *rhs, zenu_stream_t stream)
+{
+    int rc = check2(to, lhs);
+    if (!rc) rc = validate_tensor(rhs);
+    if (!rc) rc = ensure_init();
+    if (!rc) rc = check_binary(*to, *lhs, *rhs);
+    if (rc) return rc;
+    if (dtype == ZENU_F32) return binary_t<float>(op, *to, *lhs, *rhs, as_stream(stream));
+    if (dtype == ZENU_F64) return binary_t<double>(op, *to, *lhs, *rhs, as_stream(stream));
+    return ZENU_ERR_ARG;
+}
+
+int zenu_hip_binary_assign(int op, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *rhs,
+                           zenu_stream_t stream)
+{
+    int rc = check2(to, rhs);
+    if (!rc) rc = ensure_init();
+    if (!rc) rc = check_binary_assign(*to, *rhs);
+    if (rc) return rc;
+    if (dtype == ZENU_F32) return binary_t<float>(op, *to, *to, *rhs, as_stream(stream));
+    if (dtype == ZENU_F64) return binary_t<double>(op, *to, *to, *rhs, as_stream(stream));
+    return ZENU_ERR_ARG;
+}
+
+static int scalar_common(int op, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other,
+                         double scalar, const void *sp, zenu_stream_t stream)
+{
+    int rc = check2(to, other);
+    if (!rc) rc = ensure_init();
+    if (rc) return rc;
+    if (to->ndim < other->ndim) return ZENU_ERR_RANK;   // with_clousers.rs:42-50
+    if (!same_shape(*to, *other)) return ZENU_ERR_SHAPE;
+    if (dtype == ZENU_F32)
+        return scalar_t<float>(op, *to, *other, (float)scalar, static_cast<const float *>(sp),
+                               as_stream(stream));
+    if (dtype == ZENU_F64)
+        return scalar_t<double>(op, *to, *other, scalar, static_cast<const double *>(sp),
+                                as_stream(stream));
+    return ZENU_ERR_ARG;
+}
+
+int zenu_hip_binary_scalar(int op, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other,
+                           double scalar, zenu_stream_t stream)
+{
+    return scalar_common(op, dtype, to, other, scalar, nullptr, stream);
+}
+
+int zenu_hip_binary_scalar_assign(int op, int dtype, const zenu_tensor_t *to, double scalar,
+                                  zenu_stream_t stream)
+{
+    return scalar_common(op, dtype, to, to, scalar, nullptr, stream);
+}
+
+int zenu_hip_binary_scalar_ptr(int op, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other,
+                               const void *scalar_dev, zenu_stream_t stream)
+{
+    if (!scalar_dev) return ZENU_ERR_ARG;
+    return scalar_common(op, dtype, to, other, 0.0, scalar_dev, stream);
+}
+
+int zenu_hip_binary_scalar_assign_ptr(int op, int dtype, const zenu_tensor_t *to,
+                                      const void *scalar_dev, zenu_stream_t stream)
+{
+    if (!scalar_dev) return ZENU_ERR_ARG;
+    return scalar_common(op, dtype, to, to, 0.0, scalar_dev, stream);
+}
+
+int zenu_hip_unary(int fn, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other,
+                   zenu_stream_t stream)
+{
+    int rc = check2(to, other);
+    if (!rc) rc = ensure_init();
+    if (rc) return rc;
+    if (!same_shape(*to, *other)) return ZENU_ERR_SHAPE;  // "Matrix shape mismatch"
+    if (dtype == ZENU_F32) return unary_t<float>(fn, *to, *other, as_stream(stream));
+    if (dtype == ZENU_F64) return unary_t<double>(fn, *to, *other, as_stream(stream));
+    return ZENU_ERR_ARG;
+}
+
+int zenu_hip_unary_assign(int fn, int dtype, const zenu_tensor_t *to, zenu_stream_t stream)
+{
+    return zenu_hip_unary(fn, dtype, to, to, stream);
+}
+
+int zenu_hip_powf(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other, double scalar,
+                  zenu_stream_t stream)
+{
+    int rc = check2(to, other);
+    if (!rc) rc = ensure_init();
+    if (rc) return rc;
+    if (!same_shape(*to, *other)) return ZENU_ERR_SHAPE;
+    if (dtype == ZENU_F32) { PowF<float> f; f.s = (float)scalar; return run1<float>(*to, *other, f, as_stream(stream)); }
+    if (dtype == ZENU_F64) { PowF<double> f; f.s = scalar; return run1<double>(*to, *other, f, as_stream(stream)); }
+    return ZENU_ERR_ARG;
+}
+
+int zenu_hip_relu(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other, double alpha,
+                  zenu_stream_t stream)
+{
+    int rc = check2(to, other);
+    if (!rc) rc = ensure_init();
+    if (rc) return rc;
+    if (!same_shape(*to, *other)) return ZENU_ERR_SHAPE;  // "shape mismatch"
+    if (dtype == ZENU_F32) { ReluF<float> f; f.alpha = (float)alpha; return run1<float>(*to, *other, f, as_stream(stream)); }
+    if (dtype == ZENU_F64) { ReluF<double> f; f.alpha = alpha; return run1<double>(*to, *other, f, as_stream(stream)); }
+    return ZENU_ERR_ARG;
+}
+
+int zenu_hip_relu_backward_mask(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other,
+                                double alpha, zenu_stream_t stream)
+{
+    int rc = check2(to, other);
+    if (!rc) rc = ensure_init();
+    if (rc) return rc;
+    if (!same_shape(*to, *other)) return ZENU_ERR_SHAPE;
+    if (dtype == ZENU_F32) { ReluMaskF<float> f; f.alpha = (float)alpha; return run1<float>(*to, *other, f, as_stream(stream)); }
+    if (dtype == ZENU_F64) { ReluMaskF<double> f; f.alpha = alpha; return run1<double>(*to, *other, f, as_stream(stream)); }
+    return ZENU_ERR_ARG;
+}
+
+int zenu_hip_copy(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *src, zenu_stream_t stream)
+{
+    int rc = check2(to, src);
+    if (!rc) rc = ensure_init();
+    if (rc) return rc;
+    if (!same_shape(*to, *src)) return ZENU_ERR_SHAPE;
+    if (dtype == ZENU_F32) return run1<float>(*to, *src, CopyF<float>(), as_stream(stream));
+    if (dtype == ZENU_F64) return run1<double>(*to, *src, CopyF<double>(), as_stream(stream));
+    return ZENU_ERR_ARG;
+}
+
+}  // extern "C"

@@ -1,0 +1,812 @@
+// reduce.hip -- axis reductions for gfx950: sum, asum, max, arg-max (first index wins ties).
+//
+// The reference reduces by host recursion: `sum` issues shape[axis] whole-slice `+=` launches
+// (zenu-matrix/src/operation/sum.rs:12-31) and `max_axis` one alloc + copy + kernel + two
+// blocking single-element copies per output element (zenu-matrix/src/operation/max.rs:45-99).
+// Here a contiguous source is seen as [outer, R, inner] with R the reduced axis and one of two
+// kernels runs:
+//
+//   rows : inner == 1 (the reduced axis is contiguous) -- one workgroup (or one wavefront when
+//          the row is short) per row, 128-bit loads, four independent accumulators per lane,
+//          wave64 butterfly built from DPP (quad_perm, row_half_mirror, row_mirror), ds_swizzle
+//          and one cross-half exchange, then a fixed-order combine of the 4 waves through LDS.
+//          Also used with an element stride for small `inner`.
+//   cols : inner > 1 -- a 64 x 4 thread tile: 64 lanes own 64 column vectors (coalesced 128-bit
+//          loads), 4 row lanes walk the reduced axis, combined through LDS in fixed order.
+//
+// Both kernels can split the reduced axis over several workgroups; the partial results go to a
+// small workspace and a second launch of the SAME kernel folds them.  No atomics touch data:
+// the combination tree is fixed by the launch geometry, so results are bit-reproducible.
+//
+// Arg-max follows MaxIdx for Cpu (max.rs:19-34): start from element 0 and replace on strict '>'.
+// That is "largest value, lowest index on ties", except for NaN: a NaN at position 0 is never
+// replaced, a NaN anywhere else never replaces.  Mapping NaN to +inf at position 0 and to -inf
+// elsewhere turns the scan into an associative, commutative (key, index) maximum that any tree
+// reproduces; the value written is re-read from the source at the winning index so its bits
+// (NaN payload, sign of zero) are the source's.
+#include <math.h>
+
+#include "common.hpp"
+
+namespace zenu {
+
+// out[o] = src[q * outer_stride + c + idx[o] * elem_stride] with o = q * inner + c
+int gather_axis(const void *src, const int64_t *idx, void *out, int64_t nout, int64_t inner,
+                int64_t outer_stride, int64_t elem_stride, int elem_size, hipStream_t s);
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWave = 64;
+constexpr int kWaves = kBlock / kWave;
+
+template <typename T> struct VecOf;
+template <> struct VecOf<float> { typedef float4 type; static constexpr int N = 4; };
+template <> struct VecOf<double> { typedef double2 type; static constexpr int N = 2; };
+
+// ---- wave64 exchange primitives (word-wise so any POD accumulator works) ---------------------------
+
+template <int CTRL> __device__ __forceinline__ int dpp_word(int v)
+{
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false);
+}
+
+enum { kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140 };
+
+template <typename A, typename WordFn> __device__ __forceinline__ A map_words(A v, WordFn fn)
+{
+    static_assert(sizeof(A) % 4 == 0, "accumulator must be a multiple of 4 bytes");
+    constexpr int W = sizeof(A) / 4;
+    int w[W];
+    __builtin_memcpy(w, &v, sizeof(A));
+#pragma unroll
+    for (int i = 0; i < W; i++) w[i] = fn(w[i]);
+    A r;
+    __builtin_memcpy(&r, w, sizeof(A));
+    return r;
+}
+
+// After this every lane of the wavefront holds the reduction of all 64 lanes.  The merge
+// operator must be commutative so both partners compute identical bits.
+template <typename Tr> __device__ __forceinline__ typename Tr::Acc wave_allreduce(typename Tr::Acc a)
+{
+    typedef typename Tr::Acc A;
+    a = Tr::merge(a, map_words<A>(a, [](int w) { return dpp_word<kDppXor1>(w); }));
+    a = Tr::merge(a, map_words<A>(a, [](int w) { return dpp_word<kDppXor2>(w); }));
+    a = Tr::merge(a, map_words<A>(a, [](int w) { return dpp_word<kDppHalfMirror>(w); }));
+    a = Tr::merge(a, map_words<A>(a, [](int w) { return dpp_word<kDppMirror>(w); }));
+    // lane ^ 16 inside each half: ds_swizzle bit mode (and 0x1f, or 0, xor 0x10)
+    a = Tr::merge(a, map_words<A>(a, [](int w) { return __builtin_amdgcn_ds_swizzle(w, 0x401F); }));
+    // lane ^ 32: the two halves of the wavefront
+    a = Tr::merge(a, map_words<A>(a, [](int w) { return __shfl_xor(w, 32, kWave); }));
+    return a;
+}
+
+// Block-wide reduction; the result is valid in every thread.
+template <typename Tr> __device__ __forceinline__ typename Tr::Acc block_allreduce(typename Tr::Acc a)
+{
+    typedef typename Tr::Acc A;
+    __shared__ A lds[kWaves];
+    a = wave_allreduce<Tr>(a);
+    const int wave = threadIdx.x / kWave;
+    if ((threadIdx.x & (kWave - 1)) == 0) lds[wave] = a;
+    __syncthreads();
+    A r = lds[0];
+#pragma unroll
+    for (int w = 1; w < kWaves; w++) r = Tr::merge(r, lds[w]);
+    __syncthreads();
+    return r;
+}
+
+// ---- accumulator traits ------------------------------------------------------------------------------
+
+template <typename T> struct SumTr {
+    typedef T Acc;
+    static constexpr bool kHasIdx = false;
+    __device__ __forceinline__ static Acc identity() { return (T)0; }
+    __device__ __forceinline__ static Acc from_elem(T x, int64_t) { return x; }
+    __device__ __forceinline__ static Acc from_partial(T x, int64_t) { return x; }
+    __device__ __forceinline__ static Acc merge(Acc a, Acc b) { return a + b; }
+    __device__ __forceinline__ static T key(Acc a) { return a; }
+    __device__ __forceinline__ static int64_t idx(Acc) { return 0; }
+};
+
+template <typename T> struct AsumTr : SumTr<T> {
+    __device__ __forceinline__ static T from_elem(T x, int64_t) { return fabs(x); }
+};
+
+template <typename T> struct ArgPair {
+    T key;
+    int64_t idx;
+};
+
+template <typename T> struct ArgmaxTr {
+    typedef ArgPair<T> Acc;
+    static constexpr bool kHasIdx = true;
+    __device__ __forceinline__ static Acc identity()
+    {
+        Acc a;
+        a.key = -INFINITY;
+        a.idx = 0x7fffffffffffffffLL;
+        return a;
+    }
+    __device__ __forceinline__ static Acc from_elem(T x, int64_t pos)
+    {
+        Acc a;
+        a.key = (x != x) ? (pos == 0 ? (T)INFINITY : (T)-INFINITY) : x;
+        a.idx = pos;
+        return a;
+    }
+    __device__ __forceinline__ static Acc from_partial(T k, int64_t i)
+    {
+        Acc a;
+        a.key = k;
+        a.idx = i;
+        return a;
+    }
+    __device__ __forceinline__ static Acc merge(Acc a, Acc b)
+    {
+        const bool take_b = (b.key > a.key) || (b.key == a.key && b.idx < a.idx);
+        return take_b ? b : a;
+    }
+    __device__ __forceinline__ static T key(Acc a) { return a.key; }
+    __device__ __forceinline__ static int64_t idx(Acc a) { return a.idx; }
+};
+
+// ---- kernel parameters ---------------------------------------------------------------------------------
+
+template <typename T> struct RedParams {
+    const T *in;             // source values, or partial keys on a folding pass
+    const int64_t *in_idx;   // partial indices on a folding pass (arg-max only)
+    // geometry: output element o = (q, c) with q = o / inner, c = o % inner;
+    // its R values sit at in[q * outer_stride + c + r * elem_stride]
+    int64_t nout;            // number of outputs = outer * inner
+    int64_t R;               // reduced length
+    int64_t inner;
+    int64_t outer_stride;
+    int64_t elem_stride;
+    int splits;              // workgroups along R
+    int64_t seg;             // R elements per split
+    // results
+    T *out_val;              // final value (may be null)
+    int64_t *out_idx;        // final index (may be null)
+    T *part_key;             // partial outputs when splits > 1
+    int64_t *part_idx;
+    // value gather for max: value = gsrc[q * g_outer_stride + c + idx * g_elem_stride]
+    const T *gsrc;
+    int64_t g_outer_stride, g_elem_stride;
+};
+
+template <typename T, typename Tr>
+__device__ __forceinline__ void emit(const RedParams<T> &p, int64_t o, int split, typename Tr::Acc r)
+{
+    if (p.splits > 1) {
+        p.part_key[o * p.splits + split] = Tr::key(r);
+        if (Tr::kHasIdx) p.part_idx[o * p.splits + split] = Tr::idx(r);
+        return;
+    }
+    if (Tr::kHasIdx) {
+        if (p.out_idx) p.out_idx[o] = Tr::idx(r);
+        if (p.out_val) {
+            const int64_t q = o / p.inner, c = o - q * p.inner;
+            p.out_val[o] = p.gsrc[q * p.g_outer_stride + c + Tr::idx(r) * p.g_elem_stride];
+        }
+    } else {
+        p.out_val[o] = Tr::key(r);
+    }
+}
+
+// ---- kernel A: rows --------------------------------------------------------------------------------------
+// VEC > 1 requires elem_stride == 1, 16-byte aligned rows and seg % VEC == 0 (checked on the host).
+// WAVE_ROW: one wavefront per output (4 outputs per workgroup), otherwise one workgroup per
+// (output, split).
+
+template <typename T, typename Tr, int VEC, bool WAVE_ROW, bool FOLD>
+__global__ __launch_bounds__(kBlock) void reduce_rows_kernel(RedParams<T> p)
+{
+    typedef typename Tr::Acc A;
+    const int lane_n = WAVE_ROW ? kWave : kBlock;
+    const int lane = WAVE_ROW ? (threadIdx.x & (kWave - 1)) : threadIdx.x;
+    int64_t o;
+    int split;
+    if (WAVE_ROW) {
+        o = (int64_t)blockIdx.x * kWaves + threadIdx.x / kWave;
+        split = 0;
+    } else {
+        o = (int64_t)blockIdx.x / p.splits;
+        split = (int)(blockIdx.x - o * p.splits);
+    }
+    const bool active = o < p.nout;
+    A acc[4] = {Tr::identity(), Tr::identity(), Tr::identity(), Tr::identity()};
+    if (active) {
+        const int64_t q = o / p.inner, c = o - q * p.inner;
+        const int64_t base = q * p.outer_stride + c;
+        const int64_t r0 = (int64_t)split * p.seg;
+        int64_t r1 = r0 + p.seg;
+        if (r1 > p.R) r1 = p.R;
+        if (VEC > 1) {
+            typedef typename VecOf<T>::type V;
+            const T *row = p.in + base;
+            const int64_t step = (int64_t)lane_n * VEC;
+            int64_t r = r0 + (int64_t)lane * VEC;
+            // four vectors in flight per lane
+            for (; r + 3 * step + VEC <= r1; r += 4 * step) {
+                V x0 = *reinterpret_cast<const V *>(row + r);
+                V x1 = *reinterpret_cast<const V *>(row + r + step);
+                V x2 = *reinterpret_cast<const V *>(row + r + 2 * step);
+                V x3 = *reinterpret_cast<const V *>(row + r + 3 * step);
+                T e0[VEC], e1[VEC], e2[VEC], e3[VEC];
+                __builtin_memcpy(e0, &x0, sizeof(V));
+                __builtin_memcpy(e1, &x1, sizeof(V));
+                __builtin_memcpy(e2, &x2, sizeof(V));
+                __builtin_memcpy(e3, &x3, sizeof(V));
+#pragma unroll
+                for (int j = 0; j < VEC; j++) {
+                    acc[0] = Tr::merge(acc[0], Tr::from_elem(e0[j], r + j));
+                    acc[1] = Tr::merge(acc[1], Tr::from_elem(e1[j], r + step + j));
+                    acc[2] = Tr::merge(acc[2], Tr::from_elem(e2[j], r + 2 * step + j));
+                    acc[3] = Tr::merge(acc[3], Tr::from_elem(e3[j], r + 3 * step + j));
+                }
+            }
+            for (; r + VEC <= r1; r += step) {
+                V x0 = *reinterpret_cast<const V *>(row + r);
+                T e0[VEC];
+                __builtin_memcpy(e0, &x0, sizeof(V));
+#pragma unroll
+                for (int j = 0; j < VEC; j++) acc[0] = Tr::merge(acc[0], Tr::from_elem(e0[j], r + j));
+            }
+            // ragged end of the row (R % VEC != 0 only happens on the last split)
+            if (r < r1)
+                for (int j = 0; r + j < r1; j++)
+                    acc[0] = Tr::merge(acc[0], Tr::from_elem(row[r + j], r + j));
+        } else {
+            int64_t r = r0 + lane;
+            for (; r + 3 * (int64_t)lane_n < r1; r += 4 * (int64_t)lane_n) {
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int64_t rr = r + (int64_t)u * lane_n;
+                    const int64_t off = base + rr * p.elem_stride;
+                    acc[u] = Tr::merge(acc[u], FOLD ? Tr::from_partial(p.in[off], Tr::kHasIdx ? p.in_idx[off] : 0)
+                                                    : Tr::from_elem(p.in[off], rr));
+                }
+            }
+            for (; r < r1; r += lane_n) {
+                const int64_t off = base + r * p.elem_stride;
+                acc[0] = Tr::merge(acc[0], FOLD ? Tr::from_partial(p.in[off], Tr::kHasIdx ? p.in_idx[off] : 0)
+                                                : Tr::from_elem(p.in[off], r));
+            }
+        }
+    }
+    A a = Tr::merge(Tr::merge(acc[0], acc[1]), Tr::merge(acc[2], acc[3]));
+    if (WAVE_ROW) {
+        a = wave_allreduce<Tr>(a);
+        if (active && lane == 0) emit<T, Tr>(p, o, 0, a);
+    } else {
+        a = block_allreduce<Tr>(a);
+        if (active && lane == 0) emit<T, Tr>(p, o, split, a);
+    }
+}
+
+// ---- kernel B: cols ---------------------------------------------------------------------------------------
+// Source [outer, R, inner], inner contiguous.  Thread (tx, ty): tx in 0..63 owns VEC columns,
+// ty in 0..3 walks rows ty, ty+4, ... of its split.  grid = outer * col_tiles * splits.
+
+template <typename T, typename Tr, int VEC, bool FOLD>
+__global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int64_t col_tiles)
+{
+    typedef typename Tr::Acc A;
+    constexpr int TY = kBlock / kWave;
+    const int tx = threadIdx.x & (kWave - 1);
+    const int ty = threadIdx.x / kWave;
+    int64_t blk = blockIdx.x;
+    const int split = (int)(blk % p.splits);
+    blk /= p.splits;
+    const int64_t ct = blk % col_tiles;
+    const int64_t q = blk / col_tiles;
+    const int64_t c = (ct * kWave + tx) * VEC;
+    const int64_t r0 = (int64_t)split * p.seg;
+    int64_t r1 = r0 + p.seg;
+    if (r1 > p.R) r1 = p.R;
+
+    A acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) acc[j] = Tr::identity();
+
+    const int ncol = (c + VEC <= p.inner) ? VEC : (c < p.inner ? (int)(p.inner - c) : 0);
+    const T *src = p.in + q * p.outer_stride + c;
+    const int64_t *srci = FOLD && Tr::kHasIdx ? p.in_idx + q * p.outer_stride + c : nullptr;
+    if (ncol == VEC && VEC > 1 && !FOLD) {
+        typedef typename VecOf<T>::type V;
+        int64_t r = r0 + ty;
+        for (; r + 3 * TY < r1; r += 4 * TY) {
+            V x[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) x[u] = *reinterpret_cast<const V *>(src + (r + u * TY) * p.elem_stride);
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                T e[VEC];
+                __builtin_memcpy(e, &x[u], sizeof(V));
+#pragma unroll
+                for (int j = 0; j < VEC; j++) acc[j] = Tr::merge(acc[j], Tr::from_elem(e[j], r + u * TY));
+            }
+        }
+        for (; r < r1; r += TY) {
+            V x = *reinterpret_cast<const V *>(src + r * p.elem_stride);
+            T e[VEC];
+            __builtin_memcpy(e, &x, sizeof(V));
+#pragma unroll
+            for (int j = 0; j < VEC; j++) acc[j] = Tr::merge(acc[j], Tr::from_elem(e[j], r));
+        }
+    } else if (ncol > 0) {
+        for (int64_t r = r0 + ty; r < r1; r += TY) {
+            for (int j = 0; j < ncol; j++) {
+                const int64_t off = r * p.elem_stride + j;
+                acc[j] = Tr::merge(acc[j], FOLD ? Tr::from_partial(src[off], Tr::kHasIdx ? srci[off] : 0)
+                                                : Tr::from_elem(src[off], r));
+            }
+        }
+    }
+
+    // combine the TY row lanes in fixed order
+    __shared__ A lds[TY][kWave][VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) lds[ty][tx][j] = acc[j];
+    __syncthreads();
+    if (ty == 0) {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            A r = lds[0][tx][j];
+#pragma unroll
+            for (int w = 1; w < TY; w++) r = Tr::merge(r, lds[w][tx][j]);
+            if (j < ncol) emit<T, Tr>(p, q * p.inner + c + j, split, r);
+        }
+    }
+}
+
+// ---- host side ---------------------------------------------------------------------------------------------
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+template <typename T, typename Tr, bool FOLD>
+int launch_rows(const RedParams<T> &p, hipStream_t s)
+{
+    constexpr int VEC = VecOf<T>::N;
+    const bool vec = !FOLD && p.elem_stride == 1 && p.inner == 1 && aligned16(p.in) &&
+                     p.outer_stride % VEC == 0 && p.seg % VEC == 0;
+    const bool wave_row = p.splits == 1 && p.R <= 1024;
+    if (wave_row) {
+        int64_t grid = (p.nout + kWaves - 1) / kWaves;
+        if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
+        if (vec) reduce_rows_kernel<T, Tr, VEC, true, FOLD><<<(unsigned)grid, kBlock, 0, s>>>(p);
+        else     reduce_rows_kernel<T, Tr, 1, true, FOLD><<<(unsigned)grid, kBlock, 0, s>>>(p);
+    } else {
+        int64_t grid = p.nout * p.splits;
+        if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
+        if (vec) reduce_rows_kernel<T, Tr, VEC, false, FOLD><<<(unsigned)grid, kBlock, 0, s>>>(p);
+        else     reduce_rows_kernel<T, Tr, 1, false, FOLD><<<(unsigned)grid, kBlock, 0, s>>>(p);
+    }
+    ZENU_LAUNCH_CHECK();
+    return ZENU_OK;
+}
+
+template <typename T, typename Tr, bool FOLD>
+int launch_cols(const RedParams<T> &p, hipStream_t s)
+{
+    constexpr int VEC = VecOf<T>::N;
+    const bool vec = aligned16(p.in) && p.inner % VEC == 0 && p.outer_stride % VEC == 0 &&
+                     p.elem_stride % VEC == 0;
+    const int v = vec ? VEC : 1;
+    const int64_t col_tiles = (p.inner + (int64_t)kWave * v - 1) / ((int64_t)kWave * v);
+    const int64_t outer = p.nout / p.inner;
+    int64_t grid = outer * col_tiles * p.splits;
+    if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
+    if (vec) reduce_cols_kernel<T, Tr, VEC, FOLD><<<(unsigned)grid, kBlock, 0, s>>>(p, col_tiles);
+    else     reduce_cols_kernel<T, Tr, 1, FOLD><<<(unsigned)grid, kBlock, 0, s>>>(p, col_tiles);
+    ZENU_LAUNCH_CHECK();
+    return ZENU_OK;
+}
+
+// Reduce a contiguous [outer, R, inner] source into contiguous outputs of outer*inner elements.
+template <typename T, typename Tr>
+int reduce_contiguous(const T *src, int64_t outer, int64_t R, int64_t inner, T *out_val,
+                      int64_t *out_idx, hipStream_t s)
+{
+    constexpr int VEC = VecOf<T>::N;
+    const int64_t nout = outer * inner;
+    if (nout == 0) return ZENU_OK;
+    if (R <= 0) return ZENU_ERR_SHAPE;
+    const int64_t target_blocks = (int64_t)device_info().num_cus * 8;
+
+    RedParams<T> p;
+    p.in = src;
+    p.in_idx = nullptr;
+    p.nout = nout;
+    p.R = R;
+    p.inner = inner;
+    p.outer_stride = R * inner;
+    p.elem_stride = inner;
+    p.out_val = out_val;
+    p.out_idx = out_idx;
+    p.part_key = nullptr;
+    p.part_idx = nullptr;
+    p.gsrc = src;
+    p.g_outer_stride = R * inner;
+    p.g_elem_stride = inner;
+
+    const bool use_cols = inner >= 16;
+    int64_t splits = 1;
+    if (use_cols) {
+        const int64_t col_tiles = (inner + (int64_t)kWave * VEC - 1) / ((int64_t)kWave * VEC);
+        const int64_t blocks = outer * col_tiles;
+        if (blocks < target_blocks) {
+            splits = (target_blocks + blocks - 1) / blocks;
+            const int64_t max_splits = (R + 31) / 32;  // at least 32 rows per workgroup
+            if (splits > max_splits) splits = max_splits;
+        }
+    } else {
+        if (nout < target_blocks) {
+            splits = (target_blocks + nout - 1) / nout;
+            const int64_t per_block = (int64_t)kBlock * VEC * 8;  // keep >= 8 vectors per lane
+            const int64_t max_splits = (R + per_block - 1) / per_block;
+            if (splits > max_splits) splits = max_splits;
+        }
+    }
+    if (splits < 1) splits = 1;
+    if (splits > 4096) splits = 4096;
+    int64_t seg = (R + splits - 1) / splits;
+    seg = (seg + 15) / 16 * 16;  // keep vector alignment of every split
+    splits = (R + seg - 1) / seg;
+    p.splits = (int)splits;
+    p.seg = seg;
+
+    if (splits == 1) {
+        return use_cols ? launch_cols<T, Tr, false>(p, s) : launch_rows<T, Tr, false>(p, s);
+    }
+
+    // two launches: partials [nout, splits] in a workspace, then fold them
+    const size_t key_bytes = ((size_t)nout * splits * sizeof(T) + 255) / 256 * 256;
+    const size_t idx_bytes = Tr::kHasIdx ? (size_t)nout * splits * sizeof(int64_t) : 0;
+    Workspace ws(key_bytes + idx_bytes, s);
+    if (ws.status) return ws.status;
+    p.part_key = static_cast<T *>(ws.ptr);
+    p.part_idx = Tr::kHasIdx ? reinterpret_cast<int64_t *>(static_cast<char *>(ws.ptr) + key_bytes) : nullptr;
+    int rc = use_cols ? launch_cols<T, Tr, false>(p, s) : launch_rows<T, Tr, false>(p, s);
+    if (rc) return rc;
+
+    RedParams<T> f = p;
+    f.in = p.part_key;
+    f.in_idx = p.part_idx;
+    f.R = splits;
+    f.inner = 1;           // partials are [nout, splits]: a rows problem
+    f.outer_stride = splits;
+    f.elem_stride = 1;
+    f.splits = 1;
+    f.seg = (splits + 15) / 16 * 16;
+    f.part_key = nullptr;
+    f.part_idx = nullptr;
+    // the value gather still addresses the original source: output o = (q, c)
+    // (emit() derives q and c from f.inner, so keep the source geometry for the gather)
+    if (Tr::kHasIdx && out_val) {
+        // gather needs the original inner; run the fold for indices only, then gather below
+        Workspace wi(out_idx ? 0 : (size_t)nout * sizeof(int64_t), s);
+        int64_t *idx_buf = out_idx;
+        if (!idx_buf) {
+            if (wi.status) return wi.status;
+            idx_buf = static_cast<int64_t *>(wi.ptr);
+        }
+        f.out_val = nullptr;
+        f.out_idx = idx_buf;
+        rc = launch_rows<T, Tr, true>(f, s);
+        if (rc) return rc;
+        return gather_axis(src, idx_buf, out_val, nout, inner, R * inner, inner, (int)sizeof(T), s);
+    }
+    return launch_rows<T, Tr, true>(f, s);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void gather_axis_kernel(const T *src, const int64_t *idx, T *out,
+                                                             int64_t nout, int64_t inner,
+                                                             int64_t outer_stride, int64_t elem_stride)
+{
+    int64_t o = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (o >= nout) return;
+    const int64_t q = o / inner, c = o - q * inner;
+    out[o] = src[q * outer_stride + c + idx[o] * elem_stride];
+}
+
+}  // namespace
+
+int gather_axis(const void *src, const int64_t *idx, void *out, int64_t nout, int64_t inner,
+                int64_t outer_stride, int64_t elem_stride, int elem_size, hipStream_t s)
+{
+    int64_t grid = (nout + kBlock - 1) / kBlock;
+    if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
+    if (elem_size == 4)
+        gather_axis_kernel<float><<<(unsigned)grid, kBlock, 0, s>>>(
+            static_cast<const float *>(src), idx, static_cast<float *>(out), nout, inner, outer_stride,
+            elem_stride);
+    else
+        gather_axis_kernel<double><<<(unsigned)grid, kBlock, 0, s>>>(
+            static_cast<const double *>(src), idx, static_cast<double *>(out), nout, inner, outer_stride,
+            elem_stride);
+    ZENU_LAUNCH_CHECK();
+    return ZENU_OK;
+}
+
+namespace {
+
+// ---- tensor-level wrappers ------------------------------------------------------------------------------------
+
+zenu_tensor_t default_view(void *ptr, int ndim, const int64_t *shape)
+{
+    zenu_tensor_t t;
+    t.ptr = ptr;
+    t.ndim = ndim;
+    t.reserved = 0;
+    int64_t s = 1;
+    for (int i = 0; i < kMaxDim; i++) { t.shape[i] = 0; t.stride[i] = 0; }
+    for (int i = ndim - 1; i >= 0; i--) {
+        t.shape[i] = shape[i];
+        t.stride[i] = s;
+        s *= shape[i];
+    }
+    return t;
+}
+
+// out must hold src's shape minus `axis`, or with that axis kept as 1 (keep_dim)
+bool reduced_shape_ok(const zenu_tensor_t &out, const zenu_tensor_t &src, int axis)
+{
+    if (out.ndim == src.ndim - 1) {
+        int k = 0;
+        for (int i = 0; i < src.ndim; i++) {
+            if (i == axis) continue;
+            if (out.shape[k++] != src.shape[i]) return false;
+        }
+        return true;
+    }
+    if (out.ndim == src.ndim) {
+        for (int i = 0; i < src.ndim; i++)
+            if (out.shape[i] != (i == axis ? 1 : src.shape[i])) return false;
+        return true;
+    }
+    return false;
+}
+
+enum RedKind { kSum, kAsum, kMax };
+
+template <typename T>
+int reduce_axis_t(int kind, int dtype, const zenu_tensor_t *out, int64_t *out_idx,
+                  const zenu_tensor_t &src, int axis, hipStream_t s)
+{
+    const int64_t n = num_elm(src);
+    // contiguous source, or a contiguous copy of it (to_default_stride, as max.rs:49 does)
+    const T *sp = static_cast<const T *>(src.ptr);
+    Workspace wsrc(is_default_stride_strict(src) ? 0 : (size_t)n * sizeof(T), s);
+    if (!is_default_stride_strict(src)) {
+        if (wsrc.status) return wsrc.status;
+        zenu_tensor_t tmp = default_view(wsrc.ptr, src.ndim, src.shape);
+        int rc = zenu_hip_copy(dtype, &tmp, &src, s);
+        if (rc) return rc;
+        sp = static_cast<const T *>(wsrc.ptr);
+    }
+    int64_t outer = 1, inner = 1;
+    for (int i = 0; i < axis; i++) outer *= src.shape[i];
+    for (int i = axis + 1; i < src.ndim; i++) inner *= src.shape[i];
+    const int64_t R = src.shape[axis];
+    const int64_t nout = outer * inner;
+
+    // contiguous destination, or a temporary that is copied out afterwards
+    T *ov = nullptr;
+    bool need_copy = false;
+    Workspace wout((out && !is_default_stride_strict(*out)) ? (size_t)(nout ? nout : 1) * sizeof(T) : 0, s);
+    if (out) {
+        if (is_default_stride_strict(*out)) {
+            ov = static_cast<T *>(out->ptr);
+        } else {
+            if (wout.status) return wout.status;
+            ov = static_cast<T *>(wout.ptr);
+            need_copy = true;
+        }
+    }
+    int rc;
+    if (kind == kSum) rc = reduce_contiguous<T, SumTr<T>>(sp, outer, R, inner, ov, nullptr, s);
+    else if (kind == kAsum) rc = reduce_contiguous<T, AsumTr<T>>(sp, outer, R, inner, ov, nullptr, s);
+    else rc = reduce_contiguous<T, ArgmaxTr<T>>(sp, outer, R, inner, ov, out_idx, s);
+    if (rc) return rc;
+    if (need_copy) {
+        zenu_tensor_t tmp = default_view(ov, out->ndim, out->shape);
+        rc = zenu_hip_copy(dtype, out, &tmp, s);
+    }
+    return rc;
+}
+
+int reduce_axis(int kind, int dtype, const zenu_tensor_t *out, int64_t *out_idx, const zenu_tensor_t *src,
+                int axis, hipStream_t s)
+{
+    int rc = validate_tensor(src);
+    if (!rc && out) rc = validate_tensor(out);
+    if (!rc) rc = ensure_init();
+    if (rc) return rc;
+    if (axis < 0 || axis >= src->ndim) return ZENU_ERR_AXIS;
+    if (out && !reduced_shape_ok(*out, *src, axis)) return ZENU_ERR_SHAPE;
+    if (dtype == ZENU_F32) return reduce_axis_t<float>(kind, dtype, out, out_idx, *src, axis, s);
+    if (dtype == ZENU_F64) return reduce_axis_t<double>(kind, dtype, out, out_idx, *src, axis, s);
+    return ZENU_ERR_ARG;
+}
+
+// whole-tensor reductions: view the (contiguous copy of the) source as one row
+int reduce_all(int kind, int dtype, void *out_val, int64_t *out_idx, const zenu_tensor_t *src, hipStream_t s)
+{
+    int rc = validate_tensor(src);
+    if (!rc) rc = ensure_init();
+    if (rc) return rc;
+    const int64_t n = num_elm(*src);
+    if (n <= 0) return ZENU_ERR_SHAPE;
+    zenu_tensor_t flat;
+    const size_t esz = dtype == ZENU_F32 ? 4 : 8;
+    if (dtype != ZENU_F32 && dtype != ZENU_F64) return ZENU_ERR_ARG;
+    Workspace wsrc(is_default_stride_strict(*src) ? 0 : (size_t)n * esz, s);
+    const void *sp = src->ptr;
+    if (!is_default_stride_strict(*src)) {
+        if (wsrc.status) return wsrc.status;
+        zenu_tensor_t tmp = default_view(wsrc.ptr, src->ndim, src->shape);
+        rc = zenu_hip_copy(dtype, &tmp, src, s);
+        if (rc) return rc;
+        sp = wsrc.ptr;
+    }
+    (void)flat;
+    if (dtype == ZENU_F32) {
+        const float *f = static_cast<const float *>(sp);
+        float *ov = static_cast<float *>(out_val);
+        if (kind == kSum) return reduce_contiguous<float, SumTr<float>>(f, 1, n, 1, ov, nullptr, s);
+        if (kind == kAsum) return reduce_contiguous<float, AsumTr<float>>(f, 1, n, 1, ov, nullptr, s);
+        return reduce_contiguous<float, ArgmaxTr<float>>(f, 1, n, 1, ov, out_idx, s);
+    }
+    const double *d = static_cast<const double *>(sp);
+    double *ov = static_cast<double *>(out_val);
+    if (kind == kSum) return reduce_contiguous<double, SumTr<double>>(d, 1, n, 1, ov, nullptr, s);
+    if (kind == kAsum) return reduce_contiguous<double, AsumTr<double>>(d, 1, n, 1, ov, nullptr, s);
+    return reduce_contiguous<double, ArgmaxTr<double>>(d, 1, n, 1, ov, out_idx, s);
+}
+
+}  // namespace
+}  // namespace zenu
+
+using namespace zenu;
+
+extern "C" {
+
+int zenu_hip_sum_axis(int dtype, const zenu_tensor_t *out, const zenu_tensor_t *src, int axis,
+                      zenu_stream_t stream)
+{
+    if (!out) return ZENU_ERR_ARG;
+    return reduce_axis(kSum, dtype, out, nullptr, src, axis, as_stream(stream));
+}
+
+int zenu_hip_sum_all(int dtype, void *out_dev, const zenu_tensor_t *src, zenu_stream_t stream)
+{
+    if (!out_dev) return ZENU_ERR_ARG;
+    return reduce_all(kSum, dtype, out_dev, nullptr, src, as_stream(stream));
+}
+
+// ShapeStride::is_contiguous (zenu-matrix/src/shape_stride.rs:65-83) on dims k.. of `t`
+static bool ref_is_contiguous(const zenu_tensor_t &t, int k)
+{
+    const int nd = t.ndim - k;
+    if (nd <= 0) return true;
+    int order[kMaxDim];
+    for (int i = 0; i < nd; i++) order[i] = k + i;
+    for (int i = 1; i < nd; i++) {  // stable, by decreasing stride
+        int o = order[i], j = i - 1;
+        while (j >= 0 && t.stride[order[j]] < t.stride[o]) { order[j + 1] = order[j]; j--; }
+        order[j + 1] = o;
+    }
+    int64_t d[kMaxDim];
+    d[nd - 1] = 1;
+    for (int i = nd - 2; i >= 0; i--) d[i] = d[i + 1] * t.shape[order[i + 1]];
+    const int64_t s0 = t.stride[order[0]];
+    if (s0 == 0 || d[0] % s0 != 0) return false;
+    const int64_t n = d[0] / s0;
+    for (int i = 0; i < nd; i++)
+        if (d[i] * n != t.stride[order[i]]) return false;
+    return true;
+}
+
+int zenu_hip_asum(int dtype, void *out_dev, const zenu_tensor_t *src, zenu_stream_t stream)
+{
+    if (!out_dev) return ZENU_ERR_ARG;
+    int rc = validate_tensor(src);
+    if (rc) return rc;
+    // Matrix::asum (asum.rs:49-68) peels leading axes until the remaining view is contiguous and
+    // sums |x| there; a view that never becomes contiguous bottoms out at 0-d items, which are
+    // returned raw (no abs).  Same result here, in one reduction.
+    if (src->ndim == 0) {
+        const size_t esz = dtype == ZENU_F32 ? 4 : 8;
+        return zenu_hip_memcpy_d2d(out_dev, src->ptr, esz, stream);
+    }
+    bool abs_sum = false;
+    for (int k = 0; k < src->ndim && !abs_sum; k++) abs_sum = ref_is_contiguous(*src, k);
+    return reduce_all(abs_sum ? kAsum : kSum, dtype, out_dev, nullptr, src, as_stream(stream));
+}
+
+int zenu_hip_max_axis(int dtype, const zenu_tensor_t *out, const zenu_tensor_t *src, int axis,
+                      zenu_stream_t stream)
+{
+    if (!out) return ZENU_ERR_ARG;
+    return reduce_axis(kMax, dtype, out, nullptr, src, axis, as_stream(stream));
+}
+
+int zenu_hip_max_axis_idx(int dtype, int64_t *out_idx_dev, const zenu_tensor_t *src, int axis,
+                          zenu_stream_t stream)
+{
+    if (!out_idx_dev) return ZENU_ERR_ARG;
+    return reduce_axis(kMax, dtype, nullptr, out_idx_dev, src, axis, as_stream(stream));
+}
+
+int zenu_hip_max_idx(int dtype, int64_t *out_flat_idx_dev, void *out_val_dev, const zenu_tensor_t *src,
+                     zenu_stream_t stream)
+{
+    if (!out_flat_idx_dev && !out_val_dev) return ZENU_ERR_ARG;
+    return reduce_all(kMax, dtype, out_val_dev, out_flat_idx_dev, src, as_stream(stream));
+}
+
+int zenu_hip_sum_to(int dtype, const zenu_tensor_t *target, const zenu_tensor_t *src, zenu_stream_t stream)
+{
+    // sum.rs:35-94
+    int rc = validate_tensor(src);
+    if (!rc) rc = validate_tensor(target);
+    if (!rc) rc = ensure_init();
+    if (rc) return rc;
+    if (dtype != ZENU_F32 && dtype != ZENU_F64) return ZENU_ERR_ARG;
+    if (src->ndim < target->ndim) return ZENU_ERR_RANK;
+    hipStream_t s = as_stream(stream);
+    if (same_shape(*src, *target)) return zenu_hip_copy(dtype, target, src, stream);
+    const size_t esz = dtype == ZENU_F32 ? 4 : 8;
+    const int diff = src->ndim - target->ndim;
+
+    // list of axes to reduce, in the order the reference reduces them
+    int axes[kMaxDim * 2], keep[kMaxDim * 2], na = 0;
+    if (diff == 0) {
+        for (int i = 0; i < src->ndim; i++) {
+            if (src->shape[i] == target->shape[i]) continue;
+            if (target->shape[i] != 1) return ZENU_ERR_SHAPE;
+            axes[na] = i; keep[na] = 1; na++;
+        }
+    } else {
+        // trailing dims must match exactly (is_include), leading axes are summed away
+        for (int i = 0; i < target->ndim; i++)
+            if (src->shape[diff + i] != target->shape[i]) return ZENU_ERR_SHAPE;
+        for (int i = 0; i < diff; i++) { axes[na] = 0; keep[na] = 0; na++; }
+    }
+
+    zenu_tensor_t cur = *src;
+    void *cur_buf = nullptr;  // workspace owning `cur`, if any
+    for (int a = 0; a < na; a++) {
+        int64_t oshape[kMaxDim];
+        int ond = 0;
+        for (int i = 0; i < cur.ndim; i++) {
+            if (i == axes[a]) { if (keep[a]) oshape[ond++] = 1; continue; }
+            oshape[ond++] = cur.shape[i];
+        }
+        const bool last = (a == na - 1);
+        zenu_tensor_t dst;
+        void *dst_buf = nullptr;
+        if (last) {
+            dst = *target;
+        } else {
+            int64_t cnt = 1;
+            for (int i = 0; i < ond; i++) cnt *= oshape[i];
+            rc = zenu_hip_malloc(&dst_buf, (size_t)(cnt ? cnt : 1) * esz, stream);
+            if (rc) { if (cur_buf) zenu_hip_free(cur_buf, stream); return rc; }
+            dst = default_view(dst_buf, ond, oshape);
+        }
+        rc = reduce_axis(kSum, dtype, &dst, nullptr, &cur, axes[a], s);
+        if (cur_buf) zenu_hip_free(cur_buf, stream);
+        cur_buf = dst_buf;
+        if (rc) { if (cur_buf) zenu_hip_free(cur_buf, stream); return rc; }
+        cur = dst;
+    }
+    return ZENU_OK;
+}
+
+}  // extern "C"

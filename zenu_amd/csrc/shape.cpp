@@ -1,0 +1,161 @@
+// shape.cpp -- host-side shape / stride / broadcast algebra of the tensor-kernel library.
+//
+// ZeNu resolves N-d, strided and broadcast operands by recursing over the leading axis and
+// issuing one 1-D kernel per row (zenu-matrix/src/with_clousers.rs:180-223).  Here the same
+// legality rules are checked once, the operands are folded into one iteration space, and a
+// single launch covers it.
+#include <algorithm>
+#include <utility>
+
+#include "common.hpp"
+
+namespace zenu {
+
+int validate_tensor(const zenu_tensor_t *t)
+{
+    if (!t) return ZENU_ERR_ARG;
+    if (t->ndim < 0 || t->ndim > kMaxDim) return ZENU_ERR_ARG;
+    for (int i = 0; i < t->ndim; i++)
+        if (t->shape[i] < 0 || t->stride[i] < 0) return ZENU_ERR_ARG;
+    if (!t->ptr && num_elm(*t) > 0) return ZENU_ERR_ARG;
+    return ZENU_OK;
+}
+
+bool same_shape(const zenu_tensor_t &a, const zenu_tensor_t &b)
+{
+    if (a.ndim != b.ndim) return false;
+    for (int i = 0; i < a.ndim; i++)
+        if (a.shape[i] != b.shape[i]) return false;
+    return true;
+}
+
+bool is_default_stride_strict(const zenu_tensor_t &t)
+{
+    int64_t s = 1;
+    for (int i = t.ndim - 1; i >= 0; i--) {
+        if (t.stride[i] != s) return false;
+        s *= t.shape[i];
+    }
+    return true;
+}
+
+// DimDyn::is_include, dim_dyn.rs:119-130: trailing dims equal.
+static bool dims_include(const zenu_tensor_t &s, const zenu_tensor_t &o)
+{
+    if (s.ndim < o.ndim) return dims_include(o, s);
+    for (int i = 0; i < o.ndim; i++)
+        if (s.shape[s.ndim - 1 - i] != o.shape[o.ndim - 1 - i]) return false;
+    return true;
+}
+
+// DimDyn::is_include_bradcast, dim_dyn.rs:137-148: trailing dims equal or 1 on the other side.
+static bool dims_include_broadcast(const zenu_tensor_t &s, const zenu_tensor_t &o)
+{
+    if (s.ndim < o.ndim) return false;
+    for (int i = 0; i < o.ndim; i++) {
+        int64_t od = o.shape[o.ndim - 1 - i];
+        if (s.shape[s.ndim - 1 - i] == od || od == 1) continue;
+        return false;
+    }
+    return true;
+}
+
+// larger_shape_is_x, dim_dyn.rs:24-47.  1: x larger, 0: y larger, -1: the reference panics.
+static int larger_is_x(const zenu_tensor_t &x, const zenu_tensor_t &y)
+{
+    if (x.ndim < y.ndim) return dims_include(y, x) ? 0 : -1;
+    if (x.ndim > y.ndim) return dims_include(x, y) ? 1 : -1;
+    if (dims_include_broadcast(x, y)) return 1;
+    if (dims_include_broadcast(y, x)) return 0;
+    return -1;
+}
+
+int check_binary(const zenu_tensor_t &to, const zenu_tensor_t &lhs, const zenu_tensor_t &rhs)
+{
+    // array_array_array_check, with_clousers.rs:155-178
+    int lx = larger_is_x(lhs, rhs);
+    if (lx < 0) return ZENU_ERR_SHAPE;
+    const zenu_tensor_t &larger = lx ? lhs : rhs;
+    const zenu_tensor_t &smaller = lx ? rhs : lhs;
+    if (!dims_include(larger, smaller)) {
+        if (to.ndim < smaller.ndim) return ZENU_ERR_RANK;
+        if (!dims_include_broadcast(to, smaller)) return ZENU_ERR_SHAPE;
+    }
+    // The reference also admits a destination shaped like the smaller operand, which its
+    // recursion then walks out of bounds; only the larger shape is accepted here.
+    if (!same_shape(to, larger)) return ZENU_ERR_SHAPE;
+    return ZENU_OK;
+}
+
+int check_binary_assign(const zenu_tensor_t &to, const zenu_tensor_t &rhs)
+{
+    // array_array_check, with_clousers.rs:87-107
+    if (to.ndim < rhs.ndim) return ZENU_ERR_RANK;
+    if (!dims_include_broadcast(to, rhs)) return ZENU_ERR_SHAPE;
+    return ZENU_OK;
+}
+
+void ew_set_operand(EwProblem &p, int slot, const zenu_tensor_t &t, int out_ndim,
+                    const int64_t *out_shape)
+{
+    p.ptr[slot] = t.ptr;
+    int lead = out_ndim - t.ndim;
+    for (int d = 0; d < out_ndim; d++) {
+        int td = d - lead;
+        if (td < 0) {
+            p.stride[slot][d] = 0;  // missing leading dim: get_tmp_matrix passes it through
+        } else if (t.shape[td] == 1 && out_shape[d] != 1) {
+            p.stride[slot][d] = 0;  // size-1 dim: index 0 every time (with_clousers.rs:16-17)
+        } else {
+            p.stride[slot][d] = t.stride[td];
+        }
+    }
+}
+
+void ew_collapse(EwProblem &p)
+{
+    p.numel = 1;
+    for (int d = 0; d < p.ndim; d++) p.numel *= p.shape[d];
+
+    // 1. drop size-1 dims
+    int nd = 0;
+    for (int d = 0; d < p.ndim; d++) {
+        if (p.shape[d] == 1) continue;
+        p.shape[nd] = p.shape[d];
+        for (int o = 0; o < p.nops; o++) p.stride[o][nd] = p.stride[o][d];
+        nd++;
+    }
+    p.ndim = nd;
+    if (nd == 0) return;
+
+    // 2. order dims by decreasing output stride (stable), so the output is written as
+    //    sequentially as its layout allows.  Elementwise work is order independent.
+    int order[kMaxDim];
+    for (int d = 0; d < nd; d++) order[d] = d;
+    std::stable_sort(order, order + nd,
+                     [&](int a, int b) { return p.stride[0][a] > p.stride[0][b]; });
+    EwProblem q = p;
+    for (int d = 0; d < nd; d++) {
+        p.shape[d] = q.shape[order[d]];
+        for (int o = 0; o < p.nops; o++) p.stride[o][d] = q.stride[o][order[d]];
+    }
+
+    // 3. merge dim d+1 into d when stride[d] == stride[d+1]*shape[d+1] for every operand
+    int w = 0;
+    for (int d = 1; d < nd; d++) {
+        bool mergeable = true;
+        for (int o = 0; o < p.nops; o++)
+            if (p.stride[o][w] != p.stride[o][d] * p.shape[d]) { mergeable = false; break; }
+        if (mergeable) {
+            p.shape[w] *= p.shape[d];
+            for (int o = 0; o < p.nops; o++) p.stride[o][w] = p.stride[o][d];
+        } else {
+            w++;
+            p.shape[w] = p.shape[d];
+            for (int o = 0; o < p.nops; o++) p.stride[o][w] = p.stride[o][d];
+        }
+    }
+    p.ndim = w + 1;
+}
+
+}  // namespace zenu

@@ -1,0 +1,143 @@
+// shims.cpp -- the reference's own 1-D entry points (zenu-cuda-kernel-sys/kernel/*.h), so the
+// unchanged wrappers of zenu-cuda/src/kernel/mod.rs and kernel/activation.rs link against this
+// library.  Same names, same argument order, `int` sizes and element strides, launches on the
+// null stream, no return value (the reference's functions return void and check nothing).
+// Each one forwards to the N-d entry point with a 1-D strided view.
+#include "common.hpp"
+
+namespace {
+
+zenu_tensor_t view1d(const void *p, int n, int stride)
+{
+    zenu_tensor_t t;
+    t.ptr = const_cast<void *>(p);
+    t.ndim = 1;
+    t.reserved = 0;
+    for (int i = 0; i < ZENU_MAX_DIM; i++) { t.shape[i] = 0; t.stride[i] = 0; }
+    t.shape[0] = n;
+    t.stride[0] = stride;
+    return t;
+}
+
+template <typename T> constexpr int dtype_of();
+template <> constexpr int dtype_of<float>() { return ZENU_F32; }
+template <> constexpr int dtype_of<double>() { return ZENU_F64; }
+
+template <typename T>
+void aa(int op, T *a, int sa, T *b, int sb, T *c, int sc, int n)
+{
+    zenu_tensor_t ta = view1d(a, n, sa), tb = view1d(b, n, sb), tc = view1d(c, n, sc);
+    (void)zenu_hip_binary(op, dtype_of<T>(), &tc, &ta, &tb, nullptr);
+}
+template <typename T> void aa_assign(int op, T *a, int sa, T *b, int sb, int n)
+{
+    zenu_tensor_t ta = view1d(a, n, sa), tb = view1d(b, n, sb);
+    (void)zenu_hip_binary_assign(op, dtype_of<T>(), &ta, &tb, nullptr);
+}
+template <typename T> void as(int op, T *a, int n, int sa, T s, T *out, int so)
+{
+    zenu_tensor_t ta = view1d(a, n, sa), to = view1d(out, n, so);
+    (void)zenu_hip_binary_scalar(op, dtype_of<T>(), &to, &ta, (double)s, nullptr);
+}
+template <typename T> void as_assign(int op, T *a, int n, int sa, T s)
+{
+    zenu_tensor_t ta = view1d(a, n, sa);
+    (void)zenu_hip_binary_scalar_assign(op, dtype_of<T>(), &ta, (double)s, nullptr);
+}
+template <typename T> void asp(int op, T *a, int n, int sa, T *s, T *out, int so)
+{
+    zenu_tensor_t ta = view1d(a, n, sa), to = view1d(out, n, so);
+    (void)zenu_hip_binary_scalar_ptr(op, dtype_of<T>(), &to, &ta, s, nullptr);
+}
+template <typename T> void asp_assign(int op, T *a, int n, int sa, T *s)
+{
+    zenu_tensor_t ta = view1d(a, n, sa);
+    (void)zenu_hip_binary_scalar_assign_ptr(op, dtype_of<T>(), &ta, s, nullptr);
+}
+template <typename T> void un(int fn, T *a, int n, int si, T *out, int so)
+{
+    zenu_tensor_t ta = view1d(a, n, si), to = view1d(out, n, so);
+    (void)zenu_hip_unary(fn, dtype_of<T>(), &to, &ta, nullptr);
+}
+template <typename T> void un_assign(int fn, T *a, int n, int s)
+{
+    zenu_tensor_t ta = view1d(a, n, s);
+    (void)zenu_hip_unary_assign(fn, dtype_of<T>(), &ta, nullptr);
+}
+
+template <typename T> void max_idx(T *a, int size, int stride, int *out)
+{
+    // `out` is host memory (zenu-cuda/src/kernel/mod.rs:570-588): blocking, like the reference
+    zenu_tensor_t ta = view1d(a, size, stride);
+    void *d = nullptr;
+    if (zenu_hip_malloc(&d, sizeof(int64_t), nullptr) != ZENU_OK) return;
+    int64_t h = 0;
+    if (zenu_hip_max_idx(dtype_of<T>(), static_cast<int64_t *>(d), nullptr, &ta, nullptr) == ZENU_OK &&
+        zenu_hip_memcpy_d2h(&h, d, sizeof h, nullptr) == ZENU_OK)
+        *out = (int)h;
+    (void)zenu_hip_free(d, nullptr);
+}
+
+}  // namespace
+
+extern "C" {
+
+#define ZENU_DEF_1D(T, S)                                                                                  \
+    void array_array_add_##S(T *a, int sa, T *b, int sb, T *c, int sc, int n) { aa<T>(ZENU_ADD, a, sa, b, sb, c, sc, n); } \
+    void array_array_sub_##S(T *a, int sa, T *b, int sb, T *c, int sc, int n) { aa<T>(ZENU_SUB, a, sa, b, sb, c, sc, n); } \
+    void array_array_mul_##S(T *a, int sa, T *b, int sb, T *c, int sc, int n) { aa<T>(ZENU_MUL, a, sa, b, sb, c, sc, n); } \
+    void array_array_div_##S(T *a, int sa, T *b, int sb, T *c, int sc, int n) { aa<T>(ZENU_DIV, a, sa, b, sb, c, sc, n); } \
+    void array_array_add_assign_##S(T *a, int sa, T *b, int sb, int n) { aa_assign<T>(ZENU_ADD, a, sa, b, sb, n); } \
+    void array_array_sub_assign_##S(T *a, int sa, T *b, int sb, int n) { aa_assign<T>(ZENU_SUB, a, sa, b, sb, n); } \
+    void array_array_mul_assign_##S(T *a, int sa, T *b, int sb, int n) { aa_assign<T>(ZENU_MUL, a, sa, b, sb, n); } \
+    void array_array_div_assign_##S(T *a, int sa, T *b, int sb, int n) { aa_assign<T>(ZENU_DIV, a, sa, b, sb, n); } \
+    void array_scalar_add_##S(T *a, int n, int sa, T s, T *o, int so) { as<T>(ZENU_ADD, a, n, sa, s, o, so); } \
+    void array_scalar_sub_##S(T *a, int n, int sa, T s, T *o, int so) { as<T>(ZENU_SUB, a, n, sa, s, o, so); } \
+    void array_scalar_mul_##S(T *a, int n, int sa, T s, T *o, int so) { as<T>(ZENU_MUL, a, n, sa, s, o, so); } \
+    void array_scalar_div_##S(T *a, int n, int sa, T s, T *o, int so) { as<T>(ZENU_DIV, a, n, sa, s, o, so); } \
+    void array_scalar_add_assign_##S(T *a, int n, int sa, T s) { as_assign<T>(ZENU_ADD, a, n, sa, s); } \
+    void array_scalar_sub_assign_##S(T *a, int n, int sa, T s) { as_assign<T>(ZENU_SUB, a, n, sa, s); } \
+    void array_scalar_mul_assign_##S(T *a, int n, int sa, T s) { as_assign<T>(ZENU_MUL, a, n, sa, s); } \
+    void array_scalar_div_assign_##S(T *a, int n, int sa, T s) { as_assign<T>(ZENU_DIV, a, n, sa, s); } \
+    void array_scalar_pointer_add_##S(T *a, int n, int sa, T *s, T *o, int so) { asp<T>(ZENU_ADD, a, n, sa, s, o, so); } \
+    void array_scalar_pointer_sub_##S(T *a, int n, int sa, T *s, T *o, int so) { asp<T>(ZENU_SUB, a, n, sa, s, o, so); } \
+    void array_scalar_pointer_mul_##S(T *a, int n, int sa, T *s, T *o, int so) { asp<T>(ZENU_MUL, a, n, sa, s, o, so); } \
+    void array_scalar_pointer_div_##S(T *a, int n, int sa, T *s, T *o, int so) { asp<T>(ZENU_DIV, a, n, sa, s, o, so); } \
+    void array_scalar_pointer_add_assign_##S(T *a, int n, int sa, T *s) { asp_assign<T>(ZENU_ADD, a, n, sa, s); } \
+    void array_scalar_pointer_sub_assign_##S(T *a, int n, int sa, T *s) { asp_assign<T>(ZENU_SUB, a, n, sa, s); } \
+    void array_scalar_pointer_mul_assign_##S(T *a, int n, int sa, T *s) { asp_assign<T>(ZENU_MUL, a, n, sa, s); } \
+    void array_scalar_pointer_div_assign_##S(T *a, int n, int sa, T *s) { asp_assign<T>(ZENU_DIV, a, n, sa, s); } \
+    void array_exp_##S(T *a, int n, int si, T *o, int so) { un<T>(ZENU_EXP, a, n, si, o, so); }            \
+    void array_log_##S(T *a, int n, int si, T *o, int so) { un<T>(ZENU_LOG, a, n, si, o, so); }            \
+    void array_tanh_##S(T *a, int n, int si, T *o, int so) { un<T>(ZENU_TANH, a, n, si, o, so); }          \
+    void array_sqrt_##S(T *a, int n, int si, T *o, int so) { un<T>(ZENU_SQRT, a, n, si, o, so); }          \
+    void array_abs_##S(T *a, int n, int si, T *o, int so) { un<T>(ZENU_ABS, a, n, si, o, so); }            \
+    void array_exp_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_EXP, a, n, s); }                     \
+    void array_log_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_LOG, a, n, s); }                     \
+    void array_tanh_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_TANH, a, n, s); }                   \
+    void array_sqrt_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_SQRT, a, n, s); }                   \
+    void array_abs_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_ABS, a, n, s); }                     \
+    void relu_##S(T *in, T *out, T alpha, int n, int si, int so)                                           \
+    {                                                                                                      \
+        zenu_tensor_t ti = view1d(in, n, si), to = view1d(out, n, so);                                     \
+        (void)zenu_hip_relu(dtype_of<T>(), &to, &ti, (double)alpha, nullptr);                              \
+    }                                                                                                      \
+    void relu_backward_mask_##S(T *in, T *mask, T alpha, int n, int si, int sm)                            \
+    {                                                                                                      \
+        zenu_tensor_t ti = view1d(in, n, si), tm = view1d(mask, n, sm);                                    \
+        (void)zenu_hip_relu_backward_mask(dtype_of<T>(), &tm, &ti, (double)alpha, nullptr);                \
+    }                                                                                                      \
+    void array_max_idx_##S(T *a, int size, int stride, int *out) { max_idx<T>(a, size, stride, out); }     \
+    void memory_access_##S(T *array, int offset, T *result)                                                \
+    {                                                                                                      \
+        (void)zenu_hip_memcpy_d2h(result, array + offset, sizeof(T), nullptr);                             \
+    }                                                                                                      \
+    void memory_set_##S(T *array, int offset, T value)                                                     \
+    {                                                                                                      \
+        (void)zenu_hip_memcpy_h2d(array + offset, &value, sizeof(T), nullptr);                             \
+    }
+
+ZENU_DEF_1D(float, float)
+ZENU_DEF_1D(double, double)
+
+}  // extern "C"

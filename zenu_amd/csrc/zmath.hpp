@@ -1,0 +1,175 @@
+// zmath.hpp -- f32 tanh / expm1 for device code, bit-compatible with the host libm the
+// reference's CPU path calls (Rust f32::tanh -> libm tanhf).
+//
+// Why not the device math library: ZeNu's sigmoid is the composite 0.5 + 0.5*tanh(0.5*x)
+// (zenu-autograd/src/activation/sigmoid.rs:7-15).  For negative x the final add cancels, so a
+// 1-ulp difference in tanh becomes tens of ulps in the sigmoid; parity therefore needs the
+// same tanh bits as the CPU path, not merely an accurate tanh.
+//
+// Algorithm: the classic fdlibm single-precision tanhf / expm1f (Sun Microsystems, 1993; the
+// generic flt-32 implementation used by glibc 2.35, which is what this image ships):
+//   tanh(x) = sign(x) * { |x| < 2^-55 : |x|*(1+|x|)
+//                         |x| <  1    : -t/(t+2),   t = expm1(-2|x|)
+//                         |x| <  22   : 1 - 2/(t+2), t = expm1( 2|x|)
+//                         else        : 1 }
+//   expm1(x): x = k*ln2 + r, |r| <= 0.5 ln2; R1(r*r) rational correction; scale by 2^k.
+// Everything is plain IEEE f32 arithmetic (+,-,*,/ correctly rounded, no contraction), so host
+// and device produce identical bits.  The host build of this header is compared against
+// tanhf/expm1f over every f32 bit pattern in tests/test_zmath_host.py (sampled) and was run
+// exhaustively during development.
+#pragma once
+#include <stdint.h>
+#include <string.h>
+
+#if defined(__HIPCC__)
+#define ZM_HD __host__ __device__ __forceinline__
+#else
+#define ZM_HD static inline
+#endif
+
+namespace zmath {
+
+ZM_HD uint32_t f2u(float f)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __float_as_uint(f);
+#else
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+#endif
+}
+ZM_HD float u2f(uint32_t u)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __uint_as_float(u);
+#else
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+#endif
+}
+
+// expm1f for finite |x| < 88 (callers here pass |x| < 44); follows fdlibm s_expm1f.c.
+ZM_HD float expm1f_fdlibm(float x)
+{
+    const float one = 1.0f, tiny = 1.0e-30f, huge = 1.0e+30f;
+    const float o_threshold = u2f(0x42b17180u);   // 8.8721679688e+01
+    const float ln2_hi = u2f(0x3f317180u);        // 6.9313812256e-01
+    const float ln2_lo = u2f(0x3717f7d1u);        // 9.0580006145e-06
+    const float invln2 = u2f(0x3fb8aa3bu);        // 1.4426950216e+00
+    const float Q1 = u2f(0xbd088889u);            // -3.3333335072e-02
+    const float Q2 = u2f(0x3ad00d01u);            //  1.5873016091e-03
+    const float Q3 = u2f(0xb8a670cdu);            // -7.9365076090e-05
+    const float Q4 = u2f(0x36867e54u);            //  4.0082177293e-06
+    const float Q5 = u2f(0xb457edbbu);            // -2.0109921195e-07
+
+    float y, hi, lo, c = 0.0f, t, e, hxs, hfx, r1;
+    int32_t k;
+    uint32_t hx = f2u(x);
+    const uint32_t xsb = hx & 0x80000000u;
+    hx &= 0x7fffffffu;
+
+    // huge and non-finite arguments
+    if (hx >= 0x4195b844u) {            // |x| >= 27*ln2
+        if (hx >= 0x42b17218u) {        // |x| >= 88.721...
+            if (hx > 0x7f800000u) return x + x;                     // NaN
+            if (hx == 0x7f800000u) return (xsb == 0) ? x : -1.0f;   // +-inf
+            if (x > o_threshold) return huge * huge;                // overflow
+        }
+        if (xsb != 0) return tiny - one;                            // x < -27 ln2 -> -1
+    }
+
+    // argument reduction
+    if (hx > 0x3eb17218u) {             // |x| > 0.5 ln2
+        if (hx < 0x3F851592u) {         // |x| < 1.5 ln2
+            if (xsb == 0) { hi = x - ln2_hi; lo = ln2_lo;  k = 1; }
+            else          { hi = x + ln2_hi; lo = -ln2_lo; k = -1; }
+        } else {
+            k = (int32_t)(invln2 * x + ((xsb == 0) ? 0.5f : -0.5f));
+            t = (float)k;
+            hi = x - t * ln2_hi;
+            lo = t * ln2_lo;
+        }
+        x = hi - lo;
+        c = (hi - x) - lo;
+    } else if (hx < 0x33000000u) {      // |x| < 2^-25
+        t = huge + x;
+        return x - (t - (huge + x));
+    } else {
+        k = 0;
+    }
+
+    // x is now in the primary range
+    hfx = 0.5f * x;
+    hxs = x * hfx;
+    r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    t = 3.0f - r1 * hfx;
+    e = hxs * ((r1 - t) / (6.0f - x * t));
+    if (k == 0) return x - (x * e - hxs);
+    e = (x * (e - c) - c);
+    e -= hxs;
+    if (k == -1) return 0.5f * (x - e) - 0.5f;
+    if (k == 1) {
+        if (x < -0.25f) return -2.0f * (e - (x + 0.5f));
+        return one + 2.0f * (x - e);
+    }
+    if (k <= -2 || k > 56) {            // suffices to return exp(x) - 1
+        y = one - (e - x);
+        y = u2f(f2u(y) + ((uint32_t)k << 23));
+        return y - one;
+    }
+    if (k < 23) {
+        t = u2f(0x3f800000u - (0x1000000u >> k));   // 1 - 2^-k
+        y = t - (e - x);
+        y = u2f(f2u(y) + ((uint32_t)k << 23));
+    } else {
+        t = u2f((uint32_t)(0x7f - k) << 23);        // 2^-k
+        y = x - (e + t);
+        y += one;
+        y = u2f(f2u(y) + ((uint32_t)k << 23));
+    }
+    return y;
+}
+
+// tanhf following fdlibm s_tanhf.c.
+ZM_HD float tanhf_fdlibm(float x)
+{
+    const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
+    const uint32_t jx = f2u(x);
+    const uint32_t ix = jx & 0x7fffffffu;
+    const bool neg = (jx >> 31) != 0;
+    float t, z;
+
+    if (ix >= 0x7f800000u) {            // inf or NaN
+        if (!neg) return one / x + one; // tanh(+inf) = 1, NaN stays NaN
+        return one / x - one;
+    }
+    if (ix < 0x41b00000u) {             // |x| < 22
+        if (ix == 0) return x;          // +-0
+        if (ix < 0x24000000u) return x * (one + x);   // |x| < 2^-55
+        const float ax = u2f(ix);
+        if (ix >= 0x3f800000u) {        // |x| >= 1
+            t = expm1f_fdlibm(two * ax);
+            z = one - two / (t + two);
+        } else {
+            t = expm1f_fdlibm(-two * ax);
+            z = -t / (t + two);
+        }
+    } else {
+        z = one - tiny;                 // |x| >= 22: 1 (inexact)
+    }
+    return neg ? -z : z;
+}
+
+// ZeNu's sigmoid composite in f32: each step rounded to f32, as the four autograd ops do.
+ZM_HD float sigmoidf_zenu(float x)
+{
+    const float half = 0.5f;
+    float xh = x * half;
+    float th = tanhf_fdlibm(xh);
+    float ht = half * th;
+    return half + ht;
+}
+
+}  // namespace zmath
