@@ -1,0 +1,340 @@
+#!/usr/bin/env python3
+"""Benchmark of the device tensor-kernel layer on one MI355X.
+
+A "step" is one pass of the hot path over synthetic inputs: every op of BASELINE.json's
+configs[0..3] once (contiguous / broadcast / transposed elementwise, activations, axis
+reductions in f32 and f64, one fused AdamW step over 25 M parameters), each on device-resident
+buffers.  `value` is whole-step throughput: the algorithmic bytes of one step divided by the
+wall time of a step, with K steps timed between two stream synchronisations.
+
+Besides the whole-step figure every op is timed on its own with HIP events recorded on the
+stream the kernels are launched on (`ops` in the JSON line), rotating through enough buffer
+sets (>= 1 GiB per op) that the 256 MB memory-side cache cannot serve the inputs.  `roofline`
+describes the dominant kernel of the step (the fused AdamW update).  `cpu_baseline` is the CPU
+oracle (a single-threaded restatement of ZeNu's CPU path, reference-shaped: one leaf loop per
+row / slice, whole-array passes with temporaries for Adam) timed on this box's host cores on
+one pass of the same step.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload suite|c0|c1|c2|c3]
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBPS = 8000.0  # MI355X published HBM3E peak
+
+HP = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.01, step=10)
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+class Hip:
+    """the few HIP runtime calls the harness needs (events), bound with ctypes"""
+
+    def __init__(self):
+        self.rt = C.CDLL("libamdhip64.so")
+        self.rt.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.rt.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.rt.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.rt.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+
+    def event(self):
+        e = C.c_void_p()
+        assert self.rt.hipEventCreate(C.byref(e)) == 0
+        return e
+
+    def record(self, e, stream):
+        assert self.rt.hipEventRecord(e, stream) == 0
+
+    def elapsed_ms(self, a, b):
+        assert self.rt.hipEventSynchronize(b) == 0
+        ms = C.c_float()
+        assert self.rt.hipEventElapsedTime(C.byref(ms), a, b) == 0
+        return ms.value
+
+
+class Op:
+    """one op of the step: a list of pre-bound launch closures, one per rotating buffer set"""
+
+    def __init__(self, name, config, dtype, alg_bytes, elems, launches, cpu_fn, kernel=None):
+        self.name, self.config, self.dtype = name, config, dtype
+        self.alg_bytes, self.elems = alg_bytes, elems
+        self.launches = launches
+        self.cpu_fn = cpu_fn
+        self.kernel = kernel
+        self.i = 0
+
+    def launch(self):
+        self.launches[self.i % len(self.launches)]()
+        self.i += 1
+
+
+def build_ops(z, workload, stream):
+    """allocate device buffers, upload seeded inputs, return the list of ops"""
+    from zenu_amd import _lib
+    from zenu_amd._lib import check
+    import zenu_oracle as zo
+
+    l = z.lib()
+    M = z.Matrix
+    ops = []
+    GiB = 1 << 30
+
+    def nsets(bytes_per_set):
+        return max(2, -(-GiB // bytes_per_set))
+
+    def ref(t):
+        return C.byref(t)
+
+    want = lambda c: workload in ("suite", c)
+
+    # ---- config[0]: contiguous f32 [2^24], uniform[-1,1), seed 0 ------------------------------
+    def add_c0():
+        r = np.random.default_rng(0)
+        n = 1 << 24
+        a = r.uniform(-1, 1, n).astype(np.float32)
+        b = r.uniform(-1, 1, n).astype(np.float32)
+        sets = [(M.from_numpy(a), M.from_numpy(b), M.alloc([n])) for _ in range(nsets(3 * 4 * n))]
+        keep = sets
+        out_h = np.empty_like(a)
+
+        def mk_bin(op):
+            ls = []
+            for A, B, O in sets:
+                da, db, do = A.desc(), B.desc(), O.desc()
+                ls.append(lambda da=da, db=db, do=do: check(l.zenu_hip_binary(op, _lib.F32, ref(do), ref(da), ref(db), stream), "binary"))
+            return ls
+        ops.append(Op("add[2^24]", "c0", "f32", 3 * 4 * n, n, mk_bin(_lib.ADD), lambda: zo.binary_array(zo.ADD, out_h, a, b)))
+        ops.append(Op("mul[2^24]", "c0", "f32", 3 * 4 * n, n, mk_bin(_lib.MUL), lambda: zo.binary_array(zo.MUL, out_h, a, b)))
+        ls = []
+        for A, B, O in sets:
+            da, do = A.desc(), O.desc()
+            ls.append(lambda da=da, do=do: check(l.zenu_hip_relu(_lib.F32, ref(do), ref(da), 0.0, stream), "relu"))
+        ops.append(Op("relu[2^24]", "c0", "f32", 2 * 4 * n, n, ls, lambda: zo.relu(out_h, a, 0.0)))
+        ops[-1].keep = keep
+
+    # ---- config[1]: [4096,4096] f32, normal(0,1), seed 1 ----------------------------------------
+    def add_c1():
+        r = np.random.default_rng(1)
+        a = r.standard_normal((4096, 4096)).astype(np.float32)
+        b = r.standard_normal((4096, 4096)).astype(np.float32)
+        row = r.standard_normal((1, 4096)).astype(np.float32)
+        n = a.size
+        sets = [(M.from_numpy(a), M.from_numpy(b), M.from_numpy(row), M.alloc([4096, 4096])) for _ in range(nsets(3 * 4 * n))]
+        out_h = np.empty_like(a)
+
+        def mk(fn):
+            return [fn(A.desc(), B.desc(), B.transpose().desc(), R.desc(), O.desc()) for A, B, R, O in sets]
+        ops.append(Op("a+b[1,4096]", "c1", "f32", 2 * 4 * n + 4 * 4096, n,
+                      mk(lambda da, db, dbt, dr, do: (lambda: check(l.zenu_hip_binary(_lib.ADD, _lib.F32, ref(do), ref(da), ref(dr), stream), "bcast"))),
+                      lambda: zo.binary_array(zo.ADD, out_h, a, row)))
+        ops.append(Op("a+b^T", "c1", "f32", 3 * 4 * n, n,
+                      mk(lambda da, db, dbt, dr, do: (lambda: check(l.zenu_hip_binary(_lib.ADD, _lib.F32, ref(do), ref(da), ref(dbt), stream), "transposed"))),
+                      lambda: zo.binary_array(zo.ADD, out_h, a, b.T)))
+        ops.append(Op("a*0.5", "c1", "f32", 2 * 4 * n, n,
+                      mk(lambda da, db, dbt, dr, do: (lambda: check(l.zenu_hip_binary_scalar(_lib.MUL, _lib.F32, ref(do), ref(da), 0.5, stream), "scalar"))),
+                      lambda: zo.binary_scalar(zo.MUL, out_h, a, 0.5)))
+        for name, fn, zfn in (("sigmoid", _lib.SIGMOID, None), ("tanh", _lib.TANH, zo.TANH), ("exp", _lib.EXP, zo.EXP)):
+            cpu = (lambda: zo.sigmoid(out_h, a)) if zfn is None else (lambda zfn=zfn: zo.unary(zfn, out_h, a))
+            ops.append(Op(name, "c1", "f32", 2 * 4 * n, n,
+                          mk(lambda da, db, dbt, dr, do, fn=fn: (lambda: check(l.zenu_hip_unary(fn, _lib.F32, ref(do), ref(da), stream), "unary"))),
+                          cpu))
+        ops[-1].keep = sets
+
+    def add_c2(dt, dcode, dname):
+        r = np.random.default_rng(2)
+        x = r.standard_normal((8192, 4096)).astype(dt)
+        for row in r.choice(8192, size=82, replace=False):
+            x[row, int(r.integers(0, 4096))] = x[row].max()
+        inb = x.nbytes
+        sets = []
+        for _ in range(nsets(inb)):
+            X = M.from_numpy(x)
+            sets.append((X, M.alloc([4096], dt), M.alloc([8192], dt), M.alloc([8192], np.int64), M.alloc([], dt)))
+        isz = np.dtype(dt).itemsize
+        cpu_all = np.zeros((), dtype=dt)
+
+        def mk(fn):
+            return [fn(X.desc(), o0.desc(), o1.desc(), oi.as_ptr(), oa.as_ptr()) for X, o0, o1, oi, oa in sets]
+        ops.append(Op(f"sum axis0 {dname}", "c2", dname, inb + 4096 * isz, x.size,
+                      mk(lambda dx, d0, d1, pi, pa: (lambda: check(l.zenu_hip_sum_axis(dcode, ref(d0), ref(dx), 0, stream), "sum0"))),
+                      lambda: zo.sum_axis(x, 0)))
+        ops.append(Op(f"sum axis1 {dname}", "c2", dname, inb + 8192 * isz, x.size,
+                      mk(lambda dx, d0, d1, pi, pa: (lambda: check(l.zenu_hip_sum_axis(dcode, ref(d1), ref(dx), 1, stream), "sum1"))),
+                      lambda: zo.sum_axis(x, 1)))
+        ops.append(Op(f"max axis1 {dname}", "c2", dname, inb + 8192 * isz, x.size,
+                      mk(lambda dx, d0, d1, pi, pa: (lambda: check(l.zenu_hip_max_axis(dcode, ref(d1), ref(dx), 1, stream), "max1"))),
+                      lambda: zo.max_axis(x, 1)))
+        ops.append(Op(f"argmax axis1 {dname}", "c2", dname, inb + 8192 * 8, x.size,
+                      mk(lambda dx, d0, d1, pi, pa: (lambda: check(l.zenu_hip_max_axis_idx(dcode, pi, ref(dx), 1, stream), "argmax1"))),
+                      lambda: zo.max_axis_idx_ravel(x, 1)))
+        ops.append(Op(f"sum all {dname}", "c2", dname, inb + isz, x.size,
+                      mk(lambda dx, d0, d1, pi, pa: (lambda: check(l.zenu_hip_sum_all(dcode, pa, ref(dx), stream), "sumall"))),
+                      lambda: zo.sum_to(x, cpu_all)))
+        ops[-1].keep = sets
+
+    # ---- config[2]: [8192,4096] f32 and f64, normal(0,1), seed 2, ~1% duplicate maxima -------------
+
+    # ---- config[3]: fused AdamW over 25 M f32 parameters, seed 3 ---------------------------------------
+    def add_c3():
+        r = np.random.default_rng(3)
+        n = 25_000_000
+        p = (r.standard_normal(n) * 0.02).astype(np.float32)
+        g = (r.standard_normal(n) * 1e-3).astype(np.float32)
+        m = (r.standard_normal(n) * 1e-4).astype(np.float32)
+        v = np.abs(r.standard_normal(n) * 1e-6).astype(np.float32)
+        sets = [tuple(M.from_numpy(t) for t in (p, g, m, v)) for _ in range(nsets(4 * 4 * n))]
+        f = np.float32
+        hp = [float(f(HP[k])) for k in ("lr", "beta1", "beta2", "eps", "wd")]
+        ls = []
+        for P, G, Mm, V in sets:
+            ls.append(lambda P=P.as_ptr(), G=G.as_ptr(), Mm=Mm.as_ptr(), V=V.as_ptr(): check(
+                l.zenu_hip_adamw_step(_lib.F32, P, G, Mm, V, n, hp[0], hp[1], hp[2], hp[3], hp[4], 1, float(HP["step"]), stream), "adamw"))
+        pc, mc, vc = p.copy(), m.copy(), v.copy()
+        op = Op("adamw 25M", "c3", "f32", 7 * 4 * n, n, ls,
+                lambda: zo.adamw_update(pc, g, mc, vc, f(HP["lr"]), f(HP["beta1"]), f(HP["beta2"]), f(HP["eps"]), f(HP["wd"]), True, f(HP["step"])),
+                kernel="adam_kernel<float, 4>")
+        op.keep = sets
+        ops.append(op)
+
+    if want("c0"):
+        add_c0()
+    if want("c1"):
+        add_c1()
+    if want("c2"):
+        add_c2(np.float32, _lib.F32, "f32")
+        add_c2(np.float64, _lib.F64, "f64")
+    if want("c3"):
+        add_c3()
+    return ops
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="suite", choices=["suite", "c0", "c1", "c2", "c3"])
+    ap.add_argument("--op-reps", type=int, default=40, help="launches per op in the per-op timing")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--profile-op", default=None, help="only launch this op (for rocprofv3 counter runs)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; every op of the path shards without communication "
+                 "(see DESIGN.md), but no multi-GPU path exists: run with --gpus 1")
+
+    import zenu_amd as z
+    from zenu_amd import _lib
+    _lib.check(z.lib().zenu_hip_init(0), "zenu_hip_init")
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+
+    stream = C.c_void_p()
+    _lib.check(z.lib().zenu_hip_stream_create(C.byref(stream)), "stream_create")
+    z.set_stream(stream)
+    hip = Hip()
+    sync = lambda: _lib.check(z.lib().zenu_hip_stream_synchronize(stream), "sync")
+
+    t0 = time.time()
+    ops = build_ops(z, args.workload, stream)
+    sync()
+    log(f"[bench] {len(ops)} ops set up in {time.time() - t0:.1f} s")
+
+    if args.profile_op:
+        sel = [o for o in ops if o.name == args.profile_op]
+        assert sel, [o.name for o in ops]
+        for _ in range(args.warmup + args.steps):
+            sel[0].launch()
+        sync()
+        return
+
+    # ---- whole-step timing -------------------------------------------------------------------------
+    for _ in range(args.warmup):
+        for o in ops:
+            o.launch()
+    sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        for o in ops:
+            o.launch()
+    sync()
+    elapsed = time.perf_counter() - t0
+    step_bytes = sum(o.alg_bytes for o in ops)
+    ms_per_step = elapsed / args.steps * 1e3
+    value = step_bytes / (elapsed / args.steps) / 1e9
+
+    # ---- per-op timing with HIP events on the launch stream ---------------------------------------------
+    e0, e1 = hip.event(), hip.event()
+    table = []
+    for o in ops:
+        for _ in range(5):
+            o.launch()
+        sync()
+        hip.record(e0, stream)
+        for _ in range(args.op_reps):
+            o.launch()
+        hip.record(e1, stream)
+        us = hip.elapsed_ms(e0, e1) / args.op_reps * 1e3
+        gbps = o.alg_bytes / (us * 1e-6) / 1e9
+        table.append(dict(op=o.name, config=o.config, dtype=o.dtype, us=round(us, 2), GBps=round(gbps, 1),
+                          frac_of_peak=round(gbps / PEAK_HBM_GBPS, 4), Gelem_per_s=round(o.elems / (us * 1e-6) / 1e9, 2),
+                          alg_bytes=o.alg_bytes))
+        log(f"[op] {o.name:22s} {us:9.2f} us  {gbps:8.1f} GB/s  {100 * gbps / PEAK_HBM_GBPS:5.1f}% of peak")
+
+    # dominant kernel of the step = the op with the largest share of the step time
+    dom = max(table, key=lambda t: t["us"])
+    dom_op = [o for o in ops if o.name == dom["op"]][0]
+    roofline = dict(bound="hbm", achieved=dom["GBps"], peak=PEAK_HBM_GBPS, unit="GB/s",
+                    frac=round(dom["GBps"] / PEAK_HBM_GBPS, 4), traffic=None,
+                    kernel=dom_op.kernel or dom["op"], algorithmic_bytes_per_launch=dom["alg_bytes"],
+                    avg_launch_us=dom["us"])
+    adam = [t for t in table if t["config"] == "c3"]
+
+    # ---- CPU baseline: the oracle, one thread, one pass of the same step -----------------------------------
+    cpu = None
+    if not args.no_cpu_baseline:
+        t0 = time.perf_counter()
+        per_op = {o.name: 0.0 for o in ops}
+        passes = 0
+        while passes < 5 and (passes == 0 or time.perf_counter() - t0 < 10.0):
+            for o in ops:
+                t1 = time.perf_counter()
+                o.cpu_fn()
+                per_op[o.name] += time.perf_counter() - t1
+            passes += 1
+        cpu_s = (time.perf_counter() - t0) / passes
+        per_op = {k: v / passes for k, v in per_op.items()}
+        for t in table:
+            t["cpu_GBps"] = round(t["alg_bytes"] / per_op[t["op"]] / 1e9, 3)
+        cpu = dict(value=round(step_bytes / cpu_s / 1e9, 3), unit="GB/s", cores=1, kind="port",
+                   sample=f"{passes} full pass(es) of the step ({len(ops)} ops, {cpu_s:.1f} s each) by the single-threaded C oracle, "
+                          f"reference-shaped (one leaf loop per row/slice, Adam as whole-array passes); "
+                          f"host has {os.cpu_count()} logical CPUs")
+        log(f"[cpu] one step on the CPU oracle: {cpu_s:.2f} s = {cpu['value']} GB/s")
+
+    out = {
+        "metric": "achieved HBM GB/s (% of MI355X peak) per op; Adam step params/sec",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if args.workload != "suite" and args.workload != "c2" else "f32+f64", "data": "synthetic",
+        "config": {"workload": {"suite": "configs[0..3]: every op once per step", "c0": "configs[0]", "c1": "configs[1]",
+                                "c2": "configs[2]", "c3": "configs[3]"}[args.workload],
+                   "ops_per_step": len(ops), "algorithmic_bytes_per_step": step_bytes},
+        "frac_of_peak_whole_step": round(value / PEAK_HBM_GBPS, 4),
+        "adam_step_params_per_sec": (round(adam[0]["Gelem_per_s"] * 1e9) if adam else None),
+        "roofline": roofline, "cpu_baseline": cpu, "ops": table,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -41,7 +41,7 @@ def max_ulp(a, b):
 
 
 def bits_equal(a, b):
-    return a.shape == b.shape and np.array_equal(a.view(np.uint8), b.view(np.uint8))
+    return a.shape == b.shape and np.array_equal(a.reshape(-1).view(np.uint8), b.reshape(-1).view(np.uint8))
 
 
 def assert_bits(got, exp, what):
@@ -55,11 +55,18 @@ def sum_tol(dtype):
     return 1e-5 if np.dtype(dtype) == np.float32 else 1e-12
 
 
-def assert_sum_close(got, cpu, x, axis, what):
+def assert_sum_close(got, cpu, x, axis, what, cpu_slack=False):
+    """cpu_slack: for rows much longer than the BASELINE ones the sequential CPU sum itself is
+    off by about eps * sum|x| (its a-priori bound is (n-1) * eps * sum|x|); allow 4 * eps * sum|x|
+    on top when comparing against it.  The comparison with the exact f64 sum stays strict."""
     n = x.size if axis is None else x.shape[axis]
-    scale = np.abs(x.astype(np.float64)).sum(axis=axis) / np.sqrt(n)
+    sabs = np.abs(x.astype(np.float64)).sum(axis=axis)
+    scale = sabs / np.sqrt(n)
     denom = np.maximum(np.abs(cpu.astype(np.float64)), scale)
-    err = np.abs(got.astype(np.float64) - cpu.astype(np.float64)) / denom
+    diff = np.abs(got.astype(np.float64) - cpu.astype(np.float64))
+    if cpu_slack:
+        diff = np.maximum(diff - 4 * np.finfo(x.dtype).eps * sabs, 0)
+    err = diff / denom
     assert err.max() <= sum_tol(x.dtype), f"{what}: rel err {err.max():.3e}"
     exact = x.astype(np.float64).sum(axis=axis)
     err64 = np.abs(got.astype(np.float64) - exact) / np.maximum(np.abs(exact), scale)
@@ -304,7 +311,7 @@ def test_strided_broadcast_binary(hip, idx, dt):
         exp = np.empty(shape, dtype=dt)
         zo.binary_array(op, exp, lhs, rhs)
         brute = {"add": np.add, "sub": np.subtract, "mul": np.multiply, "div": np.divide}[name](lhs, rhs)
-        assert_bits(exp, np.ascontiguousarray(np.broadcast_to(brute, shape)), "oracle vs brute force")
+        assert_bits(exp, np.broadcast_to(brute, shape).copy(), "oracle vs brute force")
         out = hip.Matrix.alloc(shape, dt)
         getattr(out, f"{name}_array")(L, R)
         assert_bits(out.to_numpy(), exp, f"{name} case {idx}")
@@ -411,9 +418,15 @@ def test_reduction_shapes(hip, shape, dt):
     y = r.standard_normal(shape).astype(dt)
     Y = hip.Matrix.from_numpy(y)
     for axis in range(len(shape)):
-        assert_sum_close(Y.sum(axis).to_numpy(), zo.sum_axis(y, axis), y, axis, f"sum {shape} axis {axis}")
+        assert_sum_close(Y.sum(axis).to_numpy(), zo.sum_axis(y, axis), y, axis, f"sum {shape} axis {axis}",
+                         cpu_slack=True)
+    # asum: the reference calls OpenBLAS s/dasum whose accumulation order is unspecified (parity
+    # unpinned); the device result must be within the bar of the exact sum, and within the
+    # a-priori bound n * eps * sum|x| of the oracle's plain in-order loop
     a = float(Y.asum())
-    assert abs(a - float(zo.asum(y))) <= sum_tol(dt) * np.abs(y).sum()   # order unpinned: tolerance
+    exact = float(np.abs(y.astype(np.float64)).sum())
+    assert abs(a - exact) <= sum_tol(dt) * exact
+    assert abs(a - float(zo.asum(y))) <= y.size * np.finfo(dt).eps * exact
 
 
 def test_reduction_strided_views(hip):
