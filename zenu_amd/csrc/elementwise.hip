@@ -24,6 +24,7 @@
 #include <math.h>
 
 #include "common.hpp"
+#include "vecmem.hpp"
 #include "zmath.hpp"
 
 namespace zenu {
@@ -31,43 +32,6 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kUnroll = 4;
-
-template <typename T> struct VecOf;
-template <> struct VecOf<float> { typedef float4 type; static constexpr int N = 4; };
-template <> struct VecOf<double> { typedef double2 type; static constexpr int N = 2; };
-
-template <typename T, int N> struct Pack { T v[N]; };
-
-template <typename T, int N> __device__ __forceinline__ Pack<T, N> load_pack(const T *p)
-{
-    Pack<T, N> r;
-    if constexpr (N == 1) {
-        r.v[0] = *p;
-    } else {
-        typedef typename VecOf<T>::type V;
-        V x = *reinterpret_cast<const V *>(p);
-        __builtin_memcpy(&r, &x, sizeof(V));
-    }
-    return r;
-}
-template <typename T, int N> __device__ __forceinline__ void store_pack(T *p, const Pack<T, N> &r)
-{
-    if constexpr (N == 1) {
-        *p = r.v[0];
-    } else {
-        typedef typename VecOf<T>::type V;
-        V x;
-        __builtin_memcpy(&x, &r, sizeof(V));
-        *reinterpret_cast<V *>(p) = x;
-    }
-}
-template <typename T, int N> __device__ __forceinline__ Pack<T, N> splat(T s)
-{
-    Pack<T, N> r;
-#pragma unroll
-    for (int i = 0; i < N; i++) r.v[i] = s;
-    return r;
-}
 
 // ---- functors -----------------------------------------------------------------------------------
 
@@ -94,7 +58,7 @@ template <typename T, int OP> struct ScalarF {
     __device__ __forceinline__ T operator()(T a, T) const { return bin_apply<T, OP>(a, s); }
 };
 
-__device__ __forceinline__ float dev_tanh(float x) { return zmath::tanhf_fdlibm(x); }
+__device__ __forceinline__ float dev_tanh(float x) { return zmath::tanhf_simd(x); }
 __device__ __forceinline__ double dev_tanh(double x) { return tanh(x); }
 __device__ __forceinline__ float dev_sigmoid(float x) { return zmath::sigmoidf_zenu(x); }
 __device__ __forceinline__ double dev_sigmoid(double x)
@@ -165,7 +129,7 @@ __device__ __forceinline__ Pack<T, N> apply_pack(const F &f, const Pack<T, N> &a
 
 // ---- kernel 1: contiguous ------------------------------------------------------------------------
 
-template <typename T, int VEC, typename F>
+template <typename T, int VEC, bool NT, typename F>
 __global__ __launch_bounds__(kBlock) void ew_contig_kernel(T *out, const T *a, const T *b,
                                                            int64_t n, F f)
 {
@@ -178,14 +142,14 @@ __global__ __launch_bounds__(kBlock) void ew_contig_kernel(T *out, const T *a, c
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             int64_t i = base + ((int64_t)u * kBlock + tid) * VEC;
-            va[u] = load_pack<T, VEC>(a + i);
-            if constexpr (F::NIN == 2) vb[u] = load_pack<T, VEC>(b + i);
+            va[u] = load_pack<T, VEC, NT>(a + i);
+            if constexpr (F::NIN == 2) vb[u] = load_pack<T, VEC, NT>(b + i);
             else vb[u] = va[u];
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             int64_t i = base + ((int64_t)u * kBlock + tid) * VEC;
-            store_pack<T, VEC>(out + i, apply_pack<T, VEC, F>(f, va[u], vb[u]));
+            store_pack<T, VEC, NT>(out + i, apply_pack<T, VEC, F>(f, va[u], vb[u]));
         }
     } else {
         for (int u = 0; u < kUnroll; u++) {
@@ -243,7 +207,10 @@ struct RowsParams {
     int64_t col_tiles; // column tiles per row
 };
 
-template <typename T, int VEC, typename F>
+// NTA / NTB: input a / b is streamed once (not broadcast along an outer dim); the output is
+// streamed when either is.  Template parameters, because a run-time choice between a hinted and
+// a plain load is merged by the compiler into one plain load.
+template <typename T, int VEC, bool NTA, bool NTB, typename F>
 __global__ __launch_bounds__(kBlock) void ew_rows_kernel(T *out, const T *a, const T *b,
                                                          RowsParams p, F f)
 {
@@ -274,23 +241,23 @@ __global__ __launch_bounds__(kBlock) void ew_rows_kernel(T *out, const T *a, con
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             int64_t c = c0 + ((int64_t)u * tx_n + tx) * VEC;
-            va[u] = p.inner_a ? load_pack<T, VEC>(arow + c) : sa;
-            if constexpr (F::NIN == 2) vb[u] = p.inner_b ? load_pack<T, VEC>(brow + c) : sb;
+            va[u] = p.inner_a ? load_pack<T, VEC, NTA>(arow + c) : sa;
+            if constexpr (F::NIN == 2) vb[u] = p.inner_b ? load_pack<T, VEC, NTB>(brow + c) : sb;
             else vb[u] = va[u];
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             int64_t c = c0 + ((int64_t)u * tx_n + tx) * VEC;
-            store_pack<T, VEC>(orow + c, apply_pack<T, VEC, F>(f, va[u], vb[u]));
+            store_pack<T, VEC, (NTA || NTB)>(orow + c, apply_pack<T, VEC, F>(f, va[u], vb[u]));
         }
     } else {
         for (int u = 0; u < kUnroll; u++) {
             int64_t c = c0 + ((int64_t)u * tx_n + tx) * VEC;
             if (c + VEC <= p.ncols) {
-                Pack<T, VEC> x = p.inner_a ? load_pack<T, VEC>(arow + c) : sa;
+                Pack<T, VEC> x = p.inner_a ? load_pack<T, VEC, false>(arow + c) : sa;
                 Pack<T, VEC> y = x;
-                if constexpr (F::NIN == 2) y = p.inner_b ? load_pack<T, VEC>(brow + c) : sb;
-                store_pack<T, VEC>(orow + c, apply_pack<T, VEC, F>(f, x, y));
+                if constexpr (F::NIN == 2) y = p.inner_b ? load_pack<T, VEC, false>(brow + c) : sb;
+                store_pack<T, VEC, false>(orow + c, apply_pack<T, VEC, F>(f, x, y));
             } else {
                 for (int j = 0; j < VEC; j++) {
                     if (c + j < p.ncols) {
@@ -321,7 +288,7 @@ struct TileParams {
     int64_t tiles_r, tiles_c;
 };
 
-template <typename T, typename F>
+template <typename T, bool NT, typename F>
 __global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, const T *b,
                                                          TileParams p, F f)
 {
@@ -359,13 +326,13 @@ __global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, con
             for (int k = 0; k < kTile / RPP; k++) {
                 const int c = tid / VPR + k * RPP;
                 if (p.trans_a) {
-                    Pack<T, VEC> x = load_pack<T, VEC>(abase + rv + (int64_t)c * p.ldc[1]);
+                    Pack<T, VEC> x = load_pack<T, VEC, NT>(abase + rv + (int64_t)c * p.ldc[1]);
 #pragma unroll
                     for (int j = 0; j < VEC; j++) lds_a[(rv + j) * kPitch + c] = x.v[j];
                 }
                 if constexpr (F::NIN == 2) {
                     if (p.trans_b) {
-                        Pack<T, VEC> x = load_pack<T, VEC>(bbase + rv + (int64_t)c * p.ldc[2]);
+                        Pack<T, VEC> x = load_pack<T, VEC, NT>(bbase + rv + (int64_t)c * p.ldc[2]);
 #pragma unroll
                         for (int j = 0; j < VEC; j++) lds_b[(rv + j) * kPitch + c] = x.v[j];
                     }
@@ -398,7 +365,7 @@ __global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, con
             } else if (p.ldc[1] == 0) {
                 x = splat<T, VEC>(abase[(int64_t)r * p.ldr[1]]);
             } else {
-                x = load_pack<T, VEC>(abase + (int64_t)r * p.ldr[1] + cv);
+                x = load_pack<T, VEC, NT>(abase + (int64_t)r * p.ldr[1] + cv);
             }
             if constexpr (F::NIN == 2) {
                 if (p.trans_b) {
@@ -407,12 +374,12 @@ __global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, con
                 } else if (p.ldc[2] == 0) {
                     y = splat<T, VEC>(bbase[(int64_t)r * p.ldr[2]]);
                 } else {
-                    y = load_pack<T, VEC>(bbase + (int64_t)r * p.ldr[2] + cv);
+                    y = load_pack<T, VEC, NT>(bbase + (int64_t)r * p.ldr[2] + cv);
                 }
             } else {
                 y = x;
             }
-            store_pack<T, VEC>(obase + (int64_t)r * p.ldr[0] + cv, apply_pack<T, VEC, F>(f, x, y));
+            store_pack<T, VEC, NT>(obase + (int64_t)r * p.ldr[0] + cv, apply_pack<T, VEC, F>(f, x, y));
         }
     } else {
         for (int e = tid; e < kTile * kTile; e += kBlock) {
@@ -453,8 +420,6 @@ __global__ __launch_bounds__(kBlock) void ew_generic_kernel(T *out, const T *a, 
 
 // ---- host dispatch ---------------------------------------------------------------------------------
 
-inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
-
 template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t stream)
 {
     constexpr int VEC = VecOf<T>::N;
@@ -464,6 +429,8 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
     const T *a = static_cast<const T *>(p.ptr[1]);
     const T *b = (F::NIN == 2) ? static_cast<const T *>(p.ptr[2]) : a;
     const int nin = F::NIN;
+    // operands are streamed once: hint the caches when the op is larger than they are
+    const bool nt = p.numel * (int64_t)sizeof(T) * (nin + 1) >= kStreamBytes;
     if (p.ndim == 0) {  // a single element
         p.ndim = 1;
         p.shape[0] = 1;
@@ -482,12 +449,13 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
             int64_t tile = (int64_t)kBlock * VEC * kUnroll;
             int64_t grid = (n + tile - 1) / tile;
             if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-            ew_contig_kernel<T, VEC, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, n, f);
+            if (nt) ew_contig_kernel<T, VEC, true, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, n, f);
+            else    ew_contig_kernel<T, VEC, false, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, n, f);
         } else {
             int64_t tile = (int64_t)kBlock * kUnroll;
             int64_t grid = (n + tile - 1) / tile;
             if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-            ew_contig_kernel<T, 1, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, n, f);
+            ew_contig_kernel<T, 1, false, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, n, f);
         }
         ZENU_LAUNCH_CHECK();
         return ZENU_OK;
@@ -510,6 +478,11 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
         rp.nrows = p.numel / rp.ncols;
         rp.inner_a = (int)p.stride[1][last];
         rp.inner_b = nin == 2 ? (int)p.stride[2][last] : 1;
+        bool nta = nt && rp.inner_a == 1, ntb = nt && nin == 2 && rp.inner_b == 1;
+        for (int d = 0; d < p.ndim - 1; d++) {
+            if (p.stride[1][d] == 0) nta = false;   // re-read for every outer index: keep it cached
+            if (nin == 2 && p.stride[2][d] == 0) ntb = false;
+        }
         bool vec = aligned16(out) && (rp.ncols % VEC == 0);
         for (int o = 1; o <= nin && vec; o++)
             if (p.stride[o][last] == 1 && !aligned16(p.ptr[o])) vec = false;
@@ -528,8 +501,11 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
         int64_t rows_per_blk = kBlock >> shift;
         int64_t grid = ((rp.nrows + rows_per_blk - 1) / rows_per_blk) * rp.col_tiles;
         if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-        if (vec) ew_rows_kernel<T, VEC, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, rp, f);
-        else     ew_rows_kernel<T, 1, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, rp, f);
+        if (!vec)            ew_rows_kernel<T, 1, false, false, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, rp, f);
+        else if (nta && ntb) ew_rows_kernel<T, VEC, true, true, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, rp, f);
+        else if (nta)        ew_rows_kernel<T, VEC, true, false, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, rp, f);
+        else if (ntb)        ew_rows_kernel<T, VEC, false, true, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, rp, f);
+        else                 ew_rows_kernel<T, VEC, false, false, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, rp, f);
         ZENU_LAUNCH_CHECK();
         return ZENU_OK;
     }
@@ -587,7 +563,8 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
             tp.tiles_c = (tp.C + kTile - 1) / kTile;
             int64_t grid = tp.nbatch * tp.tiles_r * tp.tiles_c;
             if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-            ew_tile_kernel<T, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, tp, f);
+            if (nt) ew_tile_kernel<T, true, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, tp, f);
+            else    ew_tile_kernel<T, false, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, tp, f);
             ZENU_LAUNCH_CHECK();
             return ZENU_OK;
         }

@@ -14,9 +14,11 @@
 //   cols : inner > 1 -- a 64 x 4 thread tile: 64 lanes own 64 column vectors (coalesced 128-bit
 //          loads), 4 row lanes walk the reduced axis, combined through LDS in fixed order.
 //
-// Both kernels can split the reduced axis over several workgroups; the partial results go to a
-// small workspace and a second launch of the SAME kernel folds them.  No atomics touch data:
-// the combination tree is fixed by the launch geometry, so results are bit-reproducible.
+// Both kernels can split the reduced axis over several workgroups.  Partial results go to a
+// small workspace; each workgroup then bumps an arrival counter and the one that arrives last
+// folds the partials of its outputs, always in split order.  No workgroup waits for another and
+// no atomic touches data: the combination tree is fixed by the launch geometry, so results are
+// bit-reproducible, and the whole reduction is ONE launch.
 //
 // Arg-max follows MaxIdx for Cpu (max.rs:19-34): start from element 0 and replace on strict '>'.
 // That is "largest value, lowest index on ties", except for NaN: a NaN at position 0 is never
@@ -27,12 +29,12 @@
 #include <math.h>
 
 #include "common.hpp"
+#include "vecmem.hpp"
 
 namespace zenu {
 
-// out[o] = src[q * outer_stride + c + idx[o] * elem_stride] with o = q * inner + c
-int gather_axis(const void *src, const int64_t *idx, void *out, int64_t nout, int64_t inner,
-                int64_t outer_stride, int64_t elem_stride, int elem_size, hipStream_t s);
+// `n` consecutive arrival counters (zero at rest) from the library's ring, or nullptr
+int *reserve_counters(int64_t n);
 
 namespace {
 
@@ -40,9 +42,6 @@ constexpr int kBlock = 256;
 constexpr int kWave = 64;
 constexpr int kWaves = kBlock / kWave;
 
-template <typename T> struct VecOf;
-template <> struct VecOf<float> { typedef float4 type; static constexpr int N = 4; };
-template <> struct VecOf<double> { typedef double2 type; static constexpr int N = 2; };
 
 // ---- wave64 exchange primitives (word-wise so any POD accumulator works) ---------------------------
 
@@ -100,11 +99,15 @@ template <typename Tr> __device__ __forceinline__ typename Tr::Acc block_allredu
 
 // ---- accumulator traits ------------------------------------------------------------------------------
 
+// Accumulator traits.  `update` folds the next element (in increasing position order) into a
+// lane's accumulator and is the only code in the per-element hot loop; `merge` combines two
+// accumulators (lanes, waves, workgroups) and must be commutative and associative.
 template <typename T> struct SumTr {
     typedef T Acc;
     static constexpr bool kHasIdx = false;
     __device__ __forceinline__ static Acc identity() { return (T)0; }
-    __device__ __forceinline__ static Acc from_elem(T x, int64_t) { return x; }
+    __device__ __forceinline__ static Acc update(Acc a, T x, int64_t) { return a + x; }
+    __device__ __forceinline__ static Acc first(Acc a, T) { return a; }
     __device__ __forceinline__ static Acc from_partial(T x, int64_t) { return x; }
     __device__ __forceinline__ static Acc merge(Acc a, Acc b) { return a + b; }
     __device__ __forceinline__ static T key(Acc a) { return a; }
@@ -112,14 +115,23 @@ template <typename T> struct SumTr {
 };
 
 template <typename T> struct AsumTr : SumTr<T> {
-    __device__ __forceinline__ static T from_elem(T x, int64_t) { return fabs(x); }
+    __device__ __forceinline__ static T update(T a, T x, int64_t) { return a + fabs(x); }
 };
 
 template <typename T> struct ArgPair {
     T key;
-    int64_t idx;
+    int32_t idx;
 };
 
+// Arg-max with the semantics of the sequential scan of max.rs:23-31.
+//   * In a lane, elements arrive in increasing position, so "replace on strict >" keeps the first
+//     index, ignores NaN (NaN > key is false) and costs one compare and two selects.
+//   * -inf elements never pass the strict test against the -inf identity; if nothing does, every
+//     element is -inf or NaN and the scan would have stayed at index 0: idx() maps the untouched
+//     identity index to 0.
+//   * A NaN at position 0 is never replaced by the scan: first() turns it into a +inf key at
+//     index 0, which no later element beats and which wins every tie by index.
+constexpr int32_t kNoIdx = 0x7fffffff;
 template <typename T> struct ArgmaxTr {
     typedef ArgPair<T> Acc;
     static constexpr bool kHasIdx = true;
@@ -127,21 +139,30 @@ template <typename T> struct ArgmaxTr {
     {
         Acc a;
         a.key = -INFINITY;
-        a.idx = 0x7fffffffffffffffLL;
+        a.idx = kNoIdx;
         return a;
     }
-    __device__ __forceinline__ static Acc from_elem(T x, int64_t pos)
+    __device__ __forceinline__ static Acc update(Acc a, T x, int64_t pos)
     {
-        Acc a;
-        a.key = (x != x) ? (pos == 0 ? (T)INFINITY : (T)-INFINITY) : x;
-        a.idx = pos;
+        const bool gt = x > a.key;
+        a.key = gt ? x : a.key;
+        a.idx = gt ? (int32_t)pos : a.idx;
+        return a;
+    }
+    // `x` is the element at position 0 of the reduced axis, already folded in by update()
+    __device__ __forceinline__ static Acc first(Acc a, T x)
+    {
+        if (x != x) {
+            a.key = INFINITY;
+            a.idx = 0;
+        }
         return a;
     }
     __device__ __forceinline__ static Acc from_partial(T k, int64_t i)
     {
         Acc a;
         a.key = k;
-        a.idx = i;
+        a.idx = (int32_t)i;
         return a;
     }
     __device__ __forceinline__ static Acc merge(Acc a, Acc b)
@@ -150,14 +171,13 @@ template <typename T> struct ArgmaxTr {
         return take_b ? b : a;
     }
     __device__ __forceinline__ static T key(Acc a) { return a.key; }
-    __device__ __forceinline__ static int64_t idx(Acc a) { return a.idx; }
+    __device__ __forceinline__ static int64_t idx(Acc a) { return a.idx == kNoIdx ? 0 : a.idx; }
 };
 
 // ---- kernel parameters ---------------------------------------------------------------------------------
 
 template <typename T> struct RedParams {
-    const T *in;             // source values, or partial keys on a folding pass
-    const int64_t *in_idx;   // partial indices on a folding pass (arg-max only)
+    const T *in;
     // geometry: output element o = (q, c) with q = o / inner, c = o % inner;
     // its R values sit at in[q * outer_stride + c + r * elem_stride]
     int64_t nout;            // number of outputs = outer * inner
@@ -170,21 +190,19 @@ template <typename T> struct RedParams {
     // results
     T *out_val;              // final value (may be null)
     int64_t *out_idx;        // final index (may be null)
-    T *part_key;             // partial outputs when splits > 1
-    int64_t *part_idx;
+    // cross-workgroup stage (splits > 1): partial results and one arrival counter per group of
+    // workgroups that share outputs; the counters are zero at rest
+    T *part_key;
+    int32_t *part_idx;
+    int *counters;
     // value gather for max: value = gsrc[q * g_outer_stride + c + idx * g_elem_stride]
     const T *gsrc;
     int64_t g_outer_stride, g_elem_stride;
 };
 
 template <typename T, typename Tr>
-__device__ __forceinline__ void emit(const RedParams<T> &p, int64_t o, int split, typename Tr::Acc r)
+__device__ __forceinline__ void emit_final(const RedParams<T> &p, int64_t o, typename Tr::Acc r)
 {
-    if (p.splits > 1) {
-        p.part_key[o * p.splits + split] = Tr::key(r);
-        if (Tr::kHasIdx) p.part_idx[o * p.splits + split] = Tr::idx(r);
-        return;
-    }
     if (Tr::kHasIdx) {
         if (p.out_idx) p.out_idx[o] = Tr::idx(r);
         if (p.out_val) {
@@ -196,12 +214,77 @@ __device__ __forceinline__ void emit(const RedParams<T> &p, int64_t o, int split
     }
 }
 
+// Cross-workgroup hand-off.  The workgroups of one launch run on 8 XCDs with separate L2s, so the
+// partials travel with device-scope (write-through / L2-bypassing) accesses instead of a
+// device-scope fence: a release fence would write back and invalidate the whole L2 in every
+// workgroup (measured: 20x slower).  Order of events in a producer: device-scope stores of the
+// partials, wait until they are acknowledged (workgroup-scope release = s_waitcnt), barrier, then
+// one device-scope atomic increment by thread 0.  The consumer (the workgroup that reads
+// expected-1 from the counter) loads the partials with device-scope loads.
+template <typename U> __device__ __forceinline__ void store_agent(U *p, U v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename U> __device__ __forceinline__ U load_agent(const U *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <typename T, typename Tr>
+__device__ __forceinline__ void emit_partial(const RedParams<T> &p, int64_t slot, typename Tr::Acc r)
+{
+    const T k = Tr::key(r);
+    if constexpr (sizeof(T) == 4) {
+        uint32_t u;
+        __builtin_memcpy(&u, &k, 4);
+        store_agent(reinterpret_cast<uint32_t *>(p.part_key + slot), u);
+    } else {
+        uint64_t u;
+        __builtin_memcpy(&u, &k, 8);
+        store_agent(reinterpret_cast<uint64_t *>(p.part_key + slot), u);
+    }
+    if (Tr::kHasIdx) store_agent(p.part_idx + slot, (int32_t)Tr::idx(r));  // only -inf/NaN: (-inf, 0)
+}
+
+template <typename T, typename Tr>
+__device__ __forceinline__ typename Tr::Acc load_partial(const RedParams<T> &p, int64_t slot)
+{
+    T k;
+    if constexpr (sizeof(T) == 4) {
+        uint32_t u = load_agent(reinterpret_cast<const uint32_t *>(p.part_key + slot));
+        __builtin_memcpy(&k, &u, 4);
+    } else {
+        uint64_t u = load_agent(reinterpret_cast<const uint64_t *>(p.part_key + slot));
+        __builtin_memcpy(&k, &u, 8);
+    }
+    int32_t i = 0;
+    if (Tr::kHasIdx) i = load_agent(p.part_idx + slot);
+    return Tr::from_partial(k, i);
+}
+
+// Called by every thread of a workgroup after its partials are stored.  Returns true in the
+// workgroup that arrives last at `counter` among `expected`; it performs the fold.  No workgroup
+// waits for another.
+__device__ __forceinline__ bool arrive_last(int *counter, int expected)
+{
+    __shared__ int s_last;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // this thread's partial stores are acknowledged
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int t = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (t == expected - 1);
+    }
+    __syncthreads();
+    return s_last != 0;
+}
+
 // ---- kernel A: rows --------------------------------------------------------------------------------------
 // VEC > 1 requires elem_stride == 1, 16-byte aligned rows and seg % VEC == 0 (checked on the host).
-// WAVE_ROW: one wavefront per output (4 outputs per workgroup), otherwise one workgroup per
-// (output, split).
+// WAVE_ROW: one wavefront per output (4 outputs per workgroup, never split), otherwise one
+// workgroup per (output, split); with splits > 1 the last workgroup of an output to finish folds
+// that output's partials in a fixed order.
 
-template <typename T, typename Tr, int VEC, bool WAVE_ROW, bool FOLD>
+template <typename T, typename Tr, int VEC, bool WAVE_ROW, bool NT>
 __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(RedParams<T> p)
 {
     typedef typename Tr::Acc A;
@@ -225,85 +308,99 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(RedParams<T> p)
         int64_t r1 = r0 + p.seg;
         if (r1 > p.R) r1 = p.R;
         if (VEC > 1) {
-            typedef typename VecOf<T>::type V;
             const T *row = p.in + base;
             const int64_t step = (int64_t)lane_n * VEC;
             int64_t r = r0 + (int64_t)lane * VEC;
             // four vectors in flight per lane
             for (; r + 3 * step + VEC <= r1; r += 4 * step) {
-                V x0 = *reinterpret_cast<const V *>(row + r);
-                V x1 = *reinterpret_cast<const V *>(row + r + step);
-                V x2 = *reinterpret_cast<const V *>(row + r + 2 * step);
-                V x3 = *reinterpret_cast<const V *>(row + r + 3 * step);
-                T e0[VEC], e1[VEC], e2[VEC], e3[VEC];
-                __builtin_memcpy(e0, &x0, sizeof(V));
-                __builtin_memcpy(e1, &x1, sizeof(V));
-                __builtin_memcpy(e2, &x2, sizeof(V));
-                __builtin_memcpy(e3, &x3, sizeof(V));
+                Pack<T, VEC> x[4];
 #pragma unroll
-                for (int j = 0; j < VEC; j++) {
-                    acc[0] = Tr::merge(acc[0], Tr::from_elem(e0[j], r + j));
-                    acc[1] = Tr::merge(acc[1], Tr::from_elem(e1[j], r + step + j));
-                    acc[2] = Tr::merge(acc[2], Tr::from_elem(e2[j], r + 2 * step + j));
-                    acc[3] = Tr::merge(acc[3], Tr::from_elem(e3[j], r + 3 * step + j));
+                for (int u = 0; u < 4; u++) x[u] = load_pack<T, VEC, NT>(row + r + u * step);
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+#pragma unroll
+                    for (int j = 0; j < VEC; j++) acc[u] = Tr::update(acc[u], x[u].v[j], r + u * step + j);
                 }
             }
             for (; r + VEC <= r1; r += step) {
-                V x0 = *reinterpret_cast<const V *>(row + r);
-                T e0[VEC];
-                __builtin_memcpy(e0, &x0, sizeof(V));
+                Pack<T, VEC> x = load_pack<T, VEC, false>(row + r);
 #pragma unroll
-                for (int j = 0; j < VEC; j++) acc[0] = Tr::merge(acc[0], Tr::from_elem(e0[j], r + j));
+                for (int j = 0; j < VEC; j++) acc[0] = Tr::update(acc[0], x.v[j], r + j);
             }
             // ragged end of the row (R % VEC != 0 only happens on the last split)
             if (r < r1)
-                for (int j = 0; r + j < r1; j++)
-                    acc[0] = Tr::merge(acc[0], Tr::from_elem(row[r + j], r + j));
+                for (int j = 0; r + j < r1; j++) acc[0] = Tr::update(acc[0], row[r + j], r + j);
+            if (r0 == 0 && lane == 0) acc[0] = Tr::first(acc[0], row[0]);
         } else {
             int64_t r = r0 + lane;
             for (; r + 3 * (int64_t)lane_n < r1; r += 4 * (int64_t)lane_n) {
 #pragma unroll
                 for (int u = 0; u < 4; u++) {
                     const int64_t rr = r + (int64_t)u * lane_n;
-                    const int64_t off = base + rr * p.elem_stride;
-                    acc[u] = Tr::merge(acc[u], FOLD ? Tr::from_partial(p.in[off], Tr::kHasIdx ? p.in_idx[off] : 0)
-                                                    : Tr::from_elem(p.in[off], rr));
+                    acc[u] = Tr::update(acc[u], p.in[base + rr * p.elem_stride], rr);
                 }
             }
-            for (; r < r1; r += lane_n) {
-                const int64_t off = base + r * p.elem_stride;
-                acc[0] = Tr::merge(acc[0], FOLD ? Tr::from_partial(p.in[off], Tr::kHasIdx ? p.in_idx[off] : 0)
-                                                : Tr::from_elem(p.in[off], r));
-            }
+            for (; r < r1; r += lane_n) acc[0] = Tr::update(acc[0], p.in[base + r * p.elem_stride], r);
+            if (r0 == 0 && lane == 0) acc[0] = Tr::first(acc[0], p.in[base]);
         }
     }
     A a = Tr::merge(Tr::merge(acc[0], acc[1]), Tr::merge(acc[2], acc[3]));
     if (WAVE_ROW) {
         a = wave_allreduce<Tr>(a);
-        if (active && lane == 0) emit<T, Tr>(p, o, 0, a);
-    } else {
-        a = block_allreduce<Tr>(a);
-        if (active && lane == 0) emit<T, Tr>(p, o, split, a);
+        if (active && lane == 0) emit_final<T, Tr>(p, o, a);
+        return;
+    }
+    a = block_allreduce<Tr>(a);
+    if (p.splits == 1) {
+        if (lane == 0) emit_final<T, Tr>(p, o, a);
+        return;
+    }
+    if (lane == 0) emit_partial<T, Tr>(p, o * p.splits + split, a);
+    if (!arrive_last(p.counters + o, p.splits)) return;
+    // fold the splits of output o: lane l takes splits l, l + 256, ...; then the fixed block tree
+    A f = Tr::identity();
+    for (int s0 = lane; s0 < p.splits; s0 += 4 * kBlock) {
+        A t[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {   // issue the loads together, merge in split order
+            const int sidx = s0 + u * kBlock;
+            t[u] = sidx < p.splits ? load_partial<T, Tr>(p, o * p.splits + sidx) : Tr::identity();
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) f = Tr::merge(f, t[u]);
+    }
+    f = block_allreduce<Tr>(f);
+    if (lane == 0) {
+        emit_final<T, Tr>(p, o, f);
+        store_agent(p.counters + o, 0);   // back to rest for the next launch
     }
 }
 
 // ---- kernel B: cols ---------------------------------------------------------------------------------------
-// Source [outer, R, inner], inner contiguous.  Thread (tx, ty): tx in 0..63 owns VEC columns,
-// ty in 0..3 walks rows ty, ty+4, ... of its split.  grid = outer * col_tiles * splits.
+// Source [outer, R, inner], inner contiguous.  The 256 threads form a (ty, tx) tile with
+// tx_n = 2^tx_shift lanes along the columns (each owning VEC adjacent columns) and ty_n = 256 / tx_n
+// lanes along the reduced axis, combined through LDS in fixed order.  grid = outer * col_tiles *
+// splits; with splits > 1 partials are stored as [split][output] (coalesced) and the last
+// workgroup of a column tile to finish folds that tile's partials, split 0 first.
 
-template <typename T, typename Tr, int VEC, bool FOLD>
-__global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int64_t col_tiles)
+template <typename T, typename Tr, int VEC, bool NT>
+__global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int64_t col_tiles, int tx_shift)
 {
     typedef typename Tr::Acc A;
-    constexpr int TY = kBlock / kWave;
-    const int tx = threadIdx.x & (kWave - 1);
-    const int ty = threadIdx.x / kWave;
+    __shared__ A lds[kBlock * VEC];
+    const int tx_n = 1 << tx_shift;
+    const int ty_n = kBlock >> tx_shift;
+    const int tx = threadIdx.x & (tx_n - 1);
+    const int ty = threadIdx.x >> tx_shift;
+    // column tile fastest: workgroups that are dispatched together read adjacent pieces of the
+    // same source rows
     int64_t blk = blockIdx.x;
-    const int split = (int)(blk % p.splits);
-    blk /= p.splits;
     const int64_t ct = blk % col_tiles;
-    const int64_t q = blk / col_tiles;
-    const int64_t c = (ct * kWave + tx) * VEC;
+    blk /= col_tiles;
+    const int split = (int)(blk % p.splits);
+    const int64_t q = blk / p.splits;
+    const int64_t group = q * col_tiles + ct;   // the workgroups that share these outputs
+    const int64_t c = (ct * tx_n + tx) * VEC;
     const int64_t r0 = (int64_t)split * p.seg;
     int64_t r1 = r0 + p.seg;
     if (r1 > p.R) r1 = p.R;
@@ -314,94 +411,156 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int
 
     const int ncol = (c + VEC <= p.inner) ? VEC : (c < p.inner ? (int)(p.inner - c) : 0);
     const T *src = p.in + q * p.outer_stride + c;
-    const int64_t *srci = FOLD && Tr::kHasIdx ? p.in_idx + q * p.outer_stride + c : nullptr;
-    if (ncol == VEC && VEC > 1 && !FOLD) {
-        typedef typename VecOf<T>::type V;
+    if (ncol == VEC && VEC > 1) {
         int64_t r = r0 + ty;
-        for (; r + 3 * TY < r1; r += 4 * TY) {
-            V x[4];
+        for (; r + 3 * ty_n < r1; r += 4 * ty_n) {
+            Pack<T, VEC> x[4];
 #pragma unroll
-            for (int u = 0; u < 4; u++) x[u] = *reinterpret_cast<const V *>(src + (r + u * TY) * p.elem_stride);
+            for (int u = 0; u < 4; u++) x[u] = load_pack<T, VEC, NT>(src + (r + u * ty_n) * p.elem_stride);
 #pragma unroll
             for (int u = 0; u < 4; u++) {
-                T e[VEC];
-                __builtin_memcpy(e, &x[u], sizeof(V));
 #pragma unroll
-                for (int j = 0; j < VEC; j++) acc[j] = Tr::merge(acc[j], Tr::from_elem(e[j], r + u * TY));
+                for (int j = 0; j < VEC; j++) acc[j] = Tr::update(acc[j], x[u].v[j], r + u * ty_n);
             }
         }
-        for (; r < r1; r += TY) {
-            V x = *reinterpret_cast<const V *>(src + r * p.elem_stride);
-            T e[VEC];
-            __builtin_memcpy(e, &x, sizeof(V));
+        for (; r < r1; r += ty_n) {
+            Pack<T, VEC> x = load_pack<T, VEC, false>(src + r * p.elem_stride);
 #pragma unroll
-            for (int j = 0; j < VEC; j++) acc[j] = Tr::merge(acc[j], Tr::from_elem(e[j], r));
+            for (int j = 0; j < VEC; j++) acc[j] = Tr::update(acc[j], x.v[j], r);
         }
     } else if (ncol > 0) {
-        for (int64_t r = r0 + ty; r < r1; r += TY) {
-            for (int j = 0; j < ncol; j++) {
-                const int64_t off = r * p.elem_stride + j;
-                acc[j] = Tr::merge(acc[j], FOLD ? Tr::from_partial(src[off], Tr::kHasIdx ? srci[off] : 0)
-                                                : Tr::from_elem(src[off], r));
+        for (int64_t r = r0 + ty; r < r1; r += ty_n)
+            for (int j = 0; j < ncol; j++) acc[j] = Tr::update(acc[j], src[r * p.elem_stride + j], r);
+    }
+    if (r0 == 0 && ty == 0)
+        for (int j = 0; j < ncol; j++) acc[j] = Tr::first(acc[j], src[j]);
+
+    // combine the ty lanes in fixed order
+    if (ty_n > 1) {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) lds[threadIdx.x * VEC + j] = acc[j];
+        __syncthreads();
+        if (ty == 0) {
+#pragma unroll
+            for (int j = 0; j < VEC; j++) {
+                A r = lds[tx * VEC + j];
+                for (int w = 1; w < ty_n; w++) r = Tr::merge(r, lds[(w * tx_n + tx) * VEC + j]);
+                acc[j] = r;
             }
         }
     }
-
-    // combine the TY row lanes in fixed order
-    __shared__ A lds[TY][kWave][VEC];
+    const int64_t o0 = q * p.inner + c;
+    if (p.splits == 1) {
+        if (ty == 0)
+            for (int j = 0; j < ncol; j++) emit_final<T, Tr>(p, o0 + j, acc[j]);
+        return;
+    }
+    if (ty == 0)
+        for (int j = 0; j < ncol; j++) emit_partial<T, Tr>(p, (int64_t)split * p.nout + o0 + j, acc[j]);
+    if (!arrive_last(p.counters + group, p.splits)) return;
+    // fold this column tile: row lane ty takes splits ty, ty + ty_n, ...; then the fixed LDS order
 #pragma unroll
-    for (int j = 0; j < VEC; j++) lds[ty][tx][j] = acc[j];
-    __syncthreads();
-    if (ty == 0) {
+    for (int j = 0; j < VEC; j++) acc[j] = Tr::identity();
+    for (int s0 = ty; s0 < p.splits; s0 += 8 * ty_n) {
+        A t[8][VEC];
 #pragma unroll
-        for (int j = 0; j < VEC; j++) {
-            A r = lds[0][tx][j];
+        for (int u = 0; u < 8; u++) {       // issue the loads together, merge in split order
+            const int sidx = s0 + u * ty_n;
 #pragma unroll
-            for (int w = 1; w < TY; w++) r = Tr::merge(r, lds[w][tx][j]);
-            if (j < ncol) emit<T, Tr>(p, q * p.inner + c + j, split, r);
+            for (int j = 0; j < VEC; j++)
+                t[u][j] = (sidx < p.splits && j < ncol) ? load_partial<T, Tr>(p, (int64_t)sidx * p.nout + o0 + j)
+                                                        : Tr::identity();
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+#pragma unroll
+            for (int j = 0; j < VEC; j++) acc[j] = Tr::merge(acc[j], t[u][j]);
         }
     }
+    if (ty_n > 1) {
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < VEC; j++) lds[threadIdx.x * VEC + j] = acc[j];
+        __syncthreads();
+        if (ty == 0) {
+#pragma unroll
+            for (int j = 0; j < VEC; j++) {
+                A r = lds[tx * VEC + j];
+                for (int w = 1; w < ty_n; w++) r = Tr::merge(r, lds[(w * tx_n + tx) * VEC + j]);
+                acc[j] = r;
+            }
+        }
+    }
+    if (ty == 0)
+        for (int j = 0; j < ncol; j++) emit_final<T, Tr>(p, o0 + j, acc[j]);
+    if (threadIdx.x == 0) store_agent(p.counters + group, 0);
 }
 
 // ---- host side ---------------------------------------------------------------------------------------------
 
-inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+// the source is read once; when it is larger than the caches the loads carry the streaming hint
+template <typename T> inline bool stream_source(const RedParams<T> &p)
+{
+    return p.nout * p.R * (int64_t)sizeof(T) >= kStreamBytes;
+}
 
-template <typename T, typename Tr, bool FOLD>
+template <typename T, typename Tr>
 int launch_rows(const RedParams<T> &p, hipStream_t s)
 {
     constexpr int VEC = VecOf<T>::N;
-    const bool vec = !FOLD && p.elem_stride == 1 && p.inner == 1 && aligned16(p.in) &&
-                     p.outer_stride % VEC == 0 && p.seg % VEC == 0;
+    const bool vec = p.elem_stride == 1 && p.inner == 1 && aligned16(p.in) && p.outer_stride % VEC == 0 &&
+                     p.seg % VEC == 0;
+    const bool nt = vec && stream_source(p);
     const bool wave_row = p.splits == 1 && p.R <= 1024;
     if (wave_row) {
         int64_t grid = (p.nout + kWaves - 1) / kWaves;
         if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-        if (vec) reduce_rows_kernel<T, Tr, VEC, true, FOLD><<<(unsigned)grid, kBlock, 0, s>>>(p);
-        else     reduce_rows_kernel<T, Tr, 1, true, FOLD><<<(unsigned)grid, kBlock, 0, s>>>(p);
+        if (nt)       reduce_rows_kernel<T, Tr, VEC, true, true><<<(unsigned)grid, kBlock, 0, s>>>(p);
+        else if (vec) reduce_rows_kernel<T, Tr, VEC, true, false><<<(unsigned)grid, kBlock, 0, s>>>(p);
+        else          reduce_rows_kernel<T, Tr, 1, true, false><<<(unsigned)grid, kBlock, 0, s>>>(p);
     } else {
         int64_t grid = p.nout * p.splits;
         if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-        if (vec) reduce_rows_kernel<T, Tr, VEC, false, FOLD><<<(unsigned)grid, kBlock, 0, s>>>(p);
-        else     reduce_rows_kernel<T, Tr, 1, false, FOLD><<<(unsigned)grid, kBlock, 0, s>>>(p);
+        if (nt)       reduce_rows_kernel<T, Tr, VEC, false, true><<<(unsigned)grid, kBlock, 0, s>>>(p);
+        else if (vec) reduce_rows_kernel<T, Tr, VEC, false, false><<<(unsigned)grid, kBlock, 0, s>>>(p);
+        else          reduce_rows_kernel<T, Tr, 1, false, false><<<(unsigned)grid, kBlock, 0, s>>>(p);
     }
     ZENU_LAUNCH_CHECK();
     return ZENU_OK;
 }
 
-template <typename T, typename Tr, bool FOLD>
+// threads along the columns for a cols launch: a power of two covering the row, at most kColsTx
+constexpr int kColsTx = 32;  // 32 lanes x 16 B = 512 B of a source row per wavefront half (measured best of 8..256)
+inline int cols_tx_shift(int64_t inner, int v)
+{
+    const int64_t vcols = (inner + v - 1) / v;
+    int shift = 0;
+    while ((1 << shift) < kColsTx && ((int64_t)1 << shift) < vcols) shift++;
+    return shift;
+}
+
+template <typename T> inline bool cols_vec_ok(const RedParams<T> &p)
+{
+    constexpr int VEC = VecOf<T>::N;
+    return aligned16(p.in) && p.inner % VEC == 0 && p.outer_stride % VEC == 0 && p.elem_stride % VEC == 0;
+}
+
+template <typename T, typename Tr>
 int launch_cols(const RedParams<T> &p, hipStream_t s)
 {
     constexpr int VEC = VecOf<T>::N;
-    const bool vec = aligned16(p.in) && p.inner % VEC == 0 && p.outer_stride % VEC == 0 &&
-                     p.elem_stride % VEC == 0;
+    const bool vec = cols_vec_ok(p);
+    const bool nt = vec && stream_source(p);
     const int v = vec ? VEC : 1;
-    const int64_t col_tiles = (p.inner + (int64_t)kWave * v - 1) / ((int64_t)kWave * v);
+    const int shift = cols_tx_shift(p.inner, v);
+    const int64_t per_tile = ((int64_t)1 << shift) * v;
+    const int64_t col_tiles = (p.inner + per_tile - 1) / per_tile;
     const int64_t outer = p.nout / p.inner;
     int64_t grid = outer * col_tiles * p.splits;
     if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-    if (vec) reduce_cols_kernel<T, Tr, VEC, FOLD><<<(unsigned)grid, kBlock, 0, s>>>(p, col_tiles);
-    else     reduce_cols_kernel<T, Tr, 1, FOLD><<<(unsigned)grid, kBlock, 0, s>>>(p, col_tiles);
+    if (nt)       reduce_cols_kernel<T, Tr, VEC, true><<<(unsigned)grid, kBlock, 0, s>>>(p, col_tiles, shift);
+    else if (vec) reduce_cols_kernel<T, Tr, VEC, false><<<(unsigned)grid, kBlock, 0, s>>>(p, col_tiles, shift);
+    else          reduce_cols_kernel<T, Tr, 1, false><<<(unsigned)grid, kBlock, 0, s>>>(p, col_tiles, shift);
     ZENU_LAUNCH_CHECK();
     return ZENU_OK;
 }
@@ -415,11 +574,13 @@ int reduce_contiguous(const T *src, int64_t outer, int64_t R, int64_t inner, T *
     const int64_t nout = outer * inner;
     if (nout == 0) return ZENU_OK;
     if (R <= 0) return ZENU_ERR_SHAPE;
-    const int64_t target_blocks = (int64_t)device_info().num_cus * 8;
+    if (Tr::kHasIdx && R >= kNoIdx) return ZENU_ERR_UNSUPPORTED;  // positions are tracked in 32 bits
+    // workgroups to aim for when the outputs alone do not fill the GPU: two per CU.  More splits
+    // shorten the streaming phase but lengthen the serial hand-off at the end (measured 1..16).
+    const int64_t target_blocks = (int64_t)device_info().num_cus * 2;
 
     RedParams<T> p;
     p.in = src;
-    p.in_idx = nullptr;
     p.nout = nout;
     p.R = R;
     p.inner = inner;
@@ -429,18 +590,23 @@ int reduce_contiguous(const T *src, int64_t outer, int64_t R, int64_t inner, T *
     p.out_idx = out_idx;
     p.part_key = nullptr;
     p.part_idx = nullptr;
+    p.counters = nullptr;
     p.gsrc = src;
     p.g_outer_stride = R * inner;
     p.g_elem_stride = inner;
 
     const bool use_cols = inner >= 16;
-    int64_t splits = 1;
+    int64_t splits = 1, groups = nout;
     if (use_cols) {
-        const int64_t col_tiles = (inner + (int64_t)kWave * VEC - 1) / ((int64_t)kWave * VEC);
-        const int64_t blocks = outer * col_tiles;
-        if (blocks < target_blocks) {
-            splits = (target_blocks + blocks - 1) / blocks;
-            const int64_t max_splits = (R + 31) / 32;  // at least 32 rows per workgroup
+        const int v = cols_vec_ok(p) ? VEC : 1;
+        const int shift = cols_tx_shift(inner, v);
+        const int64_t per_tile = ((int64_t)1 << shift) * v;
+        const int64_t col_tiles = (inner + per_tile - 1) / per_tile;
+        const int64_t ty_n = kBlock >> shift;
+        groups = outer * col_tiles;
+        if (groups < target_blocks) {
+            splits = (target_blocks + groups - 1) / groups;
+            const int64_t max_splits = (R + 8 * ty_n - 1) / (8 * ty_n);  // >= 8 rows per thread
             if (splits > max_splits) splits = max_splits;
         }
     } else {
@@ -459,79 +625,22 @@ int reduce_contiguous(const T *src, int64_t outer, int64_t R, int64_t inner, T *
     p.splits = (int)splits;
     p.seg = seg;
 
-    if (splits == 1) {
-        return use_cols ? launch_cols<T, Tr, false>(p, s) : launch_rows<T, Tr, false>(p, s);
-    }
+    if (splits == 1) return use_cols ? launch_cols<T, Tr>(p, s) : launch_rows<T, Tr>(p, s);
 
-    // two launches: partials [nout, splits] in a workspace, then fold them
+    // one launch: partials in a workspace, folded by the last workgroup of each group to arrive
+    int *counters = reserve_counters(groups);
+    if (!counters) return ZENU_ERR_UNSUPPORTED;
     const size_t key_bytes = ((size_t)nout * splits * sizeof(T) + 255) / 256 * 256;
-    const size_t idx_bytes = Tr::kHasIdx ? (size_t)nout * splits * sizeof(int64_t) : 0;
+    const size_t idx_bytes = Tr::kHasIdx ? (size_t)nout * splits * sizeof(int32_t) : 0;
     Workspace ws(key_bytes + idx_bytes, s);
     if (ws.status) return ws.status;
     p.part_key = static_cast<T *>(ws.ptr);
-    p.part_idx = Tr::kHasIdx ? reinterpret_cast<int64_t *>(static_cast<char *>(ws.ptr) + key_bytes) : nullptr;
-    int rc = use_cols ? launch_cols<T, Tr, false>(p, s) : launch_rows<T, Tr, false>(p, s);
-    if (rc) return rc;
-
-    RedParams<T> f = p;
-    f.in = p.part_key;
-    f.in_idx = p.part_idx;
-    f.R = splits;
-    f.inner = 1;           // partials are [nout, splits]: a rows problem
-    f.outer_stride = splits;
-    f.elem_stride = 1;
-    f.splits = 1;
-    f.seg = (splits + 15) / 16 * 16;
-    f.part_key = nullptr;
-    f.part_idx = nullptr;
-    // the value gather still addresses the original source: output o = (q, c)
-    // (emit() derives q and c from f.inner, so keep the source geometry for the gather)
-    if (Tr::kHasIdx && out_val) {
-        // gather needs the original inner; run the fold for indices only, then gather below
-        Workspace wi(out_idx ? 0 : (size_t)nout * sizeof(int64_t), s);
-        int64_t *idx_buf = out_idx;
-        if (!idx_buf) {
-            if (wi.status) return wi.status;
-            idx_buf = static_cast<int64_t *>(wi.ptr);
-        }
-        f.out_val = nullptr;
-        f.out_idx = idx_buf;
-        rc = launch_rows<T, Tr, true>(f, s);
-        if (rc) return rc;
-        return gather_axis(src, idx_buf, out_val, nout, inner, R * inner, inner, (int)sizeof(T), s);
-    }
-    return launch_rows<T, Tr, true>(f, s);
-}
-
-template <typename T>
-__global__ __launch_bounds__(kBlock) void gather_axis_kernel(const T *src, const int64_t *idx, T *out,
-                                                             int64_t nout, int64_t inner,
-                                                             int64_t outer_stride, int64_t elem_stride)
-{
-    int64_t o = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (o >= nout) return;
-    const int64_t q = o / inner, c = o - q * inner;
-    out[o] = src[q * outer_stride + c + idx[o] * elem_stride];
+    p.part_idx = Tr::kHasIdx ? reinterpret_cast<int32_t *>(static_cast<char *>(ws.ptr) + key_bytes) : nullptr;
+    p.counters = counters;
+    return use_cols ? launch_cols<T, Tr>(p, s) : launch_rows<T, Tr>(p, s);
 }
 
 }  // namespace
-
-int gather_axis(const void *src, const int64_t *idx, void *out, int64_t nout, int64_t inner,
-                int64_t outer_stride, int64_t elem_stride, int elem_size, hipStream_t s)
-{
-    int64_t grid = (nout + kBlock - 1) / kBlock;
-    if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-    if (elem_size == 4)
-        gather_axis_kernel<float><<<(unsigned)grid, kBlock, 0, s>>>(
-            static_cast<const float *>(src), idx, static_cast<float *>(out), nout, inner, outer_stride,
-            elem_stride);
-    else
-        gather_axis_kernel<double><<<(unsigned)grid, kBlock, 0, s>>>(
-            static_cast<const double *>(src), idx, static_cast<double *>(out), nout, inner, outer_stride,
-            elem_stride);
-    ZENU_LAUNCH_CHECK();
-    return ZENU_OK;
-}
 
 namespace {
 

@@ -43,9 +43,14 @@ struct HipBackend : AllocBackend {
     int device_synchronize() override { return hipDeviceSynchronize() == hipSuccess ? 0 : 1; }
 };
 
+constexpr int64_t kNumCounters = 1 << 16;
+
 struct State {
     bool ready = false;
     bool use_pool = true;
+    int *counters = nullptr;      // arrival counters of the reductions, zero at rest
+    int64_t counter_cursor = 0;
+    std::mutex counter_mu;
     DeviceInfo info;
     HipBackend backend;
     CachingAllocator *pool = nullptr;
@@ -72,6 +77,9 @@ int init_locked(int device)
     const char *env = getenv("ZENU_USE_MEMPOOL");  // zenu-matrix/src/lib.rs:36, default "1"
     g_state.use_pool = !(env && strcmp(env, "0") == 0);
     g_state.pool = new CachingAllocator(&g_state.backend);
+    ZENU_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&g_state.counters), kNumCounters * sizeof(int)));
+    ZENU_HIP_TRY(hipMemset(g_state.counters, 0, kNumCounters * sizeof(int)));
+    g_state.counter_cursor = 0;
     g_state.ready = true;
     return ZENU_OK;
 }
@@ -87,6 +95,18 @@ __global__ void fill_zero_kernel(uint4 *dst16, size_t n16, unsigned char *tail, 
 }  // namespace
 
 const DeviceInfo &device_info() { return g_state.info; }
+
+// Consecutive launches take consecutive ranges of the ring, so a range is reused only after
+// kNumCounters counters' worth of later reductions; every kernel leaves its counters at zero.
+int *reserve_counters(int64_t n)
+{
+    if (n <= 0 || n > kNumCounters || !g_state.counters) return nullptr;
+    std::lock_guard<std::mutex> g(g_state.counter_mu);
+    if (g_state.counter_cursor + n > kNumCounters) g_state.counter_cursor = 0;
+    int *r = g_state.counters + g_state.counter_cursor;
+    g_state.counter_cursor += n;
+    return r;
+}
 
 int ensure_init()
 {
@@ -123,6 +143,8 @@ int zenu_hip_shutdown(void)
     (void)hipDeviceSynchronize();
     delete g_state.pool;
     g_state.pool = nullptr;
+    if (g_state.counters) (void)hipFree(g_state.counters);
+    g_state.counters = nullptr;
     g_state.ready = false;
     return ZENU_OK;
 }

@@ -162,12 +162,88 @@ ZM_HD float tanhf_fdlibm(float x)
     return neg ? -z : z;
 }
 
+// The same tanh, restructured for 64-wide SIMD execution: one path through the argument
+// reduction, the rational core and ONE division pair for every lane, the per-k tails computed
+// side by side and selected, so that a wavefront whose lanes hold |x| on both sides of 1 and
+// different k does not execute the branches of tanhf_fdlibm one after another.  Every
+// arithmetic operation that reaches the result is the one tanhf_fdlibm performs, on the same
+// operands, so the bits are identical; this is checked over every f32 bit pattern against
+// tanhf_fdlibm and the host libm (tests/test_zmath_host.py, dense sample; exhaustive run kept
+// out of the default suite).
+ZM_HD float tanhf_simd(float x)
+{
+    const float one = 1.0f, two = 2.0f;
+    const float ln2_hi = u2f(0x3f317180u), ln2_lo = u2f(0x3717f7d1u), invln2 = u2f(0x3fb8aa3bu);
+    const float Q1 = u2f(0xbd088889u), Q2 = u2f(0x3ad00d01u), Q3 = u2f(0xb8a670cdu),
+                Q4 = u2f(0x36867e54u), Q5 = u2f(0xb457edbbu);
+    const uint32_t jx = f2u(x);
+    const uint32_t ix = jx & 0x7fffffffu;
+    const bool neg = (jx >> 31) != 0;
+
+    if (ix >= 0x41b00000u) {                 // |x| >= 22, inf, NaN (rare)
+        if (ix >= 0x7f800000u) return neg ? one / x - one : one / x + one;
+        return neg ? -one : one;             // 1 - tiny rounds to 1
+    }
+    if (ix < 0x24000000u) return ix == 0 ? x : x * (one + x);   // |x| < 2^-55
+
+    const float ax = u2f(ix);
+    const bool big = ix >= 0x3f800000u;      // |x| >= 1: expm1(+2|x|), else expm1(-2|x|)
+    const float a = big ? two * ax : -two * ax;
+    const uint32_t ha = f2u(a) & 0x7fffffffu;
+
+    // expm1(a), a in (-2, 0) or [2, 44): k = round(a / ln2) when |a| > 0.5 ln2, else 0
+    int32_t k = (int32_t)(invln2 * a + (big ? 0.5f : -0.5f));
+    k = (ha > 0x3eb17218u) ? k : 0;
+    const float tk = (float)k;
+    const float hi = a - tk * ln2_hi;
+    const float lo = tk * ln2_lo;
+    const float xr = hi - lo;
+    const float c = (hi - xr) - lo;
+
+    const float hfx = 0.5f * xr;
+    const float hxs = xr * hfx;
+    const float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    float t = 3.0f - r1 * hfx;
+    const float e = hxs * ((r1 - t) / (6.0f - xr * t));
+
+    float em1;                               // expm1(a)
+    if (ha < 0x33000000u) {
+        em1 = a;                             // |a| < 2^-25
+    } else if (k == 0) {
+        em1 = xr - (xr * e - hxs);
+    } else {
+        float e1 = (xr * (e - c) - c);
+        e1 -= hxs;
+        if (k == -1) {
+            em1 = 0.5f * (xr - e1) - 0.5f;
+        } else if (k <= -2 || k > 56) {
+            float y = one - (e1 - xr);
+            y = u2f(f2u(y) + ((uint32_t)k << 23));
+            em1 = y - one;
+        } else if (k < 23) {                 // 2 <= k < 23 here (k == 1 needs |a| < 1.5 ln2 < 2)
+            const float tt = u2f(0x3f800000u - (0x1000000u >> k));
+            float y = tt - (e1 - xr);
+            em1 = u2f(f2u(y) + ((uint32_t)k << 23));
+        } else {
+            const float tt = u2f((uint32_t)(0x7f - k) << 23);
+            float y = xr - (e1 + tt);
+            y += one;
+            em1 = u2f(f2u(y) + ((uint32_t)k << 23));
+        }
+    }
+    // |x| >= 1: 1 - 2/(t+2);  |x| < 1: -t/(t+2) = -(t/(t+2))
+    const float num = big ? two : em1;
+    const float q = num / (em1 + two);
+    const float z = big ? one - q : -q;
+    return neg ? -z : z;
+}
+
 // ZeNu's sigmoid composite in f32: each step rounded to f32, as the four autograd ops do.
 ZM_HD float sigmoidf_zenu(float x)
 {
     const float half = 0.5f;
     float xh = x * half;
-    float th = tanhf_fdlibm(xh);
+    float th = tanhf_simd(xh);
     float ht = half * th;
     return half + ht;
 }
