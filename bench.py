@@ -121,6 +121,11 @@ def build_ops(z, workload, stream):
             da, do = A.desc(), O.desc()
             ls.append(lambda da=da, do=do: check(l.zenu_hip_relu(_lib.F32, ref(do), ref(da), 0.0, stream), "relu"))
         ops.append(Op("relu[2^24]", "c0", "f32", 2 * 4 * n, n, ls, lambda: zo.relu(out_h, a, 0.0)))
+        ls = []
+        for A, B, O in sets:
+            da, do = A.desc(), O.desc()
+            ls.append(lambda da=da, do=do: check(l.zenu_hip_copy(_lib.F32, ref(do), ref(da), stream), "copy"))
+        ops.append(Op("copy[2^24]", "c0", "f32", 2 * 4 * n, n, ls, lambda: zo.copy_from(out_h, a)))
         ops[-1].keep = keep
 
     # ---- config[1]: [4096,4096] f32, normal(0,1), seed 1 ----------------------------------------
@@ -219,6 +224,21 @@ def build_ops(z, workload, stream):
     return ops
 
 
+def measured_traffic(op):
+    """HBM bytes per launch of the op's kernel from the committed rocprofv3 --pmc summary
+    (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size), or None if not recorded."""
+    if op.config != "c3":
+        return None
+    path = os.path.join(ROOT, "profiles", "adam_kernel_c3_adamw25M_pmc_traffic.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return int(line.split(":")[1])
+    except OSError:
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -294,7 +314,7 @@ def main():
     dom = max(table, key=lambda t: t["us"])
     dom_op = [o for o in ops if o.name == dom["op"]][0]
     roofline = dict(bound="hbm", achieved=dom["GBps"], peak=PEAK_HBM_GBPS, unit="GB/s",
-                    frac=round(dom["GBps"] / PEAK_HBM_GBPS, 4), traffic=None,
+                    frac=round(dom["GBps"] / PEAK_HBM_GBPS, 4), traffic=measured_traffic(dom_op),
                     kernel=dom_op.kernel or dom["op"], algorithmic_bytes_per_launch=dom["alg_bytes"],
                     avg_launch_us=dom["us"])
     adam = [t for t in table if t["config"] == "c3"]

@@ -86,8 +86,10 @@ int zenu_hip_device_synchronize(void);
 /* Stream-ordered caching allocator: replaces zenu-matrix/src/memory_pool/mod.rs:79-145 and
  * cuda_malloc_bytes / cuda_free (runtime/mod.rs:30-60, which synchronise the stream on every
  * call).  zenu_hip_malloc never synchronises on a cache hit.  A block freed on stream S is
- * reusable at once by allocations on S, and by other streams only after an event recorded at
- * the free has completed.  On out-of-memory the cache is trimmed and the request retried once
+ * reusable at once by allocations on S; another stream takes it only behind an event (recorded
+ * on S at the moment of reuse, waited for by the new stream), never behind a host wait.  `stream`
+ * of zenu_hip_free is the last stream that used the block.
+ * On out-of-memory the cache is trimmed and the request retried once
  * (the flow zenu-matrix/src/memory_pool/mod.rs:9-20 documents).  Thread-safe.
  * Honours ZENU_USE_MEMPOOL=0 (zenu-matrix/src/lib.rs:36): every call goes to hipMalloc/hipFree. */
 int zenu_hip_malloc(void **ptr_dev, size_t bytes, zenu_stream_t stream);

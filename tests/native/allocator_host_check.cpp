@@ -1,0 +1,158 @@
+// Host-only test driver for zenu_amd/csrc/allocator.hpp with a fake device backend (the role
+// MockDeviceBase plays in zenu-matrix/src/memory_pool/test.rs:18-49): bookkeeping, stream
+// ordering, out-of-memory handling and foreign pointers, without a GPU.
+// Prints one "ok <name>" line per check; exits non-zero on the first failure.
+#include <cstdio>
+#include <cstdlib>
+#include <set>
+#include <vector>
+
+#include "../../zenu_amd/csrc/allocator.hpp"
+
+using namespace zenu;
+
+struct FakeBackend : AllocBackend {
+    size_t capacity = 1ull << 40, used = 0;
+    uintptr_t next = 0x10000000;
+    std::set<void *> live;
+    std::vector<std::pair<void *, void *>> orderings;  // (owner stream, waiter stream)
+    int syncs = 0, fail_next = 0;
+    int raw_alloc(void **p, size_t bytes) override
+    {
+        if (fail_next > 0) { fail_next--; *p = nullptr; return 1; }
+        if (used + bytes > capacity) { *p = nullptr; return 1; }
+        *p = reinterpret_cast<void *>(next);
+        next += (bytes + 0xfffff) & ~0xfffffull;
+        used += bytes;
+        live.insert(*p);
+        sizes[*p] = bytes;
+        return 0;
+    }
+    int raw_free(void *p) override
+    {
+        if (!live.count(p)) return 1;
+        live.erase(p);
+        used -= sizes[p];
+        return 0;
+    }
+    int order_after(void *owner, void *waiter) override { orderings.push_back({owner, waiter}); return 0; }
+    int device_synchronize() override { syncs++; return 0; }
+    std::map<void *, size_t> sizes;
+};
+
+#define CHECK(cond, name)                                             \
+    do {                                                              \
+        if (!(cond)) { printf("FAIL %s (line %d)\n", name, __LINE__); return 1; } \
+    } while (0)
+
+int main()
+{
+    void *S1 = reinterpret_cast<void *>(0x1), *S2 = reinterpret_cast<void *>(0x2);
+    {   // size classes: small requests share a 2 MiB segment, large ones get their own
+        FakeBackend be; CachingAllocator a(&be);
+        void *p1, *p2, *p3;
+        CHECK(a.malloc(&p1, 1000, S1) == 0 && a.malloc(&p2, 5000, S1) == 0, "small alloc");
+        CHECK(be.live.size() == 1 && a.stats().bytes_reserved == CachingAllocator::kSmallSegment, "one small segment");
+        CHECK((char *)p2 - (char *)p1 == 1024, "512-byte rounding, adjacent blocks");
+        CHECK(a.malloc(&p3, 100u << 20, S1) == 0 && be.live.size() == 2, "large alloc own segment");
+        CHECK(a.stats().bytes_in_use == 1024 + 5120 + (100u << 20), "bytes_in_use");
+        CHECK(a.free(p1, S1) == 0 && a.free(p2, S1) == 0 && a.free(p3, S1) == 0, "free");
+        CHECK(a.stats().bytes_in_use == 0 && a.stats().bytes_cached == a.stats().bytes_reserved, "all cached");
+        printf("ok size_classes\n");
+    }
+    {   // reuse on the same stream: immediate, no driver call, no ordering needed
+        FakeBackend be; CachingAllocator a(&be);
+        void *p, *q;
+        a.malloc(&p, 64u << 20, S1); a.free(p, S1);
+        a.malloc(&q, 64u << 20, S1);
+        CHECK(q == p && a.stats().n_driver_allocs == 1 && a.stats().n_cache_hits == 1, "same-stream reuse");
+        CHECK(be.orderings.empty() && be.syncs == 0, "no synchronisation on a hit");
+        a.free(q, S1);
+        printf("ok same_stream_reuse\n");
+    }
+    {   // reuse across streams goes through an event: owner stream -> waiter stream
+        FakeBackend be; CachingAllocator a(&be);
+        void *p, *q;
+        a.malloc(&p, 64u << 20, S1); a.free(p, S1);
+        a.malloc(&q, 64u << 20, S2);
+        CHECK(q == p && a.stats().n_driver_allocs == 1, "cross-stream reuse");
+        CHECK(be.orderings.size() == 1 && be.orderings[0].first == S1 && be.orderings[0].second == S2, "event ordering");
+        a.free(q, S2);
+        void *r; a.malloc(&r, 64u << 20, S2);
+        CHECK(r == p && be.orderings.size() == 1, "block now belongs to the second stream");
+        a.free(r, S2);
+        printf("ok cross_stream_reuse\n");
+    }
+    {   // holes in the middle of a segment are reusable; neighbours merge on free
+        FakeBackend be; CachingAllocator a(&be);
+        void *p[4];
+        for (int i = 0; i < 4; i++) a.malloc(&p[i], 256 << 10, S1);
+        a.free(p[1], S1);
+        void *h; a.malloc(&h, 200 << 10, S1);
+        CHECK(h == p[1], "hole reused (the reference's bump allocator cannot)");
+        a.free(h, S1); a.free(p[2], S1);
+        void *m; a.malloc(&m, 512 << 10, S1);
+        CHECK(m == p[1], "freed neighbours merged");
+        a.free(m, S1); a.free(p[0], S1); a.free(p[3], S1);
+        CHECK(a.trim() == 0 && be.live.empty() && a.stats().bytes_reserved == 0, "trim returns whole segments");
+        printf("ok split_merge_trim\n");
+    }
+    {   // out of memory: synchronise, drop the cache, retry once; then a clean error
+        FakeBackend be; be.capacity = 300u << 20; CachingAllocator a(&be);
+        void *p, *q, *r;
+        CHECK(a.malloc(&p, 200u << 20, S1) == 0, "first");
+        a.free(p, S1);
+        CHECK(a.malloc(&q, 250u << 20, S1) == 0, "retry after trimming the cache");
+        CHECK(a.stats().n_oom_retries == 1 && be.syncs == 1 && a.stats().n_driver_frees == 1, "oom path taken");
+        CHECK(a.malloc(&r, 200u << 20, S1) == CachingAllocator::kErrOom && r == nullptr, "clean OOM error");
+        a.free(q, S1);
+        printf("ok oom_retry\n");
+    }
+    {   // a failing driver call (injected) also takes the retry path
+        FakeBackend be; CachingAllocator a(&be);
+        be.fail_next = 1;
+        void *p;
+        CHECK(a.malloc(&p, 4u << 20, S1) == 0 && a.stats().n_oom_retries == 1, "transient failure retried");
+        be.fail_next = 2;
+        void *q;
+        CHECK(a.malloc(&q, 40u << 20, S1) == CachingAllocator::kErrOom, "persistent failure reported");
+        a.free(p, S1);
+        printf("ok injected_failure\n");
+    }
+    {   // foreign pointer / double free -> not owned (the caller falls back to a raw free)
+        FakeBackend be; CachingAllocator a(&be);
+        void *p; a.malloc(&p, 4096, S1);
+        CHECK(a.free(reinterpret_cast<void *>(0xdeadbeef), S1) == CachingAllocator::kErrNotOwned, "foreign pointer");
+        CHECK(a.free(p, S1) == 0 && a.free(p, S1) == CachingAllocator::kErrNotOwned, "double free");
+        CHECK(a.free(nullptr, S1) == 0, "null is a no-op");
+        printf("ok not_owned\n");
+    }
+    {   // randomized stress against a shadow model: no overlap, accounting consistent
+        FakeBackend be; CachingAllocator a(&be);
+        struct L { char *p; size_t n; void *s; };
+        std::vector<L> live;
+        unsigned x = 1;
+        auto rnd = [&]() { x = x * 1664525u + 1013904223u; return x >> 8; };
+        for (int it = 0; it < 20000; it++) {
+            if (live.empty() || rnd() % 3) {
+                size_t n = (rnd() % 4 == 0) ? (size_t)(rnd() % (32u << 20)) + 1 : (size_t)(rnd() % 70000) + 1;
+                void *s = (rnd() & 1) ? S1 : S2, *p;
+                CHECK(a.malloc(&p, n, s) == 0, "stress alloc");
+                for (auto &l : live) CHECK((char *)p + n <= l.p || l.p + l.n <= (char *)p, "no overlap");
+                live.push_back({(char *)p, n, s});
+            } else {
+                size_t i = rnd() % live.size();
+                CHECK(a.free(live[i].p, live[i].s) == 0, "stress free");
+                live[i] = live.back(); live.pop_back();
+            }
+            AllocStats st = a.stats();
+            CHECK(st.bytes_reserved == st.bytes_in_use + st.bytes_cached, "reserved = in use + cached");
+        }
+        for (auto &l : live) a.free(l.p, l.s);
+        CHECK(a.stats().bytes_in_use == 0, "all returned");
+        a.trim();
+        CHECK(be.live.empty(), "trim frees everything when nothing is live");
+        printf("ok stress\n");
+    }
+    return 0;
+}

@@ -1,0 +1,40 @@
+// Host build of zenu_amd/csrc/zmath.hpp compared with the host libm (the functions ZeNu's CPU path
+// calls through Rust's f32::tanh).  Usage: zmath_host_check <stride>; checks every stride-th f32
+// bit pattern (stride 1 = exhaustive, about a minute on 8 cores).  Prints the mismatch counts.
+#include <atomic>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <thread>
+#include <vector>
+
+#include "../../zenu_amd/csrc/zmath.hpp"
+
+int main(int argc, char **argv)
+{
+    const uint64_t stride = argc > 1 ? strtoull(argv[1], nullptr, 10) : 1;
+    const int nt = 8;
+    std::atomic<uint64_t> bad_fdlibm{0}, bad_simd{0}, bad_expm1{0}, bad_sig{0};
+    std::vector<std::thread> th;
+    for (int w = 0; w < nt; w++)
+        th.emplace_back([&, w]() {
+            uint64_t b0 = 0, b1 = 0, b2 = 0, b3 = 0;
+            for (uint64_t u = (uint64_t)w * stride; u < (1ull << 32); u += stride * nt) {
+                const float x = zmath::u2f((uint32_t)u);
+                const float ref = tanhf(x);
+                const float a = zmath::tanhf_fdlibm(x), s = zmath::tanhf_simd(x);
+                const bool nan = ref != ref;
+                if (nan ? !(a != a) : zmath::f2u(a) != zmath::f2u(ref)) b0++;
+                if (nan ? !(s != s) : zmath::f2u(s) != zmath::f2u(ref)) b1++;
+                if (fabsf(x) < 44.0f && zmath::f2u(zmath::expm1f_fdlibm(x)) != zmath::f2u(expm1f(x))) b2++;
+                const float sg = 0.5f + 0.5f * tanhf(0.5f * x), sz = zmath::sigmoidf_zenu(x);
+                if ((sg != sg) ? !(sz != sz) : zmath::f2u(sz) != zmath::f2u(sg)) b3++;
+            }
+            bad_fdlibm += b0; bad_simd += b1; bad_expm1 += b2; bad_sig += b3;
+        });
+    for (auto &t : th) t.join();
+    printf("tanhf_fdlibm %llu tanhf_simd %llu expm1f_fdlibm %llu sigmoidf_zenu %llu\n",
+           (unsigned long long)bad_fdlibm.load(), (unsigned long long)bad_simd.load(),
+           (unsigned long long)bad_expm1.load(), (unsigned long long)bad_sig.load());
+    return (bad_fdlibm + bad_simd + bad_expm1 + bad_sig) ? 1 : 0;
+}

@@ -257,8 +257,36 @@ private:
         return b;
     }
 
+    // Only after device_synchronize(): nothing is in flight, so free neighbours can be joined
+    // whatever stream they were freed on.
+    void coalesce_across_streams()
+    {
+        std::vector<Block *> all;
+        for (auto &kv : free_)
+            for (Block *b : kv.second) all.push_back(b);
+        free_.clear();
+        stats_.bytes_cached = 0;
+        std::set<Block *> dead;
+        for (Block *b : all) {
+            if (dead.count(b)) continue;
+            if (b->prev && !b->prev->allocated) continue;  // not the head of its free run
+            while (b->next && !b->next->allocated) {
+                Block *n = b->next;
+                b->size += n->size;
+                b->next = n->next;
+                if (n->next) n->next->prev = b;
+                dead.insert(n);
+            }
+        }
+        for (Block *b : all) {
+            if (dead.count(b)) delete b;
+            else insert_free(b);
+        }
+    }
+
     void release_free_segments()
     {
+        coalesce_across_streams();
         for (auto &kv : free_) {
             FreeSet &fs = kv.second;
             for (auto it = fs.begin(); it != fs.end();) {
