@@ -208,7 +208,7 @@ def build_ops(z, workload, stream):
         pc, mc, vc = p.copy(), m.copy(), v.copy()
         op = Op("adamw 25M", "c3", "f32", 7 * 4 * n, n, ls,
                 lambda: zo.adamw_update(pc, g, mc, vc, f(HP["lr"]), f(HP["beta1"]), f(HP["beta2"]), f(HP["eps"]), f(HP["wd"]), True, f(HP["step"])),
-                kernel="adam_kernel<float, 4>")
+                kernel="adam_kernel<float, 4, true>")
         op.keep = sets
         ops.append(op)
 

@@ -31,7 +31,10 @@ namespace zenu {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kUnroll = 4;
+#ifndef ZENU_EW_UNROLL
+#define ZENU_EW_UNROLL 2
+#endif
+constexpr int kUnroll = ZENU_EW_UNROLL;
 
 // ---- functors -----------------------------------------------------------------------------------
 
@@ -318,27 +321,64 @@ __global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, con
     const T *abase = a + oa + r0 * p.ldr[1] + c0 * p.ldc[1];
     const T *bbase = (F::NIN == 2) ? b + ob + r0 * p.ldr[2] + c0 * p.ldc[2] : abase;
 
-    // phase 1: transposed inputs -> LDS, reading along R (their contiguous dim)
-    if (p.trans_a || (F::NIN == 2 && p.trans_b)) {
-        if (full) {
-            const int rv = (tid % VPR) * VEC;
+    if (full) {
+        // All global loads of the tile are issued first -- the transposed inputs along R (their
+        // contiguous dim), the others along C -- so both streams are in flight together; then the
+        // transposed ones are turned through LDS.
+        constexpr int K = kTile / RPP;
+        const int lane_v = (tid % VPR) * VEC;   // vector position along the contiguous dim
+        const int lane_o = tid / VPR;           // position along the other dim, + k * RPP
+        const bool ta = p.trans_a != 0;
+        const bool tb = (F::NIN == 2) && p.trans_b != 0;
+        Pack<T, VEC> xa[K], xb[K];
 #pragma unroll
-            for (int k = 0; k < kTile / RPP; k++) {
-                const int c = tid / VPR + k * RPP;
-                if (p.trans_a) {
-                    Pack<T, VEC> x = load_pack<T, VEC, NT>(abase + rv + (int64_t)c * p.ldc[1]);
+        for (int k = 0; k < K; k++) {
+            const int o = lane_o + k * RPP;
+            if (ta) xa[k] = load_pack<T, VEC, NT>(abase + lane_v + (int64_t)o * p.ldc[1]);
+            else if (p.ldc[1] == 0) xa[k] = splat<T, VEC>(abase[(int64_t)o * p.ldr[1]]);
+            else xa[k] = load_pack<T, VEC, NT>(abase + (int64_t)o * p.ldr[1] + lane_v);
+            if constexpr (F::NIN == 2) {
+                if (tb) xb[k] = load_pack<T, VEC, NT>(bbase + lane_v + (int64_t)o * p.ldc[2]);
+                else if (p.ldc[2] == 0) xb[k] = splat<T, VEC>(bbase[(int64_t)o * p.ldr[2]]);
+                else xb[k] = load_pack<T, VEC, NT>(bbase + (int64_t)o * p.ldr[2] + lane_v);
+            }
+        }
+        if (ta || tb) {
 #pragma unroll
-                    for (int j = 0; j < VEC; j++) lds_a[(rv + j) * kPitch + c] = x.v[j];
-                }
-                if constexpr (F::NIN == 2) {
-                    if (p.trans_b) {
-                        Pack<T, VEC> x = load_pack<T, VEC, NT>(bbase + rv + (int64_t)c * p.ldc[2]);
+            for (int k = 0; k < K; k++) {
+                const int c = lane_o + k * RPP;  // the loaded vector holds rows lane_v.. of column c
 #pragma unroll
-                        for (int j = 0; j < VEC; j++) lds_b[(rv + j) * kPitch + c] = x.v[j];
+                for (int j = 0; j < VEC; j++) {
+                    if (ta) lds_a[(lane_v + j) * kPitch + c] = xa[k].v[j];
+                    if constexpr (F::NIN == 2) {
+                        if (tb) lds_b[(lane_v + j) * kPitch + c] = xb[k].v[j];
                     }
                 }
             }
-        } else {
+            __syncthreads();
+        }
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const int r = lane_o + k * RPP;
+            Pack<T, VEC> x = xa[k], y;
+            if (ta) {
+#pragma unroll
+                for (int j = 0; j < VEC; j++) x.v[j] = lds_a[r * kPitch + lane_v + j];
+            }
+            if constexpr (F::NIN == 2) {
+                y = xb[k];
+                if (tb) {
+#pragma unroll
+                    for (int j = 0; j < VEC; j++) y.v[j] = lds_b[r * kPitch + lane_v + j];
+                }
+            } else {
+                y = x;
+            }
+            store_pack<T, VEC, NT>(obase + (int64_t)r * p.ldr[0] + lane_v, apply_pack<T, VEC, F>(f, x, y));
+        }
+    } else {
+        // edge tiles and unaligned operands: element-wise with bounds checks
+        if (p.trans_a || (F::NIN == 2 && p.trans_b)) {
             for (int e = tid; e < kTile * kTile; e += kBlock) {
                 const int r = e % kTile, c = e / kTile;
                 if (r < nr && c < nc) {
@@ -348,40 +388,8 @@ __global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, con
                     }
                 }
             }
+            __syncthreads();
         }
-        __syncthreads();
-    }
-
-    // phase 2: walk the tile along C (the output's contiguous dim)
-    if (full) {
-        const int cv = (tid % VPR) * VEC;
-#pragma unroll
-        for (int k = 0; k < kTile / RPP; k++) {
-            const int r = tid / VPR + k * RPP;
-            Pack<T, VEC> x, y;
-            if (p.trans_a) {
-#pragma unroll
-                for (int j = 0; j < VEC; j++) x.v[j] = lds_a[r * kPitch + cv + j];
-            } else if (p.ldc[1] == 0) {
-                x = splat<T, VEC>(abase[(int64_t)r * p.ldr[1]]);
-            } else {
-                x = load_pack<T, VEC, NT>(abase + (int64_t)r * p.ldr[1] + cv);
-            }
-            if constexpr (F::NIN == 2) {
-                if (p.trans_b) {
-#pragma unroll
-                    for (int j = 0; j < VEC; j++) y.v[j] = lds_b[r * kPitch + cv + j];
-                } else if (p.ldc[2] == 0) {
-                    y = splat<T, VEC>(bbase[(int64_t)r * p.ldr[2]]);
-                } else {
-                    y = load_pack<T, VEC, NT>(bbase + (int64_t)r * p.ldr[2] + cv);
-                }
-            } else {
-                y = x;
-            }
-            store_pack<T, VEC, NT>(obase + (int64_t)r * p.ldr[0] + cv, apply_pack<T, VEC, F>(f, x, y));
-        }
-    } else {
         for (int e = tid; e < kTile * kTile; e += kBlock) {
             const int c = e % kTile, r = e / kTile;
             if (r < nr && c < nc) {
