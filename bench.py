@@ -224,6 +224,118 @@ def build_ops(z, workload, stream):
     return ops
 
 
+def run_c4(z, args, sync):
+    """configs[4]: the MLP training step (batch 256, 784-512-512-10, softmax-CE, backward, Adam) as
+    ZeNu's op sequence; GEMM on rocBLAS, everything else on this library.  Reports the wall time of
+    a step and, from one event-instrumented step, the time per kernel family."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import mlp_devices
+    import mlp_step
+    x, t, params = mlp_step.make_inputs()
+    dev = mlp_devices.HipDev(z, timed=False)
+    st = mlp_step.MlpStep(dev, x, t, params)
+    for _ in range(max(args.warmup, 3)):
+        st.step()
+    sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        st.step()
+    sync()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    dev.timed = True
+    dev.__init__(z, timed=True)
+    st.dev = dev
+    dev.begin()
+    st.step()
+    br = {k: round(v, 1) for k, v in dev.breakdown().items()}
+    graph = capture_and_replay_c4(z, st, args, sync)
+    cpu = None
+    if not args.no_cpu_baseline:
+        cst = mlp_step.MlpStep(mlp_devices.CpuDev(), x, t, params)
+        cst.step()
+        t1 = time.perf_counter()
+        n = 3
+        for _ in range(n):
+            cst.step()
+        cpu = dict(value=round(n / (time.perf_counter() - t1), 2), unit="steps/s", cores=1, kind="port",
+                   sample=f"{n} steps of the same op sequence on the C oracle (GEMM: numpy/OpenBLAS, its own threads)")
+    print(json.dumps({
+        "metric": "MLP training step (configs[4]): steps/s; time per kernel family", "value": round(1e3 / ms, 1),
+        "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[4]: batch 256, Linear 784-512-ReLU-512-ReLU-10, softmax-CE, Adam"},
+        "breakdown_us_one_instrumented_step": br, "hip_graph_replay": graph, "cpu_baseline": cpu}))
+
+
+def capture_and_replay_c4(z, st, args, sync):
+    """Capture one whole step (about 70 launches, all on the library's stream, all allocations
+    served by the caching pool) into a HIP graph and time its replays: the step without the
+    host's per-launch cost.  Every replay is checked against an eager step from the same state.
+    The Adam step number is a kernel argument and so is frozen in the graph."""
+    import numpy as np
+    rt = C.CDLL("libamdhip64.so")
+    stream = z.get_stream()
+    vp = C.c_void_p
+    rt.hipStreamBeginCapture.argtypes = [vp, C.c_int]
+    rt.hipStreamEndCapture.argtypes = [vp, C.POINTER(vp)]
+    rt.hipGraphInstantiate.argtypes = [C.POINTER(vp), vp, vp, vp, C.c_size_t]
+    rt.hipGraphLaunch.argtypes = [vp, vp]
+    try:
+        dev = st.dev
+        dev.timed = False
+
+        def snapshot():
+            return ({k: v.to_numpy() for k, v in st.p.items()}, {k: v.to_numpy() for k, v in st.opt.m.items()},
+                    {k: v.to_numpy() for k, v in st.opt.v.items()}, st.opt.step)
+
+        def restore(s):
+            from zenu_amd import _lib
+            for src, dst in ((s[0], st.p), (s[1], st.opt.m), (s[2], st.opt.v)):
+                for k, a in src.items():
+                    _lib.check(z.lib().zenu_hip_memcpy_h2d(dst[k].as_ptr(), a.ctypes.data, a.nbytes, stream), "h2d")
+            st.opt.step = s[3]
+
+        s0 = snapshot()
+        eager_loss, _ = st.step()
+        eager = (float(eager_loss.to_numpy()), {k: v.to_numpy() for k, v in st.p.items()})
+        for _ in range(2):      # rehearse with the live set the capture will see: every request a pool hit
+            rehearsal = st.step()
+            del rehearsal
+        restore(s0)
+        sync()
+        if rt.hipStreamBeginCapture(stream, 2) != 0:   # hipStreamCaptureModeRelaxed
+            return {"error": "hipStreamBeginCapture failed"}
+        g = vp()
+        try:
+            loss, grads = st.step()                     # recorded, not executed
+        finally:
+            rc = rt.hipStreamEndCapture(stream, C.byref(g))
+        if rc != 0:
+            return {"error": "hipStreamEndCapture failed"}
+        ge = vp()
+        if rt.hipGraphInstantiate(C.byref(ge), g, None, None, 0) != 0:
+            return {"error": "hipGraphInstantiate failed"}
+        checks = 0
+        for _ in range(3):                              # replays, each checked against the eager result
+            restore(s0)
+            st.opt.step = s0[3] + 1
+            assert rt.hipGraphLaunch(ge, stream) == 0
+            sync()
+            ok = float(loss.to_numpy()) == eager[0] and all(np.array_equal(st.p[k].to_numpy(), eager[1][k]) for k in st.p)
+            if not ok:
+                return {"error": "graph replay differs from the eager step"}
+            checks += 1
+        sync()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            rt.hipGraphLaunch(ge, stream)
+        sync()
+        ms = (time.perf_counter() - t0) / args.steps * 1e3
+        return {"ms_per_step": round(ms, 4), "steps_per_s": round(1e3 / ms, 1), "replays_checked_bit_exact": checks}
+    except Exception as e:  # the eager figures above stand on their own
+        return {"error": repr(e)}
+
+
 def measured_traffic(op):
     """HBM bytes per launch of the op's kernel from the committed rocprofv3 --pmc summary
     (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size), or None if not recorded."""
@@ -244,7 +356,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="suite", choices=["suite", "c0", "c1", "c2", "c3"])
+    ap.add_argument("--workload", default="suite", choices=["suite", "c0", "c1", "c2", "c3", "c4"])
     ap.add_argument("--op-reps", type=int, default=40, help="launches per op in the per-op timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--profile-op", default=None, help="only launch this op (for rocprofv3 counter runs)")
@@ -263,6 +375,9 @@ def main():
     z.set_stream(stream)
     hip = Hip()
     sync = lambda: _lib.check(z.lib().zenu_hip_stream_synchronize(stream), "sync")
+
+    if args.workload == "c4":
+        return run_c4(z, args, sync)
 
     t0 = time.time()
     ops = build_ops(z, args.workload, stream)

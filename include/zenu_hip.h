@@ -212,7 +212,9 @@ int zenu_hip_adamw_step(int dtype, void *p_dev, const void *g_dev, void *m_dev, 
                         int64_t n, double lr, double beta1, double beta2, double eps,
                         double weight_decay, int apply_decay, double step, zenu_stream_t stream);
 /* Multi-tensor form: one launch over a model's parameter tensors.  The pointer / size tables are
- * HOST arrays of length n_tensors; apply_decay may be NULL (no decay) or per-tensor flags. */
+ * HOST arrays of length n_tensors; apply_decay may be NULL (no decay) or per-tensor flags.
+ * The tables are copied into the kernel arguments (24 tensors per launch): no staging, no
+ * synchronisation. */
 int zenu_hip_adam_step_multi(int dtype, int n_tensors, void *const *p_dev, const void *const *g_dev,
                              void *const *m_dev, void *const *v_dev, const int64_t *sizes, double lr,
                              double beta1, double beta2, double eps, double weight_decay,

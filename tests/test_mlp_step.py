@@ -1,0 +1,75 @@
+"""BASELINE config[4]: the MLP training step on the HIP library against the same step on the CPU
+oracle (same op sequence, same inputs; GEMM on each side's library).
+
+Bars: quantities that do not pass through a GEMM-dependent chain would be bit-exact; everything
+here sits downstream of GEMMs computed by two different libraries (OpenBLAS vs rocBLAS, different
+summation order), so loss, gradients and updated parameters are compared at 1e-4 relative to the
+tensor's largest magnitude (SURVEY 8d's bar for GEMM-fed quantities)."""
+import numpy as np
+import pytest
+
+import mlp_devices
+import mlp_step
+
+
+def rel(a, b):
+    return float(np.max(np.abs(a.astype(np.float64) - b.astype(np.float64))) / max(np.max(np.abs(b)), 1e-30))
+
+
+def test_cpu_step_matches_plain_numpy():
+    """pins the op sequence itself: the oracle-run step equals a direct numpy forward/backward"""
+    x, t, params = mlp_step.make_inputs()
+    cpu = mlp_step.MlpStep(mlp_devices.CpuDev(), x, t, params)
+    loss, grads = cpu.step()
+    W1, b1, W2, b2, W3, b3 = (params[f"linear{i}.{n}"].astype(np.float64) for i in (1, 2, 3) for n in ("weight", "bias"))
+    xd, td = x.astype(np.float64), t.astype(np.float64)
+    a1 = xd @ W1.T + b1; h1 = np.maximum(a1, 0)
+    a2 = h1 @ W2.T + b2; h2 = np.maximum(a2, 0)
+    z = h2 @ W3.T + b3
+    s = np.exp(z - z.max(1, keepdims=True)); s /= s.sum(1, keepdims=True)
+    ref_loss = -(td * np.log(s)).sum() / x.shape[0]
+    gz = (s - td) / x.shape[0]
+    assert abs(float(loss.to_numpy()) - ref_loss) / ref_loss < 1e-5
+    assert rel(grads["linear3.weight"].to_numpy(), gz.T @ h2) < 1e-4
+    assert rel(grads["linear3.bias"].to_numpy(), gz.sum(0)) < 1e-4
+    g2 = (gz @ W3) * (a2 > 0)
+    assert rel(grads["linear2.weight"].to_numpy(), g2.T @ h1) < 1e-4
+    g1 = (g2 @ W2) * (a1 > 0)
+    assert rel(grads["linear1.weight"].to_numpy(), g1.T @ xd) < 1e-4
+    assert rel(grads["linear1.bias"].to_numpy(), g1.sum(0)) < 1e-4
+
+
+@pytest.mark.gpu
+def test_hip_step_matches_cpu_step(hip):
+    import zenu_oracle as zo
+    x, t, params = mlp_step.make_inputs()
+    cpu = mlp_step.MlpStep(mlp_devices.CpuDev(), x, t, params)
+    dev = mlp_devices.HipDev(hip)
+    gpu = mlp_step.MlpStep(dev, x, t, params)
+    losses = []
+    for step in range(1, 4):
+        print(f"[c4] step {step}", flush=True)
+        # both legs start the step from the GPU's state, so GEMM rounding does not accumulate
+        p0 = {k: v.to_numpy() for k, v in gpu.p.items()}
+        m0 = {k: v.to_numpy().reshape(-1) for k, v in gpu.opt.m.items()}
+        v0 = {k: v.to_numpy().reshape(-1) for k, v in gpu.opt.v.items()}
+        for k in cpu.p:
+            cpu.p[k].a[...] = p0[k]
+        closs, cgrads = cpu.step()
+        gloss, ggrads = gpu.step()
+        losses.append(float(gloss.to_numpy()))
+        # loss and gradients sit downstream of GEMMs from two libraries: 1e-4
+        assert abs(losses[-1] - float(closs.to_numpy())) / abs(float(closs.to_numpy())) < 1e-4
+        for k in cgrads:
+            assert rel(ggrads[k].to_numpy(), cgrads[k].to_numpy()) < 1e-4, (step, k)
+        # the fused Adam update, fed the GPU's own gradients, is bit-exact against the oracle
+        # (Adam's g / (|g| + eps) amplifies GEMM rounding on near-zero gradients, so the
+        # cross-library parameters are not compared directly)
+        f = np.float32
+        for k in p0:
+            pe = p0[k].reshape(-1).copy()
+            zo.adam_update(pe, ggrads[k].to_numpy().reshape(-1), m0[k], v0[k], f(1e-3), f(0.9), f(0.999), f(1e-8), f(step))
+            assert np.array_equal(pe, gpu.p[k].to_numpy().reshape(-1)), (step, k)
+            assert np.array_equal(m0[k], gpu.opt.m[k].to_numpy().reshape(-1)), (step, k)
+            assert np.array_equal(v0[k], gpu.opt.v[k].to_numpy().reshape(-1)), (step, k)
+    assert losses[2] < losses[0]          # it trains

@@ -115,7 +115,10 @@ __global__ __launch_bounds__(kBlock) void adam_kernel(T *p, const T *g, T *m, T 
     adam_span<T, VEC, NT>(p, g, m, v, n, blockIdx.x, k, decay != 0);
 }
 
-// multi-tensor: a table of tensors and a table mapping each workgroup to (tensor, tile)
+// multi-tensor: up to kMaxMulti tensors per launch, described in the kernel arguments themselves
+// (no staging buffer, no copy, nothing to synchronise; the call can sit in a captured graph).
+// first_block[i] is the first workgroup of tensor i; a workgroup finds its tensor by a short scan.
+constexpr int kMaxMulti = 24;
 struct MultiEntry {
     void *p;
     const void *g;
@@ -125,22 +128,28 @@ struct MultiEntry {
     int32_t decay;
     int32_t vec_ok;
 };
+struct MultiArgs {
+    MultiEntry e[kMaxMulti];
+    int32_t first_block[kMaxMulti + 1];
+    int32_t count;
+};
 
 template <typename T, int VEC>
-__global__ __launch_bounds__(kBlock) void adam_multi_kernel(const MultiEntry *entries,
-                                                            const int2 *block_map, AdamConsts<T> k)
+__global__ __launch_bounds__(kBlock) void adam_multi_kernel(MultiArgs a, AdamConsts<T> k)
 {
-    const int2 bm = block_map[blockIdx.x];
-    const MultiEntry e = entries[bm.x];
+    int t = 0;
+    while (t + 1 < a.count && (int)blockIdx.x >= a.first_block[t + 1]) t++;
+    const MultiEntry &e = a.e[t];
+    const int64_t tile = (int64_t)blockIdx.x - a.first_block[t];
     T *p = static_cast<T *>(e.p);
     const T *g = static_cast<const T *>(e.g);
     T *m = static_cast<T *>(e.m);
     T *v = static_cast<T *>(e.v);
-    if (e.vec_ok) adam_span<T, VEC, false>(p, g, m, v, e.n, bm.y, k, e.decay != 0);
+    if (e.vec_ok) adam_span<T, VEC, false>(p, g, m, v, e.n, tile, k, e.decay != 0);
     else {
         // unaligned tensor: same tile, scalar accesses
         constexpr int64_t kTile = (int64_t)kBlock * VEC * kUnroll;
-        const int64_t base = (int64_t)bm.y * kTile;
+        const int64_t base = tile * kTile;
         for (int64_t i = base + threadIdx.x; i < base + kTile && i < e.n; i += kBlock) {
             T pe = p[i], me = m[i], ve = v[i];
             adam_elem<T>(pe, g[i], me, ve, k, e.decay != 0);
@@ -245,48 +254,38 @@ int adam_multi_t(int nt, void *const *p, const void *const *g, void *const *m, v
 {
     constexpr int VEC = VecOf<T>::N;
     constexpr int64_t kTile = (int64_t)kBlock * VEC * kUnroll;
-    int64_t nblocks = 0;
-    for (int i = 0; i < nt; i++) {
+    for (int i = 0; i < nt; i++)
         if (sizes[i] < 0 || (sizes[i] > 0 && (!p[i] || !g[i] || !m[i] || !v[i]))) return ZENU_ERR_ARG;
-        nblocks += (sizes[i] + kTile - 1) / kTile;
+    int i = 0;
+    while (i < nt) {
+        MultiArgs a;
+        a.count = 0;
+        int64_t blocks = 0;
+        while (i < nt && a.count < kMaxMulti) {
+            const int64_t tiles = (sizes[i] + kTile - 1) / kTile;
+            if (tiles == 0) { i++; continue; }
+            if (blocks + tiles > 0x7fffffffLL) {
+                if (a.count == 0) return ZENU_ERR_UNSUPPORTED;
+                break;
+            }
+            MultiEntry &e = a.e[a.count];
+            e.p = p[i];
+            e.g = g[i];
+            e.m = m[i];
+            e.v = v[i];
+            e.n = sizes[i];
+            e.decay = decay ? decay[i] : 0;
+            e.vec_ok = aligned16(p[i]) && aligned16(g[i]) && aligned16(m[i]) && aligned16(v[i]);
+            a.first_block[a.count] = (int32_t)blocks;
+            blocks += tiles;
+            a.count++;
+            i++;
+        }
+        if (a.count == 0) break;
+        a.first_block[a.count] = (int32_t)blocks;
+        adam_multi_kernel<T, VEC><<<(unsigned)blocks, kBlock, 0, s>>>(a, k);
+        ZENU_LAUNCH_CHECK();
     }
-    if (nblocks == 0) return ZENU_OK;
-    if (nblocks > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-
-    // host staging in pinned memory so the upload is a real asynchronous copy
-    const size_t ebytes = (size_t)nt * sizeof(MultiEntry);
-    const size_t ebytes_al = (ebytes + 255) / 256 * 256;
-    const size_t bbytes = (size_t)nblocks * sizeof(int2);
-    void *host = nullptr;
-    ZENU_HIP_TRY(hipHostMalloc(&host, ebytes_al + bbytes, hipHostMallocDefault));
-    MultiEntry *he = static_cast<MultiEntry *>(host);
-    int2 *hb = reinterpret_cast<int2 *>(static_cast<char *>(host) + ebytes_al);
-    int64_t b = 0;
-    for (int i = 0; i < nt; i++) {
-        he[i].p = p[i];
-        he[i].g = g[i];
-        he[i].m = m[i];
-        he[i].v = v[i];
-        he[i].n = sizes[i];
-        he[i].decay = decay ? decay[i] : 0;
-        he[i].vec_ok = aligned16(p[i]) && aligned16(g[i]) && aligned16(m[i]) && aligned16(v[i]);
-        const int64_t tiles = (sizes[i] + kTile - 1) / kTile;
-        for (int64_t t = 0; t < tiles; t++) hb[b++] = make_int2(i, (int)t);
-    }
-    Workspace ws(ebytes_al + bbytes, s);
-    if (ws.status) { (void)hipHostFree(host); return ws.status; }
-    hipError_t e = hipMemcpyAsync(ws.ptr, host, ebytes_al + bbytes, hipMemcpyHostToDevice, s);
-    if (e == hipSuccess) {
-        adam_multi_kernel<T, VEC><<<(unsigned)nblocks, kBlock, 0, s>>>(
-            static_cast<const MultiEntry *>(ws.ptr),
-            reinterpret_cast<const int2 *>(static_cast<char *>(ws.ptr) + ebytes_al), k);
-        e = hipGetLastError();
-    }
-    // the staging buffer must outlive the copy: wait for it, then release
-    hipError_t e2 = hipStreamSynchronize(s);
-    (void)hipHostFree(host);
-    if (e != hipSuccess) { set_last_hip_error(e); return ZENU_ERR_HIP; }
-    if (e2 != hipSuccess) { set_last_hip_error(e2); return ZENU_ERR_HIP; }
     return ZENU_OK;
 }
 

@@ -412,19 +412,24 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int
     const int ncol = (c + VEC <= p.inner) ? VEC : (c < p.inner ? (int)(p.inner - c) : 0);
     const T *src = p.in + q * p.outer_stride + c;
     if (ncol == VEC && VEC > 1) {
-        int64_t r = r0 + ty;
-        for (; r + 3 * ty_n < r1; r += 4 * ty_n) {
-            Pack<T, VEC> x[4];
+        // pointer-bumping loop: the address arithmetic per load is one 64-bit add
+        constexpr int U = 4;
+        const int64_t row_step = (int64_t)ty_n * p.elem_stride;
+        const T *ptr = src + (r0 + ty) * p.elem_stride;
+        int r = (int)(r0 + ty);
+        const int rend = (int)r1;
+        for (; r + (U - 1) * ty_n < rend; r += U * ty_n, ptr += U * row_step) {
+            Pack<T, VEC> x[U];
 #pragma unroll
-            for (int u = 0; u < 4; u++) x[u] = load_pack<T, VEC, NT>(src + (r + u * ty_n) * p.elem_stride);
+            for (int u = 0; u < U; u++) x[u] = load_pack<T, VEC, NT>(ptr + u * row_step);
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
+            for (int u = 0; u < U; u++) {
 #pragma unroll
                 for (int j = 0; j < VEC; j++) acc[j] = Tr::update(acc[j], x[u].v[j], r + u * ty_n);
             }
         }
-        for (; r < r1; r += ty_n) {
-            Pack<T, VEC> x = load_pack<T, VEC, false>(src + r * p.elem_stride);
+        for (; r < rend; r += ty_n, ptr += row_step) {
+            Pack<T, VEC> x = load_pack<T, VEC, false>(ptr);
 #pragma unroll
             for (int j = 0; j < VEC; j++) acc[j] = Tr::update(acc[j], x.v[j], r);
         }
