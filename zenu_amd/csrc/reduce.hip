@@ -41,6 +41,11 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kWave = 64;
 constexpr int kWaves = kBlock / kWave;
+#ifndef ZENU_SPLIT_U
+#define ZENU_SPLIT_U 8
+#endif
+constexpr int kRowsU = 4;               // vectors in flight per lane, one workgroup or wavefront per row
+constexpr int kSplitU = ZENU_SPLIT_U;   // the same when workgroups share a row
 
 
 // ---- wave64 exchange primitives (word-wise so any POD accumulator works) ---------------------------
@@ -186,7 +191,6 @@ template <typename T> struct RedParams {
     int64_t outer_stride;
     int64_t elem_stride;
     int splits;              // workgroups along R
-    int64_t seg;             // R elements per split
     // results
     T *out_val;              // final value (may be null)
     int64_t *out_idx;        // final index (may be null)
@@ -195,6 +199,8 @@ template <typename T> struct RedParams {
     T *part_key;
     int32_t *part_idx;
     int *counters;
+    int fan;                 // splits per leaf counter of the arrival tree
+    int cstride;             // counters per group: 1 + number of leaves (1 when fan >= splits)
     // value gather for max: value = gsrc[q * g_outer_stride + c + idx * g_elem_stride]
     const T *gsrc;
     int64_t g_outer_stride, g_elem_stride;
@@ -262,32 +268,53 @@ __device__ __forceinline__ typename Tr::Acc load_partial(const RedParams<T> &p, 
     return Tr::from_partial(k, i);
 }
 
-// Called by every thread of a workgroup after its partials are stored.  Returns true in the
-// workgroup that arrives last at `counter` among `expected`; it performs the fold.  No workgroup
-// waits for another.
-__device__ __forceinline__ bool arrive_last(int *counter, int expected)
+// Called by every thread of a workgroup after its partials are stored.  Returns true in the one
+// workgroup of the group that arrives last; it performs the fold.  No workgroup waits for
+// another.  Atomics of many workgroups on ONE address are served one after the other (measured:
+// about 12 ns each, 6 us for 512 workgroups that finish together), so arrival is a two-level
+// tree: `fan` consecutive splits share a leaf counter and the last one at a leaf moves on to the
+// root.  `c` points at the group's 1 + ceil(splits / fan) counters (root first); with
+// fan >= splits only the root is used.  Leaves are reset by their last arriver, the root by
+// the folding workgroup.
+__device__ __forceinline__ bool arrive_last(int *c, int split, int splits, int fan)
 {
     __shared__ int s_last;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // this thread's partial stores are acknowledged
     __syncthreads();
     if (threadIdx.x == 0) {
-        const int t = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (t == expected - 1);
+        bool last;
+        if (fan >= splits) {
+            last = __hip_atomic_fetch_add(c, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == splits - 1;
+        } else {
+            const int leaves = (splits + fan - 1) / fan;
+            const int leaf = split / fan;
+            const int members = (leaf == leaves - 1) ? splits - leaf * fan : fan;
+            last = false;
+            if (__hip_atomic_fetch_add(c + 1 + leaf, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == members - 1) {
+                store_agent(c + 1 + leaf, 0);
+                last = __hip_atomic_fetch_add(c, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == leaves - 1;
+            }
+        }
+        s_last = last;
     }
     __syncthreads();
     return s_last != 0;
 }
 
 // ---- kernel A: rows --------------------------------------------------------------------------------------
-// VEC > 1 requires elem_stride == 1, 16-byte aligned rows and seg % VEC == 0 (checked on the host).
+// VEC > 1 requires elem_stride == 1, 16-byte aligned rows (checked on the host).
 // WAVE_ROW: one wavefront per output (4 outputs per workgroup, never split), otherwise one
 // workgroup per (output, split); with splits > 1 the last workgroup of an output to finish folds
 // that output's partials in a fixed order.
 
-template <typename T, typename Tr, int VEC, bool WAVE_ROW, bool NT>
+enum { kWaveRow = 0, kBlockRow = 1, kSplitRow = 2 };
+
+template <typename T, typename Tr, int VEC, int MODE, bool NT, int U>
 __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(RedParams<T> p)
 {
     typedef typename Tr::Acc A;
+    constexpr bool WAVE_ROW = MODE == kWaveRow;
+    const int nsplit = MODE == kSplitRow ? p.splits : 1;
     const int lane_n = WAVE_ROW ? kWave : kBlock;
     const int lane = WAVE_ROW ? (threadIdx.x & (kWave - 1)) : threadIdx.x;
     int64_t o;
@@ -295,68 +322,92 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(RedParams<T> p)
     if (WAVE_ROW) {
         o = (int64_t)blockIdx.x * kWaves + threadIdx.x / kWave;
         split = 0;
+    } else if (MODE == kBlockRow) {
+        o = blockIdx.x;
+        split = 0;
     } else {
-        o = (int64_t)blockIdx.x / p.splits;
-        split = (int)(blockIdx.x - o * p.splits);
+        o = (int64_t)(blockIdx.x / (unsigned)nsplit);
+        split = (int)(blockIdx.x - (unsigned)o * (unsigned)nsplit);
     }
     const bool active = o < p.nout;
-    A acc[4] = {Tr::identity(), Tr::identity(), Tr::identity(), Tr::identity()};
+    A acc[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) acc[u] = Tr::identity();
     if (active) {
-        const int64_t q = o / p.inner, c = o - q * p.inner;
+        int64_t q = o, c = 0;
+        if (p.inner != 1) {
+            q = o / p.inner;
+            c = o - q * p.inner;
+        }
         const int64_t base = q * p.outer_stride + c;
-        const int64_t r0 = (int64_t)split * p.seg;
-        int64_t r1 = r0 + p.seg;
-        if (r1 > p.R) r1 = p.R;
+        // The splits of an output interleave chunk by chunk (split s takes chunks s, s + splits,
+        // ...), so the workgroups of a launch sweep the source together as one moving window
+        // instead of each streaming its own far-apart segment in lockstep.
+        const int64_t R = p.R;
         if (VEC > 1) {
             const T *row = p.in + base;
             const int64_t step = (int64_t)lane_n * VEC;
-            int64_t r = r0 + (int64_t)lane * VEC;
-            // four vectors in flight per lane
-            for (; r + 3 * step + VEC <= r1; r += 4 * step) {
-                Pack<T, VEC> x[4];
+            const int64_t chunk = U * step;
+            const int64_t stride = chunk * nsplit;
+            for (int64_t b = (int64_t)split * chunk; b < R; b += stride) {
+                int64_t r = b + (int64_t)lane * VEC;
+                if (b + chunk <= R) {      // U vectors in flight per lane
+                    Pack<T, VEC> x[U];
 #pragma unroll
-                for (int u = 0; u < 4; u++) x[u] = load_pack<T, VEC, NT>(row + r + u * step);
+                    for (int u = 0; u < U; u++) x[u] = load_pack<T, VEC, NT>(row + r + u * step);
 #pragma unroll
-                for (int u = 0; u < 4; u++) {
+                    for (int u = 0; u < U; u++) {
 #pragma unroll
-                    for (int j = 0; j < VEC; j++) acc[u] = Tr::update(acc[u], x[u].v[j], r + u * step + j);
+                        for (int j = 0; j < VEC; j++) acc[u] = Tr::update(acc[u], x[u].v[j], r + u * step + j);
+                    }
+                } else {                   // the last, partial chunk of the row
+                    for (; r + VEC <= R; r += step) {
+                        Pack<T, VEC> x = load_pack<T, VEC, false>(row + r);
+#pragma unroll
+                        for (int j = 0; j < VEC; j++) acc[0] = Tr::update(acc[0], x.v[j], r + j);
+                    }
+                    if (r < R)             // ragged end (R % VEC != 0): one lane
+                        for (int j = 0; r + j < R; j++) acc[0] = Tr::update(acc[0], row[r + j], r + j);
                 }
             }
-            for (; r + VEC <= r1; r += step) {
-                Pack<T, VEC> x = load_pack<T, VEC, false>(row + r);
-#pragma unroll
-                for (int j = 0; j < VEC; j++) acc[0] = Tr::update(acc[0], x.v[j], r + j);
-            }
-            // ragged end of the row (R % VEC != 0 only happens on the last split)
-            if (r < r1)
-                for (int j = 0; r + j < r1; j++) acc[0] = Tr::update(acc[0], row[r + j], r + j);
-            if (r0 == 0 && lane == 0) acc[0] = Tr::first(acc[0], row[0]);
+            if (split == 0 && lane == 0) acc[0] = Tr::first(acc[0], row[0]);
         } else {
-            int64_t r = r0 + lane;
-            for (; r + 3 * (int64_t)lane_n < r1; r += 4 * (int64_t)lane_n) {
+            const int64_t chunk = (int64_t)U * lane_n;
+            const int64_t stride = chunk * nsplit;
+            for (int64_t b = (int64_t)split * chunk; b < R; b += stride) {
+                int64_t r = b + lane;
+                if (b + chunk <= R) {
 #pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    const int64_t rr = r + (int64_t)u * lane_n;
-                    acc[u] = Tr::update(acc[u], p.in[base + rr * p.elem_stride], rr);
+                    for (int u = 0; u < U; u++) {
+                        const int64_t rr = r + (int64_t)u * lane_n;
+                        acc[u] = Tr::update(acc[u], p.in[base + rr * p.elem_stride], rr);
+                    }
+                } else {
+                    for (; r < R; r += lane_n) acc[0] = Tr::update(acc[0], p.in[base + r * p.elem_stride], r);
                 }
             }
-            for (; r < r1; r += lane_n) acc[0] = Tr::update(acc[0], p.in[base + r * p.elem_stride], r);
-            if (r0 == 0 && lane == 0) acc[0] = Tr::first(acc[0], p.in[base]);
+            if (split == 0 && lane == 0) acc[0] = Tr::first(acc[0], p.in[base]);
         }
     }
-    A a = Tr::merge(Tr::merge(acc[0], acc[1]), Tr::merge(acc[2], acc[3]));
+    // fixed tree over the U accumulators
+#pragma unroll
+    for (int w = 1; w < U; w *= 2) {
+#pragma unroll
+        for (int u = 0; u + w < U; u += 2 * w) acc[u] = Tr::merge(acc[u], acc[u + w]);
+    }
+    A a = acc[0];
     if (WAVE_ROW) {
         a = wave_allreduce<Tr>(a);
         if (active && lane == 0) emit_final<T, Tr>(p, o, a);
         return;
     }
     a = block_allreduce<Tr>(a);
-    if (p.splits == 1) {
+    if (MODE != kSplitRow) {
         if (lane == 0) emit_final<T, Tr>(p, o, a);
         return;
     }
     if (lane == 0) emit_partial<T, Tr>(p, o * p.splits + split, a);
-    if (!arrive_last(p.counters + o, p.splits)) return;
+    if (!arrive_last(p.counters + o * p.cstride, split, p.splits, p.fan)) return;
     // fold the splits of output o: lane l takes splits l, l + 256, ...; then the fixed block tree
     A f = Tr::identity();
     for (int s0 = lane; s0 < p.splits; s0 += 4 * kBlock) {
@@ -372,7 +423,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(RedParams<T> p)
     f = block_allreduce<Tr>(f);
     if (lane == 0) {
         emit_final<T, Tr>(p, o, f);
-        store_agent(p.counters + o, 0);   // back to rest for the next launch
+        store_agent(p.counters + o * p.cstride, 0);   // back to rest for the next launch
     }
 }
 
@@ -401,9 +452,6 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int
     const int64_t q = blk / p.splits;
     const int64_t group = q * col_tiles + ct;   // the workgroups that share these outputs
     const int64_t c = (ct * tx_n + tx) * VEC;
-    const int64_t r0 = (int64_t)split * p.seg;
-    int64_t r1 = r0 + p.seg;
-    if (r1 > p.R) r1 = p.R;
 
     A acc[VEC];
 #pragma unroll
@@ -411,33 +459,41 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int
 
     const int ncol = (c + VEC <= p.inner) ? VEC : (c < p.inner ? (int)(p.inner - c) : 0);
     const T *src = p.in + q * p.outer_stride + c;
+    // the splits interleave in chunks of U * ty_n source rows: all workgroups of a launch sweep
+    // the source top to bottom together
+    constexpr int U = 4;
+    const int64_t R = p.R;
+    const int64_t chunk = U * ty_n;
+    const int64_t row_step = (int64_t)ty_n * p.elem_stride;
     if (ncol == VEC && VEC > 1) {
-        // pointer-bumping loop: the address arithmetic per load is one 64-bit add
-        constexpr int U = 4;
-        const int64_t row_step = (int64_t)ty_n * p.elem_stride;
-        const T *ptr = src + (r0 + ty) * p.elem_stride;
-        int r = (int)(r0 + ty);
-        const int rend = (int)r1;
-        for (; r + (U - 1) * ty_n < rend; r += U * ty_n, ptr += U * row_step) {
-            Pack<T, VEC> x[U];
+        const T *ptr = src + ((int64_t)split * chunk + ty) * p.elem_stride;
+        const int64_t ptr_step = (int64_t)p.splits * chunk * p.elem_stride;
+        for (int64_t b = split * chunk; b < R; b += p.splits * chunk, ptr += ptr_step) {
+            const int64_t r = b + ty;
+            if (b + chunk <= R) {
+                Pack<T, VEC> x[U];
 #pragma unroll
-            for (int u = 0; u < U; u++) x[u] = load_pack<T, VEC, NT>(ptr + u * row_step);
+                for (int u = 0; u < U; u++) x[u] = load_pack<T, VEC, NT>(ptr + u * row_step);
 #pragma unroll
-            for (int u = 0; u < U; u++) {
+                for (int u = 0; u < U; u++) {
 #pragma unroll
-                for (int j = 0; j < VEC; j++) acc[j] = Tr::update(acc[j], x[u].v[j], r + u * ty_n);
+                    for (int j = 0; j < VEC; j++) acc[j] = Tr::update(acc[j], x[u].v[j], r + u * ty_n);
+                }
+            } else {
+                const T *pt = ptr;
+                for (int64_t rr = r; rr < R; rr += ty_n, pt += row_step) {
+                    Pack<T, VEC> x = load_pack<T, VEC, false>(pt);
+#pragma unroll
+                    for (int j = 0; j < VEC; j++) acc[j] = Tr::update(acc[j], x.v[j], rr);
+                }
             }
         }
-        for (; r < rend; r += ty_n, ptr += row_step) {
-            Pack<T, VEC> x = load_pack<T, VEC, false>(ptr);
-#pragma unroll
-            for (int j = 0; j < VEC; j++) acc[j] = Tr::update(acc[j], x.v[j], r);
-        }
     } else if (ncol > 0) {
-        for (int64_t r = r0 + ty; r < r1; r += ty_n)
-            for (int j = 0; j < ncol; j++) acc[j] = Tr::update(acc[j], src[r * p.elem_stride + j], r);
+        for (int64_t b = split * chunk; b < R; b += p.splits * chunk)
+            for (int64_t r = b + ty; r < R && r < b + chunk; r += ty_n)
+                for (int j = 0; j < ncol; j++) acc[j] = Tr::update(acc[j], src[r * p.elem_stride + j], r);
     }
-    if (r0 == 0 && ty == 0)
+    if (split == 0 && ty == 0)
         for (int j = 0; j < ncol; j++) acc[j] = Tr::first(acc[j], src[j]);
 
     // combine the ty lanes in fixed order
@@ -462,7 +518,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int
     }
     if (ty == 0)
         for (int j = 0; j < ncol; j++) emit_partial<T, Tr>(p, (int64_t)split * p.nout + o0 + j, acc[j]);
-    if (!arrive_last(p.counters + group, p.splits)) return;
+    if (!arrive_last(p.counters + group * p.cstride, split, p.splits, p.fan)) return;
     // fold this column tile: row lane ty takes splits ty, ty + ty_n, ...; then the fixed LDS order
 #pragma unroll
     for (int j = 0; j < VEC; j++) acc[j] = Tr::identity();
@@ -498,7 +554,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int
     }
     if (ty == 0)
         for (int j = 0; j < ncol; j++) emit_final<T, Tr>(p, o0 + j, acc[j]);
-    if (threadIdx.x == 0) store_agent(p.counters + group, 0);
+    if (threadIdx.x == 0) store_agent(p.counters + group * p.cstride, 0);
 }
 
 // ---- host side ---------------------------------------------------------------------------------------------
@@ -513,22 +569,27 @@ template <typename T, typename Tr>
 int launch_rows(const RedParams<T> &p, hipStream_t s)
 {
     constexpr int VEC = VecOf<T>::N;
-    const bool vec = p.elem_stride == 1 && p.inner == 1 && aligned16(p.in) && p.outer_stride % VEC == 0 &&
-                     p.seg % VEC == 0;
+    const bool vec = p.elem_stride == 1 && p.inner == 1 && aligned16(p.in) && p.outer_stride % VEC == 0;
     const bool nt = vec && stream_source(p);
     const bool wave_row = p.splits == 1 && p.R <= 1024;
     if (wave_row) {
         int64_t grid = (p.nout + kWaves - 1) / kWaves;
         if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-        if (nt)       reduce_rows_kernel<T, Tr, VEC, true, true><<<(unsigned)grid, kBlock, 0, s>>>(p);
-        else if (vec) reduce_rows_kernel<T, Tr, VEC, true, false><<<(unsigned)grid, kBlock, 0, s>>>(p);
-        else          reduce_rows_kernel<T, Tr, 1, true, false><<<(unsigned)grid, kBlock, 0, s>>>(p);
+        if (nt)       reduce_rows_kernel<T, Tr, VEC, kWaveRow, true, kRowsU><<<(unsigned)grid, kBlock, 0, s>>>(p);
+        else if (vec) reduce_rows_kernel<T, Tr, VEC, kWaveRow, false, kRowsU><<<(unsigned)grid, kBlock, 0, s>>>(p);
+        else          reduce_rows_kernel<T, Tr, 1, kWaveRow, false, kRowsU><<<(unsigned)grid, kBlock, 0, s>>>(p);
     } else {
         int64_t grid = p.nout * p.splits;
         if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-        if (nt)       reduce_rows_kernel<T, Tr, VEC, false, true><<<(unsigned)grid, kBlock, 0, s>>>(p);
-        else if (vec) reduce_rows_kernel<T, Tr, VEC, false, false><<<(unsigned)grid, kBlock, 0, s>>>(p);
-        else          reduce_rows_kernel<T, Tr, 1, false, false><<<(unsigned)grid, kBlock, 0, s>>>(p);
+        if (p.splits > 1) {
+            if (nt)       reduce_rows_kernel<T, Tr, VEC, kSplitRow, true, kSplitU><<<(unsigned)grid, kBlock, 0, s>>>(p);
+            else if (vec) reduce_rows_kernel<T, Tr, VEC, kSplitRow, false, kRowsU><<<(unsigned)grid, kBlock, 0, s>>>(p);
+            else          reduce_rows_kernel<T, Tr, 1, kSplitRow, false, kRowsU><<<(unsigned)grid, kBlock, 0, s>>>(p);
+        } else {
+            if (nt)       reduce_rows_kernel<T, Tr, VEC, kBlockRow, true, kRowsU><<<(unsigned)grid, kBlock, 0, s>>>(p);
+            else if (vec) reduce_rows_kernel<T, Tr, VEC, kBlockRow, false, kRowsU><<<(unsigned)grid, kBlock, 0, s>>>(p);
+            else          reduce_rows_kernel<T, Tr, 1, kBlockRow, false, kRowsU><<<(unsigned)grid, kBlock, 0, s>>>(p);
+        }
     }
     ZENU_LAUNCH_CHECK();
     return ZENU_OK;
@@ -596,6 +657,8 @@ int reduce_contiguous(const T *src, int64_t outer, int64_t R, int64_t inner, T *
     p.part_key = nullptr;
     p.part_idx = nullptr;
     p.counters = nullptr;
+    p.fan = 1;
+    p.cstride = 1;
     p.gsrc = src;
     p.g_outer_stride = R * inner;
     p.g_elem_stride = inner;
@@ -624,17 +687,27 @@ int reduce_contiguous(const T *src, int64_t outer, int64_t R, int64_t inner, T *
     }
     if (splits < 1) splits = 1;
     if (splits > 4096) splits = 4096;
-    int64_t seg = (R + splits - 1) / splits;
-    seg = (seg + 15) / 16 * 16;  // keep vector alignment of every split
-    splits = (R + seg - 1) / seg;
     p.splits = (int)splits;
-    p.seg = seg;
 
     if (splits == 1) return use_cols ? launch_cols<T, Tr>(p, s) : launch_rows<T, Tr>(p, s);
 
     // one launch: partials in a workspace, folded by the last workgroup of each group to arrive
-    int *counters = reserve_counters(groups);
+    // arrival tree: about sqrt(splits) splits per leaf once a flat counter would serialise
+    int fan = (int)splits, cstride = 1;
+    if (splits > 32) {
+        fan = 1;
+        while ((int64_t)fan * fan < splits) fan++;
+        cstride = 1 + (int)((splits + fan - 1) / fan);
+    }
+    int *counters = reserve_counters(groups * cstride);
+    if (!counters && cstride > 1) {   // too many groups for trees: flat counters
+        fan = (int)splits;
+        cstride = 1;
+        counters = reserve_counters(groups);
+    }
     if (!counters) return ZENU_ERR_UNSUPPORTED;
+    p.fan = fan;
+    p.cstride = cstride;
     const size_t key_bytes = ((size_t)nout * splits * sizeof(T) + 255) / 256 * 256;
     const size_t idx_bytes = Tr::kHasIdx ? (size_t)nout * splits * sizeof(int32_t) : 0;
     Workspace ws(key_bytes + idx_bytes, s);
