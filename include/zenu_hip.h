@@ -163,6 +163,18 @@ int zenu_hip_relu(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other
 int zenu_hip_relu_backward_mask(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other,
                                 double alpha, zenu_stream_t stream);
 
+/* gx = gy * mask(x): the two backward ops of zenu-autograd/src/activation/relu.rs:35-44 in one pass. */
+int zenu_hip_relu_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *gy,
+                           const zenu_tensor_t *x, double alpha, zenu_stream_t stream);
+
+/* to = clip(other, min, max); mask = 1 inside [min, max] (and for NaN), 0 outside
+ * (zenu-matrix/src/operation/clip.rs:289-318).  The assign forms are to == other.  The mask is
+ * written with the mask's own stride (clip.rs:90-96 indexes it with the input's). */
+int zenu_hip_clip(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other, double min,
+                  double max, zenu_stream_t stream);
+int zenu_hip_clip_backward_mask(int dtype, const zenu_tensor_t *mask, const zenu_tensor_t *other,
+                                double min, double max, zenu_stream_t stream);
+
 /* Strided copy, same shapes (copy_from, zenu-matrix/src/operation/copy_from.rs:211-267;
  * to_default_stride, to_default_stride.rs:7-15). */
 int zenu_hip_copy(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *src, zenu_stream_t stream);
@@ -194,6 +206,34 @@ int zenu_hip_max_idx(int dtype, int64_t *out_flat_idx_dev, void *out_val_dev,
                      const zenu_tensor_t *src, zenu_stream_t stream);
 /* *out_dev = sum |x| (Asum, zenu-matrix/src/operation/asum.rs:14-68). */
 int zenu_hip_asum(int dtype, void *out_dev, const zenu_tensor_t *src, zenu_stream_t stream);
+
+/* ------------------------------------------------------------------------- */
+/* Fused classifier-head chains (each replaces a sequence of the ops above)    */
+/* ------------------------------------------------------------------------- */
+
+/* to = softmax(src) along `axis` (softmax_assign, zenu-matrix/src/operation/softmax.rs:10-25:
+ * src - max_axis(axis), exp, / sum(axis)); to may be src. */
+int zenu_hip_softmax(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *src, int axis,
+                     zenu_stream_t stream);
+/* gx = y*gy - y * sum(y*gy, axis) (SoftMax::backward, zenu-autograd/src/loss/softmax.rs:33-40). */
+int zenu_hip_softmax_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *y,
+                              const zenu_tensor_t *gy, int axis, zenu_stream_t stream);
+/* cross_entropy(pred, ans), zenu-autograd/src/loss/cross_entropy.rs:12-23, pred and ans [N, C]:
+ * prob = softmax(pred, 1) (kept for the backward pass), loss (0-d) = sum(ans * log(prob)) / -N. */
+int zenu_hip_softmax_cross_entropy(int dtype, const zenu_tensor_t *loss, const zenu_tensor_t *prob,
+                                   const zenu_tensor_t *pred, const zenu_tensor_t *ans,
+                                   zenu_stream_t stream);
+/* Gradient of that loss with respect to pred, following the backward of div, sum_to, mul, log
+ * and softmax op by op; gloss (0-d, device) is the gradient arriving at the loss, NULL = 1. */
+int zenu_hip_softmax_cross_entropy_backward(int dtype, const zenu_tensor_t *gpred,
+                                            const zenu_tensor_t *prob, const zenu_tensor_t *ans,
+                                            const zenu_tensor_t *gloss, zenu_stream_t stream);
+/* pre = z + bias (bias [F] broadcast over the leading dims of z [.., F]), act = relu(pre, alpha):
+ * Linear::call followed by relu (zenu-layer/src/layers/linear.rs:27-31,
+ * zenu-autograd/src/activation/relu.rs:24-33).  pre may be NULL. */
+int zenu_hip_bias_add_relu(int dtype, const zenu_tensor_t *pre, const zenu_tensor_t *act,
+                           const zenu_tensor_t *z, const zenu_tensor_t *bias, double alpha,
+                           zenu_stream_t stream);
 
 /* ------------------------------------------------------------------------- */
 /* Fused optimizer updates (one launch, 4 loads + 3 stores per element)        */
@@ -264,6 +304,15 @@ int zenu_hip_adam_step_multi(int dtype, int n_tensors, void *const *p_dev, const
     void array_tanh_assign_##S(T *a, int size, int stride);                                       \
     void array_sqrt_assign_##S(T *a, int size, int stride);                                       \
     void array_abs_assign_##S(T *a, int size, int stride);                                        \
+    /* array_scalar.h:97-106 */                                                                    \
+    void array_clip_##S(T *input, T *output, int size, int stride_in, int stride_out, T min, T max); \
+    void array_clip_assign_##S(T *input, int size, int stride, T min, T max);                     \
+    void array_clip_backward_##S(T *input, T *mask, T max, T min, int size, int stride_in,        \
+                                 int stride_mask);                                                 \
+    void array_clip_backward_assign_##S(T *input, T max, T min, int size, int stride);            \
+    /* array_array.h:27-28: output[i] = input[i] + bias[(i / channel_stride) % bias_size] */      \
+    void conv_bias_add_##S(const T *input, T *output, int channel_stride, const T *bias,          \
+                           int bias_size, int total_elements);                                     \
     /* activations.h:7-11 */                                                                       \
     void relu_##S(T *input, T *output, T alpha, int size, int input_stride, int output_stride);   \
     void relu_backward_mask_##S(T *input, T *mask, T alpha, int size, int input_stride,           \

@@ -131,6 +131,17 @@ def relu(to, other, alpha):
     _chk(getattr(lib(), f"zo_relu_{s}")(C.byref(view(to)), C.byref(view(other)), ct(alpha)), "relu")
 
 
+def clip(to, other, lo, hi):
+    s, ct = _sfx(to.dtype)
+    _chk(getattr(lib(), f"zo_clip_{s}")(C.byref(view(to)), C.byref(view(other)), ct(lo), ct(hi)), "clip")
+
+
+def clip_backward_mask(mask, other, lo, hi):
+    s, ct = _sfx(mask.dtype)
+    _chk(getattr(lib(), f"zo_clip_backward_mask_{s}")(C.byref(view(mask)), C.byref(view(other)), ct(lo), ct(hi)),
+         "clip_backward_mask")
+
+
 def relu_backward_mask(to, other, alpha):
     s, ct = _sfx(to.dtype)
     _chk(getattr(lib(), f"zo_relu_backward_mask_{s}")(C.byref(view(to)), C.byref(view(other)), ct(alpha)),

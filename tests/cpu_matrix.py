@@ -123,6 +123,44 @@ class CpuMatrix:
     def relu(self, other, alpha): zo.relu(self.a, other.a, alpha)
     def relu_backward_mask(self, other, alpha): zo.relu_backward_mask(self.a, other.a, alpha)
 
+    def relu_backward(self, gy, x, alpha):
+        """zenu-autograd/src/activation/relu.rs:35-44: mask, then gy * mask"""
+        mask = x.alloc_like()
+        mask.relu_backward_mask(x, alpha)
+        self.mul_array(gy, mask)
+
+    # clip.rs:289-318
+    def clip(self, lo, hi):
+        out = self.alloc_like()
+        zo.clip(out.a, self.a, lo, hi)
+        return out
+
+    def clip_assign(self, lo, hi): zo.clip(self.a, self.a, lo, hi)
+
+    def clip_backward_mask(self, lo, hi):
+        out = self.alloc_like()
+        zo.clip_backward_mask(out.a, self.a, lo, hi)
+        return out
+
+    def clip_backward_assign_mask(self, lo, hi): zo.clip_backward_mask(self.a, self.a, lo, hi)
+
+    def softmax_assign(self, source, axis):
+        """softmax.rs:10-25, op by op"""
+        if not (0 <= axis < self.ndim):
+            raise zo.OracleError("axis must be less than the number of dimensions")
+        max_diff = source - source.max_axis(axis, True)
+        output = max_diff.exp()
+        total = output.sum(axis, True)
+        output /= total
+        self.copy_from(output)
+
+    def bias_add_relu(self, z, bias, alpha, pre=None):
+        """Linear::call's `+ bias` (linear.rs:27-31) followed by relu (activation/relu.rs:24-33)"""
+        a = z + bias
+        if pre is not None:
+            pre.copy_from(a)
+        self.relu(a, alpha)
+
     # reductions
     def sum(self, axis, keep_dim=False): return CpuMatrix(zo.sum_axis(self.a, axis, keep_dim))
 
@@ -167,3 +205,36 @@ for _n, _f in (("exp", zo.EXP), ("log", zo.LOG), ("tanh", zo.TANH), ("sqrt", zo.
 
 def sum_to(source, target):
     zo.sum_to(source.a, target.a)
+
+
+def softmax_backward(y, gy, axis):
+    """SoftMax::backward, zenu-autograd/src/loss/softmax.rs:33-40"""
+    gx = y * gy
+    sum_gx = gx.sum(axis, True)
+    return gx - (y * sum_gx)
+
+
+def cross_entropy(pred, ans):
+    """zenu-autograd/src/loss/cross_entropy.rs:12-23 -> (loss, softmax output)"""
+    prob = pred.alloc_like()
+    prob.softmax_assign(pred, 1)
+    y_log_pred = ans * prob.log()
+    total = CpuMatrix.zeros((), pred.dtype)
+    sum_to(y_log_pred, total)
+    neg_n = CpuMatrix.from_vec([-float(pred.shape[0])], (), pred.dtype)
+    return total / neg_n, prob
+
+
+def cross_entropy_backward(prob, ans, gloss=None):
+    """backward of div (x side), sum_to (broadcast), mul (log side), log, softmax, in that order
+    (functions/div.rs, sum_to.rs, mul.rs, log.rs, loss/softmax.rs:33-40)"""
+    dt = prob.dtype
+    if gloss is None:
+        gloss = CpuMatrix.from_vec([1.0], (), dt)
+    neg_n = CpuMatrix.from_vec([-float(prob.shape[0])], (), dt)
+    g_total = gloss / neg_n
+    g_yl = CpuMatrix.zeros(prob.shape, dt)
+    g_yl += g_total
+    g_log = ans * g_yl
+    g_prob = g_log / prob
+    return softmax_backward(prob, g_prob, 1)

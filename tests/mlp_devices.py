@@ -11,6 +11,7 @@ class CpuDev:
         import zenu_oracle as zo
         self.M = cpu_matrix.CpuMatrix
         self.sum_to = cpu_matrix.sum_to
+        self.F = cpu_matrix      # softmax_backward / cross_entropy / cross_entropy_backward, op by op
         self.zo = zo
 
     def tick(self, category):
@@ -44,6 +45,7 @@ class HipDev:
         self.hip = hip
         self.M = hip.Matrix
         self.sum_to = hip.sum_to
+        self.F = hip             # the fused entry points
         self.blas = C.CDLL("librocblas.so")
         self.handle = C.c_void_p()
         assert self.blas.rocblas_create_handle(C.byref(self.handle)) == 0

@@ -444,3 +444,72 @@ def shape_errors(dev):
         dev.M.zeros([2, 3]).sum(2)
     with pytest.raises(dev.Error):
         dev.M.zeros([2, 3]).max_axis(5)
+
+
+# ---- softmax / cross-entropy / clip: the chains the fused entry points replace --------------------
+# `dev.F` holds softmax_backward, cross_entropy, cross_entropy_backward (op-by-op on the CPU device)
+
+
+@case
+def softmax_cases(dev):  # zenu-matrix/src/operation/softmax.rs:37-91 (softmax_1d, softmax_2d), 1e-6 on asum
+    a = dev.M.from_vec([1., 2., 3., 4.], [4])
+    b = dev.M.zeros([4])
+    b.softmax_assign(a, 0)
+    ans = dev.M.from_vec([0.0320586, 0.08714432, 0.23688284, 0.64391428], [4])
+    assert (b - ans).asum() < 1e-6
+    a = dev.M.from_vec([1., 2., 3., 4., 5., 6.], [2, 3])
+    b = dev.M.zeros([2, 3])
+    b.softmax_assign(a, 1)
+    ans = dev.M.from_vec([0.09003057, 0.24472847, 0.66524096, 0.09003057, 0.24472847, 0.66524096], [2, 3])
+    assert (b - ans).asum() < 1e-6
+    b = dev.M.zeros([2, 3])
+    b.softmax_assign(a, 0)
+    ans = dev.M.from_vec([0.04742587, 0.04742587, 0.04742587, 0.95257413, 0.95257413, 0.95257413], [2, 3])
+    assert (b - ans).asum() < 1e-6
+    with_axis_error = False
+    try:
+        b.softmax_assign(a, 2)      # "axis must be less than the number of dimensions"
+    except dev.Error:
+        with_axis_error = True
+    assert with_axis_error
+
+
+@case
+def softmax_backward_2d_1d(dev):  # zenu-autograd/src/loss/softmax.rs:70-103, f64, 1e-6
+    x = dev.M.from_vec([1., 2., 3., 4., 5., 6., 7., 8.], [2, 4], np.float64)
+    y = dev.M.zeros([2, 4], np.float64)
+    y.softmax_assign(x, 1)
+    close(y, [0.0320586, 0.08714432, 0.23688284, 0.64391428] * 2, 1e-6, (2, 4))
+    # loss = sum(y * [1,2,3,4]) => the gradient arriving at y is [1,2,3,4] in every row
+    gy = dev.M.from_vec([1., 2., 3., 4.] * 2, [2, 4], np.float64)
+    gx = dev.F.softmax_backward(y, gy, 1)
+    close(gx, [-0.07991097, -0.13007621, -0.11670097, 0.32668814] * 2, 1e-6, (2, 4))
+
+
+@case
+def cross_entropy_cases(dev):  # zenu-autograd/src/loss/cross_entropy.rs:38-84
+    pred = dev.M.from_vec([0.1, 0.9, 0.1, 0.1], [1, 4], np.float64)
+    ans = dev.M.from_vec([0., 1., 0., 0.], [1, 4], np.float64)
+    loss, prob = dev.F.cross_entropy(pred, ans)
+    close(loss, 0.8536, 1e-4)
+    close(dev.F.cross_entropy_backward(prob, ans), [[0.1914, -0.5741, 0.1914, 0.1914]], 1e-4)
+    pred = dev.M.from_vec([0.1, 0.9, 0.1, 0.1, 0.01, 0.9, 0.2, 0.05], [2, 4])
+    ans = dev.M.from_vec([0., 1., 0., 0., 1., 0., 0., 0.], [2, 4])
+    loss, prob = dev.F.cross_entropy(pred, ans)
+    close(loss, 1.2957, 2e-5)
+    close(dev.F.cross_entropy_backward(prob, ans),
+          [[0.0957, -0.2871, 0.0957, 0.0957], [-0.4121, 0.2142, 0.1064, 0.0915]], 3e-4)
+
+
+@case
+def clip_cases(dev):  # zenu-matrix/src/operation/clip.rs:321-372; zenu-cuda/src/kernel/mod.rs:1300-1368
+    for shape in ([4], [2, 2]):
+        a = dev.M.from_vec([1., 2., 3., 4.], shape)
+        eq(a.clip(2., 3.), [2., 2., 3., 3.], shape)
+        a.clip_assign(2., 3.)
+        eq(a, [2., 2., 3., 3.], shape)
+    for dt in (np.float32, np.float64):
+        a = dev.M.from_vec([0., 1., 2., 3., 4., 5.], [6], dt)
+        eq(a.clip_backward_mask(1., 2.), [0., 1., 1., 0., 0., 0.])
+        a.clip_backward_assign_mask(1., 2.)
+        eq(a, [0., 1., 1., 0., 0., 0.])

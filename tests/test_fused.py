@@ -1,0 +1,237 @@
+"""Fused classifier-head entry points (softmax, softmax backward, cross-entropy forward and backward,
+bias add + ReLU, ReLU backward, clip) against the op-by-op chains on the CPU oracle
+(tests/cpu_matrix.py restates each chain with the reference's file:line).
+
+Bars: pure +,-,*,/ and compare work is bit-exact wherever the chain's own summation order is the
+fused kernel's (one thread per softmax line: reduced length <= 64 or an inner stride); exp/log
+within 2 ulp per call, so softmax outputs within a few ulp (rel 2e-6 f32 / 1e-14 f64); tree sums
+rel 1e-5 f32 / 1e-12 f64.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import cpu_matrix
+from cpu_matrix import CpuMatrix
+
+pytestmark = pytest.mark.gpu
+
+
+def bits_equal(a, b):
+    a = np.ascontiguousarray(a).reshape(-1)
+    b = np.ascontiguousarray(b).reshape(-1)
+    ui = np.uint32 if a.dtype == np.float32 else np.uint64
+    return a.shape == b.shape and np.array_equal(a.view(ui), b.view(ui))
+
+
+def rel_err(got, ref):
+    got = got.astype(np.float64)
+    ref = ref.astype(np.float64)
+    return float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), 1e-300)))
+
+
+SOFTMAX_SHAPES = [
+    # shape, axis
+    ((256, 10), 1),        # configs[4] logits: one thread per row, index-order sum
+    ((7, 64), 1),
+    ((64, 1000), 1),       # workgroup per row, row in registers (vector loads)
+    ((33, 1027), 1),       # not a multiple of the vector width
+    ((5, 5000), 1),        # three-pass rows (f32: > 4096)
+    ((3, 9001), 1),
+    ((100, 37), 0),        # reduced axis first: one thread per column
+    ((4, 50, 6), 1),       # middle axis
+    ((2, 3, 4, 5), 3),
+    ((17,), 0),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("shape,axis", SOFTMAX_SHAPES, ids=lambda v: str(v))
+def test_softmax_forward_backward(hip, dtype, shape, axis):
+    print(f"[case] softmax {shape} axis {axis} {np.dtype(dtype).name}", flush=True)
+    r = np.random.default_rng(abs(hash((shape, axis))) % 2**31)
+    x = (r.standard_normal(shape) * 3).astype(dtype)
+    gy = r.standard_normal(shape).astype(dtype)
+    R = shape[axis]
+    inner = int(np.prod(shape[axis + 1:]))
+    in_order = R <= 64 or inner > 1     # one thread per line: the chain's own summation order
+    # exp within 2 ulp when the denominators are summed alike; otherwise the sum bar applies
+    if in_order:
+        tol = 2e-6 if dtype == np.float32 else 1e-14
+    else:
+        tol = 1e-5 if dtype == np.float32 else 1e-12
+
+    ref = CpuMatrix.zeros(shape, dtype)
+    ref.softmax_assign(CpuMatrix.from_numpy(x), axis)
+    out = hip.Matrix.zeros(shape, dtype)
+    out.softmax_assign(hip.Matrix.from_numpy(x), axis)
+    y = out.to_numpy()
+    assert rel_err(y, ref.a) <= tol
+    assert np.allclose(y.sum(axis=axis, dtype=np.float64), 1.0, atol=1e-5 if dtype == np.float32 else 1e-12)
+
+    # in place (to == src)
+    inpl = hip.Matrix.from_numpy(x)
+    inpl.softmax_assign(inpl, axis)
+    assert bits_equal(inpl.to_numpy(), y)
+
+    # backward from the SAME y on both devices: arithmetic only
+    gref = cpu_matrix.softmax_backward(CpuMatrix.from_numpy(y), CpuMatrix.from_numpy(gy), axis).a
+    g = hip.softmax_backward(hip.Matrix.from_numpy(y), hip.Matrix.from_numpy(gy), axis).to_numpy()
+    if in_order:
+        assert bits_equal(g, gref)          # index-order sum on both sides
+    else:
+        scale = np.max(np.abs(gref))
+        assert np.max(np.abs(g.astype(np.float64) - gref)) <= (1e-5 if dtype == np.float32 else 1e-12) * scale
+
+
+def test_softmax_strided_views(hip):
+    """transposed source and sliced destination go through contiguous staging"""
+    r = np.random.default_rng(5)
+    x = r.standard_normal((40, 24)).astype(np.float32)
+    ref = CpuMatrix.zeros((24, 40))
+    ref.softmax_assign(CpuMatrix.from_numpy(x).transpose(), 1)
+    big = hip.Matrix.zeros((24, 80))
+    dst = big.slice(slice(None), slice(0, 80, 2))
+    dst.softmax_assign(hip.Matrix.from_numpy(x).transpose(), 1)
+    assert rel_err(big.to_numpy()[:, ::2], ref.a) <= 2e-6
+    assert np.all(big.to_numpy()[:, 1::2] == 0)
+
+
+def test_softmax_special_rows(hip):
+    """NaN in position 0 / elsewhere and an all -inf row poison the row exactly as in the chain; a row
+    with +inf gives NaN at the inf (inf - inf) and 0 elsewhere... all NaN after the division"""
+    x = np.array([[np.nan, 1, 2, 3], [1, np.nan, 2, 3], [-np.inf] * 4, [1, np.inf, 2, 3], [5, 5, 5, 5]],
+                 dtype=np.float32)
+    ref = CpuMatrix.zeros(x.shape)
+    ref.softmax_assign(CpuMatrix.from_numpy(x), 1)
+    out = hip.Matrix.zeros(x.shape)
+    out.softmax_assign(hip.Matrix.from_numpy(x), 1)
+    got = out.to_numpy()
+    assert np.array_equal(np.isnan(got), np.isnan(ref.a))
+    assert bits_equal(got[4], ref.a[4])
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("n,c", [(256, 10), (1, 4), (1000, 64), (50, 1000), (70000, 3)])
+def test_cross_entropy(hip, dtype, n, c):
+    print(f"[case] cross_entropy {n}x{c} {np.dtype(dtype).name}", flush=True)
+    r = np.random.default_rng(n * 131 + c)
+    pred = r.standard_normal((n, c)).astype(dtype)
+    ans = np.zeros((n, c), dtype=dtype)
+    ans[np.arange(n), r.integers(0, c, n)] = 1
+    sum_tol = 1e-5 if dtype == np.float32 else 1e-12
+    tol = (2e-6 if dtype == np.float32 else 1e-14) if c <= 64 else sum_tol
+
+    loss_ref, prob_ref = cpu_matrix.cross_entropy(CpuMatrix.from_numpy(pred), CpuMatrix.from_numpy(ans))
+    loss, prob = hip.cross_entropy(hip.Matrix.from_numpy(pred), hip.Matrix.from_numpy(ans))
+    assert rel_err(prob.to_numpy(), prob_ref.a) <= tol
+    exact = -np.sum(ans.astype(np.float64) * np.log(prob_ref.a.astype(np.float64))) / n
+    assert abs(float(loss.to_numpy()) - exact) <= sum_tol * abs(exact)
+    assert abs(float(loss.to_numpy()) - float(loss_ref.a)) <= 4 * sum_tol * abs(exact)
+
+    # backward from the same softmax output on both devices
+    p = prob.to_numpy()
+    gref = cpu_matrix.cross_entropy_backward(CpuMatrix.from_numpy(p), CpuMatrix.from_numpy(ans)).a
+    g = hip.cross_entropy_backward(hip.Matrix.from_numpy(p), hip.Matrix.from_numpy(ans)).to_numpy()
+    if c <= 64:
+        assert bits_equal(g, gref)
+    else:
+        assert np.max(np.abs(g.astype(np.float64) - gref)) <= sum_tol * np.max(np.abs(gref))
+    # closed form: (softmax - onehot) / N
+    closed = (p.astype(np.float64) - ans) / n
+    assert np.max(np.abs(g - closed)) <= 1e-6 / n * 4 + (1e-6 if dtype == np.float32 else 1e-14)
+
+    # a gradient arriving at the loss scales the result
+    gl = np.array(-2.5, dtype=dtype)
+    gref2 = cpu_matrix.cross_entropy_backward(CpuMatrix.from_numpy(p), CpuMatrix.from_numpy(ans),
+                                              CpuMatrix.from_numpy(gl)).a
+    g2 = hip.cross_entropy_backward(hip.Matrix.from_numpy(p), hip.Matrix.from_numpy(ans),
+                                    hip.Matrix.from_numpy(gl)).to_numpy()
+    if c <= 64:
+        assert bits_equal(g2, gref2)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("shape", [(256, 512), (3, 5, 7), (1000, 10), (4096, 4096)])
+@pytest.mark.parametrize("alpha", [0.0, 0.2])
+def test_bias_add_relu_and_backward(hip, dtype, shape, alpha):
+    print(f"[case] bias_add_relu {shape} {np.dtype(dtype).name} alpha {alpha}", flush=True)
+    r = np.random.default_rng(shape[0])
+    z = r.standard_normal(shape).astype(dtype)
+    z.reshape(-1)[::17] = 0.0
+    z.reshape(-1)[5::29] = -0.0
+    b = r.standard_normal(shape[-1]).astype(dtype)
+    b[::3] = 0.0
+    gy = r.standard_normal(shape).astype(dtype)
+
+    pre_ref, act_ref = CpuMatrix.zeros(shape, dtype), CpuMatrix.zeros(shape, dtype)
+    act_ref.bias_add_relu(CpuMatrix.from_numpy(z), CpuMatrix.from_numpy(b), alpha, pre=pre_ref)
+    pre, act = hip.Matrix.zeros(shape, dtype), hip.Matrix.zeros(shape, dtype)
+    act.bias_add_relu(hip.Matrix.from_numpy(z), hip.Matrix.from_numpy(b), alpha, pre=pre)
+    assert bits_equal(pre.to_numpy(), pre_ref.a)
+    assert bits_equal(act.to_numpy(), act_ref.a)      # includes the -0.0 of alpha*x for alpha = 0
+    act2 = hip.Matrix.zeros(shape, dtype)
+    act2.bias_add_relu(hip.Matrix.from_numpy(z), hip.Matrix.from_numpy(b), alpha)
+    assert bits_equal(act2.to_numpy(), act_ref.a)
+
+    gref = CpuMatrix.zeros(shape, dtype)
+    gref.relu_backward(CpuMatrix.from_numpy(gy), pre_ref, alpha)
+    g = hip.Matrix.zeros(shape, dtype)
+    g.relu_backward(hip.Matrix.from_numpy(gy), pre, alpha)
+    assert bits_equal(g.to_numpy(), gref.a)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+def test_clip_parity(hip, dtype):
+    r = np.random.default_rng(11)
+    x = (r.standard_normal((257, 129)) * 2).astype(dtype)
+    x[0, :4] = [np.nan, np.inf, -np.inf, -0.0]
+    x[1, :2] = [-1.0, 1.5]                     # exactly on the bounds
+    cx, hx = CpuMatrix.from_numpy(x), hip.Matrix.from_numpy(x)
+    assert bits_equal(hx.clip(-1.0, 1.5).to_numpy(), cx.clip(-1.0, 1.5).a)
+    assert bits_equal(hx.clip_backward_mask(-1.0, 1.5).to_numpy(), cx.clip_backward_mask(-1.0, 1.5).a)
+    # strided views, same strides on both operands (the reference indexes the mask with the
+    # input's stride, clip.rs:90-96, so only equal strides are well defined there)
+    cv, hv = cx.slice(slice(None), slice(0, 129, 2)), hx.slice(slice(None), slice(0, 129, 2))
+    cv.clip_assign(-0.5, 0.5)
+    hv.clip_assign(-0.5, 0.5)
+    assert bits_equal(hx.to_numpy(), cx.a)
+    cv.clip_backward_assign_mask(-0.25, 0.25)
+    hv.clip_backward_assign_mask(-0.25, 0.25)
+    assert bits_equal(hx.to_numpy(), cx.a)
+
+
+def test_reference_named_clip_and_conv_bias_add(hip):
+    """array_clip_* / conv_bias_add_* keep the reference's names and argument order
+    (zenu-cuda-kernel-sys/kernel/array_scalar.h:97-106, array_array.h:27-28)"""
+    L = hip.lib()
+    fp = C.POINTER(C.c_float)
+    a = np.arange(6, dtype=np.float32)
+    d = hip.Matrix.from_numpy(a)
+    o = hip.Matrix.zeros([6])
+    L.array_clip_float.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float]
+    L.array_clip_float.restype = None
+    L.array_clip_float(d.as_ptr(), o.as_ptr(), 6, 1, 1, 1.0, 2.0)
+    assert np.array_equal(o.to_numpy(), [1, 1, 2, 2, 2, 2])
+    L.array_clip_backward_float.argtypes = [C.c_void_p, C.c_void_p, C.c_float, C.c_float, C.c_int, C.c_int, C.c_int]
+    L.array_clip_backward_float.restype = None
+    L.array_clip_backward_float(d.as_ptr(), d.as_ptr(), 2.0, 1.0, 6, 1, 1)   # kernel/mod.rs:1316
+    assert np.array_equal(d.to_numpy(), [0, 1, 1, 0, 0, 0])
+
+    # conv_bias_add: [N, C, H*W] + bias[C], plus totals that end inside an image / a channel
+    r = np.random.default_rng(3)
+    n, c, hw = 3, 5, 14
+    x = r.standard_normal(n * c * hw).astype(np.float64)
+    bias = r.standard_normal(c).astype(np.float64)
+    L.conv_bias_add_double.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int]
+    L.conv_bias_add_double.restype = None
+    for total in (n * c * hw, n * c * hw - hw, n * c * hw - 3, 9):
+        dx, db = hip.Matrix.from_numpy(x), hip.Matrix.from_numpy(bias)
+        out = hip.Matrix.zeros([n * c * hw], np.float64)
+        L.conv_bias_add_double(dx.as_ptr(), out.as_ptr(), hw, db.as_ptr(), c, total)
+        idx = np.arange(total)
+        exp = np.zeros_like(x)
+        exp[:total] = x[:total] + bias[(idx // hw) % c]
+        assert bits_equal(out.to_numpy(), exp), total
+    del fp

@@ -11,6 +11,7 @@ def hipdev(hip):
     class HipDev:
         M = hip.Matrix
         sum_to = staticmethod(hip.sum_to)
+        F = hip
         Error = hip.ZenuHipError
     return HipDev
 

@@ -4,7 +4,7 @@ oracle (same op sequence, same inputs; GEMM on each side's library).
 Bars: quantities that do not pass through a GEMM-dependent chain would be bit-exact; everything
 here sits downstream of GEMMs computed by two different libraries (OpenBLAS vs rocBLAS, different
 summation order), so loss, gradients and updated parameters are compared at 1e-4 relative to the
-tensor's largest magnitude (SURVEY 8d's bar for GEMM-fed quantities)."""
+tensor's largest magnitude."""
 import numpy as np
 import pytest
 
@@ -37,6 +37,37 @@ def test_cpu_step_matches_plain_numpy():
     g1 = (g2 @ W2) * (a1 > 0)
     assert rel(grads["linear1.weight"].to_numpy(), g1.T @ xd) < 1e-4
     assert rel(grads["linear1.bias"].to_numpy(), g1.sum(0)) < 1e-4
+
+
+def test_cpu_fused_spelling_is_the_same_chain():
+    """on the CPU device the fused names are the op-by-op chains: identical bits"""
+    x, t, params = mlp_step.make_inputs()
+    a = mlp_step.MlpStep(mlp_devices.CpuDev(), x, t, params)
+    b = mlp_step.MlpStep(mlp_devices.CpuDev(), x, t, params, fused=True)
+    la, ga = a.step()
+    lb, gb = b.step()
+    assert np.array_equal(la.to_numpy(), lb.to_numpy())
+    for k in ga:
+        assert np.array_equal(ga[k].to_numpy(), gb[k].to_numpy()), k
+        assert np.array_equal(a.p[k].to_numpy(), b.p[k].to_numpy()), k
+
+
+@pytest.mark.gpu
+def test_hip_fused_step_matches_hip_step(hip):
+    """fused entry points against the op sequence on the same device and the same GEMMs: they differ
+    only in summation order (softmax denominators over 10 classes, the loss), far below 1e-5"""
+    x, t, params = mlp_step.make_inputs()
+    dev = mlp_devices.HipDev(hip)
+    a = mlp_step.MlpStep(dev, x, t, params)
+    b = mlp_step.MlpStep(dev, x, t, params, fused=True)
+    for step in range(3):
+        for k in a.p:                      # same starting point each step
+            b.p[k].copy_from(a.p[k]); b.opt.m[k].copy_from(a.opt.m[k]); b.opt.v[k].copy_from(a.opt.v[k])
+        la, ga = a.step()
+        lb, gb = b.step()
+        assert abs(float(la.to_numpy()) - float(lb.to_numpy())) <= 1e-5 * abs(float(la.to_numpy()))
+        for k in ga:
+            assert rel(gb[k].to_numpy(), ga[k].to_numpy()) < 1e-5, (step, k)
 
 
 @pytest.mark.gpu

@@ -10,6 +10,7 @@ import zenu_oracle as zo
 class CpuDev:
     M = cpu_matrix.CpuMatrix
     sum_to = staticmethod(cpu_matrix.sum_to)
+    F = cpu_matrix
     Error = (zo.OracleError, Exception)
 
 

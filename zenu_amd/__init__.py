@@ -5,5 +5,6 @@ include/zenu_hip.h.  This package is the thin host-side mirror of zenu-matrix's 
 zenu-optimizer's optimizers used by the tests and the benchmark.
 """
 from ._lib import ZenuHipError, lib, LIB_PATH  # noqa: F401
-from .matrix import Matrix, sum_to, larger_shape, set_stream, get_stream, synchronize, default_stride  # noqa: F401
+from .matrix import (Matrix, sum_to, larger_shape, set_stream, get_stream, synchronize, default_stride,  # noqa: F401
+                     softmax_backward, cross_entropy, cross_entropy_backward)
 from .optim import SGD, Adam, AdamW  # noqa: F401

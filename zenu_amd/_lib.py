@@ -71,7 +71,15 @@ SIGNATURES = {
     "zenu_hip_powf": [_i, _TP, _TP, _d, _vp],
     "zenu_hip_relu": [_i, _TP, _TP, _d, _vp],
     "zenu_hip_relu_backward_mask": [_i, _TP, _TP, _d, _vp],
+    "zenu_hip_relu_backward": [_i, _TP, _TP, _TP, _d, _vp],
+    "zenu_hip_clip": [_i, _TP, _TP, _d, _d, _vp],
+    "zenu_hip_clip_backward_mask": [_i, _TP, _TP, _d, _d, _vp],
     "zenu_hip_copy": [_i, _TP, _TP, _vp],
+    "zenu_hip_softmax": [_i, _TP, _TP, _i, _vp],
+    "zenu_hip_softmax_backward": [_i, _TP, _TP, _TP, _i, _vp],
+    "zenu_hip_softmax_cross_entropy": [_i, _TP, _TP, _TP, _TP, _vp],
+    "zenu_hip_softmax_cross_entropy_backward": [_i, _TP, _TP, _TP, _TP, _vp],
+    "zenu_hip_bias_add_relu": [_i, _TP, _TP, _TP, _TP, _d, _vp],
     "zenu_hip_sum_axis": [_i, _TP, _TP, _i, _vp],
     "zenu_hip_sum_all": [_i, _vp, _TP, _vp],
     "zenu_hip_sum_to": [_i, _TP, _TP, _vp],
@@ -102,7 +110,9 @@ def reference_named_symbols():
         for fn in _UN:
             names += [f"array_{fn}_{s}", f"array_{fn}_assign_{s}"]
         names += [f"relu_{s}", f"relu_backward_mask_{s}", f"array_max_idx_{s}",
-                  f"memory_access_{s}", f"memory_set_{s}"]
+                  f"memory_access_{s}", f"memory_set_{s}",
+                  f"array_clip_{s}", f"array_clip_assign_{s}", f"array_clip_backward_{s}",
+                  f"array_clip_backward_assign_{s}", f"conv_bias_add_{s}"]
     return names
 
 

@@ -55,6 +55,8 @@ inline int64_t num_elm(const zenu_tensor_t &t)
 int validate_tensor(const zenu_tensor_t *t);  // ZENU_OK or ZENU_ERR_ARG
 bool same_shape(const zenu_tensor_t &a, const zenu_tensor_t &b);
 bool is_default_stride_strict(const zenu_tensor_t &t);
+// a row-major (default stride, dim/mod.rs:70-92) view of `ptr` with the given shape
+zenu_tensor_t default_view(void *ptr, int ndim, const int64_t *shape);
 
 // Broadcasting legality, restated from zenu-matrix/src/dim/dim_dyn.rs:24-58,119-148 and
 // zenu-matrix/src/with_clousers.rs:87-107,155-178.

@@ -115,6 +115,27 @@ template <typename T> struct ReluMaskF {
     __device__ __forceinline__ void init() {}
     __device__ __forceinline__ T operator()(T a, T) const { return (a > (T)0) ? (T)1 : alpha * (T)-1; }
 };
+// relu.rs backward: gx = gy * mask(x), the mask of ReluMaskF (zenu-autograd/src/activation/relu.rs:35-44)
+template <typename T> struct ReluBwdF {
+    static constexpr int NIN = 2;
+    T alpha;
+    __device__ __forceinline__ void init() {}
+    __device__ __forceinline__ T operator()(T gy, T x) const { return gy * ((x > (T)0) ? (T)1 : alpha * (T)-1); }
+};
+// clip.rs:50-57: below min -> min, above max -> max, NaN passes through
+template <typename T> struct ClipF {
+    static constexpr int NIN = 1;
+    T lo, hi;
+    __device__ __forceinline__ void init() {}
+    __device__ __forceinline__ T operator()(T a, T) const { return a < lo ? lo : (a > hi ? hi : a); }
+};
+// clip.rs:90-96: 0 outside [min, max], 1 inside (and for NaN)
+template <typename T> struct ClipMaskF {
+    static constexpr int NIN = 1;
+    T lo, hi;
+    __device__ __forceinline__ void init() {}
+    __device__ __forceinline__ T operator()(T a, T) const { return (a < lo || a > hi) ? (T)0 : (T)1; }
+};
 template <typename T> struct CopyF {
     static constexpr int NIN = 1;
     __device__ __forceinline__ void init() {}
@@ -808,6 +829,43 @@ int zenu_hip_relu_backward_mask(int dtype, const zenu_tensor_t *to, const zenu_t
     if (!same_shape(*to, *other)) return ZENU_ERR_SHAPE;
     if (dtype == ZENU_F32) { ReluMaskF<float> f; f.alpha = (float)alpha; return run1<float>(*to, *other, f, as_stream(stream)); }
     if (dtype == ZENU_F64) { ReluMaskF<double> f; f.alpha = alpha; return run1<double>(*to, *other, f, as_stream(stream)); }
+    return ZENU_ERR_ARG;
+}
+
+int zenu_hip_relu_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *gy, const zenu_tensor_t *x,
+                           double alpha, zenu_stream_t stream)
+{
+    int rc = check2(gx, gy);
+    if (!rc) rc = validate_tensor(x);
+    if (!rc) rc = ensure_init();
+    if (rc) return rc;
+    if (!same_shape(*gx, *gy) || !same_shape(*gx, *x)) return ZENU_ERR_SHAPE;
+    if (dtype == ZENU_F32) { ReluBwdF<float> f; f.alpha = (float)alpha; return run2<float>(*gx, *gy, *x, f, as_stream(stream)); }
+    if (dtype == ZENU_F64) { ReluBwdF<double> f; f.alpha = alpha; return run2<double>(*gx, *gy, *x, f, as_stream(stream)); }
+    return ZENU_ERR_ARG;
+}
+
+int zenu_hip_clip(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other, double min, double max,
+                  zenu_stream_t stream)
+{
+    int rc = check2(to, other);
+    if (!rc) rc = ensure_init();
+    if (rc) return rc;
+    if (!same_shape(*to, *other)) return ZENU_ERR_SHAPE;
+    if (dtype == ZENU_F32) { ClipF<float> f; f.lo = (float)min; f.hi = (float)max; return run1<float>(*to, *other, f, as_stream(stream)); }
+    if (dtype == ZENU_F64) { ClipF<double> f; f.lo = min; f.hi = max; return run1<double>(*to, *other, f, as_stream(stream)); }
+    return ZENU_ERR_ARG;
+}
+
+int zenu_hip_clip_backward_mask(int dtype, const zenu_tensor_t *mask, const zenu_tensor_t *other, double min,
+                                double max, zenu_stream_t stream)
+{
+    int rc = check2(mask, other);
+    if (!rc) rc = ensure_init();
+    if (rc) return rc;
+    if (!same_shape(*mask, *other)) return ZENU_ERR_SHAPE;
+    if (dtype == ZENU_F32) { ClipMaskF<float> f; f.lo = (float)min; f.hi = (float)max; return run1<float>(*mask, *other, f, as_stream(stream)); }
+    if (dtype == ZENU_F64) { ClipMaskF<double> f; f.lo = min; f.hi = max; return run1<double>(*mask, *other, f, as_stream(stream)); }
     return ZENU_ERR_ARG;
 }
 

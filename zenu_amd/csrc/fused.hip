@@ -1,0 +1,572 @@
+// fused.hip -- single-launch forms of the op chains ZeNu issues around a classifier head:
+//   softmax_assign                  zenu-matrix/src/operation/softmax.rs:10-25
+//                                   (x - max_axis(keep) ; exp ; sum(axis, keep) ; /= ; copy_from)
+//   SoftMax::backward               zenu-autograd/src/loss/softmax.rs:33-40
+//                                   (gx = y*gy ; sum(gx, axis, keep) ; gx - y*sum)
+//   cross_entropy (+ its backward)  zenu-autograd/src/loss/cross_entropy.rs:12-23
+//                                   (softmax(pred,1) ; log ; * ans ; sum_to([]) ; / -N)
+//   Linear bias add + ReLU          zenu-layer/src/layers/linear.rs:27-31, zenu-autograd/src/activation/relu.rs:24-33
+//
+// Every element goes through the same sequence of individually rounded operations as in the
+// chain (no contraction, exp/log from the device math library), so the fused results differ
+// from the chain only where the chain itself is order dependent: the sums.  The "lines" kernels
+// (one thread per softmax line) add in index order, exactly like sum.rs:20-25; the
+// workgroup-per-row kernels add in a fixed tree.
+//
+// Geometry: operands are row-major [outer, R, inner] with the softmax axis R in the middle;
+// views that are not in default stride are staged through a contiguous temporary.
+#include <math.h>
+
+#include "common.hpp"
+#include "vecmem.hpp"
+
+namespace zenu {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWaves = kBlock / 64;
+constexpr int kLineMaxR = 64;   // rows up to this length: one thread per row
+constexpr int kRegPacks = 4;    // workgroup-per-row: vectors a thread keeps in registers
+
+// ---- workgroup reductions in a fixed order ------------------------------------------------------------
+
+template <typename T, bool MAX> __device__ __forceinline__ T combine(T a, T b)
+{
+    if (MAX) return b > a ? b : a;   // a NaN never replaces (max.rs:27)
+    return a + b;
+}
+
+template <typename T, bool MAX> __device__ __forceinline__ T block_red(T v, T *lds)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = combine<T, MAX>(v, __shfl_xor(v, o));
+    __syncthreads();   // lds may still be read from the previous reduction
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+    __syncthreads();
+    T r = lds[0];
+#pragma unroll
+    for (int w = 1; w < kWaves; w++) r = combine<T, MAX>(r, lds[w]);
+    return r;
+}
+
+// ---- forward ---------------------------------------------------------------------------------------------
+// CE: additionally rowloss[line] = sum_r target * log(softmax)   (inner == 1 only)
+
+template <typename T, bool CE>
+__global__ __launch_bounds__(kBlock) void softmax_lines_kernel(const T *x, T *y, int64_t lines, int64_t R,
+                                                                int64_t inner, const T *target, T *rowloss)
+{
+    const int64_t line = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (line >= lines) return;
+    int64_t q = line, c = 0;
+    if (inner != 1) {
+        q = line / inner;
+        c = line - q * inner;
+    }
+    const int64_t base = q * R * inner + c;
+    const T *xl = x + base;
+    T *yl = y + base;
+    // max_axis: strict '>' from element 0 (max.rs:19-34)
+    T m = xl[0];
+    for (int64_t r = 1; r < R; r++) {
+        const T v = xl[r * inner];
+        if (v > m) m = v;
+    }
+    // exp(x - max), summed in index order starting from zero (sum.rs:20-25)
+    T sum = (T)0;
+    for (int64_t r = 0; r < R; r++) {
+        const T e = exp(xl[r * inner] - m);
+        yl[r * inner] = e;
+        sum = sum + e;
+    }
+    T acc = (T)0;
+    for (int64_t r = 0; r < R; r++) {
+        const T s = yl[r * inner] / sum;
+        yl[r * inner] = s;
+        if (CE) acc = acc + target[base + r * inner] * log(s);
+    }
+    if (CE) rowloss[line] = acc;
+}
+
+template <typename T, int VEC, bool CE, bool REG>
+__global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, int64_t R, const T *target,
+                                                               T *rowloss)
+{
+    __shared__ T lds[kWaves];
+    const int64_t row = blockIdx.x;
+    const T *xr = x + row * R;
+    T *yr = y + row * R;
+    const T *tr = CE ? target + row * R : nullptr;
+    const int64_t first = (int64_t)threadIdx.x * VEC;
+    constexpr int64_t step = (int64_t)kBlock * VEC;
+    const T x0 = xr[0];
+    T acc = (T)0;
+
+    if (REG) {   // R <= kRegPacks * step: the row lives in registers, one read and one write
+        Pack<T, VEC> v[kRegPacks];
+        T m = -INFINITY;
+#pragma unroll
+        for (int k = 0; k < kRegPacks; k++) {
+            const int64_t r = first + k * step;
+            v[k] = r < R ? load_pack<T, VEC, false>(xr + r) : splat<T, VEC>(-INFINITY);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) m = combine<T, true>(m, v[k].v[j]);
+        }
+        m = block_red<T, true>(m, lds);
+        if (x0 != x0) m = x0;   // a NaN in position 0 is never replaced
+        T sum = (T)0;
+#pragma unroll
+        for (int k = 0; k < kRegPacks; k++) {
+            if (first + k * step < R) {
+#pragma unroll
+                for (int j = 0; j < VEC; j++) {
+                    v[k].v[j] = exp(v[k].v[j] - m);
+                    sum = sum + v[k].v[j];
+                }
+            }
+        }
+        sum = block_red<T, false>(sum, lds);
+#pragma unroll
+        for (int k = 0; k < kRegPacks; k++) {
+            const int64_t r = first + k * step;
+            if (r < R) {
+                Pack<T, VEC> t;
+                if (CE) t = load_pack<T, VEC, false>(tr + r);
+#pragma unroll
+                for (int j = 0; j < VEC; j++) {
+                    const T s = v[k].v[j] / sum;
+                    v[k].v[j] = s;
+                    if (CE) acc = acc + t.v[j] * log(s);
+                }
+                store_pack<T, VEC, false>(yr + r, v[k]);
+            }
+        }
+    } else {     // long rows: three passes; the second and third find the row in cache
+        T m = -INFINITY;
+        for (int64_t r = first; r < R; r += step) {
+            const Pack<T, VEC> v = load_pack<T, VEC, false>(xr + r);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) m = combine<T, true>(m, v.v[j]);
+        }
+        m = block_red<T, true>(m, lds);
+        if (x0 != x0) m = x0;
+        T sum = (T)0;
+        for (int64_t r = first; r < R; r += step) {
+            Pack<T, VEC> v = load_pack<T, VEC, false>(xr + r);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) {
+                v.v[j] = exp(v.v[j] - m);
+                sum = sum + v.v[j];
+            }
+            store_pack<T, VEC, false>(yr + r, v);
+        }
+        sum = block_red<T, false>(sum, lds);
+        for (int64_t r = first; r < R; r += step) {   // each thread re-reads what it wrote itself
+            Pack<T, VEC> v = load_pack<T, VEC, false>(yr + r);
+            Pack<T, VEC> t;
+            if (CE) t = load_pack<T, VEC, false>(tr + r);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) {
+                const T s = v.v[j] / sum;
+                v.v[j] = s;
+                if (CE) acc = acc + t.v[j] * log(s);
+            }
+            store_pack<T, VEC, false>(yr + r, v);
+        }
+    }
+    if (CE) {
+        acc = block_red<T, false>(acc, lds);
+        if (threadIdx.x == 0) rowloss[row] = acc;
+    }
+}
+
+// loss = (sum of the row terms) / (-N), one workgroup
+template <typename T>
+__global__ __launch_bounds__(kBlock) void ce_finalize_kernel(const T *rowloss, int64_t n, T *loss, T neg_n)
+{
+    __shared__ T lds[kWaves];
+    T acc = (T)0;
+    for (int64_t i = threadIdx.x; i < n; i += kBlock) acc = acc + rowloss[i];
+    acc = block_red<T, false>(acc, lds);
+    if (threadIdx.x == 0) *loss = acc / neg_n;
+}
+
+// ---- backward --------------------------------------------------------------------------------------------
+// gx = t - y * sum(t), t = y * gy.  CE: gy = (target * g_total) / y with g_total = gout / (-N), the
+// chain div -> sum_to -> mul -> log backward of cross_entropy.rs:18-22.
+
+template <typename T, bool CE> struct GySource {
+    const T *p;        // gy, or the target when CE
+    T g_total;
+    __device__ __forceinline__ T get(int64_t off, T yv) const
+    {
+        if (CE) return (p[off] * g_total) / yv;
+        return p[off];
+    }
+};
+
+template <typename T, bool CE>
+__global__ __launch_bounds__(kBlock) void softmax_bwd_lines_kernel(const T *y, const T *gy_or_target, T *gx,
+                                                                    int64_t lines, int64_t R, int64_t inner,
+                                                                    const T *gout, T neg_n)
+{
+    const int64_t line = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (line >= lines) return;
+    GySource<T, CE> src;
+    src.p = gy_or_target;
+    src.g_total = CE ? (gout ? *gout : (T)1) / neg_n : (T)0;
+    int64_t q = line, c = 0;
+    if (inner != 1) {
+        q = line / inner;
+        c = line - q * inner;
+    }
+    const int64_t base = q * R * inner + c;
+    T sum = (T)0;
+    for (int64_t r = 0; r < R; r++) {
+        const int64_t off = base + r * inner;
+        const T yv = y[off];
+        const T t = yv * src.get(off, yv);
+        gx[off] = t;
+        sum = sum + t;
+    }
+    for (int64_t r = 0; r < R; r++) {
+        const int64_t off = base + r * inner;
+        gx[off] = gx[off] - y[off] * sum;
+    }
+}
+
+template <typename T, bool CE>
+__global__ __launch_bounds__(kBlock) void softmax_bwd_rows_kernel(const T *y, const T *gy_or_target, T *gx,
+                                                                   int64_t R, const T *gout, T neg_n)
+{
+    __shared__ T lds[kWaves];
+    GySource<T, CE> src;
+    src.p = gy_or_target;
+    src.g_total = CE ? (gout ? *gout : (T)1) / neg_n : (T)0;
+    const int64_t base = (int64_t)blockIdx.x * R;
+    T sum = (T)0;
+    for (int64_t r = threadIdx.x; r < R; r += kBlock) {
+        const T yv = y[base + r];
+        const T t = yv * src.get(base + r, yv);
+        gx[base + r] = t;
+        sum = sum + t;
+    }
+    sum = block_red<T, false>(sum, lds);
+    for (int64_t r = threadIdx.x; r < R; r += kBlock) gx[base + r] = gx[base + r] - y[base + r] * sum;
+}
+
+// ---- bias add + ReLU ----------------------------------------------------------------------------------------
+// pre = z + bias (broadcast over rows), act = pre > 0 ? pre : alpha * pre  (relu.rs:44-48)
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void bias_relu_kernel(const T *z, const T *bias, T *pre, T *act,
+                                                            int64_t rows, int64_t packs_per_row, T alpha)
+{
+    const int64_t total = rows * packs_per_row;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
+        const int64_t row = i / packs_per_row;
+        const int64_t col = (i - row * packs_per_row) * VEC;
+        const int64_t off = i * VEC;
+        const Pack<T, VEC> v = load_pack<T, VEC, false>(z + off);
+        const Pack<T, VEC> b = load_pack<T, VEC, false>(bias + col);
+        Pack<T, VEC> a, h;
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            a.v[j] = v.v[j] + b.v[j];
+            h.v[j] = a.v[j] > (T)0 ? a.v[j] : alpha * a.v[j];
+        }
+        if (pre) store_pack<T, VEC, false>(pre + off, a);
+        store_pack<T, VEC, false>(act + off, h);
+    }
+}
+
+// ---- host side ------------------------------------------------------------------------------------------------
+
+// a tensor as a contiguous device buffer: itself, or a temporary copy
+template <typename T> struct ContigIn {
+    Workspace ws;
+    const T *ptr;
+    int status;
+    ContigIn(const zenu_tensor_t &t, int dtype, hipStream_t s)
+        : ws(is_default_stride_strict(t) ? 0 : (size_t)num_elm(t) * sizeof(T), s),
+          ptr(static_cast<const T *>(t.ptr)), status(ws.status)
+    {
+        if (is_default_stride_strict(t) || status) return;
+        zenu_tensor_t tmp = default_view(ws.ptr, t.ndim, t.shape);
+        status = zenu_hip_copy(dtype, &tmp, &t, reinterpret_cast<zenu_stream_t>(s));
+        ptr = static_cast<const T *>(ws.ptr);
+    }
+};
+
+// a contiguous buffer to write into: the tensor itself, or a temporary that finish() copies out
+template <typename T> struct ContigOut {
+    Workspace ws;
+    const zenu_tensor_t &t;
+    T *ptr;
+    int status;
+    int dtype;
+    bool temp;
+    ContigOut(const zenu_tensor_t &t_, int dtype_, hipStream_t s)
+        : ws(is_default_stride_strict(t_) ? 0 : (size_t)num_elm(t_) * sizeof(T), s), t(t_),
+          ptr(static_cast<T *>(t_.ptr)), status(ws.status), dtype(dtype_), temp(!is_default_stride_strict(t_))
+    {
+        if (temp && !status) ptr = static_cast<T *>(ws.ptr);
+    }
+    int finish()
+    {
+        if (!temp) return ZENU_OK;
+        zenu_tensor_t tmp = default_view(ws.ptr, t.ndim, t.shape);
+        return zenu_hip_copy(dtype, &t, &tmp, reinterpret_cast<zenu_stream_t>(ws.stream));
+    }
+};
+
+struct Geometry { int64_t outer, R, inner; };
+
+Geometry geometry(const zenu_tensor_t &t, int axis)
+{
+    Geometry g = {1, t.shape[axis], 1};
+    for (int i = 0; i < axis; i++) g.outer *= t.shape[i];
+    for (int i = axis + 1; i < t.ndim; i++) g.inner *= t.shape[i];
+    return g;
+}
+
+inline bool grid_ok(int64_t blocks) { return blocks > 0 && blocks <= 0x7fffffffLL; }
+
+template <typename T, bool CE>
+int softmax_forward_launch(const T *x, T *y, Geometry g, const T *target, T *rowloss, hipStream_t s)
+{
+    constexpr int VEC = VecOf<T>::N;
+    const int64_t lines = g.outer * g.inner;
+    if (g.inner != 1 || g.R <= kLineMaxR) {
+        const int64_t blocks = (lines + kBlock - 1) / kBlock;
+        if (!grid_ok(blocks)) return ZENU_ERR_UNSUPPORTED;
+        softmax_lines_kernel<T, CE><<<(unsigned)blocks, kBlock, 0, s>>>(x, y, lines, g.R, g.inner, target, rowloss);
+    } else {
+        if (!grid_ok(lines)) return ZENU_ERR_UNSUPPORTED;
+        const bool vec = g.R % VEC == 0 && aligned16(x) && aligned16(y) && (!CE || aligned16(target));
+        const bool reg = g.R <= (int64_t)kRegPacks * kBlock * (vec ? VEC : 1);
+        const unsigned grid = (unsigned)lines;
+        if (vec && reg)       softmax_rows_kernel<T, VEC, CE, true><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
+        else if (vec)         softmax_rows_kernel<T, VEC, CE, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
+        else if (reg)         softmax_rows_kernel<T, 1, CE, true><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
+        else                  softmax_rows_kernel<T, 1, CE, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
+    }
+    ZENU_LAUNCH_CHECK();
+    return ZENU_OK;
+}
+
+template <typename T, bool CE>
+int softmax_backward_launch(const T *y, const T *gy_or_target, T *gx, Geometry g, const T *gout, T neg_n,
+                            hipStream_t s)
+{
+    const int64_t lines = g.outer * g.inner;
+    if (g.inner != 1 || g.R <= kLineMaxR) {
+        const int64_t blocks = (lines + kBlock - 1) / kBlock;
+        if (!grid_ok(blocks)) return ZENU_ERR_UNSUPPORTED;
+        softmax_bwd_lines_kernel<T, CE><<<(unsigned)blocks, kBlock, 0, s>>>(y, gy_or_target, gx, lines, g.R, g.inner,
+                                                                             gout, neg_n);
+    } else {
+        if (!grid_ok(lines)) return ZENU_ERR_UNSUPPORTED;
+        softmax_bwd_rows_kernel<T, CE><<<(unsigned)lines, kBlock, 0, s>>>(y, gy_or_target, gx, g.R, gout, neg_n);
+    }
+    ZENU_LAUNCH_CHECK();
+    return ZENU_OK;
+}
+
+template <typename T>
+int softmax_t(int dtype, const zenu_tensor_t &to, const zenu_tensor_t &src, int axis, hipStream_t s)
+{
+    if (num_elm(src) == 0) return ZENU_OK;
+    ContigIn<T> in(src, dtype, s);
+    if (in.status) return in.status;
+    ContigOut<T> out(to, dtype, s);
+    if (out.status) return out.status;
+    int rc = softmax_forward_launch<T, false>(in.ptr, out.ptr, geometry(src, axis), nullptr, nullptr, s);
+    return rc ? rc : out.finish();
+}
+
+template <typename T>
+int softmax_backward_t(int dtype, const zenu_tensor_t &gx, const zenu_tensor_t &y, const zenu_tensor_t &gy,
+                       int axis, hipStream_t s)
+{
+    if (num_elm(y) == 0) return ZENU_OK;
+    ContigIn<T> yin(y, dtype, s);
+    if (yin.status) return yin.status;
+    ContigIn<T> gin(gy, dtype, s);
+    if (gin.status) return gin.status;
+    ContigOut<T> out(gx, dtype, s);
+    if (out.status) return out.status;
+    int rc = softmax_backward_launch<T, false>(yin.ptr, gin.ptr, out.ptr, geometry(y, axis), nullptr, (T)0, s);
+    return rc ? rc : out.finish();
+}
+
+template <typename T>
+int cross_entropy_t(int dtype, const zenu_tensor_t &loss, const zenu_tensor_t &prob, const zenu_tensor_t &pred,
+                    const zenu_tensor_t &ans, hipStream_t s)
+{
+    const int64_t n = pred.shape[0];
+    if (num_elm(pred) == 0) return ZENU_ERR_SHAPE;
+    ContigIn<T> in(pred, dtype, s);
+    if (in.status) return in.status;
+    ContigIn<T> tin(ans, dtype, s);
+    if (tin.status) return tin.status;
+    ContigOut<T> out(prob, dtype, s);
+    if (out.status) return out.status;
+    Workspace rows((size_t)n * sizeof(T), s);
+    if (rows.status) return rows.status;
+    T *rowloss = static_cast<T *>(rows.ptr);
+    int rc = softmax_forward_launch<T, true>(in.ptr, out.ptr, geometry(pred, 1), tin.ptr, rowloss, s);
+    if (rc) return rc;
+    // n = T::from_usize(rows); Variable::from(-n)  (cross_entropy.rs:20-21)
+    const T neg_n = -(T)n;
+    if (n <= 65536) {
+        ce_finalize_kernel<T><<<1, kBlock, 0, s>>>(rowloss, n, static_cast<T *>(loss.ptr), neg_n);
+        ZENU_LAUNCH_CHECK();
+    } else {
+        Workspace tot(sizeof(T), s);
+        if (tot.status) return tot.status;
+        const int64_t shape1[1] = {n};
+        zenu_tensor_t rv = default_view(rowloss, 1, shape1);
+        zenu_tensor_t tv = default_view(tot.ptr, 0, nullptr);
+        rc = zenu_hip_sum_all(dtype, tot.ptr, &rv, reinterpret_cast<zenu_stream_t>(s));
+        if (!rc) rc = zenu_hip_binary_scalar(ZENU_DIV, dtype, &loss, &tv, (double)neg_n, reinterpret_cast<zenu_stream_t>(s));
+        if (rc) return rc;
+    }
+    return out.finish();
+}
+
+template <typename T>
+int cross_entropy_backward_t(int dtype, const zenu_tensor_t &gpred, const zenu_tensor_t &prob,
+                             const zenu_tensor_t &ans, const zenu_tensor_t *gloss, hipStream_t s)
+{
+    if (num_elm(prob) == 0) return ZENU_OK;
+    ContigIn<T> yin(prob, dtype, s);
+    if (yin.status) return yin.status;
+    ContigIn<T> tin(ans, dtype, s);
+    if (tin.status) return tin.status;
+    ContigOut<T> out(gpred, dtype, s);
+    if (out.status) return out.status;
+    const T neg_n = -(T)prob.shape[0];
+    const T *gout = gloss ? static_cast<const T *>(gloss->ptr) : nullptr;
+    int rc = softmax_backward_launch<T, true>(yin.ptr, tin.ptr, out.ptr, geometry(prob, 1), gout, neg_n, s);
+    return rc ? rc : out.finish();
+}
+
+template <typename T>
+int bias_relu_t(int dtype, const zenu_tensor_t *pre, const zenu_tensor_t &act, const zenu_tensor_t &z,
+                const zenu_tensor_t &bias, double alpha, hipStream_t s)
+{
+    constexpr int VEC = VecOf<T>::N;
+    const int64_t n = num_elm(z);
+    if (n == 0) return ZENU_OK;
+    const int64_t F = bias.shape[0];
+    ContigIn<T> zin(z, dtype, s);
+    if (zin.status) return zin.status;
+    ContigIn<T> bin(bias, dtype, s);
+    if (bin.status) return bin.status;
+    ContigOut<T> aout(act, dtype, s);
+    if (aout.status) return aout.status;
+    // `pre` is optional; when absent its ContigOut wraps `act` and is never written or finished
+    ContigOut<T> pout(pre ? *pre : act, dtype, s);
+    if (pre && pout.status) return pout.status;
+    T *pp = pre ? pout.ptr : nullptr;
+    const int64_t rows = n / F;
+    const bool vec = F % VEC == 0 && aligned16(zin.ptr) && aligned16(bin.ptr) && aligned16(aout.ptr) &&
+                     (!pp || aligned16(pp));
+    const int64_t packs = vec ? F / VEC : F;
+    int64_t blocks = (rows * packs + kBlock - 1) / kBlock;
+    const int64_t cap = (int64_t)device_info().num_cus * 16;
+    if (blocks > cap) blocks = cap;
+    if (vec) bias_relu_kernel<T, VEC><<<(unsigned)blocks, kBlock, 0, s>>>(zin.ptr, bin.ptr, pp, aout.ptr, rows, packs, (T)alpha);
+    else     bias_relu_kernel<T, 1><<<(unsigned)blocks, kBlock, 0, s>>>(zin.ptr, bin.ptr, pp, aout.ptr, rows, packs, (T)alpha);
+    ZENU_LAUNCH_CHECK();
+    int rc = aout.finish();
+    if (!rc && pre) rc = pout.finish();
+    return rc;
+}
+
+int check_all(const zenu_tensor_t *const *ts, int n)
+{
+    for (int i = 0; i < n; i++) {
+        if (!ts[i]) return ZENU_ERR_ARG;
+        int rc = validate_tensor(ts[i]);
+        if (rc) return rc;
+    }
+    return ensure_init();
+}
+
+}  // namespace
+}  // namespace zenu
+
+using namespace zenu;
+
+extern "C" {
+
+int zenu_hip_softmax(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *src, int axis, zenu_stream_t stream)
+{
+    const zenu_tensor_t *ts[] = {to, src};
+    int rc = check_all(ts, 2);
+    if (rc) return rc;
+    if (axis < 0 || axis >= src->ndim) return ZENU_ERR_ARG;      // "axis must be less than the number of dimensions"
+    if (!same_shape(*to, *src)) return ZENU_ERR_SHAPE;           // "softmax shape mismatch"
+    if (dtype == ZENU_F32) return softmax_t<float>(dtype, *to, *src, axis, as_stream(stream));
+    if (dtype == ZENU_F64) return softmax_t<double>(dtype, *to, *src, axis, as_stream(stream));
+    return ZENU_ERR_ARG;
+}
+
+int zenu_hip_softmax_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *y, const zenu_tensor_t *gy,
+                              int axis, zenu_stream_t stream)
+{
+    const zenu_tensor_t *ts[] = {gx, y, gy};
+    int rc = check_all(ts, 3);
+    if (rc) return rc;
+    if (axis < 0 || axis >= y->ndim) return ZENU_ERR_ARG;
+    if (!same_shape(*gx, *y) || !same_shape(*gy, *y)) return ZENU_ERR_SHAPE;
+    if (dtype == ZENU_F32) return softmax_backward_t<float>(dtype, *gx, *y, *gy, axis, as_stream(stream));
+    if (dtype == ZENU_F64) return softmax_backward_t<double>(dtype, *gx, *y, *gy, axis, as_stream(stream));
+    return ZENU_ERR_ARG;
+}
+
+int zenu_hip_softmax_cross_entropy(int dtype, const zenu_tensor_t *loss, const zenu_tensor_t *prob,
+                                   const zenu_tensor_t *pred, const zenu_tensor_t *ans, zenu_stream_t stream)
+{
+    const zenu_tensor_t *ts[] = {loss, prob, pred, ans};
+    int rc = check_all(ts, 4);
+    if (rc) return rc;
+    if (pred->ndim != 2 || loss->ndim != 0) return ZENU_ERR_SHAPE;   // softmax(pred, 1), sum_to(.., [])
+    if (!same_shape(*prob, *pred) || !same_shape(*ans, *pred)) return ZENU_ERR_SHAPE;
+    if (dtype == ZENU_F32) return cross_entropy_t<float>(dtype, *loss, *prob, *pred, *ans, as_stream(stream));
+    if (dtype == ZENU_F64) return cross_entropy_t<double>(dtype, *loss, *prob, *pred, *ans, as_stream(stream));
+    return ZENU_ERR_ARG;
+}
+
+int zenu_hip_softmax_cross_entropy_backward(int dtype, const zenu_tensor_t *gpred, const zenu_tensor_t *prob,
+                                            const zenu_tensor_t *ans, const zenu_tensor_t *gloss,
+                                            zenu_stream_t stream)
+{
+    const zenu_tensor_t *ts[] = {gpred, prob, ans};
+    int rc = check_all(ts, 3);
+    if (rc) return rc;
+    if (gloss && (validate_tensor(gloss) || gloss->ndim != 0)) return ZENU_ERR_SHAPE;
+    if (prob->ndim != 2) return ZENU_ERR_SHAPE;
+    if (!same_shape(*gpred, *prob) || !same_shape(*ans, *prob)) return ZENU_ERR_SHAPE;
+    if (dtype == ZENU_F32) return cross_entropy_backward_t<float>(dtype, *gpred, *prob, *ans, gloss, as_stream(stream));
+    if (dtype == ZENU_F64) return cross_entropy_backward_t<double>(dtype, *gpred, *prob, *ans, gloss, as_stream(stream));
+    return ZENU_ERR_ARG;
+}
+
+int zenu_hip_bias_add_relu(int dtype, const zenu_tensor_t *pre, const zenu_tensor_t *act, const zenu_tensor_t *z,
+                           const zenu_tensor_t *bias, double alpha, zenu_stream_t stream)
+{
+    const zenu_tensor_t *ts[] = {act, z, bias};
+    int rc = check_all(ts, 3);
+    if (rc) return rc;
+    if (pre && validate_tensor(pre)) return ZENU_ERR_ARG;
+    if (z->ndim < 1 || bias->ndim != 1 || bias->shape[0] != z->shape[z->ndim - 1]) return ZENU_ERR_SHAPE;
+    if (!same_shape(*act, *z) || (pre && !same_shape(*pre, *z))) return ZENU_ERR_SHAPE;
+    if (dtype == ZENU_F32) return bias_relu_t<float>(dtype, pre, *act, *z, *bias, alpha, as_stream(stream));
+    if (dtype == ZENU_F64) return bias_relu_t<double>(dtype, pre, *act, *z, *bias, alpha, as_stream(stream));
+    return ZENU_ERR_ARG;
+}
+
+}  // extern "C"

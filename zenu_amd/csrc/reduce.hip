@@ -724,22 +724,6 @@ namespace {
 
 // ---- tensor-level wrappers ------------------------------------------------------------------------------------
 
-zenu_tensor_t default_view(void *ptr, int ndim, const int64_t *shape)
-{
-    zenu_tensor_t t;
-    t.ptr = ptr;
-    t.ndim = ndim;
-    t.reserved = 0;
-    int64_t s = 1;
-    for (int i = 0; i < kMaxDim; i++) { t.shape[i] = 0; t.stride[i] = 0; }
-    for (int i = ndim - 1; i >= 0; i--) {
-        t.shape[i] = shape[i];
-        t.stride[i] = s;
-        s *= shape[i];
-    }
-    return t;
-}
-
 // out must hold src's shape minus `axis`, or with that axis kept as 1 (keep_dim)
 bool reduced_shape_ok(const zenu_tensor_t &out, const zenu_tensor_t &src, int axis)
 {

@@ -39,6 +39,22 @@ bool is_default_stride_strict(const zenu_tensor_t &t)
     return true;
 }
 
+zenu_tensor_t default_view(void *ptr, int ndim, const int64_t *shape)
+{
+    zenu_tensor_t t;
+    t.ptr = ptr;
+    t.ndim = ndim;
+    t.reserved = 0;
+    int64_t s = 1;
+    for (int i = 0; i < kMaxDim; i++) { t.shape[i] = 0; t.stride[i] = 0; }
+    for (int i = ndim - 1; i >= 0; i--) {
+        t.shape[i] = shape[i];
+        t.stride[i] = s;
+        s *= shape[i];
+    }
+    return t;
+}
+
 // DimDyn::is_include, dim_dyn.rs:119-130: trailing dims equal.
 static bool dims_include(const zenu_tensor_t &s, const zenu_tensor_t &o)
 {

@@ -65,6 +65,42 @@ template <typename T> void un_assign(int fn, T *a, int n, int s)
     (void)zenu_hip_unary_assign(fn, dtype_of<T>(), &ta, nullptr);
 }
 
+zenu_tensor_t view3d(const void *p, int64_t d0, int64_t d1, int64_t d2, int64_t s0, int64_t s1, int64_t s2)
+{
+    zenu_tensor_t t = view1d(p, 0, 0);
+    t.ndim = 3;
+    t.shape[0] = d0; t.shape[1] = d1; t.shape[2] = d2;
+    t.stride[0] = s0; t.stride[1] = s1; t.stride[2] = s2;
+    return t;
+}
+
+// output[i] = input[i] + bias[(i / channel_stride) % bias_size] (array_array.cu:49-57) as broadcast
+// adds: whole [C, channel_stride] images, then the channels and the partial channel left over
+template <typename T>
+void conv_bias(const T *in, T *out, int cs, const T *bias, int C, int total)
+{
+    if (cs <= 0 || C <= 0 || total <= 0) return;
+    const int64_t image = (int64_t)C * cs;
+    const int64_t images = total / image;
+    if (images > 0) {
+        zenu_tensor_t ti = view3d(in, images, C, cs, image, cs, 1), to = view3d(out, images, C, cs, image, cs, 1);
+        zenu_tensor_t tb = view3d(bias, 1, C, 1, C, 1, 1);
+        (void)zenu_hip_binary(ZENU_ADD, dtype_of<T>(), &to, &ti, &tb, nullptr);
+    }
+    int64_t done = images * image;
+    const int64_t chans = (total - done) / cs;
+    if (chans > 0) {
+        zenu_tensor_t ti = view3d(in + done, 1, chans, cs, image, cs, 1), to = view3d(out + done, 1, chans, cs, image, cs, 1);
+        zenu_tensor_t tb = view3d(bias, 1, chans, 1, C, 1, 1);
+        (void)zenu_hip_binary(ZENU_ADD, dtype_of<T>(), &to, &ti, &tb, nullptr);
+        done += chans * cs;
+    }
+    if (done < total) {
+        zenu_tensor_t ti = view1d(in + done, (int)(total - done), 1), to = view1d(out + done, (int)(total - done), 1);
+        (void)zenu_hip_binary_scalar_ptr(ZENU_ADD, dtype_of<T>(), &to, &ti, bias + chans, nullptr);
+    }
+}
+
 template <typename T> void max_idx(T *a, int size, int stride, int *out)
 {
     // `out` is host memory (zenu-cuda/src/kernel/mod.rs:570-588): blocking, like the reference
@@ -117,6 +153,30 @@ extern "C" {
     void array_tanh_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_TANH, a, n, s); }                   \
     void array_sqrt_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_SQRT, a, n, s); }                   \
     void array_abs_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_ABS, a, n, s); }                     \
+    void array_clip_##S(T *in, T *out, int n, int si, int so, T lo, T hi)                                  \
+    {                                                                                                      \
+        zenu_tensor_t ti = view1d(in, n, si), to = view1d(out, n, so);                                     \
+        (void)zenu_hip_clip(dtype_of<T>(), &to, &ti, (double)lo, (double)hi, nullptr);                     \
+    }                                                                                                      \
+    void array_clip_assign_##S(T *a, int n, int s, T lo, T hi)                                             \
+    {                                                                                                      \
+        zenu_tensor_t t = view1d(a, n, s);                                                                 \
+        (void)zenu_hip_clip(dtype_of<T>(), &t, &t, (double)lo, (double)hi, nullptr);                       \
+    }                                                                                                      \
+    void array_clip_backward_##S(T *in, T *mask, T hi, T lo, int n, int si, int sm)                        \
+    {                                                                                                      \
+        zenu_tensor_t ti = view1d(in, n, si), tm = view1d(mask, n, sm);                                    \
+        (void)zenu_hip_clip_backward_mask(dtype_of<T>(), &tm, &ti, (double)lo, (double)hi, nullptr);       \
+    }                                                                                                      \
+    void array_clip_backward_assign_##S(T *a, T hi, T lo, int n, int s)                                    \
+    {                                                                                                      \
+        zenu_tensor_t t = view1d(a, n, s);                                                                 \
+        (void)zenu_hip_clip_backward_mask(dtype_of<T>(), &t, &t, (double)lo, (double)hi, nullptr);         \
+    }                                                                                                      \
+    void conv_bias_add_##S(const T *in, T *out, int channel_stride, const T *bias, int bias_size, int total) \
+    {                                                                                                      \
+        conv_bias<T>(in, out, channel_stride, bias, bias_size, total);                                     \
+    }                                                                                                      \
     void relu_##S(T *in, T *out, T alpha, int n, int si, int so)                                           \
     {                                                                                                      \
         zenu_tensor_t ti = view1d(in, n, si), to = view1d(out, n, so);                                     \

@@ -322,6 +322,46 @@ class Matrix:
                                                      C.byref(other.desc()), float(alpha), _stream),
               "relu_backward_mask")
 
+    def relu_backward(self, gy, x, alpha):
+        """self = gy * relu_backward_mask(x): zenu-autograd/src/activation/relu.rs:35-44 in one pass"""
+        check(_lib.lib().zenu_hip_relu_backward(_dt(self.dtype), C.byref(self.desc()), C.byref(gy.desc()),
+                                                C.byref(x.desc()), float(alpha), _stream), "relu_backward")
+
+    # ---- clip (zenu-matrix/src/operation/clip.rs:289-318) -----------------------------------
+    def clip(self, lo, hi):
+        out = self.alloc_like()
+        check(_lib.lib().zenu_hip_clip(_dt(self.dtype), C.byref(out.desc()), C.byref(self.desc()),
+                                       float(lo), float(hi), _stream), "clip")
+        return out
+
+    def clip_assign(self, lo, hi):
+        check(_lib.lib().zenu_hip_clip(_dt(self.dtype), C.byref(self.desc()), C.byref(self.desc()),
+                                       float(lo), float(hi), _stream), "clip_assign")
+
+    def clip_backward_mask(self, lo, hi):
+        out = self.alloc_like()
+        check(_lib.lib().zenu_hip_clip_backward_mask(_dt(self.dtype), C.byref(out.desc()), C.byref(self.desc()),
+                                                     float(lo), float(hi), _stream), "clip_backward_mask")
+        return out
+
+    def clip_backward_assign_mask(self, lo, hi):
+        check(_lib.lib().zenu_hip_clip_backward_mask(_dt(self.dtype), C.byref(self.desc()), C.byref(self.desc()),
+                                                     float(lo), float(hi), _stream), "clip_backward_assign_mask")
+
+    # ---- fused chains -----------------------------------------------------------------------
+    def softmax_assign(self, source, axis):
+        """softmax.rs:10-25, one launch"""
+        if not (0 <= axis < self.ndim):
+            raise ZenuHipError(_lib.ERR_AXIS, "softmax_assign", "axis must be less than the number of dimensions")
+        check(_lib.lib().zenu_hip_softmax(_dt(self.dtype), C.byref(self.desc()), C.byref(source.desc()),
+                                          axis, _stream), "softmax_assign")
+
+    def bias_add_relu(self, z, bias, alpha, pre=None):
+        """self = relu(z + bias, alpha); pre (optional) receives z + bias"""
+        check(_lib.lib().zenu_hip_bias_add_relu(_dt(self.dtype), C.byref(pre.desc()) if pre is not None else None,
+                                                C.byref(self.desc()), C.byref(z.desc()), C.byref(bias.desc()),
+                                                float(alpha), _stream), "bias_add_relu")
+
     # ---- reductions ---------------------------------------------------------------------
     def sum(self, axis, keep_dim=False):
         """sum.rs:9-32"""
@@ -437,6 +477,33 @@ def larger_shape(x, y):
     if is_include_broadcast(y, x):
         return y
     raise ZenuHipError(_lib.ERR_SHAPE, "larger_shape", "This is bug please make issue")
+
+
+def softmax_backward(y, gy, axis):
+    """gx = y*gy - y*sum(y*gy, axis) (zenu-autograd/src/loss/softmax.rs:33-40), one launch"""
+    gx = y.alloc_like()
+    check(_lib.lib().zenu_hip_softmax_backward(_dt(y.dtype), C.byref(gx.desc()), C.byref(y.desc()),
+                                               C.byref(gy.desc()), axis, _stream), "softmax_backward")
+    return gx
+
+
+def cross_entropy(pred, ans):
+    """(loss, prob) of zenu-autograd/src/loss/cross_entropy.rs:12-23 for pred, ans [N, C]"""
+    loss = Matrix.alloc((), pred.dtype)
+    prob = pred.alloc_like()
+    check(_lib.lib().zenu_hip_softmax_cross_entropy(_dt(pred.dtype), C.byref(loss.desc()), C.byref(prob.desc()),
+                                                    C.byref(pred.desc()), C.byref(ans.desc()), _stream),
+          "cross_entropy")
+    return loss, prob
+
+
+def cross_entropy_backward(prob, ans, gloss=None):
+    """d loss / d pred from the softmax output kept by cross_entropy()"""
+    gpred = prob.alloc_like()
+    check(_lib.lib().zenu_hip_softmax_cross_entropy_backward(
+        _dt(prob.dtype), C.byref(gpred.desc()), C.byref(prob.desc()), C.byref(ans.desc()),
+        C.byref(gloss.desc()) if gloss is not None else None, _stream), "cross_entropy_backward")
+    return gpred
 
 
 def sum_to(source, target):
