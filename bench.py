@@ -15,7 +15,7 @@ oracle (a single-threaded restatement of ZeNu's CPU path, reference-shaped: one 
 row / slice, whole-array passes with temporaries for Adam) timed on this box's host cores on
 one pass of the same step.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload suite|c0|c1|c2|c3]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload suite|c0|c1|c2|c3|c4|fused]
 """
 import argparse
 import ctypes as C
@@ -212,6 +212,49 @@ def build_ops(z, workload, stream):
         op.keep = sets
         ops.append(op)
 
+    # ---- not a BASELINE config: the fused entry points at configs[2]'s size, seed 5 ---------------------
+    def add_fused():
+        r = np.random.default_rng(5)
+        shape = (8192, 4096)
+        x = r.standard_normal(shape).astype(np.float32)
+        t = np.zeros(shape, dtype=np.float32)
+        t[np.arange(shape[0]), r.integers(0, shape[1], shape[0])] = 1
+        bias = r.standard_normal(shape[1]).astype(np.float32)
+        n = x.size
+        sets = [(M.from_numpy(x), M.from_numpy(t), M.alloc(shape), M.alloc(shape), M.from_numpy(bias), M.alloc([]))
+                for _ in range(nsets(4 * 4 * n))]
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        import cpu_matrix
+        cx, ct, cb = (cpu_matrix.CpuMatrix.from_numpy(v) for v in (x, t, bias))
+        co = cpu_matrix.CpuMatrix.zeros(shape)
+
+        def mk(fn):
+            return [fn(X.desc(), T.desc(), O.desc(), P.desc(), B.desc(), L.desc()) for X, T, O, P, B, L in sets]
+        ops.append(Op("softmax rows", "fused", "f32", 2 * 4 * n, n,
+                      mk(lambda dx, dt, do, dp, db, dl: (lambda: check(l.zenu_hip_softmax(_lib.F32, ref(do), ref(dx), 1, stream), "softmax"))),
+                      lambda: co.softmax_assign(cx, 1)))
+        ops.append(Op("softmax backward", "fused", "f32", 3 * 4 * n, n,
+                      mk(lambda dx, dt, do, dp, db, dl: (lambda: check(l.zenu_hip_softmax_backward(_lib.F32, ref(do), ref(dp), ref(dx), 1, stream), "softmax_bwd"))),
+                      lambda: cpu_matrix.softmax_backward(co, cx, 1)))
+        ops.append(Op("softmax cross-entropy", "fused", "f32", 3 * 4 * n, n,
+                      mk(lambda dx, dt, do, dp, db, dl: (lambda: check(l.zenu_hip_softmax_cross_entropy(_lib.F32, ref(dl), ref(dp), ref(dx), ref(dt), stream), "ce"))),
+                      lambda: cpu_matrix.cross_entropy(cx, ct)))
+        ops.append(Op("cross-entropy backward", "fused", "f32", 3 * 4 * n, n,
+                      mk(lambda dx, dt, do, dp, db, dl: (lambda: check(l.zenu_hip_softmax_cross_entropy_backward(_lib.F32, ref(do), ref(dp), ref(dt), None, stream), "ce_bwd"))),
+                      lambda: cpu_matrix.cross_entropy_backward(co, ct)))
+        ops.append(Op("bias add + relu (2 outputs)", "fused", "f32", 3 * 4 * n + 4 * shape[1], n,
+                      mk(lambda dx, dt, do, dp, db, dl: (lambda: check(l.zenu_hip_bias_add_relu(_lib.F32, ref(dp), ref(do), ref(dx), ref(db), 0.0, stream), "bias_relu"))),
+                      lambda: co.bias_add_relu(cx, cb, 0.0, pre=co)))
+        ops.append(Op("relu backward", "fused", "f32", 3 * 4 * n, n,
+                      mk(lambda dx, dt, do, dp, db, dl: (lambda: check(l.zenu_hip_relu_backward(_lib.F32, ref(do), ref(dt), ref(dx), 0.0, stream), "relu_bwd"))),
+                      lambda: co.relu_backward(ct, cx, 0.0)))
+        ops.append(Op("clip", "fused", "f32", 2 * 4 * n, n,
+                      mk(lambda dx, dt, do, dp, db, dl: (lambda: check(l.zenu_hip_clip(_lib.F32, ref(do), ref(dx), -1.0, 1.0, stream), "clip"))),
+                      lambda: cx.clip(-1.0, 1.0)))
+        ops[-1].keep = sets
+
+    if workload == "fused":
+        add_fused()
     if want("c0"):
         add_c0()
     if want("c1"):
@@ -364,7 +407,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="suite", choices=["suite", "c0", "c1", "c2", "c3", "c4"])
+    ap.add_argument("--workload", default="suite", choices=["suite", "c0", "c1", "c2", "c3", "c4", "fused"])
     ap.add_argument("--op-reps", type=int, default=40, help="launches per op in the per-op timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--profile-op", default=None, help="only launch this op (for rocprofv3 counter runs)")
@@ -470,7 +513,8 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32" if args.workload != "suite" and args.workload != "c2" else "f32+f64", "data": "synthetic",
         "config": {"workload": {"suite": "configs[0..3]: every op once per step", "c0": "configs[0]", "c1": "configs[1]",
-                                "c2": "configs[2]", "c3": "configs[3]"}[args.workload],
+                                "c2": "configs[2]", "c3": "configs[3]",
+                                "fused": "fused entry points on [8192,4096] f32 (not a BASELINE config)"}[args.workload],
                    "ops_per_step": len(ops), "algorithmic_bytes_per_step": step_bytes},
         "frac_of_peak_whole_step": round(value / PEAK_HBM_GBPS, 4),
         "adam_step_params_per_sec": (round(adam[0]["Gelem_per_s"] * 1e9) if adam else None),

@@ -88,7 +88,7 @@ __global__ __launch_bounds__(kBlock) void softmax_lines_kernel(const T *x, T *y,
     if (CE) rowloss[line] = acc;
 }
 
-template <typename T, int VEC, bool CE, bool REG>
+template <typename T, int VEC, bool CE, bool REG, bool NT>
 __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, int64_t R, const T *target,
                                                                T *rowloss)
 {
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
 #pragma unroll
         for (int k = 0; k < kRegPacks; k++) {
             const int64_t r = first + k * step;
-            v[k] = r < R ? load_pack<T, VEC, false>(xr + r) : splat<T, VEC>(-INFINITY);
+            v[k] = r < R ? load_pack<T, VEC, NT>(xr + r) : splat<T, VEC>(-INFINITY);
 #pragma unroll
             for (int j = 0; j < VEC; j++) m = combine<T, true>(m, v[k].v[j]);
         }
@@ -131,14 +131,14 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
             const int64_t r = first + k * step;
             if (r < R) {
                 Pack<T, VEC> t;
-                if (CE) t = load_pack<T, VEC, false>(tr + r);
+                if (CE) t = load_pack<T, VEC, NT>(tr + r);
 #pragma unroll
                 for (int j = 0; j < VEC; j++) {
                     const T s = v[k].v[j] / sum;
                     v[k].v[j] = s;
                     if (CE) acc = acc + t.v[j] * log(s);
                 }
-                store_pack<T, VEC, false>(yr + r, v[k]);
+                store_pack<T, VEC, NT && !CE>(yr + r, v[k]);   // the CE output is read again by the backward pass
             }
         }
     } else {     // long rows: three passes; the second and third find the row in cache
@@ -235,24 +235,67 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_lines_kernel(const T *y, c
     }
 }
 
-template <typename T, bool CE>
+template <typename T, int VEC, bool CE, bool REG, bool NT>
 __global__ __launch_bounds__(kBlock) void softmax_bwd_rows_kernel(const T *y, const T *gy_or_target, T *gx,
                                                                    int64_t R, const T *gout, T neg_n)
 {
     __shared__ T lds[kWaves];
-    GySource<T, CE> src;
-    src.p = gy_or_target;
-    src.g_total = CE ? (gout ? *gout : (T)1) / neg_n : (T)0;
+    const T g_total = CE ? (gout ? *gout : (T)1) / neg_n : (T)0;
     const int64_t base = (int64_t)blockIdx.x * R;
+    const T *yr = y + base;
+    const T *sr = gy_or_target + base;
+    T *gr = gx + base;
+    const int64_t first = (int64_t)threadIdx.x * VEC;
+    constexpr int64_t step = (int64_t)kBlock * VEC;
     T sum = (T)0;
-    for (int64_t r = threadIdx.x; r < R; r += kBlock) {
-        const T yv = y[base + r];
-        const T t = yv * src.get(base + r, yv);
-        gx[base + r] = t;
-        sum = sum + t;
+    if (REG) {   // the row of y and of t = y * gy stays in registers: two reads, one write
+        Pack<T, VEC> yv[kRegPacks], t[kRegPacks];
+#pragma unroll
+        for (int k = 0; k < kRegPacks; k++) {
+            const int64_t r = first + k * step;
+            if (r < R) {
+                yv[k] = load_pack<T, VEC, NT && !CE>(yr + r);
+                const Pack<T, VEC> g = load_pack<T, VEC, NT>(sr + r);
+#pragma unroll
+                for (int j = 0; j < VEC; j++) {
+                    const T gyv = CE ? (g.v[j] * g_total) / yv[k].v[j] : g.v[j];
+                    t[k].v[j] = yv[k].v[j] * gyv;
+                    sum = sum + t[k].v[j];
+                }
+            }
+        }
+        sum = block_red<T, false>(sum, lds);
+#pragma unroll
+        for (int k = 0; k < kRegPacks; k++) {
+            const int64_t r = first + k * step;
+            if (r < R) {
+#pragma unroll
+                for (int j = 0; j < VEC; j++) t[k].v[j] = t[k].v[j] - yv[k].v[j] * sum;
+                store_pack<T, VEC, NT>(gr + r, t[k]);
+            }
+        }
+    } else {     // long rows: t goes to gx first; the second pass finds both rows in cache
+        for (int64_t r = first; r < R; r += step) {
+            const Pack<T, VEC> yv = load_pack<T, VEC, false>(yr + r);
+            const Pack<T, VEC> g = load_pack<T, VEC, false>(sr + r);
+            Pack<T, VEC> t;
+#pragma unroll
+            for (int j = 0; j < VEC; j++) {
+                const T gyv = CE ? (g.v[j] * g_total) / yv.v[j] : g.v[j];
+                t.v[j] = yv.v[j] * gyv;
+                sum = sum + t.v[j];
+            }
+            store_pack<T, VEC, false>(gr + r, t);
+        }
+        sum = block_red<T, false>(sum, lds);
+        for (int64_t r = first; r < R; r += step) {
+            const Pack<T, VEC> yv = load_pack<T, VEC, false>(yr + r);
+            Pack<T, VEC> t = load_pack<T, VEC, false>(gr + r);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) t.v[j] = t.v[j] - yv.v[j] * sum;
+            store_pack<T, VEC, false>(gr + r, t);
+        }
     }
-    sum = block_red<T, false>(sum, lds);
-    for (int64_t r = threadIdx.x; r < R; r += kBlock) gx[base + r] = gx[base + r] - y[base + r] * sum;
 }
 
 // ---- bias add + ReLU ----------------------------------------------------------------------------------------
@@ -269,6 +312,49 @@ __global__ __launch_bounds__(kBlock) void bias_relu_kernel(const T *z, const T *
         const int64_t off = i * VEC;
         const Pack<T, VEC> v = load_pack<T, VEC, false>(z + off);
         const Pack<T, VEC> b = load_pack<T, VEC, false>(bias + col);
+        Pack<T, VEC> a, h;
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            a.v[j] = v.v[j] + b.v[j];
+            h.v[j] = a.v[j] > (T)0 ? a.v[j] : alpha * a.v[j];
+        }
+        if (pre) store_pack<T, VEC, false>(pre + off, a);
+        store_pack<T, VEC, false>(act + off, h);
+    }
+}
+
+// Wide rows: a thread owns one vector of columns (its bias stays in registers) and walks down the
+// rows, so there is no index division; grid = (column tiles, row groups).
+template <typename T, int VEC, bool NT>
+__global__ __launch_bounds__(kBlock) void bias_relu_cols_kernel(const T *z, const T *bias, T *pre, T *act,
+                                                                 int64_t rows, int64_t F, T alpha)
+{
+    const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * VEC;
+    if (col >= F) return;
+    const Pack<T, VEC> b = load_pack<T, VEC, false>(bias + col);
+    constexpr int U = 4;
+    const int64_t rstep = gridDim.y;
+    int64_t r = blockIdx.y;
+    for (; r + (U - 1) * rstep < rows; r += U * rstep) {
+        Pack<T, VEC> v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) v[u] = load_pack<T, VEC, NT>(z + (r + u * rstep) * F + col);
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            Pack<T, VEC> a, h;
+#pragma unroll
+            for (int j = 0; j < VEC; j++) {
+                a.v[j] = v[u].v[j] + b.v[j];
+                h.v[j] = a.v[j] > (T)0 ? a.v[j] : alpha * a.v[j];
+            }
+            const int64_t off = (r + u * rstep) * F + col;
+            if (pre) store_pack<T, VEC, NT>(pre + off, a);
+            store_pack<T, VEC, NT>(act + off, h);
+        }
+    }
+    for (; r < rows; r += rstep) {
+        const int64_t off = r * F + col;
+        const Pack<T, VEC> v = load_pack<T, VEC, false>(z + off);
         Pack<T, VEC> a, h;
 #pragma unroll
         for (int j = 0; j < VEC; j++) {
@@ -346,10 +432,12 @@ int softmax_forward_launch(const T *x, T *y, Geometry g, const T *target, T *row
         const bool vec = g.R % VEC == 0 && aligned16(x) && aligned16(y) && (!CE || aligned16(target));
         const bool reg = g.R <= (int64_t)kRegPacks * kBlock * (vec ? VEC : 1);
         const unsigned grid = (unsigned)lines;
-        if (vec && reg)       softmax_rows_kernel<T, VEC, CE, true><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
-        else if (vec)         softmax_rows_kernel<T, VEC, CE, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
-        else if (reg)         softmax_rows_kernel<T, 1, CE, true><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
-        else                  softmax_rows_kernel<T, 1, CE, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
+        const bool nt = vec && reg && lines * g.R * (int64_t)sizeof(T) * 2 >= kStreamBytes;
+        if (nt)               softmax_rows_kernel<T, VEC, CE, true, true><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
+        else if (vec && reg)  softmax_rows_kernel<T, VEC, CE, true, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
+        else if (vec)         softmax_rows_kernel<T, VEC, CE, false, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
+        else if (reg)         softmax_rows_kernel<T, 1, CE, true, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
+        else                  softmax_rows_kernel<T, 1, CE, false, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
     }
     ZENU_LAUNCH_CHECK();
     return ZENU_OK;
@@ -367,7 +455,16 @@ int softmax_backward_launch(const T *y, const T *gy_or_target, T *gx, Geometry g
                                                                              gout, neg_n);
     } else {
         if (!grid_ok(lines)) return ZENU_ERR_UNSUPPORTED;
-        softmax_bwd_rows_kernel<T, CE><<<(unsigned)lines, kBlock, 0, s>>>(y, gy_or_target, gx, g.R, gout, neg_n);
+        constexpr int VEC = VecOf<T>::N;
+        const bool vec = g.R % VEC == 0 && aligned16(y) && aligned16(gy_or_target) && aligned16(gx);
+        const bool reg = g.R <= (int64_t)kRegPacks * kBlock * (vec ? VEC : 1);
+        const bool nt = vec && reg && lines * g.R * (int64_t)sizeof(T) * 3 >= kStreamBytes;
+        const unsigned grid = (unsigned)lines;
+        if (nt)              softmax_bwd_rows_kernel<T, VEC, CE, true, true><<<grid, kBlock, 0, s>>>(y, gy_or_target, gx, g.R, gout, neg_n);
+        else if (vec && reg) softmax_bwd_rows_kernel<T, VEC, CE, true, false><<<grid, kBlock, 0, s>>>(y, gy_or_target, gx, g.R, gout, neg_n);
+        else if (vec)        softmax_bwd_rows_kernel<T, VEC, CE, false, false><<<grid, kBlock, 0, s>>>(y, gy_or_target, gx, g.R, gout, neg_n);
+        else if (reg)        softmax_bwd_rows_kernel<T, 1, CE, true, false><<<grid, kBlock, 0, s>>>(y, gy_or_target, gx, g.R, gout, neg_n);
+        else                 softmax_bwd_rows_kernel<T, 1, CE, false, false><<<grid, kBlock, 0, s>>>(y, gy_or_target, gx, g.R, gout, neg_n);
     }
     ZENU_LAUNCH_CHECK();
     return ZENU_OK;
@@ -474,6 +571,21 @@ int bias_relu_t(int dtype, const zenu_tensor_t *pre, const zenu_tensor_t &act, c
     const bool vec = F % VEC == 0 && aligned16(zin.ptr) && aligned16(bin.ptr) && aligned16(aout.ptr) &&
                      (!pp || aligned16(pp));
     const int64_t packs = vec ? F / VEC : F;
+    if (vec && packs >= 64) {
+        const int64_t gx = (packs + kBlock - 1) / kBlock;
+        int64_t gy = ((int64_t)device_info().num_cus * 8 + gx - 1) / gx;
+        if (gy > rows) gy = rows;
+        if (gy > 65535) gy = 65535;
+        if (gx > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
+        const dim3 grid((unsigned)gx, (unsigned)gy);
+        const bool nt = n * (int64_t)sizeof(T) * (pp ? 3 : 2) >= kStreamBytes;
+        if (nt) bias_relu_cols_kernel<T, VEC, true><<<grid, kBlock, 0, s>>>(zin.ptr, bin.ptr, pp, aout.ptr, rows, F, (T)alpha);
+        else    bias_relu_cols_kernel<T, VEC, false><<<grid, kBlock, 0, s>>>(zin.ptr, bin.ptr, pp, aout.ptr, rows, F, (T)alpha);
+        ZENU_LAUNCH_CHECK();
+        int rc2 = aout.finish();
+        if (!rc2 && pre) rc2 = pout.finish();
+        return rc2;
+    }
     int64_t blocks = (rows * packs + kBlock - 1) / kBlock;
     const int64_t cap = (int64_t)device_info().num_cus * 16;
     if (blocks > cap) blocks = cap;
