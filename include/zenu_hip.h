@@ -179,6 +179,11 @@ int zenu_hip_clip_backward_mask(int dtype, const zenu_tensor_t *mask, const zenu
  * to_default_stride, to_default_stride.rs:7-15). */
 int zenu_hip_copy(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *src, zenu_stream_t stream);
 
+/* to = source repeated over to's leading dims and over source dims of size 1 (broadcast,
+ * zenu-matrix/src/operation/broadcast.rs:11-43): one launch instead of one copy per slice. */
+int zenu_hip_broadcast(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *source,
+                       zenu_stream_t stream);
+
 /* ------------------------------------------------------------------------- */
 /* Reductions (deterministic: fixed tree, no atomics on data)                  */
 /* ------------------------------------------------------------------------- */

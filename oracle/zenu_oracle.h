@@ -103,6 +103,8 @@ int  zo_larger_shape(int nx, const int64_t *x, int ny, const int64_t *y);
     int zo_powf_##S(const zo_view *to, const zo_view *other, T scalar);                           \
     int zo_relu_##S(const zo_view *to, const zo_view *other, T alpha);                            \
     int zo_relu_backward_mask_##S(const zo_view *to, const zo_view *other, T alpha);              \
+    /* zenu-matrix/src/operation/broadcast.rs:11-43 */                                             \
+    int zo_broadcast_##S(const zo_view *to, const zo_view *source);                               \
     /* zenu-matrix/src/operation/clip.rs:39-110, 205-318 */                                        \
     int zo_clip_##S(const zo_view *to, const zo_view *other, T min, T max);                       \
     int zo_clip_backward_mask_##S(const zo_view *mask, const zo_view *other, T min, T max);       \

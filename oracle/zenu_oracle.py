@@ -158,6 +158,11 @@ def copy_from(to, src):
     _chk(getattr(lib(), f"zo_copy_from_{s}")(C.byref(view(to)), C.byref(view(src))), "copy_from")
 
 
+def broadcast(to, source):
+    s, _ = _sfx(to.dtype)
+    _chk(getattr(lib(), f"zo_broadcast_{s}")(C.byref(view(to)), C.byref(view(source))), "broadcast")
+
+
 def sum_axis(src, axis, keep_dim=False):
     s, _ = _sfx(src.dtype)
     if not (0 <= axis < src.ndim):

@@ -76,6 +76,8 @@ class CpuMatrix:
     def copy_from(self, src):
         zo.copy_from(self.a, src.a)
 
+    def broadcast(self, source): zo.broadcast(self.a, source.a)
+
     def to_default_stride(self):
         out = self.alloc_like()
         out.copy_from(self)

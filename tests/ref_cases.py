@@ -513,3 +513,19 @@ def clip_cases(dev):  # zenu-matrix/src/operation/clip.rs:321-372; zenu-cuda/src
         eq(a.clip_backward_mask(1., 2.), [0., 1., 1., 0., 0., 0.])
         a.clip_backward_assign_mask(1., 2.)
         eq(a, [0., 1., 1., 0., 0., 0.])
+
+
+@case
+def broadcast_cases(dev):  # zenu-matrix/src/operation/broadcast.rs:53-165
+    for src, sshape, dshape in (([1.], [], [3]), ([1.], [], [2, 3]), ([1., 2., 3.], [3], [2, 3]),
+                                ([1., 2.], [1, 2], [2, 3, 1, 2]), ([1., 2., 3., 4.], [1, 1, 1, 4], [2, 3, 4, 4])):
+        s = dev.M.from_vec(src, sshape)
+        res = dev.M.zeros(dshape)
+        res.broadcast(s)
+        eq(res, np.broadcast_to(np.asarray(src, dtype=np.float32).reshape(sshape), dshape))
+    bad = False
+    try:
+        dev.M.zeros([2, 3]).broadcast(dev.M.from_vec([1., 2.], [2]))
+    except dev.Error:
+        bad = True
+    assert bad

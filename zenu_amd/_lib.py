@@ -75,6 +75,7 @@ SIGNATURES = {
     "zenu_hip_clip": [_i, _TP, _TP, _d, _d, _vp],
     "zenu_hip_clip_backward_mask": [_i, _TP, _TP, _d, _d, _vp],
     "zenu_hip_copy": [_i, _TP, _TP, _vp],
+    "zenu_hip_broadcast": [_i, _TP, _TP, _vp],
     "zenu_hip_softmax": [_i, _TP, _TP, _i, _vp],
     "zenu_hip_softmax_backward": [_i, _TP, _TP, _TP, _i, _vp],
     "zenu_hip_softmax_cross_entropy": [_i, _TP, _TP, _TP, _TP, _vp],

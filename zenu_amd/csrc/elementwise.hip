@@ -832,6 +832,17 @@ int zenu_hip_relu_backward_mask(int dtype, const zenu_tensor_t *to, const zenu_t
     return ZENU_ERR_ARG;
 }
 
+int zenu_hip_broadcast(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *source, zenu_stream_t stream)
+{
+    int rc = check2(to, source);
+    if (!rc) rc = ensure_init();
+    if (!rc) rc = check_binary_assign(*to, *source);   // is_include || is_include_bradcast, broadcast.rs:13-17
+    if (rc) return rc;
+    if (dtype == ZENU_F32) return run1<float>(*to, *source, CopyF<float>(), as_stream(stream));
+    if (dtype == ZENU_F64) return run1<double>(*to, *source, CopyF<double>(), as_stream(stream));
+    return ZENU_ERR_ARG;
+}
+
 int zenu_hip_relu_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *gy, const zenu_tensor_t *x,
                            double alpha, zenu_stream_t stream)
 {

@@ -224,6 +224,11 @@ class Matrix:
         check(_lib.lib().zenu_hip_copy(_dt(self.dtype), C.byref(self.desc()), C.byref(src.desc()), _stream),
               "copy_from")
 
+    def broadcast(self, source):
+        """broadcast.rs:11-43"""
+        check(_lib.lib().zenu_hip_broadcast(_dt(self.dtype), C.byref(self.desc()), C.byref(source.desc()), _stream),
+              "broadcast")
+
     def to_default_stride(self):
         out = self.alloc_like()
         out.copy_from(self)
