@@ -27,6 +27,8 @@
 #include "vecmem.hpp"
 #include "zmath.hpp"
 
+#include <type_traits>
+
 namespace zenu {
 namespace {
 
@@ -226,7 +228,10 @@ __device__ __forceinline__ void decompose(const OuterDesc &d, int64_t lin, int64
     o0 = o1 = o2 = 0;
     for (int k = d.nouter - 1; k >= 0; k--) {
         int64_t q, r;
-        if (lin < 0x7fffffffLL && d.shape[k] < 0x7fffffffLL) {
+        if (k == 0) {                 // the slowest dim takes what is left: no division
+            q = 0;
+            r = lin;
+        } else if (lin < 0x7fffffffLL && d.shape[k] < 0x7fffffffLL) {
             uint32_t l32 = (uint32_t)lin, s32 = (uint32_t)d.shape[k];
             q = l32 / s32;
             r = l32 - (uint32_t)q * s32;
@@ -256,7 +261,7 @@ struct RowsParams {
 // NTA / NTB: input a / b is streamed once (not broadcast along an outer dim); the output is
 // streamed when either is.  Template parameters, because a run-time choice between a hinted and
 // a plain load is merged by the compiler into one plain load.
-template <typename T, int VEC, bool NTA, bool NTB, typename F>
+template <typename T, int VEC, bool NTA, bool NTB, typename F, int kBlock, int kUnroll>
 __global__ __launch_bounds__(kBlock) void ew_rows_kernel(T *out, const T *a, const T *b,
                                                          RowsParams p, F f)
 {
@@ -265,9 +270,10 @@ __global__ __launch_bounds__(kBlock) void ew_rows_kernel(T *out, const T *a, con
     const int ty_n = kBlock >> p.tx_shift;
     const int tx = threadIdx.x & (tx_n - 1);
     const int ty = threadIdx.x >> p.tx_shift;
-    const int64_t blk = blockIdx.x;
-    const int64_t row_blk = blk / p.col_tiles;
-    const int64_t col_tile = blk - row_blk * p.col_tiles;
+    // grid and col_tiles fit 32 bits (checked at launch)
+    const uint32_t row_blk32 = blockIdx.x / (uint32_t)p.col_tiles;
+    const int64_t row_blk = row_blk32;
+    const int64_t col_tile = blockIdx.x - row_blk32 * (uint32_t)p.col_tiles;
     const int64_t row = row_blk * ty_n + ty;
     if (row >= p.nrows) return;
     int64_t oo, oa, ob;
@@ -546,19 +552,36 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
         }
         const int v = vec ? VEC : 1;
         int64_t vcols = (rp.ncols + v - 1) / v;
-        int shift = 0;
-        while ((1 << shift) < kBlock && ((int64_t)1 << shift) < vcols) shift++;
-        rp.tx_shift = shift;
-        int64_t cols_per_tile = ((int64_t)1 << shift) * v * kUnroll;
-        rp.col_tiles = (rp.ncols + cols_per_tile - 1) / cols_per_tile;
-        int64_t rows_per_blk = kBlock >> shift;
-        int64_t grid = ((rp.nrows + rows_per_blk - 1) / rows_per_blk) * rp.col_tiles;
-        if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-        if (!vec)            ew_rows_kernel<T, 1, false, false, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, rp, f);
-        else if (nta && ntb) ew_rows_kernel<T, VEC, true, true, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, rp, f);
-        else if (nta)        ew_rows_kernel<T, VEC, true, false, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, rp, f);
-        else if (ntb)        ew_rows_kernel<T, VEC, false, true, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, rp, f);
-        else                 ew_rows_kernel<T, VEC, false, false, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, rp, f);
+        // full-size streams of this launch: the output plus every input that is neither a scalar
+        // per row nor re-read for every outer index; two of them take the small workgroup shape
+        int streams = 1;
+        for (int o = 1; o <= nin; o++) {
+            bool full = p.stride[o][last] == 1;
+            for (int d = 0; d < p.ndim - 1; d++)
+                if (p.stride[o][d] == 0 && p.shape[d] > 1) full = false;
+            if (full) streams++;
+        }
+        const bool small = streams <= 2 && !IsValuBound<F>::value;
+        auto launch = [&](auto block_c, auto unroll_c) -> int {
+            constexpr int B = decltype(block_c)::value, U = decltype(unroll_c)::value;
+            int shift = 0;
+            while ((1 << shift) < B && ((int64_t)1 << shift) < vcols) shift++;
+            rp.tx_shift = shift;
+            int64_t cols_per_tile = ((int64_t)1 << shift) * v * U;
+            rp.col_tiles = (rp.ncols + cols_per_tile - 1) / cols_per_tile;
+            int64_t rows_per_blk = B >> shift;
+            int64_t grid = ((rp.nrows + rows_per_blk - 1) / rows_per_blk) * rp.col_tiles;
+            if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
+            if (!vec)            ew_rows_kernel<T, 1, false, false, F, B, U><<<(unsigned)grid, B, 0, stream>>>(out, a, b, rp, f);
+            else if (nta && ntb) ew_rows_kernel<T, VEC, true, true, F, B, U><<<(unsigned)grid, B, 0, stream>>>(out, a, b, rp, f);
+            else if (nta)        ew_rows_kernel<T, VEC, true, false, F, B, U><<<(unsigned)grid, B, 0, stream>>>(out, a, b, rp, f);
+            else if (ntb)        ew_rows_kernel<T, VEC, false, true, F, B, U><<<(unsigned)grid, B, 0, stream>>>(out, a, b, rp, f);
+            else                 ew_rows_kernel<T, VEC, false, false, F, B, U><<<(unsigned)grid, B, 0, stream>>>(out, a, b, rp, f);
+            return ZENU_OK;
+        };
+        int rc = small ? launch(std::integral_constant<int, ZENU_EW1_BLOCK>(), std::integral_constant<int, ZENU_EW1_UNROLL>())
+                       : launch(std::integral_constant<int, kBlock>(), std::integral_constant<int, kUnroll>());
+        if (rc) return rc;
         ZENU_LAUNCH_CHECK();
         return ZENU_OK;
     }
