@@ -36,16 +36,17 @@ template <typename T, bool MAX> __device__ __forceinline__ T combine(T a, T b)
     return a + b;
 }
 
-template <typename T, bool MAX> __device__ __forceinline__ T block_red(T v, T *lds)
+template <typename T, bool MAX, int BLOCK = kBlock> __device__ __forceinline__ T block_red(T v, T *lds)
 {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v = combine<T, MAX>(v, __shfl_xor(v, o));
+    if (BLOCK == 64) return v;   // one wavefront: every lane already holds the result
     __syncthreads();   // lds may still be read from the previous reduction
     if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
     __syncthreads();
     T r = lds[0];
 #pragma unroll
-    for (int w = 1; w < kWaves; w++) r = combine<T, MAX>(r, lds[w]);
+    for (int w = 1; w < BLOCK / 64; w++) r = combine<T, MAX>(r, lds[w]);
     return r;
 }
 
@@ -88,11 +89,11 @@ __global__ __launch_bounds__(kBlock) void softmax_lines_kernel(const T *x, T *y,
     if (CE) rowloss[line] = acc;
 }
 
-template <typename T, int VEC, bool CE, bool REG, bool NT>
+template <typename T, int VEC, bool CE, bool REG, bool NT, int kBlock = 256, int kRegPacks = 4>
 __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, int64_t R, const T *target,
                                                                T *rowloss)
 {
-    __shared__ T lds[kWaves];
+    __shared__ T lds[4];
     const int64_t row = blockIdx.x;
     const T *xr = x + row * R;
     T *yr = y + row * R;
@@ -112,7 +113,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
 #pragma unroll
             for (int j = 0; j < VEC; j++) m = combine<T, true>(m, v[k].v[j]);
         }
-        m = block_red<T, true>(m, lds);
+        m = block_red<T, true, kBlock>(m, lds);
         if (x0 != x0) m = x0;   // a NaN in position 0 is never replaced
         T sum = (T)0;
 #pragma unroll
@@ -125,7 +126,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
                 }
             }
         }
-        sum = block_red<T, false>(sum, lds);
+        sum = block_red<T, false, kBlock>(sum, lds);
 #pragma unroll
         for (int k = 0; k < kRegPacks; k++) {
             const int64_t r = first + k * step;
@@ -148,7 +149,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
 #pragma unroll
             for (int j = 0; j < VEC; j++) m = combine<T, true>(m, v.v[j]);
         }
-        m = block_red<T, true>(m, lds);
+        m = block_red<T, true, kBlock>(m, lds);
         if (x0 != x0) m = x0;
         T sum = (T)0;
         for (int64_t r = first; r < R; r += step) {
@@ -160,7 +161,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
             }
             store_pack<T, VEC, false>(yr + r, v);
         }
-        sum = block_red<T, false>(sum, lds);
+        sum = block_red<T, false, kBlock>(sum, lds);
         for (int64_t r = first; r < R; r += step) {   // each thread re-reads what it wrote itself
             Pack<T, VEC> v = load_pack<T, VEC, false>(yr + r);
             Pack<T, VEC> t;
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
         }
     }
     if (CE) {
-        acc = block_red<T, false>(acc, lds);
+        acc = block_red<T, false, kBlock>(acc, lds);
         if (threadIdx.x == 0) rowloss[row] = acc;
     }
 }
@@ -323,47 +324,28 @@ __global__ __launch_bounds__(kBlock) void bias_relu_kernel(const T *z, const T *
     }
 }
 
-// Wide rows: a thread owns one vector of columns (its bias stays in registers) and walks down the
-// rows, so there is no index division; grid = (column tiles, row groups).
+// Rows that are a whole number of 64-lane vectors: a 64-thread workgroup per contiguous piece of a
+// row, one vector per lane (the shape that streams best when most of the traffic is stores); the
+// row / column split is one 32-bit division per workgroup on the scalar unit.
+constexpr int kTileLanes = 64;
 template <typename T, int VEC, bool NT>
-__global__ __launch_bounds__(kBlock) void bias_relu_cols_kernel(const T *z, const T *bias, T *pre, T *act,
-                                                                 int64_t rows, int64_t F, T alpha)
+__global__ __launch_bounds__(kTileLanes) void bias_relu_tile_kernel(const T *z, const T *bias, T *pre, T *act,
+                                                                     uint32_t tiles_per_row, T alpha)
 {
-    const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * VEC;
-    if (col >= F) return;
+    const uint32_t row = blockIdx.x / tiles_per_row;
+    const uint32_t tile = blockIdx.x - row * tiles_per_row;
+    const int64_t col = ((int64_t)tile * kTileLanes + threadIdx.x) * VEC;
+    const int64_t off = (int64_t)blockIdx.x * kTileLanes * VEC + (int64_t)threadIdx.x * VEC;
+    const Pack<T, VEC> v = load_pack<T, VEC, NT>(z + off);
     const Pack<T, VEC> b = load_pack<T, VEC, false>(bias + col);
-    constexpr int U = 4;
-    const int64_t rstep = gridDim.y;
-    int64_t r = blockIdx.y;
-    for (; r + (U - 1) * rstep < rows; r += U * rstep) {
-        Pack<T, VEC> v[U];
+    Pack<T, VEC> a, h;
 #pragma unroll
-        for (int u = 0; u < U; u++) v[u] = load_pack<T, VEC, NT>(z + (r + u * rstep) * F + col);
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            Pack<T, VEC> a, h;
-#pragma unroll
-            for (int j = 0; j < VEC; j++) {
-                a.v[j] = v[u].v[j] + b.v[j];
-                h.v[j] = a.v[j] > (T)0 ? a.v[j] : alpha * a.v[j];
-            }
-            const int64_t off = (r + u * rstep) * F + col;
-            if (pre) store_pack<T, VEC, NT>(pre + off, a);
-            store_pack<T, VEC, NT>(act + off, h);
-        }
+    for (int j = 0; j < VEC; j++) {
+        a.v[j] = v.v[j] + b.v[j];
+        h.v[j] = a.v[j] > (T)0 ? a.v[j] : alpha * a.v[j];
     }
-    for (; r < rows; r += rstep) {
-        const int64_t off = r * F + col;
-        const Pack<T, VEC> v = load_pack<T, VEC, false>(z + off);
-        Pack<T, VEC> a, h;
-#pragma unroll
-        for (int j = 0; j < VEC; j++) {
-            a.v[j] = v.v[j] + b.v[j];
-            h.v[j] = a.v[j] > (T)0 ? a.v[j] : alpha * a.v[j];
-        }
-        if (pre) store_pack<T, VEC, false>(pre + off, a);
-        store_pack<T, VEC, false>(act + off, h);
-    }
+    if (pre) store_pack<T, VEC, NT>(pre + off, a);
+    store_pack<T, VEC, NT>(act + off, h);
 }
 
 // ---- host side ------------------------------------------------------------------------------------------------
@@ -433,6 +415,7 @@ int softmax_forward_launch(const T *x, T *y, Geometry g, const T *target, T *row
         const bool reg = g.R <= (int64_t)kRegPacks * kBlock * (vec ? VEC : 1);
         const unsigned grid = (unsigned)lines;
         const bool nt = vec && reg && lines * g.R * (int64_t)sizeof(T) * 2 >= kStreamBytes;
+        // (one wavefront or 128 threads per row with more vectors per lane measured 4-9 % slower)
         if (nt)               softmax_rows_kernel<T, VEC, CE, true, true><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
         else if (vec && reg)  softmax_rows_kernel<T, VEC, CE, true, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
         else if (vec)         softmax_rows_kernel<T, VEC, CE, false, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
@@ -571,16 +554,12 @@ int bias_relu_t(int dtype, const zenu_tensor_t *pre, const zenu_tensor_t &act, c
     const bool vec = F % VEC == 0 && aligned16(zin.ptr) && aligned16(bin.ptr) && aligned16(aout.ptr) &&
                      (!pp || aligned16(pp));
     const int64_t packs = vec ? F / VEC : F;
-    if (vec && packs >= 64) {
-        const int64_t gx = (packs + kBlock - 1) / kBlock;
-        int64_t gy = ((int64_t)device_info().num_cus * 8 + gx - 1) / gx;
-        if (gy > rows) gy = rows;
-        if (gy > 65535) gy = 65535;
-        if (gx > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-        const dim3 grid((unsigned)gx, (unsigned)gy);
+    if (vec && packs % kTileLanes == 0 && rows * (packs / kTileLanes) <= 0x7fffffffLL) {
+        const uint32_t tiles = (uint32_t)(packs / kTileLanes);
+        const unsigned grid = (unsigned)(rows * tiles);
         const bool nt = n * (int64_t)sizeof(T) * (pp ? 3 : 2) >= kStreamBytes;
-        if (nt) bias_relu_cols_kernel<T, VEC, true><<<grid, kBlock, 0, s>>>(zin.ptr, bin.ptr, pp, aout.ptr, rows, F, (T)alpha);
-        else    bias_relu_cols_kernel<T, VEC, false><<<grid, kBlock, 0, s>>>(zin.ptr, bin.ptr, pp, aout.ptr, rows, F, (T)alpha);
+        if (nt) bias_relu_tile_kernel<T, VEC, true><<<grid, kTileLanes, 0, s>>>(zin.ptr, bin.ptr, pp, aout.ptr, tiles, (T)alpha);
+        else    bias_relu_tile_kernel<T, VEC, false><<<grid, kTileLanes, 0, s>>>(zin.ptr, bin.ptr, pp, aout.ptr, tiles, (T)alpha);
         ZENU_LAUNCH_CHECK();
         int rc2 = aout.finish();
         if (!rc2 && pre) rc2 = pout.finish();
