@@ -22,8 +22,14 @@
 namespace zenu {
 namespace {
 
-constexpr int kBlock = 128;   // small workgroups measured best for the 7-stream update (6.2 vs 5.9 TB/s at 256)
-constexpr int kUnroll = 2;
+#ifndef ZENU_ADAM_BLOCK
+#define ZENU_ADAM_BLOCK 128
+#endif
+#ifndef ZENU_ADAM_UNROLL
+#define ZENU_ADAM_UNROLL 2
+#endif
+constexpr int kBlock = ZENU_ADAM_BLOCK;   // small workgroups measured best for the 7-stream update (6.2 vs 5.9 TB/s at 256)
+constexpr int kUnroll = ZENU_ADAM_UNROLL;
 
 
 template <typename T> struct AdamConsts {
