@@ -299,6 +299,7 @@ def run_c4(z, args, sync):
                      "forward / backward, ReLU backward)",
              "ms_per_step": round(fms, 4), "steps_per_s": round(1e3 / fms, 1),
              "breakdown_us_one_instrumented_step": fbr, "hip_graph_replay": fgraph}
+    compiled = compiled_host_c4(x, t, params, args)
     cpu = None
     if not args.no_cpu_baseline:
         cst = mlp_step.MlpStep(mlp_devices.CpuDev(), x, t, params)
@@ -309,13 +310,43 @@ def run_c4(z, args, sync):
             cst.step()
         cpu = dict(value=round(n / (time.perf_counter() - t1), 2), unit="steps/s", cores=1, kind="port",
                    sample=f"{n} steps of the same op sequence on the C oracle (GEMM: numpy/OpenBLAS, its own threads)")
+    # headline: ZeNu's op sequence issued by the compiled host when it is built, else by the Python mirror
+    head_ms, host = ms, "python mirror (ctypes)"
+    if isinstance(compiled.get("ops"), dict) and "ms_per_step" in compiled["ops"]:
+        head_ms, host = compiled["ops"]["ms_per_step"], "compiled host (C++ API)"
     print(json.dumps({
-        "metric": "MLP training step (configs[4]): steps/s; time per kernel family", "value": round(1e3 / ms, 1),
-        "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "metric": "MLP training step (configs[4]): steps/s; time per kernel family", "value": round(1e3 / head_ms, 1),
+        "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(head_ms, 4),
+        "host": host, "python_mirror_ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[4]: batch 256, Linear 784-512-ReLU-512-ReLU-10, softmax-CE, Adam"},
         "breakdown_us_one_instrumented_step": br, "hip_graph_replay": graph, "fused_entry_points": fused,
-        "cpu_baseline": cpu}))
+        "compiled_host": compiled, "cpu_baseline": cpu}))
+
+
+def compiled_host_c4(x, t, params, args):
+    """The same step issued eagerly from a C++ host (tests/native/mlp_step_bench.cpp, built by
+    __graft_entry__.build()): wall time per step without the Python mirror's per-call cost."""
+    import subprocess
+    import tempfile
+    exe = os.path.join(ROOT, "tests", "native", "bin", "mlp_step_bench")
+    if not os.path.exists(exe):
+        return {"error": "tests/native/bin/mlp_step_bench is not built"}
+    with tempfile.TemporaryDirectory() as d:
+        path = os.path.join(d, "inputs.bin")
+        with open(path, "wb") as f:
+            for a in [x, t] + [params[f"linear{i}.{n}"] for i in (1, 2, 3) for n in ("weight", "bias")]:
+                f.write(np.ascontiguousarray(a, dtype=np.float32).tobytes())
+        out = subprocess.run([exe, "--inputs", path, "--steps", str(max(args.steps, 50)), "--warmup", "5"],
+                             capture_output=True, text=True, timeout=120)
+    if out.returncode != 0:
+        return {"error": (out.stdout + out.stderr)[-300:]}
+    res = {}
+    for line in out.stdout.splitlines():
+        w = line.split()
+        if len(w) == 3 and w[1] in ("ms_per_step", "final_loss"):
+            res.setdefault(w[0], {})[w[1]] = float(w[2])
+    return res
 
 
 def capture_and_replay_c4(z, st, args, sync):

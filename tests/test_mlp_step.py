@@ -70,6 +70,37 @@ def test_hip_fused_step_matches_hip_step(hip):
             assert rel(gb[k].to_numpy(), ga[k].to_numpy()) < 1e-5, (step, k)
 
 
+def write_inputs(path, x, t, params):
+    """raw f32 in the order tests/native/mlp_step_bench.cpp reads"""
+    with open(path, "wb") as f:
+        for a in [x, t] + [params[f"linear{i}.{n}"] for i in (1, 2, 3) for n in ("weight", "bias")]:
+            f.write(np.ascontiguousarray(a, dtype=np.float32).tobytes())
+
+
+@pytest.mark.gpu
+def test_compiled_host_step_matches_python_host(hip, tmp_path):
+    """the same step issued from C++ (include/zenu_hip.hpp + rocBLAS): same kernels, same GEMM library, so
+    the losses of the first steps agree to rounding noise of the launch-order-independent kernels"""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "tests", "native", "bin", "mlp_step_bench")
+    assert os.path.exists(exe), "run __graft_entry__.build() first"
+    x, t, params = mlp_step.make_inputs()
+    write_inputs(tmp_path / "inputs.bin", x, t, params)
+    out = subprocess.run([exe, "--inputs", str(tmp_path / "inputs.bin"), "--dump-loss", "3", "--steps", "2", "--warmup", "0"],
+                         capture_output=True, text=True, timeout=100)
+    print(out.stdout, flush=True)
+    assert out.returncode == 0, out.stdout + out.stderr
+    got = {(l.split()[0], int(l.split()[2])): float(l.split()[3]) for l in out.stdout.splitlines() if " loss " in l}
+    dev = mlp_devices.HipDev(hip)
+    for fused in (False, True):
+        st = mlp_step.MlpStep(dev, x, t, params, fused=fused)
+        for step in (1, 2, 3):
+            loss, _ = st.step()
+            ref = float(loss.to_numpy())
+            assert abs(got[("fused" if fused else "ops", step)] - ref) <= 1e-6 * abs(ref), (fused, step)
+
+
 @pytest.mark.gpu
 def test_hip_step_matches_cpu_step(hip):
     import zenu_oracle as zo
