@@ -25,6 +25,16 @@
  *                                zenu-matrix/src/operation/copy_from.rs:211-267
  *   - sigmoid composite          zenu-autograd/src/activation/sigmoid.rs:7-15
  *   - SGD / Adam / AdamW         zenu-optimizer/src/{sgd.rs:20-31,adam.rs:19-59,adamw.rs:20-70}
+ *   - clip / clip masks          zenu-matrix/src/operation/clip.rs:39-110,205-318
+ *   - broadcast                  zenu-matrix/src/operation/broadcast.rs:11-43
+ * The chains built from these (softmax_assign, SoftMax::backward, cross_entropy and its
+ * backward, bias add + relu) are composed op by op in tests/cpu_matrix.py.
+ *
+ * Pinned by the reference's own known-answer tests, restated in tests/ref_cases.py and
+ * tests/test_optimizer_net.py and run against this library by tests/test_oracle_ref_cases.py
+ * (binary/scalar/broadcast/strided ops, unary tables, relu, sigmoid, sum, sum_to, max*,
+ * copy, clip, broadcast, softmax, cross-entropy, the optimizers' net_test.rs literals).
+ * Parity unpinned: the accumulation order of asum (OpenBLAS) only.
  *
  * exp/log/tanh/pow call the host libm (expf/logf/tanhf/powf, exp/log/tanh/pow):
  * the same symbols Rust's f32::exp/ln/tanh/powf lower to.
