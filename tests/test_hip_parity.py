@@ -448,6 +448,26 @@ def test_reduction_strided_views(hip):
     assert_bits(T.to_numpy(), t, "sum_to strided target")
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_reduction_views_reduced_in_place(hip, dt):
+    """views whose kept dims form one uniform stride chain plus a unit-stride run are reduced without a
+    staging copy (transposed matrices, row slices, index_axis, leading-dim slices); the others still go
+    through the copy: both must give the oracle's answers, at sizes that take the vector, split and
+    column paths"""
+    r = rng(15)
+    x = r.integers(-6, 7, size=(6, 1200, 520)).astype(dt)
+    m = x[0]
+    views = [m.T, m[::2, :], m[3:1100:7, :], m[:, 8:264], x[:, 5, :], x[2], x[1:5], np.swapaxes(x, 0, 1),
+             x[:, :, 4], x[::2, ::3, :], m[:, ::2]]
+    for v in views:
+        V = dev_view(hip, x, v)
+        for axis in range(v.ndim):
+            what = f"view {v.shape} strides {v.strides} axis {axis}"
+            assert_bits(V.sum(axis).to_numpy(), zo.sum_axis(v, axis), what)
+            assert np.array_equal(np.array(V.max_axis_idx_ravel(axis)), zo.max_axis_idx_ravel(v, axis)), what
+            assert_bits(V.max_axis(axis, True).to_numpy(), zo.max_axis(v, axis, True), what)
+
+
 def dev_view_on(hip, M, base, view):
     off = (view.__array_interface__["data"][0] - base.__array_interface__["data"][0]) // base.itemsize
     return hip.Matrix(M.buf, off, view.shape, tuple(s // base.itemsize for s in view.strides), base.dtype)

@@ -631,10 +631,11 @@ int launch_cols(const RedParams<T> &p, hipStream_t s)
     return ZENU_OK;
 }
 
-// Reduce a contiguous [outer, R, inner] source into contiguous outputs of outer*inner elements.
+// Reduce a source addressed as src[q * outer_stride + c + r * elem_stride] (q < outer, c < inner,
+// r < R; the inner run has unit stride) into contiguous outputs of outer*inner elements.
 template <typename T, typename Tr>
-int reduce_contiguous(const T *src, int64_t outer, int64_t R, int64_t inner, T *out_val,
-                      int64_t *out_idx, hipStream_t s)
+int reduce_strided(const T *src, int64_t outer, int64_t R, int64_t inner, int64_t outer_stride,
+                   int64_t elem_stride, T *out_val, int64_t *out_idx, hipStream_t s)
 {
     constexpr int VEC = VecOf<T>::N;
     const int64_t nout = outer * inner;
@@ -650,8 +651,8 @@ int reduce_contiguous(const T *src, int64_t outer, int64_t R, int64_t inner, T *
     p.nout = nout;
     p.R = R;
     p.inner = inner;
-    p.outer_stride = R * inner;
-    p.elem_stride = inner;
+    p.outer_stride = outer_stride;
+    p.elem_stride = elem_stride;
     p.out_val = out_val;
     p.out_idx = out_idx;
     p.part_key = nullptr;
@@ -660,8 +661,8 @@ int reduce_contiguous(const T *src, int64_t outer, int64_t R, int64_t inner, T *
     p.fan = 1;
     p.cstride = 1;
     p.gsrc = src;
-    p.g_outer_stride = R * inner;
-    p.g_elem_stride = inner;
+    p.g_outer_stride = outer_stride;
+    p.g_elem_stride = elem_stride;
 
     const bool use_cols = inner >= 16;
     int64_t splits = 1, groups = nout;
@@ -718,6 +719,14 @@ int reduce_contiguous(const T *src, int64_t outer, int64_t R, int64_t inner, T *
     return use_cols ? launch_cols<T, Tr>(p, s) : launch_rows<T, Tr>(p, s);
 }
 
+// a contiguous [outer, R, inner] source
+template <typename T, typename Tr>
+int reduce_contiguous(const T *src, int64_t outer, int64_t R, int64_t inner, T *out_val,
+                      int64_t *out_idx, hipStream_t s)
+{
+    return reduce_strided<T, Tr>(src, outer, R, inner, R * inner, inner, out_val, out_idx, s);
+}
+
 }  // namespace
 
 namespace {
@@ -745,26 +754,74 @@ bool reduced_shape_ok(const zenu_tensor_t &out, const zenu_tensor_t &src, int ax
 
 enum RedKind { kSum, kAsum, kMax };
 
+struct StridedMap {
+    bool ok;
+    int64_t outer, inner, outer_stride, elem_stride;
+};
+
+// kept dims of `src` (every dim but `axis`, in order) as [outer with a uniform stride chain] x
+// [inner unit-stride run]; size-1 dims never matter
+StridedMap map_strided(const zenu_tensor_t &src, int axis)
+{
+    StridedMap m = {false, 1, 1, 0, src.stride[axis]};
+    int64_t shape[kMaxDim], stride[kMaxDim];
+    int k = 0;
+    for (int i = 0; i < src.ndim; i++) {
+        if (i == axis || src.shape[i] == 1) continue;
+        if (src.shape[i] == 0 || src.stride[i] <= 0) return m;
+        shape[k] = src.shape[i];
+        stride[k] = src.stride[i];
+        k++;
+    }
+    if (src.shape[axis] > 1 && src.stride[axis] <= 0) return m;
+    // trailing unit-stride run
+    int j = k;
+    int64_t run = 1;
+    while (j > 0 && stride[j - 1] == run) {
+        run *= shape[j - 1];
+        j--;
+    }
+    m.inner = run;
+    // the rest must chain: stride[i] == stride[i+1] * shape[i+1]
+    for (int i = 0; i + 1 < j; i++)
+        if (stride[i] != stride[i + 1] * shape[i + 1]) return m;
+    for (int i = 0; i < j; i++) m.outer *= shape[i];
+    m.outer_stride = j > 0 ? stride[j - 1] : 0;
+    // the reduced elements of one output must not run into the next output's inner run or the
+    // kernel's vector paths would mis-assume; plain strided addressing needs no further condition
+    m.ok = true;
+    return m;
+}
+
 template <typename T>
 int reduce_axis_t(int kind, int dtype, const zenu_tensor_t *out, int64_t *out_idx,
                   const zenu_tensor_t &src, int axis, hipStream_t s)
 {
     const int64_t n = num_elm(src);
-    // contiguous source, or a contiguous copy of it (to_default_stride, as max.rs:49 does)
-    const T *sp = static_cast<const T *>(src.ptr);
-    Workspace wsrc(is_default_stride_strict(src) ? 0 : (size_t)n * sizeof(T), s);
-    if (!is_default_stride_strict(src)) {
-        if (wsrc.status) return wsrc.status;
-        zenu_tensor_t tmp = default_view(wsrc.ptr, src.ndim, src.shape);
-        int rc = zenu_hip_copy(dtype, &tmp, &src, s);
-        if (rc) return rc;
-        sp = static_cast<const T *>(wsrc.ptr);
-    }
     int64_t outer = 1, inner = 1;
     for (int i = 0; i < axis; i++) outer *= src.shape[i];
     for (int i = axis + 1; i < src.ndim; i++) inner *= src.shape[i];
     const int64_t R = src.shape[axis];
     const int64_t nout = outer * inner;
+
+    // A view is reduced in place when its kept dims, in output order, split into a leading group
+    // with one uniform stride chain (the kernel's `outer`) and a trailing group that is a unit-stride
+    // run (the kernel's `inner`): transposed matrices, row slices, index_axis views.  Anything
+    // else goes through a contiguous copy first (to_default_stride, as max.rs:49 does).
+    StridedMap map = map_strided(src, axis);
+    const T *sp = static_cast<const T *>(src.ptr);
+    Workspace wsrc(map.ok ? 0 : (size_t)n * sizeof(T), s);
+    if (!map.ok) {
+        if (wsrc.status) return wsrc.status;
+        zenu_tensor_t tmp = default_view(wsrc.ptr, src.ndim, src.shape);
+        int rc = zenu_hip_copy(dtype, &tmp, &src, s);
+        if (rc) return rc;
+        sp = static_cast<const T *>(wsrc.ptr);
+        map.outer = outer;
+        map.inner = inner;
+        map.outer_stride = R * inner;
+        map.elem_stride = inner;
+    }
 
     // contiguous destination, or a temporary that is copied out afterwards
     T *ov = nullptr;
@@ -780,9 +837,9 @@ int reduce_axis_t(int kind, int dtype, const zenu_tensor_t *out, int64_t *out_id
         }
     }
     int rc;
-    if (kind == kSum) rc = reduce_contiguous<T, SumTr<T>>(sp, outer, R, inner, ov, nullptr, s);
-    else if (kind == kAsum) rc = reduce_contiguous<T, AsumTr<T>>(sp, outer, R, inner, ov, nullptr, s);
-    else rc = reduce_contiguous<T, ArgmaxTr<T>>(sp, outer, R, inner, ov, out_idx, s);
+    if (kind == kSum) rc = reduce_strided<T, SumTr<T>>(sp, map.outer, R, map.inner, map.outer_stride, map.elem_stride, ov, nullptr, s);
+    else if (kind == kAsum) rc = reduce_strided<T, AsumTr<T>>(sp, map.outer, R, map.inner, map.outer_stride, map.elem_stride, ov, nullptr, s);
+    else rc = reduce_strided<T, ArgmaxTr<T>>(sp, map.outer, R, map.inner, map.outer_stride, map.elem_stride, ov, out_idx, s);
     if (rc) return rc;
     if (need_copy) {
         zenu_tensor_t tmp = default_view(ov, out->ndim, out->shape);
