@@ -682,3 +682,65 @@ def test_allocator_device(hip):
     _lib.check(l.zenu_hip_mempool_trim(), "trim")
     l.zenu_hip_mempool_stats(C.byref(st))
     assert st.bytes_reserved == st.bytes_in_use + st.bytes_cached
+
+
+def test_empty_tensors(hip):
+    """zero-sized views: elementwise ops and copies do nothing, sums over an empty axis are zeros (the
+    reference adds nothing to a zero-initialised result, sum.rs:18-25), an arg-max over nothing is an
+    error (the reference indexes element 0, max.rs:22)"""
+    for shape in [(0,), (0, 5), (5, 0), (3, 0, 4)]:
+        a, b = hip.Matrix.zeros(shape), hip.Matrix.zeros(shape)
+        assert (a + b).to_numpy().shape == shape
+        assert a.exp().to_numpy().shape == shape
+        a.alloc_like().copy_from(b)
+        a.alloc_like().relu(a, 0.0)
+        x = np.zeros(shape, dtype=np.float32)
+        for axis in range(len(shape)):
+            out = a.sum(axis).to_numpy()
+            assert out.shape == x.sum(axis).shape and not out.any()
+            a.alloc_like().softmax_assign(a, axis)
+            if shape[axis] == 0 and out.size:
+                with pytest.raises(hip.ZenuHipError):
+                    a.max_axis(axis)
+        assert float(a.sum_all().to_numpy()) == 0.0
+        assert a.asum() == 0.0
+        with pytest.raises(hip.ZenuHipError):
+            a.max_idx()
+    p = hip.Matrix.zeros((0,))
+    hip.Adam(1e-3, 0.9, 0.999, 1e-8, {"p": (p, None)}).update({"p": (p, hip.Matrix.zeros((0,)))})
+    hip.SGD(0.1).update({"p": (p, hip.Matrix.zeros((0,)))})
+    hip.synchronize()
+
+
+def test_more_than_2_31_elements(hip):
+    """element counts beyond 32 bits (8.6 GB of f32): 64-bit indexing in the elementwise and reduction
+    kernels; only device memory is used, the host sees slices"""
+    n = (1 << 31) + 4096
+    a = hip.Matrix.zeros((n,))
+    a.add_scalar_assign(1.0)
+    tail = a.slice(slice(n - 8, n))
+    assert np.array_equal(tail.to_numpy(), np.ones(8, dtype=np.float32))
+    head = a.slice(slice(0, 8))
+    assert np.array_equal(head.to_numpy(), np.ones(8, dtype=np.float32))
+    total = float(a.sum_all().to_numpy())
+    assert abs(total - n) <= 256, total            # ulp(2^31) in f32 is 256
+    # 2-D view of the same buffer: 2^16+... rows; reduce the long axis down to 4 columns
+    v = a.reshape((n // 4, 4))
+    s = v.sum(0).to_numpy()
+    assert np.all(np.abs(s - n // 4) <= 64), s
+    tail.add_scalar_assign(4.0)                    # the last 8 elements become 5
+    m = v.max_axis(0).to_numpy()                   # per-column maximum: 5 in every column
+    assert np.array_equal(m, np.full(4, 5.0, dtype=np.float32))
+    idx = v.max_axis_idx_ravel(0)                  # first row holding a 5: n/4 - 2
+    assert idx == [n // 4 - 2] * 4
+    # the flat arg-max tracks positions in 32 bits, like the reference's `int` ABI
+    with pytest.raises(hip.ZenuHipError):
+        a.max_idx()
+    del a, v, tail, head
+    _lib_trim(hip)
+
+
+def _lib_trim(hip):
+    from zenu_amd import _lib
+    hip.synchronize()
+    _lib.check(hip.lib().zenu_hip_mempool_trim(), "trim")

@@ -640,7 +640,12 @@ int reduce_strided(const T *src, int64_t outer, int64_t R, int64_t inner, int64_
     constexpr int VEC = VecOf<T>::N;
     const int64_t nout = outer * inner;
     if (nout == 0) return ZENU_OK;
-    if (R <= 0) return ZENU_ERR_SHAPE;
+    if (R <= 0) {
+        // an empty axis: sums are zero (sum.rs:18-25 adds nothing to zeros, BLAS asum of n = 0 is 0);
+        // the arg-max scan reads element 0 (max.rs:22) -- an error, as in the reference
+        if (Tr::kHasIdx) return ZENU_ERR_SHAPE;
+        return zenu_hip_memset_zero(out_val, (size_t)nout * sizeof(T), reinterpret_cast<zenu_stream_t>(s));
+    }
     if (Tr::kHasIdx && R >= kNoIdx) return ZENU_ERR_UNSUPPORTED;  // positions are tracked in 32 bits
     // workgroups to aim for when the outputs alone do not fill the GPU: two per CU.  More splits
     // shorten the streaming phase but lengthen the serial hand-off at the end (measured 1..16).
@@ -869,10 +874,13 @@ int reduce_all(int kind, int dtype, void *out_val, int64_t *out_idx, const zenu_
     if (!rc) rc = ensure_init();
     if (rc) return rc;
     const int64_t n = num_elm(*src);
-    if (n <= 0) return ZENU_ERR_SHAPE;
-    zenu_tensor_t flat;
     const size_t esz = dtype == ZENU_F32 ? 4 : 8;
     if (dtype != ZENU_F32 && dtype != ZENU_F64) return ZENU_ERR_ARG;
+    if (n <= 0) {   // nothing to add: 0; nothing to take a maximum of: an error
+        if (kind == kMax) return ZENU_ERR_SHAPE;
+        return zenu_hip_memset_zero(out_val, esz, reinterpret_cast<zenu_stream_t>(s));
+    }
+    zenu_tensor_t flat;
     Workspace wsrc(is_default_stride_strict(*src) ? 0 : (size_t)n * esz, s);
     const void *sp = src->ptr;
     if (!is_default_stride_strict(*src)) {
