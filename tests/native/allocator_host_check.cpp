@@ -83,6 +83,22 @@ int main()
         a.free(r, S2);
         printf("ok cross_stream_reuse\n");
     }
+    {   // a stream that is destroyed hands its cached blocks to the null stream: nothing is ever
+        // ordered after the dead stream again
+        FakeBackend be; CachingAllocator a(&be);
+        void *p, *s, *q, *t;
+        a.malloc(&p, 64u << 20, S1); a.malloc(&s, 4096, S1);
+        a.free(p, S1); a.free(s, S1);
+        const uint64_t cached = a.stats().bytes_cached;
+        a.retire_stream(S1);
+        CHECK(a.stats().bytes_cached == cached, "retiring keeps the cache");
+        a.malloc(&q, 64u << 20, S2); a.malloc(&t, 4096, S2);
+        CHECK(q == p && t == s && a.stats().n_driver_allocs == 2, "blocks of the retired stream are reused");
+        for (auto &o : be.orderings) CHECK(o.first != S1, "no ordering after the retired stream");
+        CHECK(be.orderings.size() == 2 && be.orderings[0].first == nullptr, "ordered after the null stream instead");
+        a.free(q, S2); a.free(t, S2);
+        printf("ok retire_stream\n");
+    }
     {   // holes in the middle of a segment are reusable; neighbours merge on free
         FakeBackend be; CachingAllocator a(&be);
         void *p[4];

@@ -744,3 +744,40 @@ def _lib_trim(hip):
     from zenu_amd import _lib
     hip.synchronize()
     _lib.check(hip.lib().zenu_hip_mempool_trim(), "trim")
+
+
+def test_split_reductions_on_two_streams(hip):
+    """split reductions (cross-workgroup hand-off through arrival counters) interleaved on two streams:
+    each stream has its own counter ring, so launches that may overlap never share counters"""
+    import ctypes as C
+    from zenu_amd import _lib
+    l = hip.lib()
+    r = rng(21)
+    x = r.integers(-4, 5, size=(1 << 22)).astype(np.float32)      # exact sums
+    y = r.integers(-4, 5, size=(3000, 1400)).astype(np.float32)
+    X, Y = hip.Matrix.from_numpy(x), hip.Matrix.from_numpy(y)
+    sx, sy = float(x.sum(dtype=np.float64)), y.sum(0, dtype=np.float64)
+    hip.synchronize()
+    s1, s2 = C.c_void_p(), C.c_void_p()
+    _lib.check(l.zenu_hip_stream_create(C.byref(s1)), "stream")
+    _lib.check(l.zenu_hip_stream_create(C.byref(s2)), "stream")
+    old = hip.get_stream()
+    try:
+        outs = []
+        for i in range(150):
+            hip.set_stream(s1 if i % 2 == 0 else s2)
+            outs.append((X.sum_all(), Y.sum(0)))
+        for s in (s1, s2):
+            _lib.check(l.zenu_hip_stream_synchronize(s), "sync")
+        hip.set_stream(s1)
+        for a, b in outs:
+            assert float(a.to_numpy()) == sx
+            assert np.array_equal(b.to_numpy(), sy.astype(np.float32))
+        del outs, a, b
+    finally:
+        hip.set_stream(s1)
+        hip.synchronize()
+        hip.set_stream(old)
+        _lib.check(l.zenu_hip_stream_synchronize(s2), "sync")
+    _lib.check(l.zenu_hip_stream_destroy(s1), "destroy")
+    _lib.check(l.zenu_hip_stream_destroy(s2), "destroy")

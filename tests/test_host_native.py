@@ -22,7 +22,7 @@ def test_allocator_bookkeeping(tmp_path):
     exe = build("allocator_host_check.cpp", str(tmp_path / "alloc_check"))
     out = subprocess.run([exe], capture_output=True, text=True)
     assert out.returncode == 0, out.stdout + out.stderr
-    for name in ("size_classes", "same_stream_reuse", "cross_stream_reuse", "split_merge_trim", "oom_retry",
+    for name in ("size_classes", "same_stream_reuse", "cross_stream_reuse", "retire_stream", "split_merge_trim", "oom_retry",
                  "injected_failure", "not_owned", "stress"):
         assert f"ok {name}" in out.stdout
 

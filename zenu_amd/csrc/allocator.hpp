@@ -149,6 +149,25 @@ public:
         return kOk;
     }
 
+    // `stream` is about to be destroyed and has been synchronised: its cached blocks are idle,
+    // so they move to the null stream's lists (nobody may order work after a dead stream).
+    void retire_stream(void *stream)
+    {
+        if (!stream) return;
+        std::lock_guard<std::mutex> g(mu_);
+        for (int small = 0; small < 2; small++) {
+            auto it = free_.find(PoolKey{stream, small != 0});
+            if (it == free_.end()) continue;
+            std::vector<Block *> blocks(it->second.begin(), it->second.end());
+            free_.erase(it);
+            for (Block *b : blocks) {
+                stats_.bytes_cached -= b->size;
+                b->stream = nullptr;
+                insert_free(b);
+            }
+        }
+    }
+
     AllocStats stats()
     {
         std::lock_guard<std::mutex> g(mu_);

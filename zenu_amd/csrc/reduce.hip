@@ -33,8 +33,8 @@
 
 namespace zenu {
 
-// `n` consecutive arrival counters (zero at rest) from the library's ring, or nullptr
-int *reserve_counters(int64_t n);
+// `n` consecutive arrival counters (zero at rest) from the ring of `stream`, or nullptr
+int *reserve_counters(int64_t n, hipStream_t stream);
 
 namespace {
 
@@ -705,11 +705,11 @@ int reduce_strided(const T *src, int64_t outer, int64_t R, int64_t inner, int64_
         while ((int64_t)fan * fan < splits) fan++;
         cstride = 1 + (int)((splits + fan - 1) / fan);
     }
-    int *counters = reserve_counters(groups * cstride);
+    int *counters = reserve_counters(groups * cstride, s);
     if (!counters && cstride > 1) {   // too many groups for trees: flat counters
         fan = (int)splits;
         cstride = 1;
-        counters = reserve_counters(groups);
+        counters = reserve_counters(groups, s);
     }
     if (!counters) return ZENU_ERR_UNSUPPORTED;
     p.fan = fan;

@@ -6,6 +6,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <map>
 #include <mutex>
 
 #include "allocator.hpp"
@@ -48,8 +49,10 @@ constexpr int64_t kNumCounters = 1 << 16;
 struct State {
     bool ready = false;
     bool use_pool = true;
-    int *counters = nullptr;      // arrival counters of the reductions, zero at rest
-    int64_t counter_cursor = 0;
+    // arrival counters of the reductions, zero at rest: one ring per stream, because only launches
+    // on the same stream are certain to run one after the other
+    struct Ring { int *base = nullptr; int64_t cursor = 0; };
+    std::map<hipStream_t, Ring> rings;
     std::mutex counter_mu;
     DeviceInfo info;
     HipBackend backend;
@@ -58,6 +61,39 @@ struct State {
 
 State g_state;
 std::mutex g_init_mu;
+
+// allocate and clear the ring of `stream` (blocking; at init, at stream creation, or at the first
+// split reduction on a stream the library did not create)
+int *make_ring(hipStream_t stream)
+{
+    int *base = nullptr;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&base), kNumCounters * sizeof(int));
+    if (e == hipSuccess) e = hipMemset(base, 0, kNumCounters * sizeof(int));
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (e != hipSuccess) {
+        set_last_hip_error(e);
+        if (base) (void)hipFree(base);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> g(g_state.counter_mu);
+    State::Ring &r = g_state.rings[stream];
+    if (r.base) {           // another thread was faster
+        (void)hipFree(base);
+        return r.base;
+    }
+    r.base = base;
+    r.cursor = 0;
+    return base;
+}
+
+void drop_ring(hipStream_t stream)
+{
+    std::lock_guard<std::mutex> g(g_state.counter_mu);
+    auto it = g_state.rings.find(stream);
+    if (it == g_state.rings.end()) return;
+    if (it->second.base) (void)hipFree(it->second.base);
+    g_state.rings.erase(it);
+}
 
 int init_locked(int device)
 {
@@ -77,11 +113,8 @@ int init_locked(int device)
     const char *env = getenv("ZENU_USE_MEMPOOL");  // zenu-matrix/src/lib.rs:36, default "1"
     g_state.use_pool = !(env && strcmp(env, "0") == 0);
     g_state.pool = new CachingAllocator(&g_state.backend);
-    ZENU_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&g_state.counters), kNumCounters * sizeof(int)));
-    ZENU_HIP_TRY(hipMemset(g_state.counters, 0, kNumCounters * sizeof(int)));
-    g_state.counter_cursor = 0;
     g_state.ready = true;
-    return ZENU_OK;
+    return make_ring(nullptr) ? ZENU_OK : ZENU_ERR_HIP;   // the null stream's ring; created streams get theirs at creation
 }
 
 __global__ void fill_zero_kernel(uint4 *dst16, size_t n16, unsigned char *tail, size_t ntail)
@@ -96,16 +129,25 @@ __global__ void fill_zero_kernel(uint4 *dst16, size_t n16, unsigned char *tail, 
 
 const DeviceInfo &device_info() { return g_state.info; }
 
-// Consecutive launches take consecutive ranges of the ring, so a range is reused only after
-// kNumCounters counters' worth of later reductions; every kernel leaves its counters at zero.
-int *reserve_counters(int64_t n)
+// Consecutive launches on a stream take consecutive ranges of that stream's ring; a range is reused
+// by a later launch of the same stream, which runs after the earlier one.  Every kernel leaves
+// its counters at zero.
+int *reserve_counters(int64_t n, hipStream_t stream)
 {
-    if (n <= 0 || n > kNumCounters || !g_state.counters) return nullptr;
-    std::lock_guard<std::mutex> g(g_state.counter_mu);
-    if (g_state.counter_cursor + n > kNumCounters) g_state.counter_cursor = 0;
-    int *r = g_state.counters + g_state.counter_cursor;
-    g_state.counter_cursor += n;
-    return r;
+    if (n <= 0 || n > kNumCounters || !g_state.ready) return nullptr;
+    {
+        std::lock_guard<std::mutex> g(g_state.counter_mu);
+        auto it = g_state.rings.find(stream);
+        if (it != g_state.rings.end() && it->second.base) {
+            State::Ring &r = it->second;
+            if (r.cursor + n > kNumCounters) r.cursor = 0;
+            int *out = r.base + r.cursor;
+            r.cursor += n;
+            return out;
+        }
+    }
+    if (!make_ring(stream)) return nullptr;
+    return reserve_counters(n, stream);
 }
 
 int ensure_init()
@@ -143,8 +185,12 @@ int zenu_hip_shutdown(void)
     (void)hipDeviceSynchronize();
     delete g_state.pool;
     g_state.pool = nullptr;
-    if (g_state.counters) (void)hipFree(g_state.counters);
-    g_state.counters = nullptr;
+    {
+        std::lock_guard<std::mutex> gc(g_state.counter_mu);
+        for (auto &kv : g_state.rings)
+            if (kv.second.base) (void)hipFree(kv.second.base);
+        g_state.rings.clear();
+    }
     g_state.ready = false;
     return ZENU_OK;
 }
@@ -177,6 +223,10 @@ int zenu_hip_stream_create(zenu_stream_t *stream)
     // default flags and priority: ordered against the null stream, as the reference's
     // cudaStreamCreate stream is (zenu-cuda/src/runtime/mod.rs:113-121)
     ZENU_HIP_TRY(hipStreamCreate(&s));
+    if (!make_ring(s)) {
+        (void)hipStreamDestroy(s);
+        return ZENU_ERR_HIP;
+    }
     *stream = s;
     return ZENU_OK;
 }
@@ -184,6 +234,9 @@ int zenu_hip_stream_create(zenu_stream_t *stream)
 int zenu_hip_stream_destroy(zenu_stream_t stream)
 {
     if (!stream) return ZENU_ERR_ARG;
+    ZENU_HIP_TRY(hipStreamSynchronize(as_stream(stream)));   // its reductions are done with their counters
+    drop_ring(as_stream(stream));
+    if (g_state.pool) g_state.pool->retire_stream(stream);   // its cached blocks outlive it
     ZENU_HIP_TRY(hipStreamDestroy(as_stream(stream)));
     return ZENU_OK;
 }
