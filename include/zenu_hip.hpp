@@ -80,11 +80,14 @@ inline Dim default_stride(const Dim &shape)
 }
 
 // Owned device memory (Ptr<Owned<T>, D>, matrix.rs:163-171)
+// The block goes back to the pool on the stream it was taken on; a buffer that is also used on
+// another stream must be kept alive until that stream is done with it.
 struct Buffer {
     void *ptr = nullptr;
     size_t bytes = 0;
-    explicit Buffer(size_t n) : bytes(n) { check(zenu_hip_malloc(&ptr, n ? n : 1, current_stream()), "zenu_hip_malloc"); }
-    ~Buffer() { if (ptr) zenu_hip_free(ptr, current_stream()); }
+    zenu_stream_t stream;
+    explicit Buffer(size_t n) : bytes(n), stream(current_stream()) { check(zenu_hip_malloc(&ptr, n ? n : 1, stream), "zenu_hip_malloc"); }
+    ~Buffer() { if (ptr) zenu_hip_free(ptr, stream); }
     Buffer(const Buffer &) = delete;
     Buffer &operator=(const Buffer &) = delete;
 };

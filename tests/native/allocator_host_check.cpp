@@ -97,6 +97,18 @@ int main()
         for (auto &o : be.orderings) CHECK(o.first != S1, "no ordering after the retired stream");
         CHECK(be.orderings.size() == 2 && be.orderings[0].first == nullptr, "ordered after the null stream instead");
         a.free(q, S2); a.free(t, S2);
+        // a block still live when its stream died is freed in the dead stream's name: null stream too
+        void *u, *w;
+        a.malloc(&u, 32u << 20, S1);          // S1 is retired: a caller's stale handle
+        a.free(u, S1);
+        const size_t before = be.orderings.size();
+        a.malloc(&w, 32u << 20, S2);
+        CHECK(w == u && be.orderings.size() == before + 1 && be.orderings.back().first == nullptr, "stale handle mapped to the null stream");
+        a.free(w, S2);
+        a.adopt_stream(S1);                   // the handle value comes back as a new stream
+        a.malloc(&u, 48u << 20, S1); a.free(u, S1); a.malloc(&w, 48u << 20, S2);
+        CHECK(w == u && be.orderings.back().first == S1, "an adopted stream is a stream again");
+        a.free(w, S2);
         printf("ok retire_stream\n");
     }
     {   // holes in the middle of a segment are reusable; neighbours merge on free

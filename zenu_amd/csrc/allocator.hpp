@@ -132,6 +132,7 @@ public:
         live_.erase(it);
         stats_.bytes_in_use -= b->size;
         b->allocated = false;
+        if (retired_.count(stream)) stream = nullptr;  // freed after its stream was destroyed (and synchronised)
         b->stream = stream;  // the last stream to use the block: stream-ordered free
         // merge with free neighbours that belong to the same stream
         b = try_merge(b, b->prev);
@@ -155,6 +156,7 @@ public:
     {
         if (!stream) return;
         std::lock_guard<std::mutex> g(mu_);
+        retired_.insert(stream);
         for (int small = 0; small < 2; small++) {
             auto it = free_.find(PoolKey{stream, small != 0});
             if (it == free_.end()) continue;
@@ -166,6 +168,13 @@ public:
                 insert_free(b);
             }
         }
+    }
+
+    // a new stream may get the handle value of a destroyed one
+    void adopt_stream(void *stream)
+    {
+        std::lock_guard<std::mutex> g(mu_);
+        retired_.erase(stream);
     }
 
     AllocStats stats()
@@ -348,6 +357,7 @@ private:
     std::mutex mu_;
     std::map<PoolKey, FreeSet> free_;
     std::unordered_map<char *, Block *> live_;
+    std::set<void *> retired_;   // destroyed streams: blocks freed in their name go to the null stream
     AllocStats stats_;
 };
 

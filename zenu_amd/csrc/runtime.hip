@@ -227,6 +227,7 @@ int zenu_hip_stream_create(zenu_stream_t *stream)
         (void)hipStreamDestroy(s);
         return ZENU_ERR_HIP;
     }
+    if (g_state.pool) g_state.pool->adopt_stream(s);
     *stream = s;
     return ZENU_OK;
 }

@@ -63,14 +63,17 @@ class DeviceBuffer:
 
     def __init__(self, nbytes):
         p = C.c_void_p()
-        check(_lib.lib().zenu_hip_malloc(C.byref(p), nbytes, _stream), "malloc")
+        # the block is returned on the stream it was taken on: a buffer used on another stream
+        # as well must be kept alive until that stream is done with it
+        self.stream = _stream
+        check(_lib.lib().zenu_hip_malloc(C.byref(p), nbytes, self.stream), "malloc")
         self.ptr = p.value
         self.nbytes = nbytes
 
     def __del__(self):
         try:
             if getattr(self, "ptr", None):
-                _lib.lib().zenu_hip_free(self.ptr, _stream)
+                _lib.lib().zenu_hip_free(self.ptr, self.stream)
                 self.ptr = None
         except Exception:
             pass
