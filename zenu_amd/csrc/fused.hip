@@ -187,7 +187,15 @@ __global__ __launch_bounds__(kBlock) void ce_finalize_kernel(const T *rowloss, i
 {
     __shared__ T lds[kWaves];
     T acc = (T)0;
-    for (int64_t i = threadIdx.x; i < n; i += kBlock) acc = acc + rowloss[i];
+    int64_t i = threadIdx.x;
+    for (; i + 7 * kBlock < n; i += 8 * kBlock) {       // eight loads in flight, added in index order
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = rowloss[i + u * kBlock];
+#pragma unroll
+        for (int u = 0; u < 8; u++) acc = acc + v[u];
+    }
+    for (; i < n; i += kBlock) acc = acc + rowloss[i];
     acc = block_red<T, false>(acc, lds);
     if (threadIdx.x == 0) *loss = acc / neg_n;
 }
