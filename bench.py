@@ -444,8 +444,8 @@ def main():
     ap.add_argument("--profile-op", default=None, help="only launch this op (for rocprofv3 counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on ONE GPU; every op of the path shards without communication "
-                 "(see DESIGN.md), but no multi-GPU path exists: run with --gpus 1")
+        sys.exit("bench.py: this build runs on ONE GPU (every op of the path would shard without communication, "
+                 "but no multi-GPU path exists): run with --gpus 1")
 
     import zenu_amd as z
     from zenu_amd import _lib

@@ -1,4 +1,5 @@
-// elementwise.hip -- N-d elementwise engine for gfx950 (binary, scalar, unary, relu, copy).
+// elementwise.hip -- N-d elementwise engine for gfx950 (binary, scalar, unary, relu, clip, copy,
+// broadcast).
 //
 // One Matrix-level call of the reference (add_array, mul_scalar, exp_array, relu, copy_from ...,
 // zenu-matrix/src/operation/basic_operations.rs:278-381,512-611, relu.rs:169-242,
@@ -6,8 +7,9 @@
 // (zenu-matrix/src/with_clousers.rs:180-223).  After the host has folded the operands into a
 // common iteration space (shape.cpp) one of four kernels runs:
 //
-//   contig : every operand is one contiguous run.  128-bit loads/stores, 4 vectors in flight
-//            per thread, block tile = 256 threads x 4 x 16 B.                        [HBM bound]
+//   contig : every operand is one contiguous run.  128-bit loads/stores; 64 threads x one vector
+//            when one input streams (the shape that moves load + store traffic fastest), 256
+//            threads x two vectors for two inputs and for tanh / sigmoid.           [HBM bound]
 //   rows   : the innermost dim is contiguous (stride 1) or broadcast (stride 0) in every operand;
 //            outer dims are arbitrary.  Covers row / column broadcast and row-sliced views.  The
 //            outer index is decomposed once per thread, the inner dim is walked with 128-bit

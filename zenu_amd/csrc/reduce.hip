@@ -3,22 +3,26 @@
 // The reference reduces by host recursion: `sum` issues shape[axis] whole-slice `+=` launches
 // (zenu-matrix/src/operation/sum.rs:12-31) and `max_axis` one alloc + copy + kernel + two
 // blocking single-element copies per output element (zenu-matrix/src/operation/max.rs:45-99).
-// Here a contiguous source is seen as [outer, R, inner] with R the reduced axis and one of two
-// kernels runs:
+// Here the source is addressed as [outer, R, inner] with R the reduced axis (any view whose kept
+// dims form one uniform stride chain plus a unit-stride run; other views are copied first) and
+// one of two kernels runs:
 //
-//   rows : inner == 1 (the reduced axis is contiguous) -- one workgroup (or one wavefront when
-//          the row is short) per row, 128-bit loads, four independent accumulators per lane,
-//          wave64 butterfly built from DPP (quad_perm, row_half_mirror, row_mirror), ds_swizzle
-//          and one cross-half exchange, then a fixed-order combine of the 4 waves through LDS.
-//          Also used with an element stride for small `inner`.
-//   cols : inner > 1 -- a 64 x 4 thread tile: 64 lanes own 64 column vectors (coalesced 128-bit
-//          loads), 4 row lanes walk the reduced axis, combined through LDS in fixed order.
+//   rows : inner < 16, normally 1 (the reduced axis is contiguous) -- one workgroup (or one
+//          wavefront when the row is short) per row, 128-bit loads, four independent
+//          accumulators per lane (eight when workgroups share a row), wave64 butterfly built
+//          from DPP (quad_perm, row_half_mirror, row_mirror), ds_swizzle and one cross-half
+//          exchange, then a fixed-order combine of the 4 waves through LDS.
+//   cols : inner >= 16 -- a 32 x 8 thread tile: 32 lanes own 32 column vectors (512-byte row
+//          pieces, coalesced 128-bit loads), 8 row lanes walk the reduced axis with four rows in
+//          flight each, combined through LDS in fixed order.
 //
-// Both kernels can split the reduced axis over several workgroups.  Partial results go to a
-// small workspace; each workgroup then bumps an arrival counter and the one that arrives last
-// folds the partials of its outputs, always in split order.  No workgroup waits for another and
-// no atomic touches data: the combination tree is fixed by the launch geometry, so results are
-// bit-reproducible, and the whole reduction is ONE launch.
+// Both kernels can split the reduced axis over several workgroups; the splits interleave chunk
+// by chunk so the grid sweeps the source as one window.  Partial results go to a small
+// workspace; each workgroup then bumps an arrival counter (a two-level tree of counters when
+// many workgroups share an output) and the one that arrives last folds the partials of its
+// outputs, always in split order.  No workgroup waits for another and no atomic touches data:
+// the combination tree is fixed by the launch geometry, so results are bit-reproducible, and
+// the whole reduction is ONE launch.
 //
 // Arg-max follows MaxIdx for Cpu (max.rs:19-34): start from element 0 and replace on strict '>'.
 // That is "largest value, lowest index on ties", except for NaN: a NaN at position 0 is never
@@ -880,7 +884,6 @@ int reduce_all(int kind, int dtype, void *out_val, int64_t *out_idx, const zenu_
         if (kind == kMax) return ZENU_ERR_SHAPE;
         return zenu_hip_memset_zero(out_val, esz, reinterpret_cast<zenu_stream_t>(s));
     }
-    zenu_tensor_t flat;
     Workspace wsrc(is_default_stride_strict(*src) ? 0 : (size_t)n * esz, s);
     const void *sp = src->ptr;
     if (!is_default_stride_strict(*src)) {
@@ -890,7 +893,6 @@ int reduce_all(int kind, int dtype, void *out_val, int64_t *out_idx, const zenu_
         if (rc) return rc;
         sp = wsrc.ptr;
     }
-    (void)flat;
     if (dtype == ZENU_F32) {
         const float *f = static_cast<const float *>(sp);
         float *ov = static_cast<float *>(out_val);
