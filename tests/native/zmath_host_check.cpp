@@ -33,8 +33,32 @@ int main(int argc, char **argv)
             bad_fdlibm += b0; bad_simd += b1; bad_expm1 += b2; bad_sig += b3;
         });
     for (auto &t : th) t.join();
+    // double precision: every stride-th value of the HIGH word (sign, exponent, 20 mantissa bits) with
+    // a pseudo-random low word, plus low words 0 and all-ones
+    std::atomic<uint64_t> bad_tanh64{0}, bad_expm164{0}, bad_sig64{0};
+    th.clear();
+    for (int w = 0; w < nt; w++)
+        th.emplace_back([&, w]() {
+            uint64_t b0 = 0, b1 = 0, b2 = 0, rng = 0x9E3779B97F4A7C15ull * (w + 1);
+            for (uint64_t u = (uint64_t)w * stride; u < (1ull << 32); u += stride * nt) {
+                rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17;
+                const uint32_t lows[3] = {(uint32_t)rng, 0u, 0xffffffffu};
+                for (uint32_t lo : lows) {
+                    const double x = zmath::u2d((u << 32) | lo);
+                    const double ref = tanh(x), got = zmath::tanh_fdlibm(x);
+                    if ((ref != ref) ? !(got != got) : zmath::d2u(got) != zmath::d2u(ref)) b0++;
+                    if (fabs(x) < 700.0 && zmath::d2u(zmath::expm1_fdlibm(x)) != zmath::d2u(expm1(x))) b1++;
+                    const double sg = 0.5 + 0.5 * tanh(0.5 * x), sz = zmath::sigmoid_zenu(x);
+                    if ((sg != sg) ? !(sz != sz) : zmath::d2u(sz) != zmath::d2u(sg)) b2++;
+                }
+            }
+            bad_tanh64 += b0; bad_expm164 += b1; bad_sig64 += b2;
+        });
+    for (auto &t : th) t.join();
     printf("tanhf_fdlibm %llu tanhf_simd %llu expm1f_fdlibm %llu sigmoidf_zenu %llu\n",
            (unsigned long long)bad_fdlibm.load(), (unsigned long long)bad_simd.load(),
            (unsigned long long)bad_expm1.load(), (unsigned long long)bad_sig.load());
-    return (bad_fdlibm + bad_simd + bad_expm1 + bad_sig) ? 1 : 0;
+    printf("tanh_fdlibm %llu expm1_fdlibm %llu sigmoid_zenu %llu\n", (unsigned long long)bad_tanh64.load(),
+           (unsigned long long)bad_expm164.load(), (unsigned long long)bad_sig64.load());
+    return (bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64) ? 1 : 0;
 }

@@ -4,7 +4,7 @@ configurations (full size) and on edge cases.  Everything goes through the C ABI
 Bars (written where they are used):
   add/sub/mul/div, relu, max, arg-max, copy, SGD/Adam/AdamW .......... bit-exact
   exp/log (device math library) ....................................... <= 2 ulp
-  tanh, sigmoid (f32: same algorithm as the host libm) ................. bit-exact (bar: <= 2 ulp)
+  tanh, sigmoid (f32 and f64: same algorithm as the host libm) ........ bit-exact (bar: <= 2 ulp)
   sums ................................................................ |gpu - cpu| <= 1e-5 (f32) /
       1e-12 (f64) times max(|cpu|, sum|x| / sqrt(n)); the second term is the typical magnitude
       of a sum of n such terms, so a result that cancels to ~0 is not held to a relative bar
@@ -249,16 +249,30 @@ def test_unary_f64(hip):
     r = rng(11)
     x = r.standard_normal((257, 129))
     X = hip.Matrix.from_numpy(x)
-    for name, fn, bar in (("exp", zo.EXP, 2), ("tanh", zo.TANH, 4), ("sqrt", zo.SQRT, 0), ("abs", zo.ABS, 0)):
+    for name, fn, bar in (("exp", zo.EXP, 2), ("tanh", zo.TANH, 0), ("sqrt", zo.SQRT, 0), ("abs", zo.ABS, 0)):
         xx = np.abs(x) if name == "sqrt" else x
         exp = np.empty_like(xx)
         zo.unary(fn, exp, xx)
         got = getattr(hip.Matrix.from_numpy(xx), name)().to_numpy()
         u = max_ulp(got, exp)
         print(f"[f64] {name}: {u} ulp", flush=True)
-        # f64 tanh comes from the device math library: parity unpinned beyond a few ulp
         assert u <= bar, (name, u)
-    del X
+    # f64 tanh and the sigmoid composite restate the host libm's algorithm: same bits, also on a wide
+    # range, at the branch points of the algorithm and on special values
+    wide = np.concatenate([r.standard_normal(200000) * s for s in (1e-3, 0.3, 3.0, 30.0)] +
+                          [np.array([0.0, -0.0, 1.0, -1.0, 22.0, -22.0, 21.999999, 1e-300, -1e-300, 2.0 ** -55, 2.0 ** -54,
+                                     0.5 * np.log(2), 1.5 * np.log(2), 709.0, -709.0, np.inf, -np.inf, np.nan, 5e-324])])
+    W = hip.Matrix.from_numpy(wide)
+    exp = np.empty_like(wide)
+    zo.unary(zo.TANH, exp, wide)
+    got = W.tanh().to_numpy()
+    fin = ~np.isnan(exp)
+    assert np.array_equal(np.isnan(got), np.isnan(exp)) and max_ulp(got[fin], exp[fin]) == 0
+    zo.sigmoid(exp, wide)
+    got = W.sigmoid().to_numpy()
+    fin = ~np.isnan(exp)
+    assert np.array_equal(np.isnan(got), np.isnan(exp)) and max_ulp(got[fin], exp[fin]) == 0
+    del X, W
 
 
 # ---- strided / broadcast engine: randomized shapes vs brute force and oracle ------------------------------

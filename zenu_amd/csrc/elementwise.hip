@@ -72,15 +72,9 @@ template <typename T, int OP> struct ScalarF {
 };
 
 __device__ __forceinline__ float dev_tanh(float x) { return zmath::tanhf_simd(x); }
-__device__ __forceinline__ double dev_tanh(double x) { return tanh(x); }
+__device__ __forceinline__ double dev_tanh(double x) { return zmath::tanh_fdlibm(x); }
 __device__ __forceinline__ float dev_sigmoid(float x) { return zmath::sigmoidf_zenu(x); }
-__device__ __forceinline__ double dev_sigmoid(double x)
-{
-    double xh = x * 0.5;
-    double th = tanh(xh);
-    double ht = 0.5 * th;
-    return 0.5 + ht;
-}
+__device__ __forceinline__ double dev_sigmoid(double x) { return zmath::sigmoid_zenu(x); }
 
 template <typename T, int FN> struct UnaryF {
     static constexpr int NIN = 1;

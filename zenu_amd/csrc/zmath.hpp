@@ -1,5 +1,5 @@
-// zmath.hpp -- f32 tanh / expm1 for device code, bit-compatible with the host libm the
-// reference's CPU path calls (Rust f32::tanh -> libm tanhf).
+// zmath.hpp -- tanh / expm1 (f32 and f64) for device code, bit-compatible with the host libm the
+// reference's CPU path calls (Rust f32::tanh / f64::tanh -> libm tanhf / tanh).
 //
 // Why not the device math library: ZeNu's sigmoid is the composite 0.5 + 0.5*tanh(0.5*x)
 // (zenu-autograd/src/activation/sigmoid.rs:7-15).  For negative x the final add cancels, so a
@@ -236,6 +236,151 @@ ZM_HD float tanhf_simd(float x)
     const float q = num / (em1 + two);
     const float z = big ? one - q : -q;
     return neg ? -z : z;
+}
+
+// ---- double precision: fdlibm s_expm1.c / s_tanh.c as shipped by glibc 2.35 (generic dbl-64) ----------
+
+ZM_HD uint64_t d2u(double d)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return (uint64_t)__double_as_longlong(d);
+#else
+    uint64_t u;
+    memcpy(&u, &d, 8);
+    return u;
+#endif
+}
+ZM_HD double u2d(uint64_t u)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __longlong_as_double((long long)u);
+#else
+    double d;
+    memcpy(&d, &u, 8);
+    return d;
+#endif
+}
+ZM_HD uint32_t hi_word(double d) { return (uint32_t)(d2u(d) >> 32); }
+ZM_HD double add_to_hi_word(double d, uint32_t inc) { return u2d(d2u(d) + ((uint64_t)inc << 32)); }
+ZM_HD double from_hi_word(uint32_t hi) { return u2d((uint64_t)hi << 32); }
+
+// expm1 for finite arguments (tanh passes |x| < 44)
+ZM_HD double expm1_fdlibm(double x)
+{
+    const double one = 1.0, tiny = 1.0e-300, huge = 1.0e+300;
+    const double o_threshold = 7.09782712893383973096e+02;
+    const double ln2_hi = u2d(0x3fe62e42fee00000ull);   // 6.93147180369123816490e-01
+    const double ln2_lo = u2d(0x3dea39ef35793c76ull);   // 1.90821492927058770002e-10
+    const double invln2 = u2d(0x3ff71547652b82feull);   // 1.44269504088896338700e+00
+    const double Q1 = u2d(0xBFA11111111110F4ull);       // -3.33333333333331316428e-02
+    const double Q2 = u2d(0x3F5A01A019FE5585ull);       //  1.58730158725481460165e-03
+    const double Q3 = u2d(0xBF14CE199EAADBB7ull);       // -7.93650757867487942473e-05
+    const double Q4 = u2d(0x3ED0CFCA86E65239ull);       //  4.00821782732936239552e-06
+    const double Q5 = u2d(0xBE8AFDB76E09C32Dull);       // -2.01099218183624371326e-07
+
+    double y, hi, lo, c = 0.0, t, e, hxs, hfx, r1, h2, h4, R1, R2, R3;
+    int32_t k;
+    uint32_t hx = hi_word(x);
+    const uint32_t xsb = hx & 0x80000000u;
+    hx &= 0x7fffffffu;
+
+    if (hx >= 0x4043687Au) {                 // |x| >= 56 ln2
+        if (hx >= 0x40862E42u) {             // |x| >= 709.78...
+            if (hx >= 0x7ff00000u) {
+                if (((hx & 0xfffffu) | (uint32_t)d2u(x)) != 0) return x + x;   // NaN
+                return (xsb == 0) ? x : -1.0;                                 // +-inf
+            }
+            if (x > o_threshold) return huge * huge;
+        }
+        if (xsb != 0) return tiny - one;     // x < -56 ln2
+    }
+    if (hx > 0x3fd62e42u) {                  // |x| > 0.5 ln2
+        if (hx < 0x3FF0A2B2u) {              // |x| < 1.5 ln2
+            if (xsb == 0) { hi = x - ln2_hi; lo = ln2_lo;  k = 1; }
+            else          { hi = x + ln2_hi; lo = -ln2_lo; k = -1; }
+        } else {
+            k = (int32_t)(invln2 * x + ((xsb == 0) ? 0.5 : -0.5));
+            t = (double)k;
+            hi = x - t * ln2_hi;
+            lo = t * ln2_lo;
+        }
+        x = hi - lo;
+        c = (hi - x) - lo;
+    } else if (hx < 0x3c900000u) {           // |x| < 2^-54
+        t = huge + x;
+        return x - (t - (huge + x));
+    } else {
+        k = 0;
+    }
+    hfx = 0.5 * x;
+    hxs = x * hfx;
+    R1 = one + hxs * Q1;
+    h2 = hxs * hxs;
+    R2 = Q2 + hxs * Q3;
+    h4 = h2 * h2;
+    R3 = Q4 + hxs * Q5;
+    r1 = R1 + h2 * R2 + h4 * R3;
+    t = 3.0 - r1 * hfx;
+    e = hxs * ((r1 - t) / (6.0 - x * t));
+    if (k == 0) return x - (x * e - hxs);
+    e = (x * (e - c) - c);
+    e -= hxs;
+    if (k == -1) return 0.5 * (x - e) - 0.5;
+    if (k == 1) {
+        if (x < -0.25) return -2.0 * (e - (x + 0.5));
+        return one + 2.0 * (x - e);
+    }
+    if (k <= -2 || k > 56) {
+        y = one - (e - x);
+        y = add_to_hi_word(y, (uint32_t)k << 20);
+        return y - one;
+    }
+    if (k < 20) {
+        t = from_hi_word(0x3ff00000u - (0x200000u >> k));   // 1 - 2^-k
+        y = t - (e - x);
+        y = add_to_hi_word(y, (uint32_t)k << 20);
+    } else {
+        t = from_hi_word((uint32_t)(0x3ff - k) << 20);      // 2^-k
+        y = x - (e + t);
+        y += one;
+        y = add_to_hi_word(y, (uint32_t)k << 20);
+    }
+    return y;
+}
+
+ZM_HD double tanh_fdlibm(double x)
+{
+    const double one = 1.0, two = 2.0, tiny = 1.0e-300;
+    const uint64_t bits = d2u(x);
+    const uint32_t jx = (uint32_t)(bits >> 32), lx = (uint32_t)bits;
+    const uint32_t ix = jx & 0x7fffffffu;
+    const bool neg = (jx >> 31) != 0;
+    double t, z;
+    if (ix >= 0x7ff00000u) return neg ? one / x - one : one / x + one;   // inf or NaN
+    if (ix < 0x40360000u) {                  // |x| < 22
+        if ((ix | lx) == 0) return x;        // +-0
+        if (ix < 0x3c800000u) return x * (one + x);   // |x| < 2^-55
+        const double ax = u2d(bits & 0x7fffffffffffffffull);
+        if (ix >= 0x3ff00000u) {             // |x| >= 1
+            t = expm1_fdlibm(two * ax);
+            z = one - two / (t + two);
+        } else {
+            t = expm1_fdlibm(-two * ax);
+            z = -t / (t + two);
+        }
+    } else {
+        z = one - tiny;
+    }
+    return neg ? -z : z;
+}
+
+// ZeNu's sigmoid composite in f64
+ZM_HD double sigmoid_zenu(double x)
+{
+    double xh = x * 0.5;
+    double th = tanh_fdlibm(xh);
+    double ht = 0.5 * th;
+    return 0.5 + ht;
 }
 
 // ZeNu's sigmoid composite in f32: each step rounded to f32, as the four autograd ops do.
