@@ -1,5 +1,5 @@
 // Host build of zenu_amd/csrc/zmath.hpp compared with the host libm (the functions ZeNu's CPU path
-// calls through Rust's f32::tanh).  Usage: zmath_host_check <stride>; checks every stride-th f32
+// calls through Rust's f32::tanh / exp / ln and f64::tanh).  Usage: zmath_host_check <stride>; checks every stride-th f32
 // bit pattern (stride 1 = exhaustive, about a minute on 8 cores).  Prints the mismatch counts.
 #include <atomic>
 #include <cmath>
@@ -14,13 +14,17 @@ int main(int argc, char **argv)
 {
     const uint64_t stride = argc > 1 ? strtoull(argv[1], nullptr, 10) : 1;
     const int nt = 8;
-    std::atomic<uint64_t> bad_fdlibm{0}, bad_simd{0}, bad_expm1{0}, bad_sig{0};
+    std::atomic<uint64_t> bad_fdlibm{0}, bad_simd{0}, bad_expm1{0}, bad_sig{0}, bad_exp{0}, bad_log{0};
     std::vector<std::thread> th;
     for (int w = 0; w < nt; w++)
         th.emplace_back([&, w]() {
-            uint64_t b0 = 0, b1 = 0, b2 = 0, b3 = 0;
+            uint64_t b0 = 0, b1 = 0, b2 = 0, b3 = 0, b4 = 0, b5 = 0;
             for (uint64_t u = (uint64_t)w * stride; u < (1ull << 32); u += stride * nt) {
                 const float x = zmath::u2f((uint32_t)u);
+                const float er = expf(x), eg = zmath::expf_glibc(x);
+                if ((er != er) ? !(eg != eg) : zmath::f2u(eg) != zmath::f2u(er)) b4++;
+                const float lr = logf(x), lg = zmath::logf_glibc(x);
+                if ((lr != lr) ? !(lg != lg) : zmath::f2u(lg) != zmath::f2u(lr)) b5++;
                 const float ref = tanhf(x);
                 const float a = zmath::tanhf_fdlibm(x), s = zmath::tanhf_simd(x);
                 const bool nan = ref != ref;
@@ -30,7 +34,7 @@ int main(int argc, char **argv)
                 const float sg = 0.5f + 0.5f * tanhf(0.5f * x), sz = zmath::sigmoidf_zenu(x);
                 if ((sg != sg) ? !(sz != sz) : zmath::f2u(sz) != zmath::f2u(sg)) b3++;
             }
-            bad_fdlibm += b0; bad_simd += b1; bad_expm1 += b2; bad_sig += b3;
+            bad_fdlibm += b0; bad_simd += b1; bad_expm1 += b2; bad_sig += b3; bad_exp += b4; bad_log += b5;
         });
     for (auto &t : th) t.join();
     // double precision: every stride-th value of the HIGH word (sign, exponent, 20 mantissa bits) with
@@ -60,5 +64,6 @@ int main(int argc, char **argv)
            (unsigned long long)bad_expm1.load(), (unsigned long long)bad_sig.load());
     printf("tanh_fdlibm %llu expm1_fdlibm %llu sigmoid_zenu %llu\n", (unsigned long long)bad_tanh64.load(),
            (unsigned long long)bad_expm164.load(), (unsigned long long)bad_sig64.load());
-    return (bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64) ? 1 : 0;
+    printf("expf_glibc %llu logf_glibc %llu\n", (unsigned long long)bad_exp.load(), (unsigned long long)bad_log.load());
+    return (bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64 + bad_exp + bad_log) ? 1 : 0;
 }

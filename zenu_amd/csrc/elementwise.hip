@@ -78,11 +78,15 @@ __device__ __forceinline__ double dev_sigmoid(double x) { return zmath::sigmoid_
 
 template <typename T, int FN> struct UnaryF {
     static constexpr int NIN = 1;
-    __device__ __forceinline__ void init() {}
+    zmath::ExpLog<T> m;     // exp / log state (f32: tables in LDS)
+    __device__ __forceinline__ void init()
+    {
+        if constexpr (FN == ZENU_EXP || FN == ZENU_LOG) m.init(FN == ZENU_EXP, FN == ZENU_LOG);
+    }
     __device__ __forceinline__ T operator()(T a, T) const
     {
-        if constexpr (FN == ZENU_EXP) return exp(a);
-        else if constexpr (FN == ZENU_LOG) return log(a);
+        if constexpr (FN == ZENU_EXP) return m.exp(a);
+        else if constexpr (FN == ZENU_LOG) return m.log(a);
         else if constexpr (FN == ZENU_TANH) return dev_tanh(a);
         else if constexpr (FN == ZENU_SQRT) return sqrt(a);
         else if constexpr (FN == ZENU_ABS) return fabs(a);
@@ -175,7 +179,6 @@ template <typename T, int VEC, bool NT, typename F>
 __global__ __launch_bounds__(ContigShape<F>::kBlock) void ew_contig_kernel(T *out, const T *a, const T *b,
                                                                          int64_t n, F f)
 {
-    f.init();
     constexpr int kBlock = ContigShape<F>::kBlock;
     constexpr int kUnroll = ContigShape<F>::kUnroll;
     constexpr int64_t kTile = (int64_t)kBlock * VEC * kUnroll;
@@ -190,12 +193,14 @@ __global__ __launch_bounds__(ContigShape<F>::kBlock) void ew_contig_kernel(T *ou
             if constexpr (F::NIN == 2) vb[u] = load_pack<T, VEC, NT>(b + i);
             else vb[u] = va[u];
         }
+        f.init();   // after the loads are issued: what it fetches (a device scalar, a table) overlaps them
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             int64_t i = base + ((int64_t)u * kBlock + tid) * VEC;
             store_pack<T, VEC, NT>(out + i, apply_pack<T, VEC, F>(f, va[u], vb[u]));
         }
     } else {
+        f.init();
         for (int u = 0; u < kUnroll; u++) {
             int64_t i = base + ((int64_t)u * kBlock + tid) * VEC;
 #pragma unroll

@@ -8,7 +8,7 @@
 //   Linear bias add + ReLU          zenu-layer/src/layers/linear.rs:27-31, zenu-autograd/src/activation/relu.rs:24-33
 //
 // Every element goes through the same sequence of individually rounded operations as in the
-// chain (no contraction, exp/log from the device math library), so the fused results differ
+// chain (no contraction; f32 exp/log are the host libm's algorithm, zmath.hpp), so the fused results differ
 // from the chain only where the chain itself is order dependent: the sums.  The "lines" kernels
 // (one thread per softmax line) add in index order, exactly like sum.rs:20-25; the
 // workgroup-per-row kernels add in a fixed tree.
@@ -19,6 +19,7 @@
 
 #include "common.hpp"
 #include "vecmem.hpp"
+#include "zmath.hpp"
 
 namespace zenu {
 namespace {
@@ -57,6 +58,8 @@ template <typename T, bool CE>
 __global__ __launch_bounds__(kBlock) void softmax_lines_kernel(const T *x, T *y, int64_t lines, int64_t R,
                                                                 int64_t inner, const T *target, T *rowloss)
 {
+    zmath::ExpLog<T> ml;
+    ml.init(true, CE);
     const int64_t line = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (line >= lines) return;
     int64_t q = line, c = 0;
@@ -76,7 +79,7 @@ __global__ __launch_bounds__(kBlock) void softmax_lines_kernel(const T *x, T *y,
     // exp(x - max), summed in index order starting from zero (sum.rs:20-25)
     T sum = (T)0;
     for (int64_t r = 0; r < R; r++) {
-        const T e = exp(xl[r * inner] - m);
+        const T e = ml.exp(xl[r * inner] - m);
         yl[r * inner] = e;
         sum = sum + e;
     }
@@ -84,7 +87,7 @@ __global__ __launch_bounds__(kBlock) void softmax_lines_kernel(const T *x, T *y,
     for (int64_t r = 0; r < R; r++) {
         const T s = yl[r * inner] / sum;
         yl[r * inner] = s;
-        if (CE) acc = acc + target[base + r * inner] * log(s);
+        if (CE) acc = acc + target[base + r * inner] * ml.log(s);
     }
     if (CE) rowloss[line] = acc;
 }
@@ -94,6 +97,8 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
                                                                T *rowloss)
 {
     __shared__ T lds[4];
+    zmath::ExpLog<T> ml;
+    if (!REG) ml.init(true, CE);
     const int64_t row = blockIdx.x;
     const T *xr = x + row * R;
     T *yr = y + row * R;
@@ -113,6 +118,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
 #pragma unroll
             for (int j = 0; j < VEC; j++) m = combine<T, true>(m, v[k].v[j]);
         }
+        ml.init(true, CE);      // after the row's loads are issued: the table fetch overlaps them
         m = block_red<T, true, kBlock>(m, lds);
         if (x0 != x0) m = x0;   // a NaN in position 0 is never replaced
         T sum = (T)0;
@@ -121,7 +127,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
             if (first + k * step < R) {
 #pragma unroll
                 for (int j = 0; j < VEC; j++) {
-                    v[k].v[j] = exp(v[k].v[j] - m);
+                    v[k].v[j] = ml.exp(v[k].v[j] - m);
                     sum = sum + v[k].v[j];
                 }
             }
@@ -137,7 +143,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
                 for (int j = 0; j < VEC; j++) {
                     const T s = v[k].v[j] / sum;
                     v[k].v[j] = s;
-                    if (CE) acc = acc + t.v[j] * log(s);
+                    if (CE) acc = acc + t.v[j] * ml.log(s);
                 }
                 store_pack<T, VEC, NT && !CE>(yr + r, v[k]);   // the CE output is read again by the backward pass
             }
@@ -156,7 +162,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
             Pack<T, VEC> v = load_pack<T, VEC, false>(xr + r);
 #pragma unroll
             for (int j = 0; j < VEC; j++) {
-                v.v[j] = exp(v.v[j] - m);
+                v.v[j] = ml.exp(v.v[j] - m);
                 sum = sum + v.v[j];
             }
             store_pack<T, VEC, false>(yr + r, v);
@@ -170,7 +176,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
             for (int j = 0; j < VEC; j++) {
                 const T s = v.v[j] / sum;
                 v.v[j] = s;
-                if (CE) acc = acc + t.v[j] * log(s);
+                if (CE) acc = acc + t.v[j] * ml.log(s);
             }
             store_pack<T, VEC, false>(yr + r, v);
         }

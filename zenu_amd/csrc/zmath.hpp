@@ -18,6 +18,7 @@
 // tanhf/expm1f over every f32 bit pattern in tests/test_zmath_host.py (sampled) and was run
 // exhaustively during development.
 #pragma once
+#include <math.h>
 #include <stdint.h>
 #include <string.h>
 
@@ -238,6 +239,122 @@ ZM_HD float tanhf_simd(float x)
     return neg ? -z : z;
 }
 
+// ---- f32 exp and log: the table-driven routines glibc ships since 2.27 (from ARM's optimized routines) ----
+// expf:  x*N/ln2 = k + r, N = 32;  exp(x) = 2^(k/N) * 2^(r/N) ~ T[k % N] * 2^(k / N) * (C0 r^3 + C1 r^2 + C2 r + 1),
+//        evaluated in double and rounded once to float.
+// logf:  x = 2^k z, z in [0x3f330000, 2*0x3f330000) split into N = 16 intervals with centre c;
+//        log(x) = log1p(z/c - 1) + log(c) + k ln2, a cubic in r = z * (1/c) - 1, in double.
+// The reduction r = fma(InvLn2N, x, -k) is the fused form that the x86-64 build with FMA (the one a
+// CPU with FMA selects at run time) produces; with it the results equal the host libm's on every
+// f32 bit pattern (the non-fused form differs on 2 of the 2^32 inputs of expf, by one ulp).
+// Checked exhaustively by tests/native/zmath_host_check.cpp.
+
+#define ZM_EXP2F_TAB                                                                                        \
+    { 0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,           \
+      0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull,           \
+      0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull,           \
+      0x3feebfdad5362a27ull, 0x3feeb42b569d4f82ull, 0x3feeab07dd485429ull, 0x3feea47eb03a5585ull,           \
+      0x3feea09e667f3bcdull, 0x3fee9f75e8ec5f74ull, 0x3feea11473eb0187ull, 0x3feea589994cce13ull,           \
+      0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull,           \
+      0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,           \
+      0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull }
+// {1/c, log(c)} per interval
+#define ZM_LOGF_TAB                                                                                         \
+    { 0x1.661ec79f8f3bep+0, -0x1.57bf7808caadep-2, 0x1.571ed4aaf883dp+0, -0x1.2bef0a7c06ddbp-2,             \
+      0x1.49539f0f010bp+0, -0x1.01eae7f513a67p-2, 0x1.3c995b0b80385p+0, -0x1.b31d8a68224e9p-3,              \
+      0x1.30d190c8864a5p+0, -0x1.6574f0ac07758p-3, 0x1.25e227b0b8eap+0, -0x1.1aa2bc79c81p-3,                \
+      0x1.1bb4a4a1a343fp+0, -0x1.a4e76ce8c0e5ep-4, 0x1.12358f08ae5bap+0, -0x1.1973c5a611cccp-4,             \
+      0x1.0953f419900a7p+0, -0x1.252f438e10c1ep-5, 0x1p+0, 0x0p+0,                                          \
+      0x1.e608cfd9a47acp-1, 0x1.aa5aa5df25984p-5, 0x1.ca4b31f026aap-1, 0x1.c5e53aa362eb4p-4,                \
+      0x1.b2036576afce6p-1, 0x1.526e57720db08p-3, 0x1.9c2d163a1aa2dp-1, 0x1.bc2860d22477p-3,                \
+      0x1.886e6037841edp-1, 0x1.1058bc8a07ee1p-2, 0x1.767dcf5534862p-1, 0x1.4043057b6ee09p-2 }
+
+static const uint64_t kExp2fTabHost[32] = ZM_EXP2F_TAB;
+static const double kLogfTabHost[32] = ZM_LOGF_TAB;
+#if defined(__HIPCC__)
+static __device__ const uint64_t kExp2fTabDev[32] = ZM_EXP2F_TAB;
+static __device__ const double kLogfTabDev[32] = ZM_LOGF_TAB;
+#endif
+
+// the tables as seen from the code being compiled (device: global memory; kernels that evaluate
+// many elements copy them into LDS first, a gather from global memory costs a tag lookup per lane)
+ZM_HD const uint64_t *exp2f_table()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return kExp2fTabDev;
+#else
+    return kExp2fTabHost;
+#endif
+}
+ZM_HD const double *logf_table()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return kLogfTabDev;
+#else
+    return kLogfTabHost;
+#endif
+}
+
+ZM_HD uint64_t d2u(double d);
+ZM_HD double u2d(uint64_t u);
+
+ZM_HD float expf_glibc(float x, const uint64_t *tab)
+{
+    const double InvLn2N = 0x1.71547652b82fep+0 * 32, Shift = 0x1.8p+52;
+    const double C0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32, C1 = 0x1.ebfce50fac4f3p-3 / 32 / 32,
+                 C2 = 0x1.62e42ff0c52d6p-1 / 32;
+    const uint32_t ux = f2u(x);
+    const uint32_t abstop = (ux >> 20) & 0x7ffu;
+    if (abstop >= (0x42b00000u >> 20)) {                 // |x| >= 88 or NaN
+        if (ux == 0xff800000u) return 0.0f;              // -inf
+        if (abstop >= (0x7f800000u >> 20)) return x + x; // +inf, NaN
+        if (x > 0x1.62e42ep6f) return u2f(0x7f800000u);  // overflow
+        if (x < -0x1.9fe368p6f) return 0.0f;             // underflow
+    }
+    const double xd = (double)x;
+    const double z = InvLn2N * xd;
+    double kd = z + Shift;
+    const uint64_t ki = d2u(kd);
+    kd -= Shift;
+    const double r = __builtin_fma(InvLn2N, xd, -kd);
+    const uint64_t t = tab[ki % 32] + (ki << (52 - 5));
+    const double s = u2d(t);
+    const double p = __builtin_fma(C0, r, C1);
+    const double r2 = r * r;
+    double y = __builtin_fma(C2, r, 1.0);
+    y = __builtin_fma(p, r2, y);
+    y = y * s;
+    return (float)y;
+}
+
+ZM_HD float logf_glibc(float x, const double *tab)
+{
+    const double A0 = -0x1.00ea348b88334p-2, A1 = 0x1.5575b0be00b6ap-2, A2 = -0x1.ffffef20a4123p-2;
+    const double Ln2 = 0x1.62e42fefa39efp-1;
+    uint32_t ix = f2u(x);
+    if (ix == 0x3f800000u) return 0.0f;
+    if (ix - 0x00800000u >= 0x7f800000u - 0x00800000u) { // x < 2^-126, inf or NaN
+        if (ix * 2 == 0) return u2f(0xff800000u);        // log(+-0) = -inf
+        if (ix == 0x7f800000u) return x;                 // log(inf) = inf
+        if ((ix & 0x80000000u) || ix * 2 >= 0xff000000u) return (x - x) / (x - x);   // NaN
+        ix = f2u(x * 0x1p23f);                           // subnormal: normalise
+        ix -= 23u << 23;
+    }
+    const uint32_t tmp = ix - 0x3f330000u;
+    const uint32_t i = (tmp >> (23 - 4)) % 16;
+    const int32_t k = (int32_t)tmp >> 23;
+    const uint32_t iz = ix - (tmp & (0x1ffu << 23));
+    const double invc = tab[2 * i], logc = tab[2 * i + 1];
+    const double z = (double)u2f(iz);
+    const double r = __builtin_fma(z, invc, -1.0);
+    const double y0 = __builtin_fma((double)k, Ln2, logc);
+    const double r2 = r * r;
+    double y = __builtin_fma(A1, r, A2);
+    y = __builtin_fma(A0, r2, y);
+    y = __builtin_fma(y, r2, y0 + r);
+    return (float)y;
+}
+
 // ---- double precision: fdlibm s_expm1.c / s_tanh.c as shipped by glibc 2.35 (generic dbl-64) ----------
 
 ZM_HD uint64_t d2u(double d)
@@ -392,5 +509,38 @@ ZM_HD float sigmoidf_zenu(float x)
     float ht = half * th;
     return half + ht;
 }
+
+// what the kernels call: f32 from the restatements above, f64 exp / log from the math library
+ZM_HD float expf_glibc(float x) { return expf_glibc(x, exp2f_table()); }
+ZM_HD float logf_glibc(float x) { return logf_glibc(x, logf_table()); }
+
+#if defined(__HIPCC__)
+// exp / log as the kernels call them: f32 through tables copied to LDS by init(), which every
+// thread of the workgroup calls once before anything else (it synchronises); f64 from the math
+// library.
+template <typename T> struct ExpLog {
+    __device__ __forceinline__ void init(bool, bool) {}
+    __device__ __forceinline__ T exp(T x) const { return ::exp(x); }
+    __device__ __forceinline__ T log(T x) const { return ::log(x); }
+};
+template <> struct ExpLog<float> {
+    const uint64_t *etab;
+    const double *ltab;
+    __device__ __forceinline__ void init(bool need_exp, bool need_log)
+    {
+        __shared__ uint64_t lds_exp[32];
+        __shared__ double lds_log[32];
+        if (threadIdx.x < 32) {
+            if (need_exp) lds_exp[threadIdx.x] = kExp2fTabDev[threadIdx.x];
+            if (need_log) lds_log[threadIdx.x] = kLogfTabDev[threadIdx.x];
+        }
+        __syncthreads();
+        etab = lds_exp;
+        ltab = lds_log;
+    }
+    __device__ __forceinline__ float exp(float x) const { return expf_glibc(x, etab); }
+    __device__ __forceinline__ float log(float x) const { return logf_glibc(x, ltab); }
+};
+#endif
 
 }  // namespace zmath
