@@ -1,6 +1,7 @@
 // Host build of zenu_amd/csrc/zmath.hpp compared with the host libm (the functions ZeNu's CPU path
 // calls through Rust's f32::tanh / exp / ln and f64::tanh).  Usage: zmath_host_check <stride>; checks every stride-th f32
-// bit pattern (stride 1 = exhaustive, about a minute on 8 cores).  Prints the mismatch counts.
+// bit pattern (stride 1 = exhaustive, about a minute on 8 cores).  powf: every stride-th x for a set
+// of fixed exponents, and 2^32 / stride pseudo-random (x, y) pairs.  Prints the mismatch counts.
 #include <atomic>
 #include <cmath>
 #include <cstdio>
@@ -59,11 +60,36 @@ int main(int argc, char **argv)
             bad_tanh64 += b0; bad_expm164 += b1; bad_sig64 += b2;
         });
     for (auto &t : th) t.join();
+    // powf(x, y)
+    std::atomic<uint64_t> bad_pow{0};
+    th.clear();
+    for (int w = 0; w < nt; w++)
+        th.emplace_back([&, w]() {
+            uint64_t b = 0, rng = 0xD1B54A32D192ED03ull * (w + 1);
+            auto one = [&](float x, float y) {
+                const float ref = powf(x, y), got = zmath::powf_glibc(x, y);
+                if ((ref != ref) ? !(got != got) : zmath::f2u(got) != zmath::f2u(ref)) b++;
+            };
+            const float ys[] = {2.0f, 0.5f, 2.5f, -1.0f, 3.0f, 1.5f, -0.5f, 0.333333343f, 10.0f, -2.5f, 0.0f, 1.0f,
+                                INFINITY, -INFINITY, NAN, zmath::u2f(0x7f800001u), 1e-30f, 16777217.0f, 5.0f};
+            for (uint64_t u = (uint64_t)w * stride; u < (1ull << 32); u += stride * nt) {
+                for (float y : ys) one(zmath::u2f((uint32_t)u), y);
+                rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17;
+                one(zmath::u2f((uint32_t)rng), zmath::u2f((uint32_t)(rng >> 32)));
+                // moderate arguments, where the result is finite and the tables decide it
+                const float xm = zmath::u2f(0x3c000000u + (uint32_t)(rng % 0x08000000u));           // [2^-7, 2^9)
+                const float ym = zmath::u2f((0x3c000000u + (uint32_t)((rng >> 29) % 0x07000000u)) | ((uint32_t)(rng >> 63) << 31));
+                one(xm, ym);
+            }
+            bad_pow += b;
+        });
+    for (auto &t : th) t.join();
     printf("tanhf_fdlibm %llu tanhf_simd %llu expm1f_fdlibm %llu sigmoidf_zenu %llu\n",
            (unsigned long long)bad_fdlibm.load(), (unsigned long long)bad_simd.load(),
            (unsigned long long)bad_expm1.load(), (unsigned long long)bad_sig.load());
     printf("tanh_fdlibm %llu expm1_fdlibm %llu sigmoid_zenu %llu\n", (unsigned long long)bad_tanh64.load(),
            (unsigned long long)bad_expm164.load(), (unsigned long long)bad_sig64.load());
     printf("expf_glibc %llu logf_glibc %llu\n", (unsigned long long)bad_exp.load(), (unsigned long long)bad_log.load());
-    return (bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64 + bad_exp + bad_log) ? 1 : 0;
+    printf("powf_glibc %llu\n", (unsigned long long)bad_pow.load());
+    return (bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64 + bad_exp + bad_log + bad_pow) ? 1 : 0;
 }

@@ -3,9 +3,9 @@ configurations (full size) and on edge cases.  Everything goes through the C ABI
 
 Bars (written where they are used):
   add/sub/mul/div, relu, max, arg-max, copy, SGD/Adam/AdamW .......... bit-exact
-  f32 exp, log; tanh, sigmoid in f32 and f64 (the host libm's algorithms,
-      restated) ....................................................... bit-exact (bar: <= 2 ulp)
-  f64 exp, log (device math library) .................................. <= 2 ulp
+  f32 exp, log, powf; tanh, sigmoid in f32 and f64 (the host libm's
+      algorithms, restated) ........................................... bit-exact (bar: <= 2 ulp)
+  f64 exp, log, powf (device math library) ............................ <= 2 ulp
   sums ................................................................ |gpu - cpu| <= 1e-5 (f32) /
       1e-12 (f64) times max(|cpu|, sum|x| / sqrt(n)); the second term is the typical magnitude
       of a sum of n such terms, so a result that cancels to ~0 is not held to a relative bar
@@ -278,6 +278,43 @@ def test_unary_f64(hip):
     fin = ~np.isnan(exp)
     assert np.array_equal(np.isnan(got), np.isnan(exp)) and max_ulp(got[fin], exp[fin]) == 0
     del X, W
+
+
+def test_powf(hip):
+    """powf (zenu-matrix/src/device/cpu/basic_operations.rs pow: `x.powf(scalar)` per element):
+    f32 has the host libm's bits for every exponent class -- integer, half-integer, negative,
+    fractional, zero, infinite, NaN -- over bases that include negatives, zeros, subnormals and
+    non-finite values; f64 comes from the device math library (<= 2 ulp on finite results)."""
+    r = rng(17)
+    base = np.concatenate([
+        r.standard_normal(200000).astype(np.float32) * 3,
+        np.exp(r.uniform(-80, 80, 200000)).astype(np.float32),
+        r.integers(0, 1 << 32, 200000, dtype=np.uint64).astype(np.uint32).view(np.float32),
+        np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1.1754944e-38, 3e38, -3e38, 2.0, -2.0,
+                  0.5, -0.5, 3.0, -3.0], dtype=np.float32)])
+    X = hip.Matrix.from_numpy(base)
+    exp = np.empty_like(base)
+    for y in (2.0, 0.5, 3.0, -1.0, 2.5, -0.5, 1.0 / 3.0, 0.0, 1.0, 10.0, -7.0, 1e-30, 40.25, np.inf, -np.inf, np.nan):
+        with np.errstate(all="ignore"):
+            zo.powf(exp, base, y)
+        got = X.powf_array(y).to_numpy()
+        assert np.array_equal(np.isnan(got), np.isnan(exp)), y
+        fin = ~np.isnan(exp)
+        assert max_ulp(got[fin], exp[fin]) == 0, y
+    # a strided view (every other column of a transposed matrix) takes the same path
+    m = np.abs(r.standard_normal((96, 130))).astype(np.float32) + 0.01
+    Mv = hip.Matrix.from_numpy(m).transpose().slice(slice(None, None, 2))
+    e2 = np.empty((65, 96), dtype=np.float32)
+    zo.powf(e2, np.ascontiguousarray(m.T[::2]), 1.7)
+    assert max_ulp(Mv.powf_array(1.7).to_numpy(), e2) == 0
+    b64 = np.abs(r.standard_normal(100000)) * 5 + 1e-3
+    e64 = np.empty_like(b64)
+    for y in (2.0, 0.5, -1.5, 3.3):
+        zo.powf(e64, b64, y)
+        u = max_ulp(hip.Matrix.from_numpy(b64).powf_array(y).to_numpy(), e64)
+        print(f"[f64] powf {y}: {u} ulp", flush=True)
+        assert u <= 2, (y, u)
+    del X, Mv
 
 
 # ---- strided / broadcast engine: randomized shapes vs brute force and oracle ------------------------------

@@ -31,10 +31,11 @@ def test_device_tanh_matches_host_libm(tmp_path):
     """zmath.hpp (the tanh / expm1 / sigmoid the kernels use) compiled for the host with
     contraction off must give the bits of tanhf / expm1f / tanh / expm1: every 31st f32 bit pattern
     here (138 M points; stride 1, all 2^32, was run during development with the same result) and,
-    for double, every 31st high word with three low words each (415 M points)."""
+    for double, every 31st high word with three low words each (415 M points); powf on every 31st
+    base for 19 fixed exponents and on two pseudo-random (base, exponent) pairs per base."""
     exe = build("zmath_host_check.cpp", str(tmp_path / "zmath_check"), ("-ffp-contract=off", "-fno-fast-math"))
     out = subprocess.run([exe, "31"], capture_output=True, text=True)
     assert out.returncode == 0, out.stdout
     assert out.stdout.split() == ["tanhf_fdlibm", "0", "tanhf_simd", "0", "expm1f_fdlibm", "0", "sigmoidf_zenu", "0",
                                   "tanh_fdlibm", "0", "expm1_fdlibm", "0", "sigmoid_zenu", "0",
-                                  "expf_glibc", "0", "logf_glibc", "0"]
+                                  "expf_glibc", "0", "logf_glibc", "0", "powf_glibc", "0"]

@@ -105,8 +105,9 @@ template <typename T, int FN> struct UnaryF {
 template <typename T> struct PowF {
     static constexpr int NIN = 1;
     T s;
-    __device__ __forceinline__ void init() {}
-    __device__ __forceinline__ T operator()(T a, T) const { return pow(a, s); }
+    zmath::Pow<T> m;        // f32: tables in LDS
+    __device__ __forceinline__ void init() { m.init(); }
+    __device__ __forceinline__ T operator()(T a, T) const { return m.pow(a, s); }
 };
 
 // relu.rs:44-48: the non-positive branch returns the PRODUCT alpha*x (-0.0 for alpha = 0)

@@ -269,11 +269,24 @@ ZM_HD float tanhf_simd(float x)
       0x1.b2036576afce6p-1, 0x1.526e57720db08p-3, 0x1.9c2d163a1aa2dp-1, 0x1.bc2860d22477p-3,                \
       0x1.886e6037841edp-1, 0x1.1058bc8a07ee1p-2, 0x1.767dcf5534862p-1, 0x1.4043057b6ee09p-2 }
 
+// powf's {1/c, log2(c)} per interval (same centres as logf's)
+#define ZM_POWF_LOG2_TAB                                                                                    \
+    { 0x1.661ec79f8f3bep+0, -0x1.efec65b963019p-2, 0x1.571ed4aaf883dp+0, -0x1.b0b6832d4fca4p-2,             \
+      0x1.49539f0f010bp+0, -0x1.7418b0a1fb77bp-2, 0x1.3c995b0b80385p+0, -0x1.39de91a6dcf7bp-2,              \
+      0x1.30d190c8864a5p+0, -0x1.01d9bf3f2b631p-2, 0x1.25e227b0b8eap+0, -0x1.97c1d1b3b7afp-3,               \
+      0x1.1bb4a4a1a343fp+0, -0x1.2f9e393af3c9fp-3, 0x1.12358f08ae5bap+0, -0x1.960cbbf788d5cp-4,             \
+      0x1.0953f419900a7p+0, -0x1.a6f9db6475fcep-5, 0x1p+0, 0x0p+0,                                          \
+      0x1.e608cfd9a47acp-1, 0x1.338ca9f24f53dp-4, 0x1.ca4b31f026aap-1, 0x1.476a9543891bap-3,                \
+      0x1.b2036576afce6p-1, 0x1.e840b4ac4e4d2p-3, 0x1.9c2d163a1aa2dp-1, 0x1.40645f0c6651cp-2,               \
+      0x1.886e6037841edp-1, 0x1.88e9c2c1b9ff8p-2, 0x1.767dcf5534862p-1, 0x1.ce0a44eb17bccp-2 }
+
 static const uint64_t kExp2fTabHost[32] = ZM_EXP2F_TAB;
 static const double kLogfTabHost[32] = ZM_LOGF_TAB;
+static const double kPowfLog2TabHost[32] = ZM_POWF_LOG2_TAB;
 #if defined(__HIPCC__)
 static __device__ const uint64_t kExp2fTabDev[32] = ZM_EXP2F_TAB;
 static __device__ const double kLogfTabDev[32] = ZM_LOGF_TAB;
+static __device__ const double kPowfLog2TabDev[32] = ZM_POWF_LOG2_TAB;
 #endif
 
 // the tables as seen from the code being compiled (device: global memory; kernels that evaluate
@@ -292,6 +305,15 @@ ZM_HD const double *logf_table()
     return kLogfTabDev;
 #else
     return kLogfTabHost;
+#endif
+}
+
+ZM_HD const double *powf_log2_table()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return kPowfLog2TabDev;
+#else
+    return kPowfLog2TabHost;
 #endif
 }
 
@@ -353,6 +375,97 @@ ZM_HD float logf_glibc(float x, const double *tab)
     y = __builtin_fma(A0, r2, y);
     y = __builtin_fma(y, r2, y0 + r);
     return (float)y;
+}
+
+// powf (glibc's e_powf.c, same origin): x^y = 2^(y log2 x); log2 x as a quartic in r = z/c - 1 around
+// the 16 interval centres, the product y log2(x) and the 2^ step (exp2f's 32-entry table and cubic)
+// all in double, rounded once to float.  Results equal the host libm's with the fused and with
+// the unfused evaluation on every sampled input (tests/native/zmath_host_check.cpp).
+// 0 = not an integer, 1 = odd integer, 2 = even integer
+ZM_HD int powf_checkint(uint32_t iy)
+{
+    const int e = (int)(iy >> 23 & 0xffu);
+    if (e < 0x7f) return 0;
+    if (e > 0x7f + 23) return 2;
+    if (iy & ((1u << (0x7f + 23 - e)) - 1u)) return 0;
+    if (iy & (1u << (0x7f + 23 - e))) return 1;
+    return 2;
+}
+ZM_HD bool powf_zeroinfnan(uint32_t i) { return 2u * i - 1u >= 2u * 0x7f800000u - 1u; }
+ZM_HD bool powf_signaling(uint32_t i) { return 2u * (i ^ 0x00400000u) > 2u * 0x7fc00000u; }
+
+ZM_HD float powf_glibc(float x, float y, const uint64_t *etab, const double *ltab)
+{
+    const double A0 = 0x1.27616c9496e0bp-2, A1 = -0x1.71969a075c67ap-2, A2 = 0x1.ec70a6ca7baddp-2,
+                 A3 = -0x1.7154748bef6c8p-1, A4 = 0x1.71547652ab82bp0;
+    const double C0 = 0x1.c6af84b912394p-5, C1 = 0x1.ebfce50fac4f3p-3, C2 = 0x1.62e42ff0c52d6p-1;
+    const double Shift = 0x1.8p+52 / 32;
+    uint32_t sign_bias = 0;
+    uint32_t ix = f2u(x);
+    const uint32_t iy = f2u(y);
+    if (ix - 0x00800000u >= 0x7f800000u - 0x00800000u || powf_zeroinfnan(iy)) {
+        // x < 2^-126, inf or NaN; or y zero, inf or NaN
+        if (powf_zeroinfnan(iy)) {
+            if (2u * iy == 0) return powf_signaling(ix) ? x + y : 1.0f;
+            if (ix == 0x3f800000u) return powf_signaling(iy) ? x + y : 1.0f;
+            if (2u * ix > 2u * 0x7f800000u || 2u * iy > 2u * 0x7f800000u) return x + y;
+            if (2u * ix == 2u * 0x3f800000u) return 1.0f;
+            if ((2u * ix < 2u * 0x3f800000u) == !(iy & 0x80000000u)) return 0.0f;   // |x|<1, y=inf or |x|>1, y=-inf
+            return y * y;
+        }
+        if (powf_zeroinfnan(ix)) {
+            float x2 = x * x;
+            if ((ix & 0x80000000u) && powf_checkint(iy) == 1) x2 = -x2;
+            return (iy & 0x80000000u) ? 1.0f / x2 : x2;
+        }
+        if (ix & 0x80000000u) {                          // finite x < 0
+            const int yint = powf_checkint(iy);
+            if (yint == 0) return (x - x) / (x - x);
+            if (yint == 1) sign_bias = 1u << (5 + 11);
+            ix &= 0x7fffffffu;
+        }
+        if (ix < 0x00800000u) {                          // subnormal: normalise
+            ix = f2u(x * 0x1p23f);
+            ix &= 0x7fffffffu;
+            ix -= 23u << 23;
+        }
+    }
+    // log2(x) = log1p(z/c - 1)/ln2 + log2(c) + k
+    const uint32_t tmp = ix - 0x3f330000u;
+    const uint32_t i = (tmp >> (23 - 4)) % 16;
+    const uint32_t top = tmp & 0xff800000u;
+    const uint32_t iz = ix - top;
+    const int32_t k = (int32_t)top >> 23;
+    const double invc = ltab[2 * i], logc = ltab[2 * i + 1];
+    const double z = (double)u2f(iz);
+    const double r = __builtin_fma(z, invc, -1.0);
+    const double y0 = logc + (double)k;
+    const double r2 = r * r;
+    double yy = __builtin_fma(A0, r, A1);
+    const double p = __builtin_fma(A2, r, A3);
+    const double r4 = r2 * r2;
+    double q = __builtin_fma(A4, r, y0);
+    q = __builtin_fma(p, r2, q);
+    yy = __builtin_fma(yy, r4, q);
+    const double ylogx = (double)y * yy;                 // cannot overflow: y is single precision
+    if ((d2u(ylogx) >> 47 & 0xffffu) >= (d2u(126.0) >> 47)) {   // |y log2 x| >= 126
+        if (ylogx > 0x1.fffffffd1d571p+6) return u2f(sign_bias ? 0xff800000u : 0x7f800000u);
+        if (ylogx <= -150.0) return u2f(sign_bias ? 0x80000000u : 0u);
+    }
+    // 2^(y log2 x): x' = k/N + r', |r'| <= 1/(2N)
+    double kd = ylogx + Shift;
+    const uint64_t ki = d2u(kd);
+    kd -= Shift;
+    const double rr = ylogx - kd;
+    uint64_t t = etab[ki % 32];
+    t += (ki + sign_bias) << (52 - 5);
+    const double s = u2d(t);
+    const double zz = __builtin_fma(C0, rr, C1);
+    const double rr2 = rr * rr;
+    double out = __builtin_fma(C2, rr, 1.0);
+    out = __builtin_fma(zz, rr2, out);
+    out = out * s;
+    return (float)out;
 }
 
 // ---- double precision: fdlibm s_expm1.c / s_tanh.c as shipped by glibc 2.35 (generic dbl-64) ----------
@@ -513,6 +626,7 @@ ZM_HD float sigmoidf_zenu(float x)
 // what the kernels call: f32 from the restatements above, f64 exp / log from the math library
 ZM_HD float expf_glibc(float x) { return expf_glibc(x, exp2f_table()); }
 ZM_HD float logf_glibc(float x) { return logf_glibc(x, logf_table()); }
+ZM_HD float powf_glibc(float x, float y) { return powf_glibc(x, y, exp2f_table(), powf_log2_table()); }
 
 #if defined(__HIPCC__)
 // exp / log as the kernels call them: f32 through tables copied to LDS by init(), which every
@@ -540,6 +654,29 @@ template <> struct ExpLog<float> {
     }
     __device__ __forceinline__ float exp(float x) const { return expf_glibc(x, etab); }
     __device__ __forceinline__ float log(float x) const { return logf_glibc(x, ltab); }
+};
+
+// pow with the same arrangement: f32 through powf's two tables in LDS, f64 from the math library
+template <typename T> struct Pow {
+    __device__ __forceinline__ void init() {}
+    __device__ __forceinline__ T pow(T x, T y) const { return ::pow(x, y); }
+};
+template <> struct Pow<float> {
+    const uint64_t *etab;
+    const double *ltab;
+    __device__ __forceinline__ void init()
+    {
+        __shared__ uint64_t lds_exp2[32];
+        __shared__ double lds_log2[32];
+        if (threadIdx.x < 32) {
+            lds_exp2[threadIdx.x] = kExp2fTabDev[threadIdx.x];
+            lds_log2[threadIdx.x] = kPowfLog2TabDev[threadIdx.x];
+        }
+        __syncthreads();
+        etab = lds_exp2;
+        ltab = lds_log2;
+    }
+    __device__ __forceinline__ float pow(float x, float y) const { return powf_glibc(x, y, etab, ltab); }
 };
 #endif
 
