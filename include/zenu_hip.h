@@ -318,6 +318,9 @@ int zenu_hip_adam_step_multi(int dtype, int n_tensors, void *const *p_dev, const
     /* array_array.h:27-28: output[i] = input[i] + bias[(i / channel_stride) % bias_size] */      \
     void conv_bias_add_##S(const T *input, T *output, int channel_stride, const T *bias,          \
                            int bias_size, int total_elements);                                     \
+    /* conv2d_bkwd_data.h:7-17: dbias[c] = sum over n, h, w of dOut[n, c, h, w]; follows the CPU  \
+       path (zenu-matrix/src/nn/conv/cpu/bias.rs:18-25: sum(0), sum(2), sum(3)) */                \
+    void conv2d_bias_bkwd_##S(const T *dOut, T *dbias, int N, int C, int H, int W);               \
     /* activations.h:7-11 */                                                                       \
     void relu_##S(T *input, T *output, T alpha, int size, int input_stride, int output_stride);   \
     void relu_backward_mask_##S(T *input, T *mask, T alpha, int size, int input_stride,           \

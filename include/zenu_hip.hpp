@@ -523,6 +523,28 @@ Matrix<T> cross_entropy_backward(const Matrix<T> &prob, const Matrix<T> &ans, co
     return g;
 }
 
+// ---- ConvBias (zenu-matrix/src/nn/conv/mod.rs:84-107; the CPU device's definitions, cpu/bias.rs) ----------------
+
+template <typename T> bool is_channel_bias(const Matrix<T> &bias, const Matrix<T> &x)
+{
+    const Dim &b = bias.shape(), &s = x.shape();
+    return b.size() == 4 && s.size() == 4 && b[0] == 1 && b[2] == 1 && b[3] == 1 && b[1] == s[1];
+}
+
+// output[N,C,H,W] = input + bias[1,C,1,1]
+template <typename T> void conv2d_bias_add(const Matrix<T> &input, const Matrix<T> &bias, const Matrix<T> &output)
+{
+    if (input.shape() != output.shape() || !is_channel_bias(bias, output)) throw Error(ZENU_ERR_SHAPE, "conv2d_bias_add");
+    output.add_array(input, bias);
+}
+
+// d_bias[1,C,1,1] = d_output summed over axes 0, 2 and 3
+template <typename T> void conv2d_bias_bkwd(const Matrix<T> &d_output, const Matrix<T> &d_bias)
+{
+    if (!is_channel_bias(d_bias, d_output)) throw Error(ZENU_ERR_SHAPE, "conv2d_bias_bkwd");
+    d_output.sum_to(d_bias);
+}
+
 // ---- optimizers: name -> (parameter, gradient); a default-constructed gradient means "no grad" -----------------
 
 template <typename T> struct ParamGrad {

@@ -209,6 +209,16 @@ def sum_to(source, target):
     zo.sum_to(source.a, target.a)
 
 
+def conv2d_bias_add(input, bias, output):
+    """ConvBias for Cpu, zenu-matrix/src/nn/conv/cpu/bias.rs:10-16"""
+    output.add_array(input, bias)
+
+
+def conv2d_bias_bkwd(d_output, d_bias):
+    """zenu-matrix/src/nn/conv/cpu/bias.rs:18-25: sum(0, true), sum(2, true), sum(3, true), copy_from"""
+    d_bias.copy_from(d_output.sum(0, True).sum(2, True).sum(3, True))
+
+
 def softmax_backward(y, gy, axis):
     """SoftMax::backward, zenu-autograd/src/loss/softmax.rs:33-40"""
     gx = y * gy

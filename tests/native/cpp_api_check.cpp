@@ -259,6 +259,27 @@ static void broadcast_cases() // broadcast.rs:53-165
     REQUIRE(eq(r1, {1, 1, 1}));
 }
 
+static void conv_bias_cases() // zenu-matrix/src/nn/conv/mod.rs:84-107, cpu/bias.rs:10-25
+{
+    const int n = 2, c = 3, h = 2, w = 4;
+    M x = M::from_vec(iota(n * c * h * w), {n, c, h, w});
+    M b = M::from_vec({10, 20, 30}, {1, c, 1, 1});
+    M y = M::zeros({n, c, h, w});
+    conv2d_bias_add(x, b, y);
+    std::vector<float> exp = iota(n * c * h * w);
+    std::vector<float> gexp(c, 0.f);
+    for (int i = 0; i < n * c * h * w; i++) {
+        const int ch = (i / (h * w)) % c;
+        gexp[ch] += exp[i];            // small integers: exact in any order
+        exp[i] += 10.f * (ch + 1);
+    }
+    REQUIRE(eq(y, exp));
+    M g = M::zeros({1, c, 1, 1});
+    conv2d_bias_bkwd(x, g);
+    REQUIRE(eq(g, gexp));
+    REQUIRE(throws_status(ZENU_ERR_SHAPE, [&] { conv2d_bias_bkwd(x, M::zeros({c})); }));
+}
+
 // ---- softmax, cross-entropy, clip ----------------------------------------------------------------------------------
 
 static void softmax_cases()   // softmax.rs:37-91; loss/softmax.rs:70-103
@@ -394,7 +415,8 @@ int main(int argc, char **argv)
         {"broadcast_add_1x4x1x1_3x4x5x5", broadcast_add_1x4x1x1_3x4x5x5}, {"sub_mul_div", sub_mul_div},
         {"shape_errors", shape_errors}, {"unary_tables", unary_tables}, {"relu_cases", relu_cases},
         {"sigmoid_cases", sigmoid_cases}, {"sum_4d", sum_4d}, {"max_cases", max_cases}, {"asum_cases", asum_cases},
-        {"copy_cases", copy_cases}, {"broadcast_cases", broadcast_cases}, {"softmax_cases", softmax_cases},
+        {"copy_cases", copy_cases}, {"broadcast_cases", broadcast_cases}, {"conv_bias_cases", conv_bias_cases},
+        {"softmax_cases", softmax_cases},
         {"cross_entropy_cases", cross_entropy_cases}, {"clip_cases", clip_cases}, {"sgd_net_test", sgd_net_test},
         {"adam_net_test", adam_net_test}, {"adam_w_net_test", adam_w_net_test},
     };

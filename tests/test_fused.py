@@ -239,3 +239,34 @@ def test_reference_named_clip_and_conv_bias_add(hip):
         exp[:total] = x[:total] + bias[(idx // hw) % c]
         assert bits_equal(out.to_numpy(), exp), total
     del fp
+
+
+def test_conv2d_bias_add_and_backward(hip):
+    """ConvBias (zenu-matrix/src/nn/conv/mod.rs:84-107, cpu/bias.rs): the forward add is bit-exact;
+    the bias gradient is three sums (sum bar), and the reference-named entry
+    conv2d_bias_bkwd_<type> (conv2d_bkwd_data.h:7-17) gives the same numbers."""
+    r = np.random.default_rng(23)
+    for dt, tol in ((np.float32, 1e-5), (np.float64, 1e-12)):
+        for (n, c, h, w) in ((4, 3, 5, 7), (16, 64, 28, 28), (1, 8, 1, 1), (3, 1, 2, 33)):
+            x = r.standard_normal((n, c, h, w)).astype(dt)
+            b = r.standard_normal((1, c, 1, 1)).astype(dt)
+            hx, hb, ho = hip.Matrix.from_numpy(x), hip.Matrix.from_numpy(b), hip.Matrix.zeros(x.shape, dt)
+            cx, cb, co = CpuMatrix.from_numpy(x), CpuMatrix.from_numpy(b), CpuMatrix.zeros(x.shape, dt)
+            hip.conv2d_bias_add(hx, hb, ho)
+            cpu_matrix.conv2d_bias_add(cx, cb, co)
+            assert bits_equal(ho.to_numpy(), co.a)
+            hg, cg = hip.Matrix.zeros(b.shape, dt), CpuMatrix.zeros(b.shape, dt)
+            hip.conv2d_bias_bkwd(hx, hg)
+            cpu_matrix.conv2d_bias_bkwd(cx, cg)
+            scale = np.maximum(np.abs(cg.a), np.abs(x).sum(axis=(0, 2, 3)).reshape(b.shape) / np.sqrt(n * h * w))
+            assert np.all(np.abs(hg.to_numpy() - cg.a) <= tol * scale), (dt, n, c, h, w)
+            # the reference-named C entry point
+            L = hip.lib()
+            f = getattr(L, "conv2d_bias_bkwd_" + ("float" if dt == np.float32 else "double"))
+            f.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int]
+            f.restype = None
+            hg2 = hip.Matrix.zeros(b.shape, dt)
+            f(hx.as_ptr(), hg2.as_ptr(), n, c, h, w)
+            assert bits_equal(hg2.to_numpy(), hg.to_numpy())
+    with pytest.raises(hip.ZenuHipError):
+        hip.conv2d_bias_bkwd(hx, hip.Matrix.zeros((1, c + 1, 1, 1), dt))

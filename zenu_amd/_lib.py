@@ -113,7 +113,7 @@ def reference_named_symbols():
         names += [f"relu_{s}", f"relu_backward_mask_{s}", f"array_max_idx_{s}",
                   f"memory_access_{s}", f"memory_set_{s}",
                   f"array_clip_{s}", f"array_clip_assign_{s}", f"array_clip_backward_{s}",
-                  f"array_clip_backward_assign_{s}", f"conv_bias_add_{s}"]
+                  f"array_clip_backward_assign_{s}", f"conv_bias_add_{s}", f"conv2d_bias_bkwd_{s}"]
     return names
 
 

@@ -101,6 +101,27 @@ void conv_bias(const T *in, T *out, int cs, const T *bias, int C, int total)
     }
 }
 
+// d_bias[c] = sum over n, h, w of d_output[n, c, h, w] (NCHW, contiguous), as the CPU path defines it:
+// sum(0), sum(2), sum(3) in that order (zenu-matrix/src/nn/conv/cpu/bias.rs:18-25).  The CUDA kernel
+// of the same name (conv2d_bkwd_data.cu:120-156) reads channel c as ONE run of N*H*W elements, which
+// is that sum only for N = 1; the CPU path is the one followed.
+template <typename T> void conv_bias_bkwd(const T *dout, T *dbias, int N, int C, int H, int W)
+{
+    if (C <= 0) return;
+    zenu_tensor_t src = view1d(dout, 0, 0), dst = view1d(dbias, 0, 0);
+    src.ndim = dst.ndim = 4;
+    const int64_t shape[4] = {N, C, H, W};
+    int64_t st = 1;
+    for (int i = 3; i >= 0; i--) {
+        src.shape[i] = shape[i];
+        src.stride[i] = st;
+        st *= shape[i];
+        dst.shape[i] = (i == 1) ? C : 1;
+        dst.stride[i] = (i == 0) ? C : 1;
+    }
+    (void)zenu_hip_sum_to(dtype_of<T>(), &dst, &src, nullptr);
+}
+
 template <typename T> void max_idx(T *a, int size, int stride, int *out)
 {
     // `out` is host memory (zenu-cuda/src/kernel/mod.rs:570-588): blocking, like the reference
@@ -176,6 +197,10 @@ extern "C" {
     void conv_bias_add_##S(const T *in, T *out, int channel_stride, const T *bias, int bias_size, int total) \
     {                                                                                                      \
         conv_bias<T>(in, out, channel_stride, bias, bias_size, total);                                     \
+    }                                                                                                      \
+    void conv2d_bias_bkwd_##S(const T *dout, T *dbias, int N, int C, int H, int W)                         \
+    {                                                                                                      \
+        conv_bias_bkwd<T>(dout, dbias, N, C, H, W);                                                        \
     }                                                                                                      \
     void relu_##S(T *in, T *out, T alpha, int n, int si, int so)                                           \
     {                                                                                                      \

@@ -514,6 +514,25 @@ def cross_entropy_backward(prob, ans, gloss=None):
     return gpred
 
 
+def conv2d_bias_add(input, bias, output):
+    """zenu-matrix/src/nn/conv/mod.rs:84-95: output[N,C,H,W] = input + bias[1,C,1,1], one launch"""
+    if tuple(input.shape) != tuple(output.shape):
+        raise ZenuHipError(_lib.ERR_SHAPE, "conv2d_bias_add", "input and output shapes differ")
+    if bias.ndim != 4 or input.ndim != 4 or (bias.shape[0], bias.shape[2], bias.shape[3]) != (1, 1, 1) \
+            or bias.shape[1] != output.shape[1]:
+        raise ZenuHipError(_lib.ERR_SHAPE, "conv2d_bias_add", "bias must be [1, C, 1, 1]")
+    output.add_array(input, bias)
+
+
+def conv2d_bias_bkwd(d_output, d_bias):
+    """zenu-matrix/src/nn/conv/mod.rs:98-107 with the CPU device's definition (cpu/bias.rs:18-25):
+    d_bias[1,C,1,1] = d_output[N,C,H,W] summed over axes 0, 2 and 3, in that order"""
+    if d_bias.ndim != 4 or d_output.ndim != 4 or (d_bias.shape[0], d_bias.shape[2], d_bias.shape[3]) != (1, 1, 1) \
+            or d_bias.shape[1] != d_output.shape[1]:
+        raise ZenuHipError(_lib.ERR_SHAPE, "conv2d_bias_bkwd", "d_bias must be [1, C, 1, 1]")
+    sum_to(d_output, d_bias)
+
+
 def sum_to(source, target):
     """sum.rs:35-94: reduce `source` into the (smaller) `target` in place"""
     check(_lib.lib().zenu_hip_sum_to(_dt(source.dtype), C.byref(target.desc()), C.byref(source.desc()),
