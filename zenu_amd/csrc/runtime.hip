@@ -6,6 +6,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
 #include <map>
 #include <mutex>
 
@@ -47,7 +48,7 @@ struct HipBackend : AllocBackend {
 constexpr int64_t kNumCounters = 1 << 16;
 
 struct State {
-    bool ready = false;
+    std::atomic<bool> ready{false};   // read without the init lock by every entry point
     bool use_pool = true;
     // arrival counters of the reductions, zero at rest: one ring per stream, because only launches
     // on the same stream are certain to run one after the other
