@@ -3,7 +3,7 @@ configurations (full size) and on edge cases.  Everything goes through the C ABI
 
 Bars (written where they are used):
   add/sub/mul/div, relu, max, arg-max, copy, SGD/Adam/AdamW .......... bit-exact
-  f32 exp, log, powf; tanh, sigmoid in f32 and f64 (the host libm's
+  f32 exp, log, powf, sinh, cosh, sin, cos; tanh, sigmoid in f32 and f64 (the host libm's
       algorithms, restated) ........................................... bit-exact (bar: <= 2 ulp)
   f64 exp, log, powf (device math library) ............................ <= 2 ulp
   sums ................................................................ |gpu - cpu| <= 1e-5 (f32) /
@@ -210,7 +210,8 @@ def test_transcendental_special_values(hip):
                   21.9, 22.0, -22.5, 0.99999994, 1.0, 1.0000001, 0.346, 0.347, 1.039, 1.04, 9.01, 9.011,
                   3e38, -3e38, 1.1754944e-38, 5e-39], dtype=np.float32)
     X = hip.Matrix.from_numpy(x)
-    for name, fn in (("exp", zo.EXP), ("tanh", zo.TANH), ("log", zo.LOG), ("sqrt", zo.SQRT)):
+    for name, fn in (("exp", zo.EXP), ("tanh", zo.TANH), ("log", zo.LOG), ("sqrt", zo.SQRT), ("sinh", zo.SINH),
+                     ("cosh", zo.COSH), ("sin", zo.SIN), ("cos", zo.COS)):
         exp = np.empty_like(x)
         with np.errstate(all="ignore"):
             zo.unary(fn, exp, x)
@@ -248,6 +249,14 @@ def test_tanh_sigmoid_dense_sweep(hip):
     ok = ~np.isnan(exp)                                    # log of negatives and NaN is NaN on both sides
     assert np.array_equal(np.isnan(got), np.isnan(exp))
     assert max_ulp(got[ok], exp[ok]) == 0                  # includes zeros (-inf), subnormals and +inf
+    # cosh is what tanh's backward evaluates; sin / cos include the large-argument reduction
+    for name, fn in (("sinh", zo.SINH), ("cosh", zo.COSH), ("sin", zo.SIN), ("cos", zo.COS)):
+        with np.errstate(all="ignore"):
+            zo.unary(fn, exp, x)
+        got = getattr(X, name)().to_numpy()
+        ok = ~np.isnan(exp)
+        assert np.array_equal(np.isnan(got), np.isnan(exp)), name
+        assert max_ulp(got[ok], exp[ok]) == 0, name
 
 
 def test_unary_f64(hip):

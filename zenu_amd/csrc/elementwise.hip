@@ -73,6 +73,10 @@ template <typename T, int OP> struct ScalarF {
 
 __device__ __forceinline__ float dev_tanh(float x) { return zmath::tanhf_simd(x); }
 __device__ __forceinline__ double dev_tanh(double x) { return zmath::tanh_fdlibm(x); }
+__device__ __forceinline__ float dev_sin(float x) { return zmath::sinf_glibc(x); }
+__device__ __forceinline__ double dev_sin(double x) { return sin(x); }
+__device__ __forceinline__ float dev_cos(float x) { return zmath::cosf_glibc(x); }
+__device__ __forceinline__ double dev_cos(double x) { return cos(x); }
 __device__ __forceinline__ float dev_sigmoid(float x) { return zmath::sigmoidf_zenu(x); }
 __device__ __forceinline__ double dev_sigmoid(double x) { return zmath::sigmoid_zenu(x); }
 
@@ -81,7 +85,8 @@ template <typename T, int FN> struct UnaryF {
     zmath::ExpLog<T> m;     // exp / log state (f32: tables in LDS)
     __device__ __forceinline__ void init()
     {
-        if constexpr (FN == ZENU_EXP || FN == ZENU_LOG) m.init(FN == ZENU_EXP, FN == ZENU_LOG);
+        if constexpr (FN == ZENU_EXP || FN == ZENU_LOG || FN == ZENU_SINH || FN == ZENU_COSH)
+            m.init(FN != ZENU_LOG, FN == ZENU_LOG);
     }
     __device__ __forceinline__ T operator()(T a, T) const
     {
@@ -90,14 +95,14 @@ template <typename T, int FN> struct UnaryF {
         else if constexpr (FN == ZENU_TANH) return dev_tanh(a);
         else if constexpr (FN == ZENU_SQRT) return sqrt(a);
         else if constexpr (FN == ZENU_ABS) return fabs(a);
-        else if constexpr (FN == ZENU_SIN) return sin(a);
-        else if constexpr (FN == ZENU_COS) return cos(a);
+        else if constexpr (FN == ZENU_SIN) return dev_sin(a);
+        else if constexpr (FN == ZENU_COS) return dev_cos(a);
         else if constexpr (FN == ZENU_TAN) return tan(a);
         else if constexpr (FN == ZENU_ASIN) return asin(a);
         else if constexpr (FN == ZENU_ACOS) return acos(a);
         else if constexpr (FN == ZENU_ATAN) return atan(a);
-        else if constexpr (FN == ZENU_SINH) return sinh(a);
-        else if constexpr (FN == ZENU_COSH) return cosh(a);
+        else if constexpr (FN == ZENU_SINH) return m.sinh(a);
+        else if constexpr (FN == ZENU_COSH) return m.cosh(a);
         else return dev_sigmoid(a);
     }
 };

@@ -468,6 +468,144 @@ ZM_HD float powf_glibc(float x, float y, const uint64_t *etab, const double *lta
     return (float)out;
 }
 
+// sinhf / coshf (fdlibm e_sinhf.c / e_coshf.c as glibc 2.35 ships them): expm1f below 22, expf above,
+// the argument halved where exp would overflow.  `etab` is expf's table.
+ZM_HD float sinhf_fdlibm(float x, const uint64_t *etab)
+{
+    const float one = 1.0f, shuge = 1.0e37f;
+    const uint32_t jx = f2u(x);
+    const uint32_t ix = jx & 0x7fffffffu;
+    if (ix >= 0x7f800000u) return x + x;                 // inf, NaN
+    const float h = (jx & 0x80000000u) ? -0.5f : 0.5f;
+    const float ax = u2f(ix);
+    if (ix < 0x41b00000u) {                              // |x| < 22
+        if (ix < 0x31800000u) return x;                  // |x| < 2^-28
+        const float t = expm1f_fdlibm(ax);
+        if (ix < 0x3f800000u) return h * (2.0f * t - t * t / (t + one));
+        return h * (t + t / (t + one));
+    }
+    if (ix < 0x42b17180u) return h * expf_glibc(ax, etab);   // |x| < log(FLT_MAX)
+    if (ix <= 0x42b2d4fcu) {                             // up to the overflow threshold
+        const float w = expf_glibc(0.5f * ax, etab);
+        const float t = h * w;
+        return t * w;
+    }
+    return x * shuge;                                    // overflow
+}
+
+ZM_HD float coshf_fdlibm(float x, const uint64_t *etab)
+{
+    const float one = 1.0f, half = 0.5f, huge = 1.0e30f;
+    const uint32_t ix = f2u(x) & 0x7fffffffu;
+    const float ax = u2f(ix);
+    if (ix < 0x41b00000u) {                              // |x| < 22
+        if (ix < 0x3eb17218u) {                          // |x| < 0.5 ln2: 1 + expm1^2 / (2 exp)
+            if (ix < 0x24000000u) return one;
+            const float t = expm1f_fdlibm(ax);
+            const float w = one + t;
+            return one + (t * t) / (w + w);
+        }
+        const float t = expf_glibc(ax, etab);
+        return half * t + half / t;
+    }
+    if (ix < 0x42b17180u) return half * expf_glibc(ax, etab);
+    if (ix <= 0x42b2d4fcu) {
+        const float w = expf_glibc(half * ax, etab);
+        const float t = half * w;
+        return t * w;
+    }
+    if (ix >= 0x7f800000u) return x * x;                 // inf, NaN
+    return huge * huge;                                  // overflow
+}
+
+// sinf / cosf (glibc's s_sinf.c / s_cosf.c with sincosf.h, from ARM's optimized routines), in double:
+// |x| < pi/4 a polynomial; |x| < 120 one multiply-subtract reduction by pi/2 with the quadrant from a
+// scaled float-to-int conversion; larger arguments a 32 x 96 bit fixed-point product with 4/pi.
+// Every a + b*c is fused, as in the x86-64 build that CPUs with FMA select; with that the results
+// equal the host libm's on all 2^32 inputs (the unfused form differs on 12 / 22 of them).
+// 4/pi to 192 bits, 8 new bits per entry
+#define ZM_INV_PIO4_TAB                                                                                     \
+    { 0xa2u, 0xa2f9u, 0xa2f983u, 0xa2f9836eu, 0xf9836e4eu, 0x836e4e44u, 0x6e4e4415u, 0x4e441529u,           \
+      0x441529fcu, 0x1529fc27u, 0x29fc2757u, 0xfc2757d1u, 0x2757d1f5u, 0x57d1f534u, 0xd1f534ddu,            \
+      0xf534ddc0u, 0x34ddc0dbu, 0xddc0db62u, 0xc0db6295u, 0xdb629599u, 0x6295993cu, 0x95993c43u,            \
+      0x993c4390u, 0x3c439041u }
+static const uint32_t kInvPio4Host[24] = ZM_INV_PIO4_TAB;
+#if defined(__HIPCC__)
+static __device__ const uint32_t kInvPio4Dev[24] = ZM_INV_PIO4_TAB;
+#endif
+ZM_HD const uint32_t *inv_pio4_table()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return kInvPio4Dev;
+#else
+    return kInvPio4Host;
+#endif
+}
+
+// sine polynomial for an even quadrant, cosine polynomial for an odd one; `neg` flips the cosine
+ZM_HD float sincosf_poly(double x, double x2, bool neg, int n)
+{
+    if ((n & 1) == 0) {
+        const double S1 = -0x1.555545995a603p-3, S2 = 0x1.1107605230bc4p-7, S3 = -0x1.994eb3774cf24p-13;
+        const double x3 = x * x2;
+        const double s1 = __builtin_fma(x2, S3, S2);
+        const double x7 = x3 * x2;
+        const double s = __builtin_fma(x3, S1, x);
+        return (float)__builtin_fma(x7, s1, s);
+    }
+    const double sg = neg ? -1.0 : 1.0;
+    const double C0 = sg, C1 = sg * -0x1.ffffffd0c621cp-2, C2 = sg * 0x1.55553e1068f19p-5,
+                 C3 = sg * -0x1.6c087e89a359dp-10, C4 = sg * 0x1.99343027bf8c3p-16;
+    const double x4 = x2 * x2;
+    const double c2 = __builtin_fma(x2, C4, C3);
+    const double c1 = __builtin_fma(x2, C1, C0);
+    const double x6 = x4 * x2;
+    const double c = __builtin_fma(x4, C2, c1);
+    return (float)__builtin_fma(x6, c2, c);
+}
+
+// cosine = 0: sinf(y); cosine = 1: cosf(y)
+ZM_HD float sincosf_glibc(float y, int cosine)
+{
+    const double HpiInv = 0x1.45F306DC9C883p+23, Hpi = 0x1.921FB54442D18p0, Pi63 = 0x1.921FB54442D18p-62;
+    const uint32_t top = (f2u(y) >> 20) & 0x7ffu;
+    double x = (double)y;
+    int n;
+    if (top < (0x3f490fdbu >> 20)) {                     // |y| < pi/4 (by the top 12 bits)
+        if (top < (0x39800000u >> 20)) return cosine ? 1.0f : y;   // |y| < 2^-12
+        return sincosf_poly(x, x * x, false, cosine);
+    }
+    if (top < (0x42f00000u >> 20)) {                     // |y| < 120
+        const double r = x * HpiInv;
+        n = ((int32_t)r + 0x800000) >> 24;
+        x = __builtin_fma(-(double)n, Hpi, x);
+    } else if (top < (0x7f800000u >> 20)) {
+        uint32_t xi = f2u(y);
+        const int sign = (int)(xi >> 31);
+        const uint32_t *arr = inv_pio4_table() + ((xi >> 26) & 15u);
+        const int shift = (int)((xi >> 23) & 7u);
+        xi = (xi & 0xffffffu) | 0x800000u;
+        xi <<= shift;
+        uint64_t res0 = (uint64_t)(uint32_t)(xi * arr[0]);
+        const uint64_t res1 = (uint64_t)xi * arr[4];
+        const uint64_t res2 = (uint64_t)xi * arr[8];
+        res0 = (res2 >> 32) | (res0 << 32);
+        res0 += res1;
+        const uint64_t q = (res0 + (1ull << 61)) >> 62;
+        res0 -= q << 62;
+        x = (double)(int64_t)res0 * Pi63;
+        n = (int)q + sign;
+        const double s = ((n & 3) == 1 || (n & 3) == 2) ? -1.0 : 1.0;
+        return sincosf_poly(x * s, x * x, (n & 2) != 0, (int)q ^ cosine);
+    } else {
+        return (y - y) / (y - y);                        // inf, NaN
+    }
+    const double s = ((n & 3) == 1 || (n & 3) == 2) ? -1.0 : 1.0;
+    return sincosf_poly(x * s, x * x, (n & 2) != 0, n ^ cosine);
+}
+ZM_HD float sinf_glibc(float x) { return sincosf_glibc(x, 0); }
+ZM_HD float cosf_glibc(float x) { return sincosf_glibc(x, 1); }
+
 // ---- double precision: fdlibm s_expm1.c / s_tanh.c as shipped by glibc 2.35 (generic dbl-64) ----------
 
 ZM_HD uint64_t d2u(double d)
@@ -627,6 +765,8 @@ ZM_HD float sigmoidf_zenu(float x)
 ZM_HD float expf_glibc(float x) { return expf_glibc(x, exp2f_table()); }
 ZM_HD float logf_glibc(float x) { return logf_glibc(x, logf_table()); }
 ZM_HD float powf_glibc(float x, float y) { return powf_glibc(x, y, exp2f_table(), powf_log2_table()); }
+ZM_HD float sinhf_fdlibm(float x) { return sinhf_fdlibm(x, exp2f_table()); }
+ZM_HD float coshf_fdlibm(float x) { return coshf_fdlibm(x, exp2f_table()); }
 
 #if defined(__HIPCC__)
 // exp / log as the kernels call them: f32 through tables copied to LDS by init(), which every
@@ -636,6 +776,8 @@ template <typename T> struct ExpLog {
     __device__ __forceinline__ void init(bool, bool) {}
     __device__ __forceinline__ T exp(T x) const { return ::exp(x); }
     __device__ __forceinline__ T log(T x) const { return ::log(x); }
+    __device__ __forceinline__ T sinh(T x) const { return ::sinh(x); }
+    __device__ __forceinline__ T cosh(T x) const { return ::cosh(x); }
 };
 template <> struct ExpLog<float> {
     const uint64_t *etab;
@@ -654,6 +796,8 @@ template <> struct ExpLog<float> {
     }
     __device__ __forceinline__ float exp(float x) const { return expf_glibc(x, etab); }
     __device__ __forceinline__ float log(float x) const { return logf_glibc(x, ltab); }
+    __device__ __forceinline__ float sinh(float x) const { return sinhf_fdlibm(x, etab); }
+    __device__ __forceinline__ float cosh(float x) const { return coshf_fdlibm(x, etab); }
 };
 
 // pow with the same arrangement: f32 through powf's two tables in LDS, f64 from the math library
