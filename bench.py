@@ -251,6 +251,12 @@ def build_ops(z, workload, stream):
         ops.append(Op("clip", "fused", "f32", 2 * 4 * n, n,
                       mk(lambda dx, dt, do, dp, db, dl: (lambda: check(l.zenu_hip_clip(_lib.F32, ref(do), ref(dx), -1.0, 1.0, stream), "clip"))),
                       lambda: cx.clip(-1.0, 1.0)))
+        ops.append(Op("tanh backward", "fused", "f32", 3 * 4 * n, n,
+                      mk(lambda dx, dt, do, dp, db, dl: (lambda: check(l.zenu_hip_tanh_backward(_lib.F32, ref(do), ref(dt), ref(dx), stream), "tanh_bwd"))),
+                      lambda: co.tanh_backward(ct, cx)))
+        ops.append(Op("sigmoid backward", "fused", "f32", 3 * 4 * n, n,
+                      mk(lambda dx, dt, do, dp, db, dl: (lambda: check(l.zenu_hip_sigmoid_backward(_lib.F32, ref(do), ref(dt), ref(dx), stream), "sigmoid_bwd"))),
+                      lambda: co.sigmoid_backward(ct, cx)))
         ops[-1].keep = sets
 
     if workload == "fused":

@@ -167,6 +167,15 @@ int zenu_hip_relu_backward_mask(int dtype, const zenu_tensor_t *to, const zenu_t
 int zenu_hip_relu_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *gy,
                            const zenu_tensor_t *x, double alpha, zenu_stream_t stream);
 
+/* Backward of tanh and of the sigmoid composite in one pass, with the roundings of the op chains
+ * they replace: gx = gy / (cosh(x) * cosh(x)) (zenu-autograd/src/functions/tanh.rs:30-37) and
+ * gx = ((0.5 * gy) / (cosh(0.5 * x) * cosh(0.5 * x))) * 0.5 (activation/sigmoid.rs:7-15 through the
+ * backward of its mul, tanh, mul and add nodes, functions/mul.rs:35-44).  x is the forward INPUT. */
+int zenu_hip_tanh_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *gy,
+                           const zenu_tensor_t *x, zenu_stream_t stream);
+int zenu_hip_sigmoid_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *gy,
+                              const zenu_tensor_t *x, zenu_stream_t stream);
+
 /* to = clip(other, min, max); mask = 1 inside [min, max] (and for NaN), 0 outside
  * (zenu-matrix/src/operation/clip.rs:289-318).  The assign forms are to == other.  The mask is
  * written with the mask's own stride (clip.rs:90-96 indexes it with the input's). */

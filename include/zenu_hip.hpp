@@ -383,6 +383,16 @@ public:
         zenu_tensor_t t = desc(), g = gy.desc(), xx = x.desc();
         check(zenu_hip_relu_backward(dt(), &t, &g, &xx, (double)alpha, st()), "relu_backward");
     }
+    void tanh_backward(const Matrix &gy, const Matrix &x) const      // functions/tanh.rs:30-37
+    {
+        zenu_tensor_t t = desc(), g = gy.desc(), xx = x.desc();
+        check(zenu_hip_tanh_backward(dt(), &t, &g, &xx, st()), "tanh_backward");
+    }
+    void sigmoid_backward(const Matrix &gy, const Matrix &x) const   // activation/sigmoid.rs:7-15
+    {
+        zenu_tensor_t t = desc(), g = gy.desc(), xx = x.desc();
+        check(zenu_hip_sigmoid_backward(dt(), &t, &g, &xx, st()), "sigmoid_backward");
+    }
     Matrix clip(T lo, T hi) const
     {
         Matrix out = alloc_like();

@@ -125,6 +125,20 @@ class CpuMatrix:
     def relu(self, other, alpha): zo.relu(self.a, other.a, alpha)
     def relu_backward_mask(self, other, alpha): zo.relu_backward_mask(self.a, other.a, alpha)
 
+    def tanh_backward(self, gy, x):
+        """zenu-autograd/src/functions/tanh.rs:30-37: cosh(x), cosh * cosh, gy / that"""
+        c = x.cosh()
+        self.div_array(gy, c * c)
+
+    def sigmoid_backward(self, gy, x):
+        """backward of activation/sigmoid.rs:7-15, node by node: add passes gy on; mul(half, th) gives
+        half * gy (functions/mul.rs:35-44); tanh divides by cosh(x * half)^2; mul(x, half) gives g * half"""
+        half = CpuMatrix.from_vec([0.5], (), self.dtype)
+        g1 = half * gy
+        c = (x * half).cosh()
+        g2 = g1 / (c * c)
+        self.mul_array(g2, half)
+
     def relu_backward(self, gy, x, alpha):
         """zenu-autograd/src/activation/relu.rs:35-44: mask, then gy * mask"""
         mask = x.alloc_like()

@@ -270,3 +270,53 @@ def test_conv2d_bias_add_and_backward(hip):
             assert bits_equal(hg2.to_numpy(), hg.to_numpy())
     with pytest.raises(hip.ZenuHipError):
         hip.conv2d_bias_bkwd(hx, hip.Matrix.zeros((1, c + 1, 1, 1), dt))
+
+
+def test_tanh_and_sigmoid_backward(hip):
+    """One-pass backward of tanh (zenu-autograd/src/functions/tanh.rs:30-37) and of the sigmoid
+    composite (activation/sigmoid.rs:7-15) against the op-by-op chains on the CPU: bit-exact in
+    f32 (cosh is the host libm's algorithm); f64 cosh comes from the device math library, so the
+    bar there is 4 ulp (two for cosh, doubled by the square).  Also strided views and the
+    closed form d tanh = 1 - tanh^2, d sigmoid = s (1 - s)."""
+    r = np.random.default_rng(29)
+    x32 = np.concatenate([r.standard_normal(100000) * 3, r.uniform(-95, 95, 20000),
+                          [0.0, -0.0, 1e-30, 22.0, -22.0, 88.0, 89.5, -89.5, 100.0, np.inf, -np.inf, np.nan]]).astype(np.float32)
+    g32 = r.standard_normal(x32.size).astype(np.float32)
+    for dt, bar in ((np.float32, 0), (np.float64, 4)):
+        x, gy = x32.astype(dt), g32.astype(dt)
+        hx, hg = hip.Matrix.from_numpy(x), hip.Matrix.from_numpy(gy)
+        cx, cg = CpuMatrix.from_numpy(x), CpuMatrix.from_numpy(gy)
+        for name in ("tanh_backward", "sigmoid_backward"):
+            ho, co = hip.Matrix.zeros(x.shape, dt), CpuMatrix.zeros(x.shape, dt)
+            getattr(ho, name)(hg, hx)
+            with np.errstate(all="ignore"):
+                getattr(co, name)(cg, cx)
+            got, exp = ho.to_numpy(), co.a
+            assert np.array_equal(np.isnan(got), np.isnan(exp)), (name, dt)
+            ok = ~np.isnan(exp)
+            if bar == 0:
+                assert bits_equal(got[ok], exp[ok]), (name, dt)
+            else:
+                fin = ok & np.isfinite(exp) & (exp != 0)
+                assert np.max(np.abs(got[fin] - exp[fin]) / np.abs(exp[fin])) <= bar * np.finfo(dt).eps, (name, dt)
+    # closed forms, f64, moderate arguments
+    x = r.standard_normal(50000) * 2
+    one = np.ones_like(x)
+    hx, h1 = hip.Matrix.from_numpy(x), hip.Matrix.from_numpy(one)
+    o = hip.Matrix.zeros(x.shape, np.float64)
+    o.tanh_backward(h1, hx)
+    assert np.allclose(o.to_numpy(), 1 - np.tanh(x) ** 2, rtol=1e-13, atol=1e-15)
+    o.sigmoid_backward(h1, hx)
+    s = 1 / (1 + np.exp(-x))
+    assert np.allclose(o.to_numpy(), s * (1 - s), rtol=1e-13, atol=1e-15)
+    # strided views: transposed x, every other row of gy
+    m = r.standard_normal((64, 96)).astype(np.float32)
+    g = r.standard_normal((192, 64)).astype(np.float32)
+    hm, hg = hip.Matrix.from_numpy(m).transpose(), hip.Matrix.from_numpy(g).slice(slice(None, None, 2))
+    cm, cg = CpuMatrix.from_numpy(np.ascontiguousarray(m.T)), CpuMatrix.from_numpy(np.ascontiguousarray(g[::2]))
+    ho, co = hip.Matrix.zeros((96, 64)), CpuMatrix.zeros((96, 64))
+    ho.sigmoid_backward(hg, hm)
+    co.sigmoid_backward(cg, cm)
+    assert bits_equal(ho.to_numpy(), co.a)
+    with pytest.raises(hip.ZenuHipError):
+        ho.tanh_backward(hg, hip.Matrix.zeros((64, 96)))

@@ -72,6 +72,8 @@ SIGNATURES = {
     "zenu_hip_relu": [_i, _TP, _TP, _d, _vp],
     "zenu_hip_relu_backward_mask": [_i, _TP, _TP, _d, _vp],
     "zenu_hip_relu_backward": [_i, _TP, _TP, _TP, _d, _vp],
+    "zenu_hip_tanh_backward": [_i, _TP, _TP, _TP, _vp],
+    "zenu_hip_sigmoid_backward": [_i, _TP, _TP, _TP, _vp],
     "zenu_hip_clip": [_i, _TP, _TP, _d, _d, _vp],
     "zenu_hip_clip_backward_mask": [_i, _TP, _TP, _d, _d, _vp],
     "zenu_hip_copy": [_i, _TP, _TP, _vp],

@@ -136,6 +136,36 @@ template <typename T> struct ReluBwdF {
     __device__ __forceinline__ void init() {}
     __device__ __forceinline__ T operator()(T gy, T x) const { return gy * ((x > (T)0) ? (T)1 : alpha * (T)-1); }
 };
+// backward of tanh (zenu-autograd/src/functions/tanh.rs:30-37): cosh(x), its square, gy / square --
+// three ops there, each rounded once; the same roundings here in one pass
+template <typename T> struct TanhBwdF {
+    static constexpr int NIN = 2;
+    zmath::ExpLog<T> m;
+    __device__ __forceinline__ void init() { m.init(true, false); }
+    __device__ __forceinline__ T operator()(T gy, T x) const
+    {
+        const T c = m.cosh(x);
+        const T c2 = c * c;
+        return gy / c2;
+    }
+};
+// backward of the sigmoid composite (zenu-autograd/src/activation/sigmoid.rs:7-15) through its add,
+// mul, tanh and mul nodes (functions/mul.rs:35-44): ((0.5 gy) / cosh(0.5 x)^2) 0.5, every step rounded
+template <typename T> struct SigmoidBwdF {
+    static constexpr int NIN = 2;
+    zmath::ExpLog<T> m;
+    __device__ __forceinline__ void init() { m.init(true, false); }
+    __device__ __forceinline__ T operator()(T gy, T x) const
+    {
+        const T half = (T)0.5;
+        const T xh = x * half;
+        const T c = m.cosh(xh);
+        const T c2 = c * c;
+        const T g1 = half * gy;
+        const T g2 = g1 / c2;
+        return g2 * half;
+    }
+};
 // clip.rs:50-57: below min -> min, above max -> max, NaN passes through
 template <typename T> struct ClipF {
     static constexpr int NIN = 1;
@@ -174,6 +204,8 @@ __device__ __forceinline__ Pack<T, N> apply_pack(const F &f, const Pack<T, N> &a
 template <typename F> struct IsValuBound { static constexpr bool value = false; };
 template <typename T> struct IsValuBound<UnaryF<T, ZENU_TANH>> { static constexpr bool value = true; };
 template <typename T> struct IsValuBound<UnaryF<T, ZENU_SIGMOID>> { static constexpr bool value = true; };
+template <typename T> struct IsValuBound<TanhBwdF<T>> { static constexpr bool value = true; };
+template <typename T> struct IsValuBound<SigmoidBwdF<T>> { static constexpr bool value = true; };
 
 template <typename F> struct ContigShape {
     static constexpr bool kSmall = F::NIN == 1 && !IsValuBound<F>::value;
@@ -763,6 +795,20 @@ int check2(const zenu_tensor_t *a, const zenu_tensor_t *b)
 
 using namespace zenu;
 
+template <template <typename> class F>
+static int activation_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *gy, const zenu_tensor_t *x,
+                               zenu_stream_t stream)
+{
+    int rc = check2(gx, gy);
+    if (!rc) rc = validate_tensor(x);
+    if (!rc) rc = ensure_init();
+    if (rc) return rc;
+    if (!same_shape(*gx, *gy) || !same_shape(*gx, *x)) return ZENU_ERR_SHAPE;
+    if (dtype == ZENU_F32) return run2<float>(*gx, *gy, *x, F<float>(), as_stream(stream));
+    if (dtype == ZENU_F64) return run2<double>(*gx, *gy, *x, F<double>(), as_stream(stream));
+    return ZENU_ERR_ARG;
+}
+
 extern "C" {
 
 int zenu_hip_binary(int op, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *lhs,
@@ -908,6 +954,18 @@ int zenu_hip_relu_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor
     if (dtype == ZENU_F32) { ReluBwdF<float> f; f.alpha = (float)alpha; return run2<float>(*gx, *gy, *x, f, as_stream(stream)); }
     if (dtype == ZENU_F64) { ReluBwdF<double> f; f.alpha = alpha; return run2<double>(*gx, *gy, *x, f, as_stream(stream)); }
     return ZENU_ERR_ARG;
+}
+
+int zenu_hip_tanh_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *gy, const zenu_tensor_t *x,
+                           zenu_stream_t stream)
+{
+    return activation_backward<TanhBwdF>(dtype, gx, gy, x, stream);
+}
+
+int zenu_hip_sigmoid_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *gy, const zenu_tensor_t *x,
+                              zenu_stream_t stream)
+{
+    return activation_backward<SigmoidBwdF>(dtype, gx, gy, x, stream);
 }
 
 int zenu_hip_clip(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other, double min, double max,

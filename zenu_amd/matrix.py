@@ -330,6 +330,16 @@ class Matrix:
                                                      C.byref(other.desc()), float(alpha), _stream),
               "relu_backward_mask")
 
+    def tanh_backward(self, gy, x):
+        """self = gy / cosh(x)^2: zenu-autograd/src/functions/tanh.rs:30-37 in one pass"""
+        check(_lib.lib().zenu_hip_tanh_backward(_dt(self.dtype), C.byref(self.desc()), C.byref(gy.desc()),
+                                                C.byref(x.desc()), _stream), "tanh_backward")
+
+    def sigmoid_backward(self, gy, x):
+        """self = d sigmoid(x) * gy with the roundings of the autograd chain (activation/sigmoid.rs:7-15)"""
+        check(_lib.lib().zenu_hip_sigmoid_backward(_dt(self.dtype), C.byref(self.desc()), C.byref(gy.desc()),
+                                                   C.byref(x.desc()), _stream), "sigmoid_backward")
+
     def relu_backward(self, gy, x, alpha):
         """self = gy * relu_backward_mask(x): zenu-autograd/src/activation/relu.rs:35-44 in one pass"""
         check(_lib.lib().zenu_hip_relu_backward(_dt(self.dtype), C.byref(self.desc()), C.byref(gy.desc()),
