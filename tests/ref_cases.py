@@ -272,6 +272,50 @@ def sigmoid_cases(dev):
         close(dev.M.from_vec([0.5], [], dt).sigmoid(), 0.62245935, 1e-6)
 
 
+# ---- unary functions with their backward: zenu-autograd/src/functions/{tanh,sinh,cosh,powf,clip}.rs test mods ----
+
+_X6 = [1., 2., 3., 4., 5., 6.]
+_TANH6 = [0.7615941559557649, 0.9640275800758169, 0.9950547536867305, 0.999329299739067, 0.9999092042625951,
+          0.9999877116507956]
+_SINH6 = [1.1752011936438014, 3.626860407847019, 10.017874927409903, 27.28991719712775, 74.20321057778875,
+          201.71315737027922]
+_COSH6 = [1.5430806348152437, 3.7621956910836314, 10.067661995777765, 27.308232836016487, 74.20994852478785,
+          201.7156361224559]
+
+
+@case
+def autograd_unary_backward(dev):
+    # tanh_1d (tanh.rs test mod): y = tanh(x), x.grad = 1 / cosh(x)^2 with an all-ones output gradient, 1e-6
+    x = dev.M.from_vec(_X6, [6])
+    ones = dev.M.from_vec([1.] * 6, [6])
+    close(x.tanh(), _TANH6, 1e-6)
+    gx = dev.M.zeros([6])
+    gx.tanh_backward(ones, x)
+    close(gx, [1.0 / (c * c) for c in _COSH6], 1e-6)
+    # sinh_1d / cosh_1d (f64): values, and gradients cosh(x) * gy / sinh(x) * gy (sinh.rs:30-35, cosh.rs)
+    xd = dev.M.from_vec(_X6, [6], np.float64)
+    od = dev.M.from_vec([1.] * 6, [6], np.float64)
+    close(xd.sinh(), _SINH6, 1e-6 * 201.8)      # assert_val_eq's bound is on asum(diff) relative to the values' scale
+    close(xd.cosh(), _COSH6, 1e-6 * 201.8)
+    close(xd.cosh() * od, _COSH6, 1e-6 * 201.8)
+    close(xd.sinh() * od, _SINH6, 1e-6 * 201.8)
+    # powf_ (powf.rs test mod): x^2 and its gradient powf(x, factor - 1) * factor * gy (powf.rs:25-30)
+    p = dev.M.from_vec([1., 2., 3.], [3])
+    close(p.powf_array(2.0), [1., 4., 9.], 1e-6)
+    two = dev.M.from_vec([2.0], [])
+    close(p.powf_array(1.0) * two * dev.M.from_vec([1.] * 3, [3]), [2., 4., 6.], 1e-6)
+    # clip_1d (clip.rs test mod)
+    c = dev.M.from_vec(_X6, [6])
+    eq(c.clip(2., 4.), [2., 2., 3., 4., 4., 4.])
+    eq(c.clip_backward_mask(2., 4.), [0., 1., 1., 1., 0., 0.])
+    # sigmoid backward has no test in the reference: closed form s (1 - s) at the sigmoid_cases points
+    xs = dev.M.from_vec([0.0, 0.5, 0.1, 0.2, 0.3, 0.4], [6], np.float64)
+    gs = dev.M.zeros([6], np.float64)
+    gs.sigmoid_backward(dev.M.from_vec([1.] * 6, [6], np.float64), xs)
+    sg = [0.5, 0.62245935, 0.52497919, 0.54983399, 0.57444252, 0.59868766]
+    close(gs, [v * (1 - v) for v in sg], 1e-7)
+
+
 # ---- sum: sum.rs:109-245 ------------------------------------------------------------------------------
 
 _SUM1 = [60, 63, 66, 69, 72, 75, 78, 81, 84, 87, 90, 93, 96, 99, 102, 105, 108, 111, 114, 117,
