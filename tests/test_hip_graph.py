@@ -1,0 +1,124 @@
+"""The library's calls inside a captured HIP graph.
+
+What a capturing caller relies on: no entry point synchronises or calls the driver's allocator
+when the caching pool can serve the request (rehearsal runs make every request a hit), zero fills
+are kernels (no memset nodes), the arrival counters of the split reductions are back at zero after
+every run, and scratch taken from the pool during the capture stays valid for replays on the same
+stream.  The graph is replayed several times with new inputs, eager work on the same stream and
+synchronisations in between, and every replay is compared bit for bit with the eager sequence on
+the same inputs.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _hip_runtime():
+    rt = C.CDLL("libamdhip64.so")
+    vp = C.c_void_p
+    rt.hipStreamBeginCapture.argtypes = [vp, C.c_int]
+    rt.hipStreamEndCapture.argtypes = [vp, C.POINTER(vp)]
+    rt.hipGraphInstantiate.argtypes = [C.POINTER(vp), vp, vp, vp, C.c_size_t]
+    rt.hipGraphLaunch.argtypes = [vp, vp]
+    rt.hipGraphExecDestroy.argtypes = [vp]
+    rt.hipGraphDestroy.argtypes = [vp]
+    return rt
+
+
+def test_library_calls_in_a_captured_graph(hip):
+    import os
+    from zenu_amd import _lib
+    if os.environ.get("ZENU_USE_MEMPOOL") == "0":
+        pytest.skip("without the pool every scratch request is a driver allocation, which cannot be captured")
+    rt = _hip_runtime()
+    l = hip.lib()
+    M = hip.Matrix
+    stream = C.c_void_p()
+    _lib.check(l.zenu_hip_stream_create(C.byref(stream)), "stream_create")
+    old = hip.get_stream()
+    hip.set_stream(stream)
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    try:
+        r = np.random.default_rng(41)
+        rows, cols = 1024, 2048
+        inputs = [r.standard_normal((rows, cols)).astype(np.float32) * s for s in (1.0, 0.5, 2.0, 1.5)]
+        t = np.zeros((rows, cols), dtype=np.float32)
+        t[np.arange(rows), r.integers(0, cols, rows)] = 1
+        x, tgt = M.from_numpy(inputs[0]), M.from_numpy(t)
+        bias = M.from_numpy(r.standard_normal(cols).astype(np.float32))
+        act, pre, th = M.alloc((rows, cols)), M.alloc((rows, cols)), M.alloc((rows, cols))
+        colsum, total = M.alloc((cols,)), M.alloc(())
+        argmax = M.alloc((rows,))
+        p0 = r.standard_normal(rows * cols).astype(np.float32) * 0.02
+        p = M.from_numpy(p0)
+        params = {"w": (p, act)}                       # the activations double as a gradient
+        opt = hip.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, params, ["w"])
+        outs = {}
+
+        def sequence():
+            act.bias_add_relu(x, bias, 0.0, pre=pre)            # fused elementwise, two outputs
+            th.tanh_array(pre)                                  # exact tanh (VALU path)
+            hip.sum_to(act, colsum)                             # split column reduction: scratch + counters
+            l.zenu_hip_memset_zero(total.as_ptr(), 4, stream)   # a zero fill inside the capture
+            _lib.check(l.zenu_hip_sum_all(_lib.F32, total.as_ptr(), C.byref(x.desc()), stream), "sum_all")
+            argmax.copy_from(x.max_axis(1))                     # allocation + arg-max + strided copy
+            outs["loss"], outs["prob"] = hip.cross_entropy(x, tgt)
+            outs["g"] = hip.cross_entropy_backward(outs["prob"], tgt)
+            opt.update(params)
+
+        def state():
+            hip.synchronize()
+            return [v.to_numpy().copy() for v in (act, pre, th, colsum, total, argmax, outs["loss"], outs["prob"],
+                                                  outs["g"], p, opt.m["w"], opt.v["w"])]
+
+        def reset(inp):
+            _lib.check(l.zenu_hip_memcpy_h2d(x.as_ptr(), inp.ctypes.data, inp.nbytes, stream), "h2d")
+            _lib.check(l.zenu_hip_memcpy_h2d(p.as_ptr(), p0.ctypes.data, p0.nbytes, stream), "h2d")
+            for mv in (opt.m["w"], opt.v["w"]):
+                _lib.check(l.zenu_hip_memset_zero(mv.as_ptr(), p0.nbytes, stream), "zero")
+            opt.step = 0
+
+        eager = []
+        for inp in inputs:                                       # also the rehearsal: the pool holds every block
+            reset(inp)
+            sequence()
+            eager.append(state())
+        reset(inputs[0])
+        hip.synchronize()
+        assert rt.hipStreamBeginCapture(stream, 2) == 0          # hipStreamCaptureModeRelaxed
+        try:
+            sequence()                                           # recorded, not executed
+        finally:
+            rc = rt.hipStreamEndCapture(stream, C.byref(graph))
+        assert rc == 0
+        assert rt.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+        keep = dict(outs)                                        # the captured outputs' buffers
+        for i, inp in enumerate(inputs):
+            reset(inp)
+            opt.step = 1                                         # frozen in the graph as a kernel argument
+            assert rt.hipGraphLaunch(gexec, stream) == 0
+            got = state()
+            for name, a, b in zip(("act", "pre", "tanh", "colsum", "total", "argmax", "loss", "prob", "g", "p", "m", "v"),
+                                  got, eager[i]):
+                assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), (i, name)
+            # eager work between replays: other launches that use counters and pool blocks
+            y = (x + x).sum(0)
+            z = x.exp().max_axis(1)
+            del y, z
+            hip.synchronize()
+        del keep
+    finally:
+        hip.synchronize()
+        if gexec:
+            rt.hipGraphExecDestroy(gexec)
+        if graph:
+            rt.hipGraphDestroy(graph)
+        hip.set_stream(old)
+        outs.clear()
+        del x, tgt, bias, act, pre, th, colsum, total, argmax, p, opt, params
+        import gc
+        gc.collect()
+        _lib.check(l.zenu_hip_stream_destroy(stream), "stream_destroy")
