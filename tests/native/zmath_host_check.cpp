@@ -48,11 +48,11 @@ int main(int argc, char **argv)
     for (auto &t : th) t.join();
     // double precision: every stride-th value of the HIGH word (sign, exponent, 20 mantissa bits) with
     // a pseudo-random low word, plus low words 0 and all-ones
-    std::atomic<uint64_t> bad_tanh64{0}, bad_expm164{0}, bad_sig64{0};
+    std::atomic<uint64_t> bad_tanh64{0}, bad_expm164{0}, bad_sig64{0}, bad_exp64{0}, bad_sinh64{0}, bad_cosh64{0};
     th.clear();
     for (int w = 0; w < nt; w++)
         th.emplace_back([&, w]() {
-            uint64_t b0 = 0, b1 = 0, b2 = 0, rng = 0x9E3779B97F4A7C15ull * (w + 1);
+            uint64_t b0 = 0, b1 = 0, b2 = 0, b3 = 0, b4 = 0, b5 = 0, rng = 0x9E3779B97F4A7C15ull * (w + 1);
             for (uint64_t u = (uint64_t)w * stride; u < (1ull << 32); u += stride * nt) {
                 rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17;
                 const uint32_t lows[3] = {(uint32_t)rng, 0u, 0xffffffffu};
@@ -63,9 +63,25 @@ int main(int argc, char **argv)
                     if (fabs(x) < 700.0 && zmath::d2u(zmath::expm1_fdlibm(x)) != zmath::d2u(expm1(x))) b1++;
                     const double sg = 0.5 + 0.5 * tanh(0.5 * x), sz = zmath::sigmoid_zenu(x);
                     if ((sg != sg) ? !(sz != sz) : zmath::d2u(sz) != zmath::d2u(sg)) b2++;
+                    const double er = exp(x), eg = zmath::exp_glibc(x);
+                    if ((er != er) ? !(eg != eg) : zmath::d2u(eg) != zmath::d2u(er)) b3++;
+                    const double shr = sinh(x), shg = zmath::sinh_fdlibm(x);
+                    if ((shr != shr) ? !(shg != shg) : zmath::d2u(shg) != zmath::d2u(shr)) b4++;
+                    const double chr = cosh(x), chg = zmath::cosh_fdlibm(x);
+                    if ((chr != chr) ? !(chg != chg) : zmath::d2u(chg) != zmath::d2u(chr)) b5++;
+                }
+                // arguments where exp is finite and not 1: uniform in +-745 and in +-4
+                const double m = (double)(int64_t)rng / 9.2233720368547758e18;
+                for (double x : {m * 745.0, m * 4.0}) {
+                    const double er = exp(x), eg = zmath::exp_glibc(x);
+                    if (zmath::d2u(eg) != zmath::d2u(er)) b3++;
+                    const double shr = sinh(x), shg = zmath::sinh_fdlibm(x);
+                    if (zmath::d2u(shg) != zmath::d2u(shr)) b4++;
+                    const double chr = cosh(x), chg = zmath::cosh_fdlibm(x);
+                    if (zmath::d2u(chg) != zmath::d2u(chr)) b5++;
                 }
             }
-            bad_tanh64 += b0; bad_expm164 += b1; bad_sig64 += b2;
+            bad_tanh64 += b0; bad_expm164 += b1; bad_sig64 += b2; bad_exp64 += b3; bad_sinh64 += b4; bad_cosh64 += b5;
         });
     for (auto &t : th) t.join();
     // powf(x, y)
@@ -97,9 +113,11 @@ int main(int argc, char **argv)
            (unsigned long long)bad_expm1.load(), (unsigned long long)bad_sig.load());
     printf("tanh_fdlibm %llu expm1_fdlibm %llu sigmoid_zenu %llu\n", (unsigned long long)bad_tanh64.load(),
            (unsigned long long)bad_expm164.load(), (unsigned long long)bad_sig64.load());
+    printf("exp_glibc %llu sinh_fdlibm %llu cosh_fdlibm %llu\n", (unsigned long long)bad_exp64.load(),
+           (unsigned long long)bad_sinh64.load(), (unsigned long long)bad_cosh64.load());
     printf("expf_glibc %llu logf_glibc %llu\n", (unsigned long long)bad_exp.load(), (unsigned long long)bad_log.load());
     printf("powf_glibc %llu sinhf_fdlibm %llu coshf_fdlibm %llu\n", (unsigned long long)bad_pow.load(),
            (unsigned long long)bad_sinh.load(), (unsigned long long)bad_cosh.load());
     printf("sinf_glibc %llu cosf_glibc %llu\n", (unsigned long long)bad_sin.load(), (unsigned long long)bad_cos.load());
-    return (bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64 + bad_exp + bad_log + bad_pow + bad_sinh + bad_cosh + bad_sin + bad_cos) ? 1 : 0;
+    return (bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64 + bad_exp64 + bad_sinh64 + bad_cosh64 + bad_exp + bad_log + bad_pow + bad_sinh + bad_cosh + bad_sin + bad_cos) ? 1 : 0;
 }

@@ -3,9 +3,9 @@ configurations (full size) and on edge cases.  Everything goes through the C ABI
 
 Bars (written where they are used):
   add/sub/mul/div, relu, max, arg-max, copy, SGD/Adam/AdamW .......... bit-exact
-  f32 exp, log, powf, sinh, cosh, sin, cos; tanh, sigmoid in f32 and f64 (the host libm's
-      algorithms, restated) ........................................... bit-exact (bar: <= 2 ulp)
-  f64 exp, log, powf (device math library) ............................ <= 2 ulp
+  f32 exp, log, powf, sinh, cosh, sin, cos; f64 exp, sinh, cosh; tanh, sigmoid in f32 and f64
+      (the host libm's algorithms, restated) .......................... bit-exact (bar: <= 2 ulp)
+  f64 log, powf (device math library) ................................. <= 2 ulp
   sums ................................................................ |gpu - cpu| <= 1e-5 (f32) /
       1e-12 (f64) times max(|cpu|, sum|x| / sqrt(n)); the second term is the typical magnitude
       of a sum of n such terms, so a result that cancels to ~0 is not held to a relative bar
@@ -263,8 +263,9 @@ def test_unary_f64(hip):
     r = rng(11)
     x = r.standard_normal((257, 129))
     X = hip.Matrix.from_numpy(x)
-    for name, fn, bar in (("exp", zo.EXP, 2), ("tanh", zo.TANH, 0), ("sqrt", zo.SQRT, 0), ("abs", zo.ABS, 0)):
-        xx = np.abs(x) if name == "sqrt" else x
+    for name, fn, bar in (("exp", zo.EXP, 0), ("tanh", zo.TANH, 0), ("sqrt", zo.SQRT, 0), ("abs", zo.ABS, 0),
+                          ("sinh", zo.SINH, 0), ("cosh", zo.COSH, 0), ("log", zo.LOG, 2)):
+        xx = np.abs(x) if name in ("sqrt", "log") else x
         exp = np.empty_like(xx)
         zo.unary(fn, exp, xx)
         got = getattr(hip.Matrix.from_numpy(xx), name)().to_numpy()
@@ -286,7 +287,20 @@ def test_unary_f64(hip):
     got = W.sigmoid().to_numpy()
     fin = ~np.isnan(exp)
     assert np.array_equal(np.isnan(got), np.isnan(exp)) and max_ulp(got[fin], exp[fin]) == 0
-    del X, W
+    # f64 exp, sinh, cosh: the whole finite range, the subnormal results of exp and the overflow edges
+    wide2 = np.concatenate([wide, r.uniform(-745.2, 709.8, 400000), r.uniform(-1, 1, 100000) * 2.0 ** -30,
+                            np.array([709.782712893384, 709.7827128933841, -745.1332191019411, -745.1332191019412,
+                                      -708.3964185322641, 710.4758600739439, 710.475860073944, 1e308, -1e308])])
+    W2 = hip.Matrix.from_numpy(wide2)
+    exp = np.empty_like(wide2)
+    for name, fn in (("exp", zo.EXP), ("sinh", zo.SINH), ("cosh", zo.COSH)):
+        with np.errstate(all="ignore"):
+            zo.unary(fn, exp, wide2)
+        got = getattr(W2, name)().to_numpy()
+        fin = ~np.isnan(exp)
+        assert np.array_equal(np.isnan(got), np.isnan(exp)), name
+        assert np.array_equal(got[fin].view(np.uint64), exp[fin].view(np.uint64)), name
+    del X, W, W2
 
 
 def test_powf(hip):
