@@ -3,7 +3,7 @@ configurations (full size) and on edge cases.  Everything goes through the C ABI
 
 Bars (written where they are used):
   add/sub/mul/div, relu, max, arg-max, copy, SGD/Adam/AdamW .......... bit-exact
-  f32 exp, log, powf, sinh, cosh, sin, cos; f64 exp, sinh, cosh; tanh, sigmoid in f32 and f64
+  f32 exp, log, powf, sinh, cosh, sin, cos, asin, acos, atan; f64 exp, sinh, cosh; tanh, sigmoid in f32 and f64
       (the host libm's algorithms, restated) .......................... bit-exact (bar: <= 2 ulp)
   f64 log, powf (device math library) ................................. <= 2 ulp
   sums ................................................................ |gpu - cpu| <= 1e-5 (f32) /
@@ -211,7 +211,8 @@ def test_transcendental_special_values(hip):
                   3e38, -3e38, 1.1754944e-38, 5e-39], dtype=np.float32)
     X = hip.Matrix.from_numpy(x)
     for name, fn in (("exp", zo.EXP), ("tanh", zo.TANH), ("log", zo.LOG), ("sqrt", zo.SQRT), ("sinh", zo.SINH),
-                     ("cosh", zo.COSH), ("sin", zo.SIN), ("cos", zo.COS)):
+                     ("cosh", zo.COSH), ("sin", zo.SIN), ("cos", zo.COS), ("atan", zo.ATAN),
+                     ("asin", zo.ASIN), ("acos", zo.ACOS)):
         exp = np.empty_like(x)
         with np.errstate(all="ignore"):
             zo.unary(fn, exp, x)
@@ -250,7 +251,8 @@ def test_tanh_sigmoid_dense_sweep(hip):
     assert np.array_equal(np.isnan(got), np.isnan(exp))
     assert max_ulp(got[ok], exp[ok]) == 0                  # includes zeros (-inf), subnormals and +inf
     # cosh is what tanh's backward evaluates; sin / cos include the large-argument reduction
-    for name, fn in (("sinh", zo.SINH), ("cosh", zo.COSH), ("sin", zo.SIN), ("cos", zo.COS)):
+    for name, fn in (("sinh", zo.SINH), ("cosh", zo.COSH), ("sin", zo.SIN), ("cos", zo.COS), ("atan", zo.ATAN),
+                     ("asin", zo.ASIN), ("acos", zo.ACOS)):
         with np.errstate(all="ignore"):
             zo.unary(fn, exp, x)
         got = getattr(X, name)().to_numpy()

@@ -40,4 +40,5 @@ def test_device_tanh_matches_host_libm(tmp_path):
                                   "tanh_fdlibm", "0", "expm1_fdlibm", "0", "sigmoid_zenu", "0",
                                   "exp_glibc", "0", "sinh_fdlibm", "0", "cosh_fdlibm", "0",
                                   "expf_glibc", "0", "logf_glibc", "0", "powf_glibc", "0",
-                                  "sinhf_fdlibm", "0", "coshf_fdlibm", "0", "sinf_glibc", "0", "cosf_glibc", "0"]
+                                  "sinhf_fdlibm", "0", "coshf_fdlibm", "0", "sinf_glibc", "0", "cosf_glibc", "0",
+                                  "atanf_fdlibm", "0", "asinf_fdlibm", "0", "acosf_fdlibm", "0"]

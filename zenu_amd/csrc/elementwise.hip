@@ -77,6 +77,12 @@ __device__ __forceinline__ float dev_sin(float x) { return zmath::sinf_glibc(x);
 __device__ __forceinline__ double dev_sin(double x) { return sin(x); }
 __device__ __forceinline__ float dev_cos(float x) { return zmath::cosf_glibc(x); }
 __device__ __forceinline__ double dev_cos(double x) { return cos(x); }
+__device__ __forceinline__ float dev_asin(float x) { return zmath::asinf_fdlibm(x); }
+__device__ __forceinline__ double dev_asin(double x) { return asin(x); }
+__device__ __forceinline__ float dev_acos(float x) { return zmath::acosf_fdlibm(x); }
+__device__ __forceinline__ double dev_acos(double x) { return acos(x); }
+__device__ __forceinline__ float dev_atan(float x) { return zmath::atanf_fdlibm(x); }
+__device__ __forceinline__ double dev_atan(double x) { return atan(x); }
 __device__ __forceinline__ float dev_sigmoid(float x) { return zmath::sigmoidf_zenu(x); }
 __device__ __forceinline__ double dev_sigmoid(double x) { return zmath::sigmoid_zenu(x); }
 
@@ -98,9 +104,9 @@ template <typename T, int FN> struct UnaryF {
         else if constexpr (FN == ZENU_SIN) return dev_sin(a);
         else if constexpr (FN == ZENU_COS) return dev_cos(a);
         else if constexpr (FN == ZENU_TAN) return tan(a);
-        else if constexpr (FN == ZENU_ASIN) return asin(a);
-        else if constexpr (FN == ZENU_ACOS) return acos(a);
-        else if constexpr (FN == ZENU_ATAN) return atan(a);
+        else if constexpr (FN == ZENU_ASIN) return dev_asin(a);
+        else if constexpr (FN == ZENU_ACOS) return dev_acos(a);
+        else if constexpr (FN == ZENU_ATAN) return dev_atan(a);
         else if constexpr (FN == ZENU_SINH) return m.sinh(a);
         else if constexpr (FN == ZENU_COSH) return m.cosh(a);
         else return dev_sigmoid(a);

@@ -606,6 +606,122 @@ ZM_HD float sincosf_glibc(float y, int cosine)
 ZM_HD float sinf_glibc(float x) { return sincosf_glibc(x, 0); }
 ZM_HD float cosf_glibc(float x) { return sincosf_glibc(x, 1); }
 
+// atanf, asinf, acosf: fdlibm's s_atanf.c, e_asinf.c (the five-term polynomial glibc carries), e_acosf.c as
+// glibc 2.35 ships them, plain f32 arithmetic (no fused operations: these have no FMA build).  The
+// constants are the decimal literals of the sources; atanf returns pi/2 from |x| >= 2^25.  Equal to
+// the host libm on all 2^32 inputs.
+ZM_HD float atanf_fdlibm(float x)
+{
+    // atan(0.5), atan(1), atan(1.5), atan(inf) as high + low parts
+    const float hi0 = 4.6364760399e-01f, hi1 = 7.8539812565e-01f, hi2 = 9.8279368877e-01f, hi3 = 1.5707962513e+00f;
+    const float lo0 = 5.0121582440e-09f, lo1 = 3.7748947079e-08f, lo2 = 3.4473217170e-08f, lo3 = 7.5497894159e-08f;
+    const float a0 = 3.3333334327e-01f, a1 = -2.0000000298e-01f, a2 = 1.4285714924e-01f, a3 = -1.1111110449e-01f,
+                a4 = 9.0908870101e-02f, a5 = -7.6918758452e-02f, a6 = 6.6610731184e-02f, a7 = -5.8335702866e-02f,
+                a8 = 4.9768779427e-02f, a9 = -3.6531571299e-02f, a10 = 1.6285819933e-02f;
+    const float one = 1.0f;
+    const uint32_t hx = f2u(x);
+    const uint32_t ix = hx & 0x7fffffffu;
+    const bool neg = (hx >> 31) != 0;
+    if (ix >= 0x4c000000u) {                             // |x| >= 2^25
+        if (ix > 0x7f800000u) return x + x;              // NaN
+        return neg ? -hi3 - lo3 : hi3 + lo3;
+    }
+    bool reduced = false;
+    float h = 0.0f, l = 0.0f;
+    if (ix < 0x3ee00000u) {                              // |x| < 0.4375
+        if (ix < 0x31000000u) return x;                  // |x| < 2^-29
+    } else {
+        reduced = true;
+        x = u2f(ix);
+        if (ix < 0x3f980000u) {                          // |x| < 1.1875
+            if (ix < 0x3f300000u) { h = hi0; l = lo0; x = (2.0f * x - one) / (2.0f + x); }
+            else                  { h = hi1; l = lo1; x = (x - one) / (x + one); }
+        } else {
+            if (ix < 0x401c0000u) { h = hi2; l = lo2; x = (x - 1.5f) / (one + 1.5f * x); }
+            else                  { h = hi3; l = lo3; x = -1.0f / x; }
+        }
+    }
+    const float z = x * x;
+    const float w = z * z;
+    const float s1 = z * (a0 + w * (a2 + w * (a4 + w * (a6 + w * (a8 + w * a10)))));
+    const float s2 = w * (a1 + w * (a3 + w * (a5 + w * (a7 + w * a9))));
+    if (!reduced) return x - x * (s1 + s2);
+    const float r = h - ((x * (s1 + s2) - l) - x);
+    return neg ? -r : r;
+}
+
+ZM_HD float asinf_fdlibm(float x)
+{
+    const float one = 1.0f, pio2_hi = 1.57079637050628662109375f, pio2_lo = -4.37113900018624283e-8f,
+                pio4_hi = 0.785398185253143310546875f;
+    const float p0 = 1.666675248e-1f, p1 = 7.495297643e-2f, p2 = 4.547037598e-2f, p3 = 2.417951451e-2f,
+                p4 = 4.216630880e-2f;
+    const uint32_t hx = f2u(x);
+    const uint32_t ix = hx & 0x7fffffffu;
+    if (ix == 0x3f800000u) return x * pio2_hi + x * pio2_lo;     // asin(+-1) = +-pi/2
+    if (ix > 0x3f800000u) return (x - x) / (x - x);              // |x| > 1, NaN
+    if (ix < 0x3f000000u) {                              // |x| < 0.5
+        if (ix < 0x32000000u) return x;                  // |x| < 2^-27
+        const float t = x * x;
+        const float w = t * (p0 + t * (p1 + t * (p2 + t * (p3 + t * p4))));
+        return x + x * w;
+    }
+    float w = one - u2f(ix);
+    float t = w * 0.5f;
+    float p = t * (p0 + t * (p1 + t * (p2 + t * (p3 + t * p4))));
+    const float s = sqrtf(t);
+    if (ix >= 0x3F79999Au) {                             // |x| > 0.975
+        t = pio2_hi - (2.0f * (s + s * p) - pio2_lo);
+    } else {
+        w = u2f(f2u(s) & 0xfffff000u);
+        const float c = (t - w * w) / (s + w);
+        const float r = p;
+        p = 2.0f * s * r - (pio2_lo - 2.0f * c);
+        const float q = pio4_hi - 2.0f * w;
+        t = pio4_hi - (p - q);
+    }
+    return (hx >> 31) ? -t : t;
+}
+
+ZM_HD float acosf_fdlibm(float x)
+{
+    const float one = 1.0f, pi = 3.1415925026e+00f, pio2_hi = 1.5707962513e+00f, pio2_lo = 7.5497894159e-08f;
+    const float pS0 = 1.6666667163e-01f, pS1 = -3.2556581497e-01f, pS2 = 2.0121252537e-01f, pS3 = -4.0055535734e-02f,
+                pS4 = 7.9153501429e-04f, pS5 = 3.4793309169e-05f;
+    const float qS1 = -2.4033949375e+00f, qS2 = 2.0209457874e+00f, qS3 = -6.8828397989e-01f, qS4 = 7.7038154006e-02f;
+    const uint32_t hx = f2u(x);
+    const uint32_t ix = hx & 0x7fffffffu;
+    const bool neg = (hx >> 31) != 0;
+    if (ix == 0x3f800000u) return neg ? pi + 2.0f * pio2_lo : 0.0f;   // acos(-1) = pi, acos(1) = 0
+    if (ix > 0x3f800000u) return (x - x) / (x - x);                   // |x| > 1, NaN
+    if (ix < 0x3f000000u) {                              // |x| < 0.5
+        if (ix <= 0x23000000u) return pio2_hi + pio2_lo; // |x| < 2^-57
+        const float z = x * x;
+        const float p = z * (pS0 + z * (pS1 + z * (pS2 + z * (pS3 + z * (pS4 + z * pS5)))));
+        const float q = one + z * (qS1 + z * (qS2 + z * (qS3 + z * qS4)));
+        const float r = p / q;
+        return pio2_hi - (x - (pio2_lo - x * r));
+    }
+    if (neg) {                                           // x < -0.5
+        const float z = (one + x) * 0.5f;
+        const float p = z * (pS0 + z * (pS1 + z * (pS2 + z * (pS3 + z * (pS4 + z * pS5)))));
+        const float q = one + z * (qS1 + z * (qS2 + z * (qS3 + z * qS4)));
+        const float s = sqrtf(z);
+        const float r = p / q;
+        const float w = r * s - pio2_lo;
+        return pi - 2.0f * (s + w);
+    }
+    const float z = (one - x) * 0.5f;                    // x > 0.5
+    const float s = sqrtf(z);
+    const float df = u2f(f2u(s) & 0xfffff000u);
+    const float c = (z - df * df) / (s + df);
+    const float p = z * (pS0 + z * (pS1 + z * (pS2 + z * (pS3 + z * (pS4 + z * pS5)))));
+    const float q = one + z * (qS1 + z * (qS2 + z * (qS3 + z * qS4)));
+    const float r = p / q;
+    const float w = r * s + c;
+    return 2.0f * (df + w);
+}
+
 // ---- double precision exp: the table-driven routine glibc ships since 2.28 (from ARM's optimized routines) ----
 // x = k ln2/N + r, N = 128;  exp(x) = 2^(k/N) exp(r),  2^(k/N) = H[k] (1 + tail[k]) with H the nearest
 // double;  exp(r) - 1 as a degree-5 polynomial.  The table holds {tail[k], bits(H[k]) - (k << 52) / N};
