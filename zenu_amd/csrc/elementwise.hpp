@@ -1,4 +1,4 @@
-// elementwise.hip -- N-d elementwise engine for gfx950 (binary, scalar, unary, relu, clip, copy,
+// elementwise.hpp -- N-d elementwise engine for gfx950 (binary, scalar, unary, relu, clip, copy,
 // broadcast).
 //
 // One Matrix-level call of the reference (add_array, mul_scalar, exp_array, relu, copy_from ...,
@@ -23,6 +23,10 @@
 //
 // Arithmetic is plain IEEE with contraction off; + - * / sqrt are correctly rounded on gfx950,
 // so results are bit-identical to the CPU loops of basic_operations.rs:93-181.
+// This header holds the functors, the kernels and the launch logic; the entry points are spread over
+// ew_binary.hip, ew_unary.hip, ew_unary_trig.hip and ew_misc.hip so that their template
+// instantiations compile in parallel.
+#pragma once
 #include <math.h>
 
 #include "common.hpp"
@@ -744,51 +748,6 @@ int run2(const zenu_tensor_t &to, const zenu_tensor_t &x, const zenu_tensor_t &y
     return launch_ew<T, F>(p, f, s);
 }
 
-template <typename T> int binary_t(int op, const zenu_tensor_t &to, const zenu_tensor_t &l,
-                                   const zenu_tensor_t &r, hipStream_t s)
-{
-    switch (op) {
-    case ZENU_ADD: return run2<T>(to, l, r, BinF<T, ZENU_ADD>(), s);
-    case ZENU_SUB: return run2<T>(to, l, r, BinF<T, ZENU_SUB>(), s);
-    case ZENU_MUL: return run2<T>(to, l, r, BinF<T, ZENU_MUL>(), s);
-    case ZENU_DIV: return run2<T>(to, l, r, BinF<T, ZENU_DIV>(), s);
-    default: return ZENU_ERR_ARG;
-    }
-}
-
-template <typename T> int scalar_t(int op, const zenu_tensor_t &to, const zenu_tensor_t &in, T sv,
-                                   const T *sp, hipStream_t s)
-{
-    switch (op) {
-    case ZENU_ADD: { ScalarF<T, ZENU_ADD> f; f.s = sv; f.sp = sp; return run1<T>(to, in, f, s); }
-    case ZENU_SUB: { ScalarF<T, ZENU_SUB> f; f.s = sv; f.sp = sp; return run1<T>(to, in, f, s); }
-    case ZENU_MUL: { ScalarF<T, ZENU_MUL> f; f.s = sv; f.sp = sp; return run1<T>(to, in, f, s); }
-    case ZENU_DIV: { ScalarF<T, ZENU_DIV> f; f.s = sv; f.sp = sp; return run1<T>(to, in, f, s); }
-    default: return ZENU_ERR_ARG;
-    }
-}
-
-template <typename T> int unary_t(int fn, const zenu_tensor_t &to, const zenu_tensor_t &in, hipStream_t s)
-{
-    switch (fn) {
-    case ZENU_EXP: return run1<T>(to, in, UnaryF<T, ZENU_EXP>(), s);
-    case ZENU_LOG: return run1<T>(to, in, UnaryF<T, ZENU_LOG>(), s);
-    case ZENU_TANH: return run1<T>(to, in, UnaryF<T, ZENU_TANH>(), s);
-    case ZENU_SQRT: return run1<T>(to, in, UnaryF<T, ZENU_SQRT>(), s);
-    case ZENU_ABS: return run1<T>(to, in, UnaryF<T, ZENU_ABS>(), s);
-    case ZENU_SIN: return run1<T>(to, in, UnaryF<T, ZENU_SIN>(), s);
-    case ZENU_COS: return run1<T>(to, in, UnaryF<T, ZENU_COS>(), s);
-    case ZENU_TAN: return run1<T>(to, in, UnaryF<T, ZENU_TAN>(), s);
-    case ZENU_ASIN: return run1<T>(to, in, UnaryF<T, ZENU_ASIN>(), s);
-    case ZENU_ACOS: return run1<T>(to, in, UnaryF<T, ZENU_ACOS>(), s);
-    case ZENU_ATAN: return run1<T>(to, in, UnaryF<T, ZENU_ATAN>(), s);
-    case ZENU_SINH: return run1<T>(to, in, UnaryF<T, ZENU_SINH>(), s);
-    case ZENU_COSH: return run1<T>(to, in, UnaryF<T, ZENU_COSH>(), s);
-    case ZENU_SIGMOID: return run1<T>(to, in, UnaryF<T, ZENU_SIGMOID>(), s);
-    default: return ZENU_ERR_ARG;
-    }
-}
-
 int check2(const zenu_tensor_t *a, const zenu_tensor_t *b)
 {
     int rc = validate_tensor(a);
@@ -798,215 +757,3 @@ int check2(const zenu_tensor_t *a, const zenu_tensor_t *b)
 
 }  // namespace
 }  // namespace zenu
-
-using namespace zenu;
-
-template <template <typename> class F>
-static int activation_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *gy, const zenu_tensor_t *x,
-                               zenu_stream_t stream)
-{
-    int rc = check2(gx, gy);
-    if (!rc) rc = validate_tensor(x);
-    if (!rc) rc = ensure_init();
-    if (rc) return rc;
-    if (!same_shape(*gx, *gy) || !same_shape(*gx, *x)) return ZENU_ERR_SHAPE;
-    if (dtype == ZENU_F32) return run2<float>(*gx, *gy, *x, F<float>(), as_stream(stream));
-    if (dtype == ZENU_F64) return run2<double>(*gx, *gy, *x, F<double>(), as_stream(stream));
-    return ZENU_ERR_ARG;
-}
-
-extern "C" {
-
-int zenu_hip_binary(int op, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *lhs,
-                    const zenu_tensor_t *rhs, zenu_stream_t stream)
-{
-    int rc = check2(to, lhs);
-    if (!rc) rc = validate_tensor(rhs);
-    if (!rc) rc = ensure_init();
-    if (!rc) rc = check_binary(*to, *lhs, *rhs);
-    if (rc) return rc;
-    if (dtype == ZENU_F32) return binary_t<float>(op, *to, *lhs, *rhs, as_stream(stream));
-    if (dtype == ZENU_F64) return binary_t<double>(op, *to, *lhs, *rhs, as_stream(stream));
-    return ZENU_ERR_ARG;
-}
-
-int zenu_hip_binary_assign(int op, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *rhs,
-                           zenu_stream_t stream)
-{
-    int rc = check2(to, rhs);
-    if (!rc) rc = ensure_init();
-    if (!rc) rc = check_binary_assign(*to, *rhs);
-    if (rc) return rc;
-    if (dtype == ZENU_F32) return binary_t<float>(op, *to, *to, *rhs, as_stream(stream));
-    if (dtype == ZENU_F64) return binary_t<double>(op, *to, *to, *rhs, as_stream(stream));
-    return ZENU_ERR_ARG;
-}
-
-static int scalar_common(int op, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other,
-                         double scalar, const void *sp, zenu_stream_t stream)
-{
-    int rc = check2(to, other);
-    if (!rc) rc = ensure_init();
-    if (rc) return rc;
-    if (to->ndim < other->ndim) return ZENU_ERR_RANK;   // with_clousers.rs:42-50
-    if (!same_shape(*to, *other)) return ZENU_ERR_SHAPE;
-    if (dtype == ZENU_F32)
-        return scalar_t<float>(op, *to, *other, (float)scalar, static_cast<const float *>(sp),
-                               as_stream(stream));
-    if (dtype == ZENU_F64)
-        return scalar_t<double>(op, *to, *other, scalar, static_cast<const double *>(sp),
-                                as_stream(stream));
-    return ZENU_ERR_ARG;
-}
-
-int zenu_hip_binary_scalar(int op, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other,
-                           double scalar, zenu_stream_t stream)
-{
-    return scalar_common(op, dtype, to, other, scalar, nullptr, stream);
-}
-
-int zenu_hip_binary_scalar_assign(int op, int dtype, const zenu_tensor_t *to, double scalar,
-                                  zenu_stream_t stream)
-{
-    return scalar_common(op, dtype, to, to, scalar, nullptr, stream);
-}
-
-int zenu_hip_binary_scalar_ptr(int op, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other,
-                               const void *scalar_dev, zenu_stream_t stream)
-{
-    if (!scalar_dev) return ZENU_ERR_ARG;
-    return scalar_common(op, dtype, to, other, 0.0, scalar_dev, stream);
-}
-
-int zenu_hip_binary_scalar_assign_ptr(int op, int dtype, const zenu_tensor_t *to,
-                                      const void *scalar_dev, zenu_stream_t stream)
-{
-    if (!scalar_dev) return ZENU_ERR_ARG;
-    return scalar_common(op, dtype, to, to, 0.0, scalar_dev, stream);
-}
-
-int zenu_hip_unary(int fn, int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other,
-                   zenu_stream_t stream)
-{
-    int rc = check2(to, other);
-    if (!rc) rc = ensure_init();
-    if (rc) return rc;
-    if (!same_shape(*to, *other)) return ZENU_ERR_SHAPE;  // "Matrix shape mismatch"
-    if (dtype == ZENU_F32) return unary_t<float>(fn, *to, *other, as_stream(stream));
-    if (dtype == ZENU_F64) return unary_t<double>(fn, *to, *other, as_stream(stream));
-    return ZENU_ERR_ARG;
-}
-
-int zenu_hip_unary_assign(int fn, int dtype, const zenu_tensor_t *to, zenu_stream_t stream)
-{
-    return zenu_hip_unary(fn, dtype, to, to, stream);
-}
-
-int zenu_hip_powf(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other, double scalar,
-                  zenu_stream_t stream)
-{
-    int rc = check2(to, other);
-    if (!rc) rc = ensure_init();
-    if (rc) return rc;
-    if (!same_shape(*to, *other)) return ZENU_ERR_SHAPE;
-    if (dtype == ZENU_F32) { PowF<float> f; f.s = (float)scalar; return run1<float>(*to, *other, f, as_stream(stream)); }
-    if (dtype == ZENU_F64) { PowF<double> f; f.s = scalar; return run1<double>(*to, *other, f, as_stream(stream)); }
-    return ZENU_ERR_ARG;
-}
-
-int zenu_hip_relu(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other, double alpha,
-                  zenu_stream_t stream)
-{
-    int rc = check2(to, other);
-    if (!rc) rc = ensure_init();
-    if (rc) return rc;
-    if (!same_shape(*to, *other)) return ZENU_ERR_SHAPE;  // "shape mismatch"
-    if (dtype == ZENU_F32) { ReluF<float> f; f.alpha = (float)alpha; return run1<float>(*to, *other, f, as_stream(stream)); }
-    if (dtype == ZENU_F64) { ReluF<double> f; f.alpha = alpha; return run1<double>(*to, *other, f, as_stream(stream)); }
-    return ZENU_ERR_ARG;
-}
-
-int zenu_hip_relu_backward_mask(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other,
-                                double alpha, zenu_stream_t stream)
-{
-    int rc = check2(to, other);
-    if (!rc) rc = ensure_init();
-    if (rc) return rc;
-    if (!same_shape(*to, *other)) return ZENU_ERR_SHAPE;
-    if (dtype == ZENU_F32) { ReluMaskF<float> f; f.alpha = (float)alpha; return run1<float>(*to, *other, f, as_stream(stream)); }
-    if (dtype == ZENU_F64) { ReluMaskF<double> f; f.alpha = alpha; return run1<double>(*to, *other, f, as_stream(stream)); }
-    return ZENU_ERR_ARG;
-}
-
-int zenu_hip_broadcast(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *source, zenu_stream_t stream)
-{
-    int rc = check2(to, source);
-    if (!rc) rc = ensure_init();
-    if (!rc) rc = check_binary_assign(*to, *source);   // is_include || is_include_bradcast, broadcast.rs:13-17
-    if (rc) return rc;
-    if (dtype == ZENU_F32) return run1<float>(*to, *source, CopyF<float>(), as_stream(stream));
-    if (dtype == ZENU_F64) return run1<double>(*to, *source, CopyF<double>(), as_stream(stream));
-    return ZENU_ERR_ARG;
-}
-
-int zenu_hip_relu_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *gy, const zenu_tensor_t *x,
-                           double alpha, zenu_stream_t stream)
-{
-    int rc = check2(gx, gy);
-    if (!rc) rc = validate_tensor(x);
-    if (!rc) rc = ensure_init();
-    if (rc) return rc;
-    if (!same_shape(*gx, *gy) || !same_shape(*gx, *x)) return ZENU_ERR_SHAPE;
-    if (dtype == ZENU_F32) { ReluBwdF<float> f; f.alpha = (float)alpha; return run2<float>(*gx, *gy, *x, f, as_stream(stream)); }
-    if (dtype == ZENU_F64) { ReluBwdF<double> f; f.alpha = alpha; return run2<double>(*gx, *gy, *x, f, as_stream(stream)); }
-    return ZENU_ERR_ARG;
-}
-
-int zenu_hip_tanh_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *gy, const zenu_tensor_t *x,
-                           zenu_stream_t stream)
-{
-    return activation_backward<TanhBwdF>(dtype, gx, gy, x, stream);
-}
-
-int zenu_hip_sigmoid_backward(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *gy, const zenu_tensor_t *x,
-                              zenu_stream_t stream)
-{
-    return activation_backward<SigmoidBwdF>(dtype, gx, gy, x, stream);
-}
-
-int zenu_hip_clip(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other, double min, double max,
-                  zenu_stream_t stream)
-{
-    int rc = check2(to, other);
-    if (!rc) rc = ensure_init();
-    if (rc) return rc;
-    if (!same_shape(*to, *other)) return ZENU_ERR_SHAPE;
-    if (dtype == ZENU_F32) { ClipF<float> f; f.lo = (float)min; f.hi = (float)max; return run1<float>(*to, *other, f, as_stream(stream)); }
-    if (dtype == ZENU_F64) { ClipF<double> f; f.lo = min; f.hi = max; return run1<double>(*to, *other, f, as_stream(stream)); }
-    return ZENU_ERR_ARG;
-}
-
-int zenu_hip_clip_backward_mask(int dtype, const zenu_tensor_t *mask, const zenu_tensor_t *other, double min,
-                                double max, zenu_stream_t stream)
-{
-    int rc = check2(mask, other);
-    if (!rc) rc = ensure_init();
-    if (rc) return rc;
-    if (!same_shape(*mask, *other)) return ZENU_ERR_SHAPE;
-    if (dtype == ZENU_F32) { ClipMaskF<float> f; f.lo = (float)min; f.hi = (float)max; return run1<float>(*mask, *other, f, as_stream(stream)); }
-    if (dtype == ZENU_F64) { ClipMaskF<double> f; f.lo = min; f.hi = max; return run1<double>(*mask, *other, f, as_stream(stream)); }
-    return ZENU_ERR_ARG;
-}
-
-int zenu_hip_copy(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *src, zenu_stream_t stream)
-{
-    int rc = check2(to, src);
-    if (!rc) rc = ensure_init();
-    if (rc) return rc;
-    if (!same_shape(*to, *src)) return ZENU_ERR_SHAPE;
-    if (dtype == ZENU_F32) return run1<float>(*to, *src, CopyF<float>(), as_stream(stream));
-    if (dtype == ZENU_F64) return run1<double>(*to, *src, CopyF<double>(), as_stream(stream));
-    return ZENU_ERR_ARG;
-}
-
-}  // extern "C"
