@@ -280,8 +280,8 @@ int zenu_hip_adam_step_multi(int dtype, int n_tensors, void *const *p_dev, const
 /* They let the unchanged zenu-cuda/src/kernel/mod.rs wrappers link.            */
 /* ------------------------------------------------------------------------- */
 
-#define ZENU_DECL_1D(T, S)                                                                         \
-    /* array_array.h:7-28 */                                                                       \
+#define ZENU_DECL_1D(T, S)                                                                        \
+    /* array_array.h:7-28 */                                                                      \
     void array_array_add_##S(T *a, int stride_a, T *b, int stride_b, T *c, int stride_c, int n);  \
     void array_array_sub_##S(T *a, int stride_a, T *b, int stride_b, T *c, int stride_c, int n);  \
     void array_array_mul_##S(T *a, int stride_a, T *b, int stride_b, T *c, int stride_c, int n);  \
@@ -290,7 +290,7 @@ int zenu_hip_adam_step_multi(int dtype, int n_tensors, void *const *p_dev, const
     void array_array_sub_assign_##S(T *a, int stride_a, T *b, int stride_b, int n);               \
     void array_array_mul_assign_##S(T *a, int stride_a, T *b, int stride_b, int n);               \
     void array_array_div_assign_##S(T *a, int stride_a, T *b, int stride_b, int n);               \
-    /* array_scalar.h:7-44 */                                                                      \
+    /* array_scalar.h:7-44 */                                                                     \
     void array_scalar_add_##S(T *a, int size, int stride_a, T scalar, T *out, int stride_out);    \
     void array_scalar_sub_##S(T *a, int size, int stride_a, T scalar, T *out, int stride_out);    \
     void array_scalar_mul_##S(T *a, int size, int stride_a, T scalar, T *out, int stride_out);    \
@@ -307,7 +307,7 @@ int zenu_hip_adam_step_multi(int dtype, int n_tensors, void *const *p_dev, const
     void array_scalar_pointer_sub_assign_##S(T *a, int size, int stride, T *scalar);              \
     void array_scalar_pointer_mul_assign_##S(T *a, int size, int stride, T *scalar);              \
     void array_scalar_pointer_div_assign_##S(T *a, int size, int stride, T *scalar);              \
-    /* array_scalar.h:46-112 (unary) */                                                            \
+    /* array_scalar.h:46-112 (unary) */                                                           \
     void array_exp_##S(T *a, int size, int stride_in, T *out, int stride_out);                    \
     void array_log_##S(T *a, int size, int stride_in, T *out, int stride_out);                    \
     void array_tanh_##S(T *a, int size, int stride_in, T *out, int stride_out);                   \
@@ -318,22 +318,41 @@ int zenu_hip_adam_step_multi(int dtype, int n_tensors, void *const *p_dev, const
     void array_tanh_assign_##S(T *a, int size, int stride);                                       \
     void array_sqrt_assign_##S(T *a, int size, int stride);                                       \
     void array_abs_assign_##S(T *a, int size, int stride);                                        \
-    /* array_scalar.h:97-106 */                                                                    \
+    void array_sin_##S(T *a, int size, int stride_in, T *out, int stride_out);                    \
+    void array_cos_##S(T *a, int size, int stride_in, T *out, int stride_out);                    \
+    void array_tan_##S(T *a, int size, int stride_in, T *out, int stride_out);                    \
+    void array_asin_##S(T *a, int size, int stride_in, T *out, int stride_out);                   \
+    void array_acos_##S(T *a, int size, int stride_in, T *out, int stride_out);                   \
+    void array_atan_##S(T *a, int size, int stride_in, T *out, int stride_out);                   \
+    void array_sinh_##S(T *a, int size, int stride_in, T *out, int stride_out);                   \
+    void array_cosh_##S(T *a, int size, int stride_in, T *out, int stride_out);                   \
+    void array_sin_assign_##S(T *a, int size, int stride);                                        \
+    void array_cos_assign_##S(T *a, int size, int stride);                                        \
+    void array_tan_assign_##S(T *a, int size, int stride);                                        \
+    void array_asin_assign_##S(T *a, int size, int stride);                                       \
+    void array_acos_assign_##S(T *a, int size, int stride);                                       \
+    void array_atan_assign_##S(T *a, int size, int stride);                                       \
+    void array_sinh_assign_##S(T *a, int size, int stride);                                       \
+    void array_cosh_assign_##S(T *a, int size, int stride);                                       \
+    /* array_scalar.h:109-112 */                                                                  \
+    void array_pow_##S(T *a, int size, int stride_a, T scalar, T *out, int stride_o);             \
+    void array_pow_assign_##S(T *a, int size, int stride, T scalar);                              \
+    /* array_scalar.h:97-106 */                                                                   \
     void array_clip_##S(T *input, T *output, int size, int stride_in, int stride_out, T min, T max); \
     void array_clip_assign_##S(T *input, int size, int stride, T min, T max);                     \
     void array_clip_backward_##S(T *input, T *mask, T max, T min, int size, int stride_in,        \
-                                 int stride_mask);                                                 \
+                                 int stride_mask);                                                \
     void array_clip_backward_assign_##S(T *input, T max, T min, int size, int stride);            \
     /* array_array.h:27-28: output[i] = input[i] + bias[(i / channel_stride) % bias_size] */      \
     void conv_bias_add_##S(const T *input, T *output, int channel_stride, const T *bias,          \
-                           int bias_size, int total_elements);                                     \
+                           int bias_size, int total_elements);                                    \
     /* conv2d_bkwd_data.h:7-17: dbias[c] = sum over n, h, w of dOut[n, c, h, w]; follows the CPU  \
        path (zenu-matrix/src/nn/conv/cpu/bias.rs:18-25: sum(0), sum(2), sum(3)) */                \
     void conv2d_bias_bkwd_##S(const T *dOut, T *dbias, int N, int C, int H, int W);               \
-    /* activations.h:7-11 */                                                                       \
+    /* activations.h:7-11 */                                                                      \
     void relu_##S(T *input, T *output, T alpha, int size, int input_stride, int output_stride);   \
     void relu_backward_mask_##S(T *input, T *mask, T alpha, int size, int input_stride,           \
-                                int mask_stride);                                                  \
+                                int mask_stride);                                                 \
     /* element_wise.h:7-9: `out` is a HOST int (zenu-cuda/src/kernel/mod.rs:570-588); blocking */ \
     void array_max_idx_##S(T *a, int size, int stride, int *out);                                 \
     /* memory_access.h:7-11: blocking single-element copies */                                    \

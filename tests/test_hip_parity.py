@@ -716,6 +716,35 @@ def test_reference_named_entry_points(hip):
     l.memory_set_float.restype = None
     l.memory_set_float(A.as_ptr(), 17, C.c_float(42.5))
     assert A.to_numpy()[17] == np.float32(42.5)
+    # the unary family (array_scalar.h:46-95) and pow (:109-112): strided out-of-place and in-place forms
+    src = np.clip(r.standard_normal(3 * n), -0.99, 0.99).astype(np.float32)
+    for name, fn in (("exp", zo.EXP), ("log", zo.LOG), ("tanh", zo.TANH), ("sqrt", zo.SQRT), ("abs", zo.ABS),
+                     ("sin", zo.SIN), ("cos", zo.COS), ("asin", zo.ASIN), ("acos", zo.ACOS), ("atan", zo.ATAN),
+                     ("sinh", zo.SINH), ("cosh", zo.COSH)):
+        xin = np.abs(src) + np.float32(0.01) if name in ("log", "sqrt") else src
+        S = hip.Matrix.from_numpy(xin)
+        f = getattr(l, f"array_{name}_float")
+        f.argtypes, f.restype = [vp, C.c_int, C.c_int, vp, C.c_int], None
+        f(S.as_ptr(), n, 3, OUT.as_ptr(), 1)
+        exp = np.empty(n, dtype=np.float32)
+        zo.unary(fn, exp, np.ascontiguousarray(xin[::3]))
+        assert_bits(OUT.to_numpy(), exp, f"array_{name}_float")
+        g = getattr(l, f"array_{name}_assign_float")
+        g.argtypes, g.restype = [vp, C.c_int, C.c_int], None
+        g(S.as_ptr(), n, 3)
+        got = S.to_numpy()
+        assert_bits(np.ascontiguousarray(got[::3]), exp, f"array_{name}_assign_float")
+        assert_bits(np.ascontiguousarray(got[1::3]), np.ascontiguousarray(xin[1::3]),
+                    f"array_{name}_assign_float leaves the gaps alone")
+    P = hip.Matrix.from_numpy(np.abs(src) + np.float32(0.01))
+    l.array_pow_float.argtypes, l.array_pow_float.restype = [vp, C.c_int, C.c_int, C.c_float, vp, C.c_int], None
+    l.array_pow_float(P.as_ptr(), n, 3, C.c_float(2.5), OUT.as_ptr(), 1)
+    exp = np.empty(n, dtype=np.float32)
+    zo.powf(exp, np.ascontiguousarray((np.abs(src) + np.float32(0.01))[::3]), 2.5)
+    assert_bits(OUT.to_numpy(), exp, "array_pow_float")
+    l.array_pow_assign_float.argtypes, l.array_pow_assign_float.restype = [vp, C.c_int, C.c_int, C.c_float], None
+    l.array_pow_assign_float(P.as_ptr(), n, 3, C.c_float(2.5))
+    assert_bits(np.ascontiguousarray(P.to_numpy()[::3]), exp, "array_pow_assign_float")
 
 
 # ---- allocator on the device ------------------------------------------------------------------------------------

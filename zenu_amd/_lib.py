@@ -98,7 +98,7 @@ SIGNATURES = {
 }
 
 _BIN = ("add", "sub", "mul", "div")
-_UN = ("exp", "log", "tanh", "sqrt", "abs")
+_UN = ("exp", "log", "tanh", "sqrt", "abs", "sin", "cos", "tan", "asin", "acos", "atan", "sinh", "cosh")
 
 
 def reference_named_symbols():
@@ -115,7 +115,8 @@ def reference_named_symbols():
         names += [f"relu_{s}", f"relu_backward_mask_{s}", f"array_max_idx_{s}",
                   f"memory_access_{s}", f"memory_set_{s}",
                   f"array_clip_{s}", f"array_clip_assign_{s}", f"array_clip_backward_{s}",
-                  f"array_clip_backward_assign_{s}", f"conv_bias_add_{s}", f"conv2d_bias_bkwd_{s}"]
+                  f"array_clip_backward_assign_{s}", f"conv_bias_add_{s}", f"conv2d_bias_bkwd_{s}",
+                  f"array_pow_{s}", f"array_pow_assign_{s}"]
     return names
 
 

@@ -174,6 +174,32 @@ extern "C" {
     void array_tanh_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_TANH, a, n, s); }                   \
     void array_sqrt_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_SQRT, a, n, s); }                   \
     void array_abs_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_ABS, a, n, s); }                     \
+    void array_sin_##S(T *a, int n, int si, T *o, int so) { un<T>(ZENU_SIN, a, n, si, o, so); }            \
+    void array_cos_##S(T *a, int n, int si, T *o, int so) { un<T>(ZENU_COS, a, n, si, o, so); }            \
+    void array_tan_##S(T *a, int n, int si, T *o, int so) { un<T>(ZENU_TAN, a, n, si, o, so); }            \
+    void array_asin_##S(T *a, int n, int si, T *o, int so) { un<T>(ZENU_ASIN, a, n, si, o, so); }          \
+    void array_acos_##S(T *a, int n, int si, T *o, int so) { un<T>(ZENU_ACOS, a, n, si, o, so); }          \
+    void array_atan_##S(T *a, int n, int si, T *o, int so) { un<T>(ZENU_ATAN, a, n, si, o, so); }          \
+    void array_sinh_##S(T *a, int n, int si, T *o, int so) { un<T>(ZENU_SINH, a, n, si, o, so); }          \
+    void array_cosh_##S(T *a, int n, int si, T *o, int so) { un<T>(ZENU_COSH, a, n, si, o, so); }          \
+    void array_sin_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_SIN, a, n, s); }                     \
+    void array_cos_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_COS, a, n, s); }                     \
+    void array_tan_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_TAN, a, n, s); }                     \
+    void array_asin_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_ASIN, a, n, s); }                   \
+    void array_acos_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_ACOS, a, n, s); }                   \
+    void array_atan_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_ATAN, a, n, s); }                   \
+    void array_sinh_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_SINH, a, n, s); }                   \
+    void array_cosh_assign_##S(T *a, int n, int s) { un_assign<T>(ZENU_COSH, a, n, s); }                   \
+    void array_pow_##S(T *a, int n, int sa, T scalar, T *o, int so)                                        \
+    {                                                                                                      \
+        zenu_tensor_t ti = view1d(a, n, sa), to = view1d(o, n, so);                                        \
+        (void)zenu_hip_powf(dtype_of<T>(), &to, &ti, (double)scalar, nullptr);                             \
+    }                                                                                                      \
+    void array_pow_assign_##S(T *a, int n, int s, T scalar)                                                \
+    {                                                                                                      \
+        zenu_tensor_t t = view1d(a, n, s);                                                                 \
+        (void)zenu_hip_powf(dtype_of<T>(), &t, &t, (double)scalar, nullptr);                               \
+    }                                                                                                      \
     void array_clip_##S(T *in, T *out, int n, int si, int so, T lo, T hi)                                  \
     {                                                                                                      \
         zenu_tensor_t ti = view1d(in, n, si), to = view1d(out, n, so);                                     \
