@@ -442,10 +442,10 @@ def measured_traffic(op):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="suite", choices=["suite", "c0", "c1", "c2", "c3", "c4", "fused"])
-    ap.add_argument("--op-reps", type=int, default=40, help="launches per op in the per-op timing")
+    ap.add_argument("--op-reps", type=int, default=50, help="launches per op in the per-op timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--profile-op", default=None, help="only launch this op (for rocprofv3 counter runs)")
     args = ap.parse_args()
@@ -496,10 +496,14 @@ def main():
     value = step_bytes / (elapsed / args.steps) / 1e9
 
     # ---- per-op timing with HIP events on the launch stream ---------------------------------------------
+    # `us` is the mean over op_reps back-to-back launches (one event pair around the batch) and agrees
+    # with the kernel durations of a rocprofv3 trace; a second pass brackets every launch with its
+    # own events for a median and a minimum, which include the cost of one event record (~2.5 us)
     e0, e1 = hip.event(), hip.event()
+    marks = [hip.event() for _ in range(args.op_reps + 1)]
     table = []
     for o in ops:
-        for _ in range(5):
+        for _ in range(10):
             o.launch()
         sync()
         hip.record(e0, stream)
@@ -507,10 +511,15 @@ def main():
             o.launch()
         hip.record(e1, stream)
         us = hip.elapsed_ms(e0, e1) / args.op_reps * 1e3
+        hip.record(marks[0], stream)
+        for i in range(args.op_reps):
+            o.launch()
+            hip.record(marks[i + 1], stream)
+        each = sorted(hip.elapsed_ms(marks[i], marks[i + 1]) * 1e3 for i in range(args.op_reps))
         gbps = o.alg_bytes / (us * 1e-6) / 1e9
         table.append(dict(op=o.name, config=o.config, dtype=o.dtype, us=round(us, 2), GBps=round(gbps, 1),
                           frac_of_peak=round(gbps / PEAK_HBM_GBPS, 4), Gelem_per_s=round(o.elems / (us * 1e-6) / 1e9, 2),
-                          alg_bytes=o.alg_bytes))
+                          alg_bytes=o.alg_bytes, us_bracketed_median=round(each[len(each) // 2], 2), us_bracketed_min=round(each[0], 2)))
         log(f"[op] {o.name:22s} {us:9.2f} us  {gbps:8.1f} GB/s  {100 * gbps / PEAK_HBM_GBPS:5.1f}% of peak")
 
     # dominant kernel of the step = the op with the largest share of the step time
@@ -556,6 +565,8 @@ def main():
         "frac_of_peak_whole_step": round(value / PEAK_HBM_GBPS, 4),
         "adam_step_params_per_sec": (round(adam[0]["Gelem_per_s"] * 1e9) if adam else None),
         "roofline": roofline, "cpu_baseline": cpu, "ops": table,
+        "timing": f"HIP events on the launch stream; per op {args.op_reps} back-to-back launches after 10 warm-up launches: "
+                  "us = batch mean, us_bracketed_* = per-launch event pairs (each includes one event record)",
     }
     print(json.dumps(out))
 
