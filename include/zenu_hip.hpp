@@ -492,6 +492,24 @@ public:
         check(zenu_hip_memcpy_d2h(&v, val.ptr, sizeof v, st()), "memcpy_d2h");
         return v;
     }
+    Matrix mean(int axis, bool keep_dim = false) const    // mean.rs:10-13
+    {
+        return sum(axis, keep_dim) / (T)shape()[axis];
+    }
+    Matrix mean_all() const                               // mean.rs:15-19: asum / num_elm, the mean of |x|
+    {
+        return from_vec({asum() / (T)num_elm(shape())}, {});
+    }
+    Matrix variance(int axis, bool keep_dim = false) const   // var.rs:19-26
+    {
+        Matrix diff = *this - mean(axis, true);
+        return (diff * diff).mean(axis, keep_dim);
+    }
+    Matrix variance_all() const
+    {
+        Matrix diff = *this - mean_all();
+        return (diff * diff).mean_all();
+    }
     T asum() const                                        // asum.rs:49-68
     {
         Buffer val(sizeof(T));

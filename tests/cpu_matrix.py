@@ -191,6 +191,20 @@ class CpuMatrix:
     def max_axis_idx_ravel(self, axis): return [int(i) for i in zo.max_axis_idx_ravel(self.a, axis)]
     def asum(self): return zo.asum(self.a)
 
+    def mean(self, axis=None, keep_dim=False):
+        """mean.rs:9-20"""
+        if axis is not None:
+            return self.sum(axis, keep_dim) / self.dtype.type(self.shape[axis])
+        n = 1
+        for d in self.shape:
+            n *= d
+        return CpuMatrix.from_numpy(np.asarray(self.asum() / self.dtype.type(n), dtype=self.dtype))
+
+    def variance(self, axis=None, keep_dim=False):
+        """var.rs:19-26"""
+        diff = self - self.mean(axis, True)
+        return (diff * diff).mean(axis, keep_dim)
+
 
 def _named(name, op):
     setattr(CpuMatrix, f"{name}_array", lambda self, l, r: zo.binary_array(op, self.a, l.a, r.a))

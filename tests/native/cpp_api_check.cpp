@@ -259,6 +259,18 @@ static void broadcast_cases() // broadcast.rs:53-165
     REQUIRE(eq(r1, {1, 1, 1}));
 }
 
+static void mean_variance_cases() // var.rs test mod, mean.rs:9-20
+{
+    REQUIRE(close(M::from_vec({1, 2, 3, 4}, {4}).variance_all(), {1.25}, 1e-6));
+    REQUIRE(close(M::from_vec({1, 2}, {2}).variance_all(), {0.25}, 1e-6));
+    M x = M::from_vec({1, 2, 3, 4}, {2, 2});
+    REQUIRE(close(x.variance_all(), {1.25}, 1e-6));
+    REQUIRE(close(x.variance(0), {1., 1.}, 1e-6));
+    REQUIRE(close(x.variance(1), {0.25, 0.25}, 1e-6));
+    REQUIRE(close(x.mean(1, true), {1.5, 3.5}, 1e-6));
+    REQUIRE(close(M::from_vec({-1, 2, -3, 4}, {4}).mean_all(), {2.5}, 1e-6));   // the mean of |x|
+}
+
 static void conv_bias_cases() // zenu-matrix/src/nn/conv/mod.rs:84-107, cpu/bias.rs:10-25
 {
     const int n = 2, c = 3, h = 2, w = 4;
@@ -415,7 +427,7 @@ int main(int argc, char **argv)
         {"broadcast_add_1x4x1x1_3x4x5x5", broadcast_add_1x4x1x1_3x4x5x5}, {"sub_mul_div", sub_mul_div},
         {"shape_errors", shape_errors}, {"unary_tables", unary_tables}, {"relu_cases", relu_cases},
         {"sigmoid_cases", sigmoid_cases}, {"sum_4d", sum_4d}, {"max_cases", max_cases}, {"asum_cases", asum_cases},
-        {"copy_cases", copy_cases}, {"broadcast_cases", broadcast_cases}, {"conv_bias_cases", conv_bias_cases},
+        {"copy_cases", copy_cases}, {"broadcast_cases", broadcast_cases}, {"conv_bias_cases", conv_bias_cases}, {"mean_variance_cases", mean_variance_cases},
         {"softmax_cases", softmax_cases},
         {"cross_entropy_cases", cross_entropy_cases}, {"clip_cases", clip_cases}, {"sgd_net_test", sgd_net_test},
         {"adam_net_test", adam_net_test}, {"adam_w_net_test", adam_w_net_test},

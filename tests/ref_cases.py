@@ -316,6 +316,24 @@ def autograd_unary_backward(dev):
     close(gs, [v * (1 - v) for v in sg], 1e-7)
 
 
+# ---- mean / variance: zenu-matrix/src/operation/var.rs test mod, mean.rs:9-20 ------------------------------
+
+
+@case
+def mean_variance_cases(dev):
+    for dt in (np.float32, np.float64):
+        close(dev.M.from_vec([1., 2., 3., 4.], [4], dt).variance(None, False), 1.25, 1e-6)      # variance_1d
+        close(dev.M.from_vec([1., 2.], [2], dt).variance(None, False), 0.25, 1e-6)              # variance_1d_
+        x = dev.M.from_vec([1., 2., 3., 4.], [2, 2], dt)
+        close(x.variance(None, False), 1.25, 1e-6)                                              # variance_2d
+        close(x.variance(0, False), [1., 1.], 1e-6)                                             # variance_2d_0
+        close(x.variance(1, False), [0.25, 0.25], 1e-6)                                         # variance_2d_1
+        close(x.mean(0, False), [2., 3.], 1e-6)
+        close(x.mean(1, True), [[1.5], [3.5]], 1e-6)
+        # without an axis the reference averages |x| (mean.rs:15-19 calls asum)
+        close(dev.M.from_vec([-1., 2., -3., 4.], [4], dt).mean(None, False), 2.5, 1e-6)
+
+
 # ---- sum: sum.rs:109-245 ------------------------------------------------------------------------------
 
 _SUM1 = [60, 63, 66, 69, 72, 75, 78, 81, 84, 87, 90, 93, 96, 99, 102, 105, 108, 111, 114, 117,

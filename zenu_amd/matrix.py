@@ -439,6 +439,21 @@ class Matrix:
         check(_lib.lib().zenu_hip_asum(_dt(self.dtype), out.as_ptr(), C.byref(self.desc()), _stream), "asum")
         return out.to_numpy()[()]
 
+    def mean(self, axis=None, keep_dim=False):
+        """mean.rs:9-20: sum(axis) / n; without an axis asum() / num_elm -- the mean of |x|, as the
+        reference computes it -- returned as a 0-d matrix"""
+        if axis is not None:
+            return self.sum(axis, keep_dim) / self.dtype.type(self.shape[axis])
+        n = 1
+        for d in self.shape:
+            n *= d
+        return Matrix.from_numpy(np.asarray(self.asum() / self.dtype.type(n), dtype=self.dtype))
+
+    def variance(self, axis=None, keep_dim=False):
+        """var.rs:19-26: mean((x - mean(x, keep))^2), each step an operator of its own"""
+        diff = self - self.mean(axis, True)
+        return (diff * diff).mean(axis, keep_dim)
+
     def index_item(self, index):
         return self.to_numpy()[tuple(index)]
 
