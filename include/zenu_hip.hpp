@@ -551,6 +551,46 @@ Matrix<T> cross_entropy_backward(const Matrix<T> &prob, const Matrix<T> &ans, co
     return g;
 }
 
+// ---- stack / split (zenu-matrix/src/operation/stack.rs:18-58, split.rs:20-58): one strided copy per piece ------
+
+template <typename T> Matrix<T> axis_range(const Matrix<T> &m, int axis, int64_t start, int64_t stop)
+{
+    std::vector<Slice> s((size_t)axis + 1);
+    s[(size_t)axis] = Slice(start, stop);
+    return m.slice(s);
+}
+
+template <typename T> Matrix<T> stack(const std::vector<Matrix<T>> &matrices, int axis)
+{
+    if (matrices.empty()) throw Error(ZENU_ERR_ARG, "stack: No matrices to stack");
+    const Dim first = matrices[0].shape();
+    for (const Matrix<T> &m : matrices)
+        if (m.shape() != first) throw Error(ZENU_ERR_SHAPE, "stack: All matrices must have the same shape");
+    if (axis < 0 || axis >= (int)first.size()) throw Error(ZENU_ERR_AXIS, "stack");
+    const int64_t n = first[(size_t)axis];
+    Dim shape = first;
+    shape[(size_t)axis] = n * (int64_t)matrices.size();
+    Matrix<T> out = Matrix<T>::alloc(shape);
+    for (size_t i = 0; i < matrices.size(); i++) axis_range(out, axis, (int64_t)i * n, (int64_t)(i + 1) * n).copy_from(matrices[i]);
+    return out;
+}
+
+template <typename T> std::vector<Matrix<T>> split(const Matrix<T> &matrix, int axis, int num_splits)
+{
+    if (axis < 0 || axis >= matrix.ndim()) throw Error(ZENU_ERR_AXIS, "split");
+    if (num_splits <= 0 || matrix.shape()[(size_t)axis] % num_splits) throw Error(ZENU_ERR_SHAPE, "split");
+    const int64_t n = matrix.shape()[(size_t)axis] / num_splits;
+    Dim shape = matrix.shape();
+    shape[(size_t)axis] = n;
+    std::vector<Matrix<T>> outs;
+    for (int i = 0; i < num_splits; i++) {
+        Matrix<T> o = Matrix<T>::alloc(shape);
+        o.copy_from(axis_range(matrix, axis, (int64_t)i * n, (int64_t)(i + 1) * n));
+        outs.push_back(o);
+    }
+    return outs;
+}
+
 // ---- ConvBias (zenu-matrix/src/nn/conv/mod.rs:84-107; the CPU device's definitions, cpu/bias.rs) ----------------
 
 template <typename T> bool is_channel_bias(const Matrix<T> &bias, const Matrix<T> &x)

@@ -54,7 +54,8 @@ class CpuMatrix:
 
     # views
     def index_axis(self, axis, index):
-        return CpuMatrix(self.a[(slice(None),) * axis + (index,)])
+        # a view also when the result is 0-d (plain integer indexing would return a numpy scalar)
+        return CpuMatrix(np.squeeze(self.a[(slice(None),) * axis + (slice(index, index + 1),)], axis=axis))
 
     def slice(self, *slices):
         return CpuMatrix(self.a[tuple(slices)])
@@ -231,6 +232,35 @@ for _n, _f in (("exp", zo.EXP), ("log", zo.LOG), ("tanh", zo.TANH), ("sqrt", zo.
                ("sin", zo.SIN), ("cos", zo.COS), ("tan", zo.TAN), ("asin", zo.ASIN), ("acos", zo.ACOS),
                ("atan", zo.ATAN), ("sinh", zo.SINH), ("cosh", zo.COSH)):
     _unary(_n, _f)
+
+
+def stack(matrices, axis):
+    """zenu-matrix/src/operation/stack.rs:18-58, index by index as the reference copies"""
+    first = tuple(matrices[0].shape)
+    assert all(tuple(m.shape) == first for m in matrices), "All matrices must have the same shape"
+    n = first[axis]
+    shape = list(first)
+    shape[axis] = n * len(matrices)
+    out = CpuMatrix.alloc(shape, matrices[0].dtype)
+    for i, m in enumerate(matrices):
+        for j in range(n):
+            out.index_axis(axis, i * n + j).copy_from(m.index_axis(axis, j))
+    return out
+
+
+def split(matrix, axis, num_splits):
+    """zenu-matrix/src/operation/split.rs:20-58"""
+    assert matrix.shape[axis] % num_splits == 0
+    n = matrix.shape[axis] // num_splits
+    shape = list(matrix.shape)
+    shape[axis] = n
+    outs = []
+    for i in range(num_splits):
+        o = CpuMatrix.alloc(shape, matrix.dtype)
+        for j in range(n):
+            o.index_axis(axis, j).copy_from(matrix.index_axis(axis, i * n + j))
+        outs.append(o)
+    return outs
 
 
 def sum_to(source, target):

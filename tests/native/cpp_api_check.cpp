@@ -259,6 +259,21 @@ static void broadcast_cases() // broadcast.rs:53-165
     REQUIRE(eq(r1, {1, 1, 1}));
 }
 
+static void stack_split_cases() // stack.rs:71-108, split.rs:70-117
+{
+    std::vector<M> v1 = {M::from_vec({1, 2, 3}, {3}), M::from_vec({4, 5, 6}, {3}), M::from_vec({7, 8, 9}, {3})};
+    REQUIRE(eq(stack(v1, 0), {1, 2, 3, 4, 5, 6, 7, 8, 9}));
+    std::vector<M> v2 = {M::from_vec({1, 2, 3, 4}, {2, 2}), M::from_vec({5, 6, 7, 8}, {2, 2}), M::from_vec({9, 10, 11, 12}, {2, 2})};
+    M s = stack(v2, 1);
+    REQUIRE(s.shape() == Dim({2, 6}));
+    REQUIRE(eq(s, {1, 2, 5, 6, 9, 10, 3, 4, 7, 8, 11, 12}));
+    std::vector<M> p0 = split(M::from_vec({1, 2, 3, 4, 5, 6}, {3, 2}), 0, 3);
+    REQUIRE(p0.size() == 3 && p0[0].shape() == Dim({1, 2}) && eq(p0[0], {1, 2}) && eq(p0[1], {3, 4}) && eq(p0[2], {5, 6}));
+    std::vector<M> p1 = split(M::from_vec({1, 2, 3, 4, 5, 6}, {2, 3}), 1, 3);
+    REQUIRE(p1[0].shape() == Dim({2, 1}) && eq(p1[0], {1, 4}) && eq(p1[1], {2, 5}) && eq(p1[2], {3, 6}));
+    REQUIRE(throws_status(ZENU_ERR_SHAPE, [&] { split(M::from_vec({1, 2, 3}, {3}), 0, 2); }));
+}
+
 static void mean_variance_cases() // var.rs test mod, mean.rs:9-20
 {
     REQUIRE(close(M::from_vec({1, 2, 3, 4}, {4}).variance_all(), {1.25}, 1e-6));
@@ -427,7 +442,7 @@ int main(int argc, char **argv)
         {"broadcast_add_1x4x1x1_3x4x5x5", broadcast_add_1x4x1x1_3x4x5x5}, {"sub_mul_div", sub_mul_div},
         {"shape_errors", shape_errors}, {"unary_tables", unary_tables}, {"relu_cases", relu_cases},
         {"sigmoid_cases", sigmoid_cases}, {"sum_4d", sum_4d}, {"max_cases", max_cases}, {"asum_cases", asum_cases},
-        {"copy_cases", copy_cases}, {"broadcast_cases", broadcast_cases}, {"conv_bias_cases", conv_bias_cases}, {"mean_variance_cases", mean_variance_cases},
+        {"copy_cases", copy_cases}, {"broadcast_cases", broadcast_cases}, {"conv_bias_cases", conv_bias_cases}, {"mean_variance_cases", mean_variance_cases}, {"stack_split_cases", stack_split_cases},
         {"softmax_cases", softmax_cases},
         {"cross_entropy_cases", cross_entropy_cases}, {"clip_cases", clip_cases}, {"sgd_net_test", sgd_net_test},
         {"adam_net_test", adam_net_test}, {"adam_w_net_test", adam_w_net_test},

@@ -316,6 +316,30 @@ def autograd_unary_backward(dev):
     close(gs, [v * (1 - v) for v in sg], 1e-7)
 
 
+# ---- stack / split: zenu-matrix/src/operation/stack.rs:71-108, split.rs:70-117 --------------------------------
+
+
+@case
+def stack_split_cases(dev):
+    a, b, c = (dev.M.from_vec(v, [3]) for v in ([1., 2., 3.], [4., 5., 6.], [7., 8., 9.]))
+    eq(dev.F.stack([a, b, c], 0), [1., 2., 3., 4., 5., 6., 7., 8., 9.])                        # test_stack_axis0
+    a, b, c = (dev.M.from_vec(v, [2, 2]) for v in ([1., 2., 3., 4.], [5., 6., 7., 8.], [9., 10., 11., 12.]))
+    eq(dev.F.stack([a, b, c], 1), [[1., 2., 5., 6., 9., 10.], [3., 4., 7., 8., 11., 12.]])     # test_stack_axis1
+    parts = dev.F.split(dev.M.from_vec([1., 2., 3., 4., 5., 6.], [3, 2]), 0, 3)                # test_split_axis0
+    assert len(parts) == 3
+    for p, e in zip(parts, ([[1., 2.]], [[3., 4.]], [[5., 6.]])):
+        eq(p, e)
+    parts = dev.F.split(dev.M.from_vec([1., 2., 3., 4., 5., 6.], [2, 3]), 1, 3)                # test_split_axis1
+    for p, e in zip(parts, ([[1.], [4.]], [[2.], [5.]], [[3.], [6.]])):
+        eq(p, e)
+    # a transposed input and a round trip: split(stack(x)) gives the inputs back
+    t = dev.M.from_vec([1., 2., 3., 4., 5., 6.], [2, 3]).transpose()
+    st = dev.F.stack([t, t], 0)
+    eq(st, [[1., 4.], [2., 5.], [3., 6.], [1., 4.], [2., 5.], [3., 6.]])
+    for p in dev.F.split(st, 0, 2):
+        eq(p, [[1., 4.], [2., 5.], [3., 6.]])
+
+
 # ---- mean / variance: zenu-matrix/src/operation/var.rs test mod, mean.rs:9-20 ------------------------------
 
 

@@ -558,6 +558,48 @@ def conv2d_bias_bkwd(d_output, d_bias):
     sum_to(d_output, d_bias)
 
 
+def _axis_range(m, axis, start, stop):
+    return m.slice(*([slice(None)] * axis + [slice(start, stop)]))
+
+
+def stack(matrices, axis):
+    """zenu-matrix/src/operation/stack.rs:18-58: the inputs laid one after the other along `axis`
+    (the output's extent there is len(matrices) times the inputs'); one strided copy per input
+    where the reference copies index by index"""
+    if not matrices:
+        raise ZenuHipError(_lib.ERR_ARG, "stack", "No matrices to stack")
+    first = tuple(matrices[0].shape)
+    if any(tuple(m.shape) != first for m in matrices):
+        raise ZenuHipError(_lib.ERR_SHAPE, "stack", "All matrices must have the same shape")
+    if not (0 <= axis < len(first)):      # the reference admits axis == ndim and then indexes out of bounds
+        raise ZenuHipError(_lib.ERR_AXIS, "stack", "Axis out of bounds for stack")
+    n = first[axis]
+    shape = list(first)
+    shape[axis] = n * len(matrices)
+    out = Matrix.alloc(shape, matrices[0].dtype)
+    for i, m in enumerate(matrices):
+        _axis_range(out, axis, i * n, (i + 1) * n).copy_from(m)
+    return out
+
+
+def split(matrix, axis, num_splits):
+    """zenu-matrix/src/operation/split.rs:20-58: num_splits equal pieces along `axis`, each a new
+    matrix; one strided copy per piece"""
+    if not (0 <= axis < matrix.ndim):
+        raise ZenuHipError(_lib.ERR_AXIS, "split", "Axis out of bounds")
+    if num_splits <= 0 or matrix.shape[axis] % num_splits:
+        raise ZenuHipError(_lib.ERR_SHAPE, "split", "Size along axis is not divisible by num_splits")
+    n = matrix.shape[axis] // num_splits
+    shape = list(matrix.shape)
+    shape[axis] = n
+    outs = []
+    for i in range(num_splits):
+        o = Matrix.alloc(shape, matrix.dtype)
+        o.copy_from(_axis_range(matrix, axis, i * n, (i + 1) * n))
+        outs.append(o)
+    return outs
+
+
 def sum_to(source, target):
     """sum.rs:35-94: reduce `source` into the (smaller) `target` in place"""
     check(_lib.lib().zenu_hip_sum_to(_dt(source.dtype), C.byref(target.desc()), C.byref(source.desc()),
