@@ -3,6 +3,10 @@
 // Same op sequence as tests/mlp_step.py (which cites the reference's files for every line):
 //   ops   -- the sequence ZeNu's autograd issues, one library call per Matrix-level op
 //   fused -- the same step through the fused entry points
+//   lean  -- fused, and the GEMMs take their transposed operands as views (rocBLAS transpose flags)
+//            instead of the contiguous copies that ZeNu's autograd `transpose` makes
+//            (zenu-autograd/src/functions/transpose.rs:26-33); bias gradients go into
+//            uninitialised buffers (sum_to writes every element)
 // Prints one line per measurement: "<variant> <what> <value>".
 //
 //   mlp_step_bench [--inputs file] [--steps K] [--warmup W] [--dump-loss N]
@@ -34,6 +38,20 @@ static M gemm(const M &a, const M &b)
     M out = M::alloc({m, n});
     const float alpha = 1.f, beta = 0.f;
     if (rocblas_sgemm(g_blas, rocblas_operation_none, rocblas_operation_none, n, m, k, &alpha, b.as_ptr(), n, a.as_ptr(), k,
+                      &beta, out.as_ptr(), n) != rocblas_status_success) {
+        std::printf("rocblas_sgemm failed\n");
+        std::exit(1);
+    }
+    return out;
+}
+
+// row-major C[m,n] = op(A) op(B), A and B stored row-major with leading dimensions lda, ldb
+static M gemm_rm(bool ta, bool tb, int m, int n, int k, const M &a, int lda, const M &b, int ldb)
+{
+    M out = M::alloc({m, n});
+    const float alpha = 1.f, beta = 0.f;
+    if (rocblas_sgemm(g_blas, tb ? rocblas_operation_transpose : rocblas_operation_none,
+                      ta ? rocblas_operation_transpose : rocblas_operation_none, n, m, k, &alpha, b.as_ptr(), ldb, a.as_ptr(), lda,
                       &beta, out.as_ptr(), n) != rocblas_status_success) {
         std::printf("rocblas_sgemm failed\n");
         std::exit(1);
@@ -96,8 +114,49 @@ struct Step {
         opt->update(p);
     }
 
-    void run(bool fused)
+    // forward and backward with no materialised transpose: 20 launches
+    void run_lean()
     {
+        M pre[3], act_in[3];
+        M h = x, logits;
+        for (int i = 0; i < 3; i++) {
+            act_in[i] = h;
+            const int in = kLayers[i][0], out = kLayers[i][1];
+            M z = gemm_rm(false, true, kBatch, out, in, h, in, p[wk[i]].data, in);      // h W^T, W stored [out, in]
+            if (i == 2) {
+                logits = z + p[bk[i]].data;
+            } else {
+                pre[i] = z.alloc_like();
+                M a = z.alloc_like();
+                a.bias_add_relu(z, p[bk[i]].data, 0.f, &pre[i]);
+                h = a;
+            }
+        }
+        auto lp = cross_entropy(logits, t);
+        loss = lp.first;
+        M g = cross_entropy_backward(lp.second, t, &one);
+        for (int i = 2; i >= 0; i--) {
+            const int in = kLayers[i][0], out = kLayers[i][1];
+            M gb = M::alloc({out});
+            g.sum_to(gb);
+            M gW = gemm_rm(true, false, out, in, kBatch, g, out, act_in[i], in);        // dY^T X, already [out, in]
+            M w = p[wk[i]].data;
+            p[wk[i]] = ParamGrad<float>(w, gW);
+            p[bk[i]] = ParamGrad<float>(p[bk[i]].data, gb);
+            if (i > 0) {
+                M gh = gemm_rm(false, false, kBatch, in, out, g, out, w, in);           // dY W
+                M gn = gh.alloc_like();
+                gn.relu_backward(gh, pre[i - 1], 0.f);
+                g = gn;
+            }
+        }
+        opt->update(p);
+    }
+
+    void run(int variant)
+    {
+        if (variant == 2) return run_lean();
+        const bool fused = variant == 1;
         M Wt[3], pre[3], act_in[3];
         M h = x;
         M logits;
@@ -198,18 +257,18 @@ int main(int argc, char **argv)
             std::printf("rocblas init failed\n");
             return 1;
         }
-        for (int fused = 0; fused < 2; fused++) {
-            const char *name = fused ? "fused" : "ops";
+        for (int fused = 0; fused < 3; fused++) {
+            const char *name = fused == 2 ? "lean" : fused ? "fused" : "ops";
             Step st;
             st.init(buf);
             for (int i = 0; i < dump; i++) {            // the first steps' losses, for the parity test
-                st.run(fused != 0);
+                st.run(fused);
                 std::printf("%s loss %d %.9g\n", name, i + 1, (double)st.loss.to_vec()[0]);
             }
-            for (int i = 0; i < warmup; i++) st.run(fused != 0);
+            for (int i = 0; i < warmup; i++) st.run(fused);
             synchronize();
             const auto t0 = std::chrono::steady_clock::now();
-            for (int i = 0; i < steps; i++) st.run(fused != 0);
+            for (int i = 0; i < steps; i++) st.run(fused);
             synchronize();
             const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / steps;
             std::printf("%s ms_per_step %.4f\n", name, ms);
