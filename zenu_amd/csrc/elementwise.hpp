@@ -16,8 +16,9 @@
 //            accesses; a broadcast row stays in L2.                                   [HBM bound]
 //   tile   : some input is contiguous along a different dim than the output (a transposed
 //            operand).  64x64 tiles: the transposed input is read along ITS contiguous dim with
-//            128-bit loads, turned through LDS (pitch 65 words: conflict-free both ways on the
-//            64-lane wavefront), and every HBM access stays coalesced.               [HBM bound]
+//            128-bit loads in 128-byte segments, turned through LDS (pitch 65 words, eight lanes
+//            per segment: no bank conflicts in either direction, checked with the hardware
+//            counter), and every HBM access stays coalesced.                        [HBM bound]
 //   generic: anything else (strided output, gathers): one element per thread, index arithmetic
 //            per element.
 //
@@ -396,8 +397,15 @@ __global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, con
     constexpr int VEC = VecOf<T>::N;
     constexpr int kTile = TileOf<T>::N;
     constexpr int kPitch = kTile + 1;
-    constexpr int VPR = kTile / VEC;        // vectors per tile row
-    constexpr int RPP = kBlock / VPR;       // tile rows per pass
+    // Eight lanes cover one 128-byte segment of a tile row; 32 segments per pass.  With eight (not
+    // sixteen) lanes along the vector dim the 32 lanes that the LDS serves together -- eight
+    // vector positions x four rows -- fall into 32 different banks in the scatter (one element of
+    // each lane's vector per instruction, rows one pitch apart) and in the gather alike; sixteen
+    // lanes per row alias pairwise (4 m and 4 (m + 8) share a bank) whatever the pitch.
+    constexpr int VPS = 8;                  // vectors per segment
+    constexpr int SEG = kTile / (VPS * VEC);// segments per tile row (2)
+    constexpr int RPP = kBlock / VPS;       // segments per pass (32)
+    static_assert(kTile % RPP == 0 && SEG >= 1, "tile geometry");
     __shared__ T lds_a[kTile * kPitch];
     __shared__ T lds_b[(F::NIN == 2) ? kTile * kPitch : 1];
     f.init();
@@ -423,15 +431,17 @@ __global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, con
         // All global loads of the tile are issued first -- the transposed inputs along R (their
         // contiguous dim), the others along C -- so both streams are in flight together; then the
         // transposed ones are turned through LDS.
-        constexpr int K = kTile / RPP;
-        const int lane_v = (tid % VPR) * VEC;   // vector position along the contiguous dim
-        const int lane_o = tid / VPR;           // position along the other dim, + k * RPP
+        constexpr int K = kTile * SEG / RPP;    // passes: the segments of a tile, 32 at a time
+        constexpr int PPS = kTile / RPP;        // passes per segment column
+        const int seg_v = (tid % VPS) * VEC;    // vector position inside the segment
+        const int lane_o = tid / VPS;           // position along the other dim, + (k % PPS) * RPP
         const bool ta = p.trans_a != 0;
         const bool tb = (F::NIN == 2) && p.trans_b != 0;
         Pack<T, VEC> xa[K], xb[K];
 #pragma unroll
         for (int k = 0; k < K; k++) {
-            const int o = lane_o + k * RPP;
+            const int o = lane_o + (k % PPS) * RPP;
+            const int lane_v = seg_v + (k / PPS) * VPS * VEC;
             if (ta) xa[k] = load_pack<T, VEC, NT>(abase + lane_v + (int64_t)o * p.ldc[1]);
             else if (p.ldc[1] == 0) xa[k] = splat<T, VEC>(abase[(int64_t)o * p.ldr[1]]);
             else xa[k] = load_pack<T, VEC, NT>(abase + (int64_t)o * p.ldr[1] + lane_v);
@@ -444,7 +454,8 @@ __global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, con
         if (ta || tb) {
 #pragma unroll
             for (int k = 0; k < K; k++) {
-                const int c = lane_o + k * RPP;  // the loaded vector holds rows lane_v.. of column c
+                const int c = lane_o + (k % PPS) * RPP;  // the loaded vector holds rows lane_v.. of column c
+                const int lane_v = seg_v + (k / PPS) * VPS * VEC;
 #pragma unroll
                 for (int j = 0; j < VEC; j++) {
                     if (ta) lds_a[(lane_v + j) * kPitch + c] = xa[k].v[j];
@@ -457,7 +468,8 @@ __global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, con
         }
 #pragma unroll
         for (int k = 0; k < K; k++) {
-            const int r = lane_o + k * RPP;
+            const int r = lane_o + (k % PPS) * RPP;
+            const int lane_v = seg_v + (k / PPS) * VPS * VEC;
             Pack<T, VEC> x = xa[k], y;
             if (ta) {
 #pragma unroll

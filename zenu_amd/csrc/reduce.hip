@@ -503,13 +503,13 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int
     // combine the ty lanes in fixed order
     if (ty_n > 1) {
 #pragma unroll
-        for (int j = 0; j < VEC; j++) lds[threadIdx.x * VEC + j] = acc[j];
+        for (int j = 0; j < VEC; j++) lds[j * kBlock + threadIdx.x] = acc[j];   // [vector element][thread]: consecutive lanes, consecutive banks
         __syncthreads();
         if (ty == 0) {
 #pragma unroll
             for (int j = 0; j < VEC; j++) {
-                A r = lds[tx * VEC + j];
-                for (int w = 1; w < ty_n; w++) r = Tr::merge(r, lds[(w * tx_n + tx) * VEC + j]);
+                A r = lds[j * kBlock + tx];
+                for (int w = 1; w < ty_n; w++) r = Tr::merge(r, lds[j * kBlock + w * tx_n + tx]);
                 acc[j] = r;
             }
         }
@@ -545,13 +545,13 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int
     if (ty_n > 1) {
         __syncthreads();
 #pragma unroll
-        for (int j = 0; j < VEC; j++) lds[threadIdx.x * VEC + j] = acc[j];
+        for (int j = 0; j < VEC; j++) lds[j * kBlock + threadIdx.x] = acc[j];   // [vector element][thread]: consecutive lanes, consecutive banks
         __syncthreads();
         if (ty == 0) {
 #pragma unroll
             for (int j = 0; j < VEC; j++) {
-                A r = lds[tx * VEC + j];
-                for (int w = 1; w < ty_n; w++) r = Tr::merge(r, lds[(w * tx_n + tx) * VEC + j]);
+                A r = lds[j * kBlock + tx];
+                for (int w = 1; w < ty_n; w++) r = Tr::merge(r, lds[j * kBlock + w * tx_n + tx]);
                 acc[j] = r;
             }
         }
