@@ -259,8 +259,54 @@ def build_ops(z, workload, stream):
                       lambda: co.sigmoid_backward(ct, cx)))
         ops[-1].keep = sets
 
+    # ---- the neighbours of the path: strided copy / transpose / broadcast, the rest of the unary surface,
+    # powf, asum, the bias-gradient reduction (not a BASELINE config) ------------------------------------
+    def add_next():
+        r = np.random.default_rng(6)
+        n = 4096
+        a = r.standard_normal((n, n)).astype(np.float32)
+        pos = (np.abs(a) + np.float32(0.01)).astype(np.float32)
+        unit = np.clip(a, -0.99, 0.99).astype(np.float32)
+        row = r.standard_normal(n).astype(np.float32)
+        nb = 4 * n * n
+        sets = [(M.from_numpy(a), M.from_numpy(pos), M.from_numpy(unit), M.from_numpy(row), M.alloc((n, n)), M.alloc((n,)), M.alloc(()))
+                for _ in range(nsets(4 * nb))]
+        out_h = np.empty_like(a)
+        col_h = np.empty(n, dtype=np.float32)
+
+        def mk(fn):
+            return [fn(A, P, U, R, O, V, S) for A, P, U, R, O, V, S in sets]
+        ops.append(Op("transpose copy (to_default_stride of a^T)", "next", "f32", 2 * nb, n * n,
+                      mk(lambda A, P, U, R, O, V, S: (lambda d=O.desc(), s_=A.transpose().desc(): check(l.zenu_hip_copy(_lib.F32, ref(d), ref(s_), stream), "copy"))),
+                      lambda: zo.copy_from(out_h, a.T)))
+        ops.append(Op("row-sliced copy (every other row)", "next", "f32", nb, n * n // 2,
+                      mk(lambda A, P, U, R, O, V, S: (lambda d=O.slice(slice(0, n // 2)).desc(), s_=A.slice(slice(None, None, 2)).desc(): check(l.zenu_hip_copy(_lib.F32, ref(d), ref(s_), stream), "copy"))),
+                      lambda: zo.copy_from(out_h[:n // 2], a[::2])))
+        ops.append(Op("broadcast [4096] -> [4096,4096]", "next", "f32", nb + 4 * n, n * n,
+                      mk(lambda A, P, U, R, O, V, S: (lambda d=O.desc(), s_=R.desc(): check(l.zenu_hip_broadcast(_lib.F32, ref(d), ref(s_), stream), "broadcast"))),
+                      lambda: zo.broadcast(out_h, row)))
+        for name, fn, src in (("log", _lib.LOG, 1), ("sqrt", _lib.SQRT, 1), ("abs", _lib.ABS, 0), ("sin", _lib.SIN, 0), ("cos", _lib.COS, 0),
+                              ("tan", _lib.TAN, 2), ("asin", _lib.ASIN, 2), ("acos", _lib.ACOS, 2), ("atan", _lib.ATAN, 0),
+                              ("sinh", _lib.SINH, 0), ("cosh", _lib.COSH, 0)):
+            host = (a, pos, unit)[src]
+            ops.append(Op(name, "next", "f32", 2 * nb, n * n,
+                          mk(lambda A, P, U, R, O, V, S, fn=fn, src=src: (lambda d=O.desc(), s_=(A, P, U)[src].desc(): check(l.zenu_hip_unary(fn, _lib.F32, ref(d), ref(s_), stream), "unary"))),
+                          lambda fn=fn, host=host: zo.unary(fn, out_h, host)))
+        ops.append(Op("powf(x, 2.5)", "next", "f32", 2 * nb, n * n,
+                      mk(lambda A, P, U, R, O, V, S: (lambda d=O.desc(), s_=P.desc(): check(l.zenu_hip_powf(_lib.F32, ref(d), ref(s_), 2.5, stream), "powf"))),
+                      lambda: zo.powf(out_h, pos, 2.5)))
+        ops.append(Op("asum (whole tensor)", "next", "f32", nb + 4, n * n,
+                      mk(lambda A, P, U, R, O, V, S: (lambda p_=S.as_ptr(), s_=A.desc(): check(l.zenu_hip_asum(_lib.F32, p_, ref(s_), stream), "asum"))),
+                      lambda: zo.asum(a)))
+        ops.append(Op("sum_to [4096,4096] -> [4096] (bias gradient)", "next", "f32", nb + 4 * n, n * n,
+                      mk(lambda A, P, U, R, O, V, S: (lambda d=V.desc(), s_=A.desc(): check(l.zenu_hip_sum_to(_lib.F32, ref(d), ref(s_), stream), "sum_to"))),
+                      lambda: zo.sum_to(a, col_h)))
+        ops[-1].keep = sets
+
     if workload == "fused":
         add_fused()
+    if workload == "next":
+        add_next()
     if want("c0"):
         add_c0()
     if want("c1"):
@@ -444,7 +490,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="suite", choices=["suite", "c0", "c1", "c2", "c3", "c4", "fused"])
+    ap.add_argument("--workload", default="suite", choices=["suite", "c0", "c1", "c2", "c3", "c4", "fused", "next"])
     ap.add_argument("--op-reps", type=int, default=50, help="launches per op in the per-op timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--profile-op", default=None, help="only launch this op (for rocprofv3 counter runs)")
@@ -560,7 +606,9 @@ def main():
         "dtype": "f32" if args.workload != "suite" and args.workload != "c2" else "f32+f64", "data": "synthetic",
         "config": {"workload": {"suite": "configs[0..3]: every op once per step", "c0": "configs[0]", "c1": "configs[1]",
                                 "c2": "configs[2]", "c3": "configs[3]",
-                                "fused": "fused entry points on [8192,4096] f32 (not a BASELINE config)"}[args.workload],
+                                "fused": "fused entry points on [8192,4096] f32 (not a BASELINE config)",
+                                "next": "strided copy, broadcast, the remaining unary functions, powf, asum and sum_to on [4096,4096] f32 "
+                                        "(not a BASELINE config)"}[args.workload],
                    "ops_per_step": len(ops), "algorithmic_bytes_per_step": step_bytes},
         "frac_of_peak_whole_step": round(value / PEAK_HBM_GBPS, 4),
         "adam_step_params_per_sec": (round(adam[0]["Gelem_per_s"] * 1e9) if adam else None),

@@ -797,6 +797,24 @@ def test_allocator_device(hip):
     assert st.bytes_reserved == st.bytes_in_use + st.bytes_cached
 
 
+def test_memset_zero_any_alignment_and_size(hip):
+    """zenu_hip_memset_zero clears exactly [ptr, ptr + bytes): unaligned starts, sizes that are not a
+    multiple of 16 (or of 4), sizes below one vector, and a size that spans many workgroups; the
+    bytes on both sides stay untouched"""
+    from zenu_amd import _lib
+    l = hip.lib()
+    total = (1 << 20) + 64
+    for start, nbytes in [(0, 16), (4, 16), (1, 1), (3, 7), (5, 40), (12, 4), (16, 8192), (7, 8200), (9, 100001),
+                          (32, 1 << 20), (0, 0)]:
+        host = np.full(total // 4, -1.5, dtype=np.float32)      # every byte non-zero
+        buf = hip.Matrix.from_numpy(host)
+        _lib.check(l.zenu_hip_memset_zero(buf.as_ptr() + start, nbytes, hip.get_stream()), "memset_zero")
+        got = buf.to_numpy().view(np.uint8)
+        exp = host.view(np.uint8).copy()
+        exp[start:start + nbytes] = 0
+        assert np.array_equal(got, exp), (start, nbytes)
+
+
 def test_empty_tensors(hip):
     """zero-sized views: elementwise ops and copies do nothing, sums over an empty axis are zeros (the
     reference adds nothing to a zero-initialised result, sum.rs:18-25), an arg-max over nothing is an
