@@ -27,12 +27,14 @@ def test_allocator_bookkeeping(tmp_path):
         assert f"ok {name}" in out.stdout
 
 
-def test_device_tanh_matches_host_libm(tmp_path):
-    """zmath.hpp (the tanh / expm1 / sigmoid the kernels use) compiled for the host with
-    contraction off must give the bits of tanhf / expm1f / tanh / expm1: every 31st f32 bit pattern
-    here (138 M points; stride 1, all 2^32, was run during development with the same result) and,
-    for double, every 31st high word with three low words each (415 M points); powf on every 31st
-    base for 19 fixed exponents and on two pseudo-random (base, exponent) pairs per base."""
+def test_zmath_matches_host_libm(tmp_path):
+    """zmath.hpp (the transcendental functions the kernels use) compiled for the host with
+    contraction off must give the bits of the host libm: f32 tanh, expm1, exp, log, sinh, cosh, sin,
+    cos, atan, asin, acos and the sigmoid composite on every 31st f32 bit pattern (138 M points
+    each; stride 1, all 2^32, was run during development with the same result); powf on every 31st
+    base for 19 fixed exponents and on two pseudo-random (base, exponent) pairs per base; f64 tanh,
+    expm1, exp, sinh, cosh and the sigmoid composite on every 31st high word with three low words
+    each plus uniform samples in +-745 and +-4 (about 700 M points)."""
     exe = build("zmath_host_check.cpp", str(tmp_path / "zmath_check"), ("-ffp-contract=off", "-fno-fast-math"))
     out = subprocess.run([exe, "31"], capture_output=True, text=True)
     assert out.returncode == 0, out.stdout

@@ -1,22 +1,30 @@
-// zmath.hpp -- tanh / expm1 (f32 and f64) for device code, bit-compatible with the host libm the
-// reference's CPU path calls (Rust f32::tanh / f64::tanh -> libm tanhf / tanh).
+// zmath.hpp -- the transcendental functions of the kernels, bit-compatible with the host libm that
+// the reference's CPU path calls (Rust f32::tanh / exp / ln / powf ... -> libm tanhf / expf / logf /
+// powf ...; glibc 2.35 is what this image ships).
+//
+//   f32: tanh, expm1, exp, log, powf, sinh, cosh, sin, cos, atan, asin, acos, the sigmoid composite
+//   f64: tanh, expm1, exp, sinh, cosh, the sigmoid composite
 //
 // Why not the device math library: ZeNu's sigmoid is the composite 0.5 + 0.5*tanh(0.5*x)
 // (zenu-autograd/src/activation/sigmoid.rs:7-15).  For negative x the final add cancels, so a
 // 1-ulp difference in tanh becomes tens of ulps in the sigmoid; parity therefore needs the
-// same tanh bits as the CPU path, not merely an accurate tanh.
+// same tanh bits as the CPU path, not merely an accurate tanh.  The other functions follow the
+// same idea: each restates the algorithm the host libm uses (fdlibm's float and double routines,
+// ARM's table-driven expf / logf / powf / sinf / cosf / exp as glibc carries them), with the fused
+// multiply-adds exactly where the x86-64 build that CPUs with FMA select has them, so host and
+// device produce identical bits.
 //
-// Algorithm: the classic fdlibm single-precision tanhf / expm1f (Sun Microsystems, 1993; the
-// generic flt-32 implementation used by glibc 2.35, which is what this image ships):
+// tanh, the first of them: the classic fdlibm single-precision tanhf / expm1f (Sun Microsystems, 1993):
 //   tanh(x) = sign(x) * { |x| < 2^-55 : |x|*(1+|x|)
 //                         |x| <  1    : -t/(t+2),   t = expm1(-2|x|)
 //                         |x| <  22   : 1 - 2/(t+2), t = expm1( 2|x|)
 //                         else        : 1 }
 //   expm1(x): x = k*ln2 + r, |r| <= 0.5 ln2; R1(r*r) rational correction; scale by 2^k.
-// Everything is plain IEEE f32 arithmetic (+,-,*,/ correctly rounded, no contraction), so host
-// and device produce identical bits.  The host build of this header is compared against
-// tanhf/expm1f over every f32 bit pattern in tests/test_zmath_host.py (sampled) and was run
-// exhaustively during development.
+// Everything there is plain IEEE f32 arithmetic (+,-,*,/ correctly rounded, no contraction).
+//
+// The host build of this header is compared with the host libm by tests/native/zmath_host_check.cpp
+// (tests/test_host_native.py runs it on a sample; on every f32 bit pattern and on 2e10 sampled
+// f64 inputs it was run during development, without a mismatch).
 #pragma once
 #include <math.h>
 #include <stdint.h>
@@ -169,8 +177,7 @@ ZM_HD float tanhf_fdlibm(float x)
 // different k does not execute the branches of tanhf_fdlibm one after another.  Every
 // arithmetic operation that reaches the result is the one tanhf_fdlibm performs, on the same
 // operands, so the bits are identical; this is checked over every f32 bit pattern against
-// tanhf_fdlibm and the host libm (tests/test_zmath_host.py, dense sample; exhaustive run kept
-// out of the default suite).
+// tanhf_fdlibm and the host libm (tests/native/zmath_host_check.cpp).
 ZM_HD float tanhf_simd(float x)
 {
     const float one = 1.0f, two = 2.0f;
