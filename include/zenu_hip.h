@@ -256,6 +256,11 @@ int zenu_hip_bias_add_relu(int dtype, const zenu_tensor_t *pre, const zenu_tenso
 /* p -= g*lr (zenu-optimizer/src/sgd.rs:20-31). */
 int zenu_hip_sgd_step(int dtype, void *p_dev, const void *g_dev, int64_t n, double lr,
                       zenu_stream_t stream);
+
+/* The same update for n_tensors tensors in one launch (the loop of SGD::update, sgd.rs:20-31):
+ * p_dev[i], g_dev[i] are device pointers of sizes[i] elements; host arrays, read during the call. */
+int zenu_hip_sgd_step_multi(int dtype, int n_tensors, void *const *p_dev, const void *const *g_dev,
+                            const int64_t *sizes, double lr, zenu_stream_t stream);
 /* Adam (zenu-optimizer/src/adam.rs:19-59).  `step` is the counter AFTER the increment;
  * 1-beta, beta^step and 1-beta^step are formed on the host in dtype, as the reference does. */
 int zenu_hip_adam_step(int dtype, void *p_dev, const void *g_dev, void *m_dev, void *v_dev,

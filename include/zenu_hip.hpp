@@ -628,15 +628,22 @@ template <typename T> class SGD {           // zenu-optimizer/src/sgd.rs:6-31
 public:
     T learning_rate;
     explicit SGD(T lr) : learning_rate(lr) {}
-    void update(const Parameters<T> &params) const
+    void update(const Parameters<T> &params) const        // one launch for all tensors
     {
+        std::vector<void *> p;
+        std::vector<const void *> g;
+        std::vector<int64_t> n;
         for (const auto &kv : params) {
             const ParamGrad<T> &pg = kv.second;
             if (!pg.has_grad) continue;
             if (!pg.data.is_default_stride() || !pg.grad.is_default_stride()) throw std::invalid_argument("optimizer tensors must be default stride");
-            check(zenu_hip_sgd_step(DType<T>::value, pg.data.as_ptr(), pg.grad.as_ptr(), num_elm(pg.data.shape()),
-                                    (double)learning_rate, current_stream()), "sgd_step");
+            p.push_back(pg.data.as_ptr());
+            g.push_back(pg.grad.as_ptr());
+            n.push_back(num_elm(pg.data.shape()));
         }
+        if (p.empty()) return;
+        check(zenu_hip_sgd_step_multi(DType<T>::value, (int)p.size(), p.data(), g.data(), n.data(), (double)learning_rate,
+                                      current_stream()), "sgd_step_multi");
     }
 };
 

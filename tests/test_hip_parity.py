@@ -644,6 +644,38 @@ def test_sgd(hip):
         assert_bits(P.to_numpy(), p, "sgd")
 
 
+def test_sgd_multi_tensor(hip):
+    """zenu_hip_sgd_step_multi: more tensors than one launch holds (24), odd sizes, an empty tensor, an
+    unaligned tensor (a view one element into a buffer) -- bit-exact against the oracle per tensor"""
+    import ctypes as C
+    from zenu_amd import _lib
+    from zenu_amd._lib import check
+    r = rng(8)
+    for dt in (np.float32, np.float64):
+        sizes = [1, 7, 0, 4096, 100003, 2048, 33] * 5            # 35 tensors: two launches
+        host, dev = [], []
+        for i, n in enumerate(sizes):
+            p = (r.standard_normal(n + 1) * 0.05).astype(dt)
+            g = (r.standard_normal(n + 1) * 0.01).astype(dt)
+            off = 1 if i % 3 == 0 else 0                           # every third tensor starts off 16-byte alignment
+            host.append((p, g, off, n))
+            dev.append((hip.Matrix.from_numpy(p), hip.Matrix.from_numpy(g)))
+        k = len(sizes)
+        P, G, N = (C.c_void_p * k)(), (C.c_void_p * k)(), (C.c_int64 * k)()
+        isz = np.dtype(dt).itemsize
+        for i, ((p, g, off, n), (dp, dg)) in enumerate(zip(host, dev)):
+            P[i], G[i], N[i] = dp.as_ptr() + off * isz, dg.as_ptr() + off * isz, n
+        check(hip.lib().zenu_hip_sgd_step_multi(_lib.F32 if dt == np.float32 else _lib.F64, k, P, G, N, 0.3, None), "sgd_multi")
+        for (p, g, off, n), (dp, dg) in zip(host, dev):
+            exp = p.copy()
+            if n:
+                seg = np.ascontiguousarray(exp[off:off + n])
+                zo.sgd_update(seg, np.ascontiguousarray(g[off:off + n]), np.dtype(dt).type(0.3))
+                exp[off:off + n] = seg
+            assert_bits(dp.to_numpy(), exp, f"sgd_multi n={n} off={off}")
+            assert_bits(dg.to_numpy(), g, "gradient untouched")
+
+
 def test_optimizer_classes_multi_tensor(hip):
     """Optimizer::update over a model-like set of tensors: the multi-tensor launch equals the
     per-tensor launches and the oracle; AdamW decays weights only (adamw.rs:61-65)"""

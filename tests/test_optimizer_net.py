@@ -144,10 +144,11 @@ def device_params(hip, p, g):
 
 
 @pytest.mark.gpu
-def test_hip_sgd_net(hip):
+@pytest.mark.parametrize("multi", [True, False])
+def test_hip_sgd_net(hip, multi):
     p = init_parameters()
     params = device_params(hip, p, grads(p))
-    hip.SGD(0.9).update(params)
+    hip.SGD(0.9).update(params, multi_tensor=multi)
     check({k: v[0].to_numpy() for k, v in params.items()}, SGD_ANS, 1e-4)
 
 

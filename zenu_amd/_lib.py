@@ -91,6 +91,7 @@ SIGNATURES = {
     "zenu_hip_max_idx": [_i, _vp, _vp, _TP, _vp],
     "zenu_hip_asum": [_i, _vp, _TP, _vp],
     "zenu_hip_sgd_step": [_i, _vp, _vp, _i64, _d, _vp],
+    "zenu_hip_sgd_step_multi": [_i, _i, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_i64), _d, _vp],
     "zenu_hip_adam_step": [_i, _vp, _vp, _vp, _vp, _i64, _d, _d, _d, _d, _d, _vp],
     "zenu_hip_adamw_step": [_i, _vp, _vp, _vp, _vp, _i64, _d, _d, _d, _d, _d, _i, _d, _vp],
     "zenu_hip_adam_step_multi": [_i, _i, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),

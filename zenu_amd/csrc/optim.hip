@@ -166,12 +166,15 @@ __global__ __launch_bounds__(kBlock) void adam_multi_kernel(MultiArgs a, AdamCon
     }
 }
 
+constexpr int kSgdUnroll = 4;
+
+// one tile of kBlock * VEC * kSgdUnroll elements: p = p - (g * lr), two roundings (sgd.rs:23-27)
 template <typename T, int VEC>
-__global__ __launch_bounds__(kBlock) void sgd_kernel(T *p, const T *g, int64_t n, T lr)
+__device__ __forceinline__ void sgd_span(T *p, const T *g, int64_t n, int64_t blk, T lr)
 {
-    constexpr int kU = 4;
+    constexpr int kU = kSgdUnroll;
     constexpr int64_t kTile = (int64_t)kBlock * VEC * kU;
-    const int64_t base = (int64_t)blockIdx.x * kTile;
+    const int64_t base = blk * kTile;
     const int tid = threadIdx.x;
     if (VEC > 1 && base + kTile <= n) {
         Pack<T, VEC> vp[kU], vg[kU];
@@ -201,6 +204,34 @@ __global__ __launch_bounds__(kBlock) void sgd_kernel(T *p, const T *g, int64_t n
                     p[i] = p[i] - t;
                 }
             }
+        }
+    }
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void sgd_kernel(T *p, const T *g, int64_t n, T lr)
+{
+    sgd_span<T, VEC>(p, g, n, blockIdx.x, lr);
+}
+
+// multi-tensor SGD: the tensors of one SGD::update (sgd.rs:20-31 walks the parameter map) in one
+// launch; same argument layout as the multi-tensor Adam (m, v unused)
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void sgd_multi_kernel(MultiArgs a, T lr)
+{
+    int t = 0;
+    while (t + 1 < a.count && (int)blockIdx.x >= a.first_block[t + 1]) t++;
+    const MultiEntry &e = a.e[t];
+    const int64_t tile = (int64_t)blockIdx.x - a.first_block[t];
+    T *p = static_cast<T *>(e.p);
+    const T *g = static_cast<const T *>(e.g);
+    if (e.vec_ok) sgd_span<T, VEC>(p, g, e.n, tile, lr);
+    else {
+        constexpr int64_t kTile = (int64_t)kBlock * VEC * kSgdUnroll;   // same tile, scalar accesses
+        const int64_t base = tile * kTile;
+        for (int64_t i = base + threadIdx.x; i < base + kTile && i < e.n; i += kBlock) {
+            T t2 = g[i] * lr;
+            p[i] = p[i] - t2;
         }
     }
 }
@@ -295,12 +326,65 @@ int adam_multi_t(int nt, void *const *p, const void *const *g, void *const *m, v
     return ZENU_OK;
 }
 
+template <typename T>
+int sgd_multi_t(int nt, void *const *p, const void *const *g, const int64_t *sizes, T lr, hipStream_t s)
+{
+    constexpr int VEC = VecOf<T>::N;
+    constexpr int64_t kTile = (int64_t)kBlock * VEC * kSgdUnroll;
+    for (int i = 0; i < nt; i++)
+        if (sizes[i] < 0 || (sizes[i] > 0 && (!p[i] || !g[i]))) return ZENU_ERR_ARG;
+    int i = 0;
+    while (i < nt) {
+        MultiArgs a;
+        a.count = 0;
+        int64_t blocks = 0;
+        while (i < nt && a.count < kMaxMulti) {
+            const int64_t tiles = (sizes[i] + kTile - 1) / kTile;
+            if (tiles == 0) { i++; continue; }
+            if (blocks + tiles > 0x7fffffffLL) {
+                if (a.count == 0) return ZENU_ERR_UNSUPPORTED;
+                break;
+            }
+            MultiEntry &e = a.e[a.count];
+            e.p = p[i];
+            e.g = g[i];
+            e.m = nullptr;
+            e.v = nullptr;
+            e.n = sizes[i];
+            e.decay = 0;
+            e.vec_ok = aligned16(p[i]) && aligned16(g[i]);
+            a.first_block[a.count] = (int32_t)blocks;
+            blocks += tiles;
+            a.count++;
+            i++;
+        }
+        if (a.count == 0) break;
+        a.first_block[a.count] = (int32_t)blocks;
+        sgd_multi_kernel<T, VEC><<<(unsigned)blocks, kBlock, 0, s>>>(a, lr);
+        ZENU_LAUNCH_CHECK();
+    }
+    return ZENU_OK;
+}
+
 }  // namespace
 }  // namespace zenu
 
 using namespace zenu;
 
 extern "C" {
+
+int zenu_hip_sgd_step_multi(int dtype, int n_tensors, void *const *p_dev, const void *const *g_dev,
+                            const int64_t *sizes, double lr, zenu_stream_t stream)
+{
+    if (n_tensors < 0) return ZENU_ERR_ARG;
+    if (n_tensors == 0) return ZENU_OK;
+    if (!p_dev || !g_dev || !sizes) return ZENU_ERR_ARG;
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (dtype == ZENU_F32) return sgd_multi_t<float>(n_tensors, p_dev, g_dev, sizes, (float)lr, as_stream(stream));
+    if (dtype == ZENU_F64) return sgd_multi_t<double>(n_tensors, p_dev, g_dev, sizes, lr, as_stream(stream));
+    return ZENU_ERR_ARG;
+}
 
 int zenu_hip_sgd_step(int dtype, void *p_dev, const void *g_dev, int64_t n, double lr, zenu_stream_t stream)
 {

@@ -28,10 +28,22 @@ class SGD:
     def __init__(self, learning_rate):
         self.learning_rate = learning_rate
 
-    def update(self, parameters):
-        for _, (data, grad) in parameters.items():
-            if grad is None:
-                continue
+    def update(self, parameters, multi_tensor=True):
+        items = [(d, g) for _, (d, g) in parameters.items() if g is not None]
+        if not items:
+            return
+        dtype = items[0][0].dtype
+        if multi_tensor and all(d.dtype == dtype for d, _ in items):
+            n = len(items)
+            P, G = (C.c_void_p * n)(), (C.c_void_p * n)()
+            sizes = (C.c_int64 * n)()
+            for i, (d, g) in enumerate(items):
+                P[i], sizes[i] = _flat(d)
+                G[i] = _flat(g)[0]
+            check(_lib.lib().zenu_hip_sgd_step_multi(_dt(dtype), n, P, G, sizes, float(self.learning_rate),
+                                                     get_stream()), "sgd_step_multi")
+            return
+        for data, grad in items:
             p, n = _flat(data)
             g, _ = _flat(grad)
             check(_lib.lib().zenu_hip_sgd_step(_dt(data.dtype), p, g, n, float(self.learning_rate),
