@@ -303,6 +303,41 @@ def build_ops(z, workload, stream):
                       lambda: zo.sum_to(a, col_h)))
         ops[-1].keep = sets
 
+    # ---- the same kernels on larger tensors: how much of the distance to the roofline is the fixed
+    # cost of a launch at the BASELINE sizes (not a BASELINE config) --------------------------------------
+    def add_scaling():
+        r = np.random.default_rng(7)
+        for mib in (64, 256, 1024):
+            n = mib * (1 << 20) // 4
+            a = r.standard_normal(n).astype(np.float32)
+            sets = [(M.from_numpy(a), M.from_numpy(a), M.alloc([n]), M.alloc(())) for _ in range(max(2, 3072 // (3 * mib)))]
+            rows = n // 4096
+            out_h = np.empty_like(a)
+
+            def mk(fn):
+                return [fn(A, B, O, S) for A, B, O, S in sets]
+            ops.append(Op(f"copy {mib} MiB", "scaling", "f32", 2 * 4 * n, n,
+                          mk(lambda A, B, O, S: (lambda d=O.desc(), s_=A.desc(): check(l.zenu_hip_copy(_lib.F32, ref(d), ref(s_), stream), "copy"))),
+                          lambda: zo.copy_from(out_h, a)))
+            ops.append(Op(f"add {mib} MiB", "scaling", "f32", 3 * 4 * n, n,
+                          mk(lambda A, B, O, S: (lambda d=O.desc(), x=A.desc(), y=B.desc(): check(l.zenu_hip_binary(_lib.ADD, _lib.F32, ref(d), ref(x), ref(y), stream), "add"))),
+                          lambda: zo.binary_array(zo.ADD, out_h, a, a)))
+            ops.append(Op(f"sum axis1 [{rows},4096]", "scaling", "f32", 4 * n + 4 * rows, n,
+                          mk(lambda A, B, O, S: (lambda d=O.slice(slice(0, rows)).desc(), s_=A.reshape((rows, 4096)).desc(): check(l.zenu_hip_sum_axis(_lib.F32, ref(d), ref(s_), 1, stream), "sum"))),
+                          lambda: zo.sum_axis(a.reshape(rows, 4096), 1)))
+            ops.append(Op(f"sum axis0 [{rows},4096]", "scaling", "f32", 4 * n + 4 * 4096, n,
+                          mk(lambda A, B, O, S: (lambda d=O.slice(slice(0, 4096)).desc(), s_=A.reshape((rows, 4096)).desc(): check(l.zenu_hip_sum_axis(_lib.F32, ref(d), ref(s_), 0, stream), "sum"))),
+                          lambda: zo.sum_axis(a.reshape(rows, 4096), 0)))
+            ops.append(Op(f"sum all {mib} MiB", "scaling", "f32", 4 * n + 4, n,
+                          mk(lambda A, B, O, S: (lambda p_=S.as_ptr(), s_=A.desc(): check(l.zenu_hip_sum_all(_lib.F32, p_, ref(s_), stream), "sum_all"))),
+                          lambda: zo.sum_to(a, np.zeros((), dtype=np.float32))))
+            ops.append(Op(f"tanh {mib} MiB", "scaling", "f32", 2 * 4 * n, n,
+                          mk(lambda A, B, O, S: (lambda d=O.desc(), s_=A.desc(): check(l.zenu_hip_unary(_lib.TANH, _lib.F32, ref(d), ref(s_), stream), "tanh"))),
+                          lambda: zo.unary(zo.TANH, out_h, a)))
+            ops[-1].keep = sets
+
+    if workload == "scaling":
+        add_scaling()
     if workload == "fused":
         add_fused()
     if workload == "next":
@@ -490,7 +525,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="suite", choices=["suite", "c0", "c1", "c2", "c3", "c4", "fused", "next"])
+    ap.add_argument("--workload", default="suite", choices=["suite", "c0", "c1", "c2", "c3", "c4", "fused", "next", "scaling"])
     ap.add_argument("--op-reps", type=int, default=50, help="launches per op in the per-op timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--profile-op", default=None, help="only launch this op (for rocprofv3 counter runs)")
@@ -607,6 +642,7 @@ def main():
         "config": {"workload": {"suite": "configs[0..3]: every op once per step", "c0": "configs[0]", "c1": "configs[1]",
                                 "c2": "configs[2]", "c3": "configs[3]",
                                 "fused": "fused entry points on [8192,4096] f32 (not a BASELINE config)",
+                                "scaling": "copy, add, sums and tanh on 64 MiB, 256 MiB and 1 GiB f32 tensors (not a BASELINE config)",
                                 "next": "strided copy, broadcast, the remaining unary functions, powf, asum and sum_to on [4096,4096] f32 "
                                         "(not a BASELINE config)"}[args.workload],
                    "ops_per_step": len(ops), "algorithmic_bytes_per_step": step_bytes},
