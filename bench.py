@@ -292,6 +292,9 @@ def build_ops(z, workload, stream):
             ops.append(Op(name, "next", "f32", 2 * nb, n * n,
                           mk(lambda A, P, U, R, O, V, S, fn=fn, src=src: (lambda d=O.desc(), s_=(A, P, U)[src].desc(): check(l.zenu_hip_unary(fn, _lib.F32, ref(d), ref(s_), stream), "unary"))),
                           lambda fn=fn, host=host: zo.unary(fn, out_h, host)))
+        ops.append(Op("tanh, the <= 2 ulp variant (ZENU_TANH_ULP2)", "next", "f32", 2 * nb, n * n,
+                      mk(lambda A, P, U, R, O, V, S: (lambda d=O.desc(), s_=A.desc(): check(l.zenu_hip_unary(_lib.TANH_ULP2, _lib.F32, ref(d), ref(s_), stream), "unary"))),
+                      lambda: zo.unary(zo.TANH, out_h, a)))
         ops.append(Op("powf(x, 2.5)", "next", "f32", 2 * nb, n * n,
                       mk(lambda A, P, U, R, O, V, S: (lambda d=O.desc(), s_=P.desc(): check(l.zenu_hip_powf(_lib.F32, ref(d), ref(s_), 2.5, stream), "powf"))),
                       lambda: zo.powf(out_h, pos, 2.5)))

@@ -50,7 +50,13 @@ typedef enum {
     ZENU_EXP = 0, ZENU_LOG = 1, ZENU_TANH = 2, ZENU_SQRT = 3, ZENU_ABS = 4,
     ZENU_SIN = 5, ZENU_COS = 6, ZENU_TAN = 7, ZENU_ASIN = 8, ZENU_ACOS = 9, ZENU_ATAN = 10,
     ZENU_SINH = 11, ZENU_COSH = 12,
-    ZENU_SIGMOID = 13 /* 0.5 + 0.5*tanh(0.5*x), zenu-autograd/src/activation/sigmoid.rs:7-15 */
+    ZENU_SIGMOID = 13, /* 0.5 + 0.5*tanh(0.5*x), zenu-autograd/src/activation/sigmoid.rs:7-15 */
+    /* No counterpart in the reference.  ZENU_TANH returns the bits of the host library's tanhf (what
+     * ZeNu's Cpu device returns) and is bound by arithmetic, not memory.  ZENU_TANH_ULP2 is for
+     * callers that accept the usual tolerance instead: f32 tanh evaluated in f64 and rounded once,
+     * at most 2 units in the last place from ZENU_TANH on every one of the 2^32 arguments, and
+     * bound by memory.  For f64 it is ZENU_TANH. */
+    ZENU_TANH_ULP2 = 14
 } zenu_unop_t;
 
 /* A strided view: Matrix<_, DimDyn, D> flattened (zenu-matrix/src/matrix.rs:224-233). */

@@ -362,6 +362,7 @@ public:
     ZENU_HPP_UNARY(sinh, ZENU_SINH)
     ZENU_HPP_UNARY(cosh, ZENU_COSH)
     ZENU_HPP_UNARY(sigmoid, ZENU_SIGMOID)
+    ZENU_HPP_UNARY(tanh_ulp2, ZENU_TANH_ULP2)   // not in the reference: f32 tanh within 2 ulp of tanh(), memory-bound
 #undef ZENU_HPP_UNARY
     void powf(const Matrix &other, T s) const
     {

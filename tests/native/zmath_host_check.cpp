@@ -15,11 +15,11 @@ int main(int argc, char **argv)
 {
     const uint64_t stride = argc > 1 ? strtoull(argv[1], nullptr, 10) : 1;
     const int nt = 8;
-    std::atomic<uint64_t> bad_fdlibm{0}, bad_simd{0}, bad_expm1{0}, bad_sig{0}, bad_exp{0}, bad_log{0}, bad_sinh{0}, bad_cosh{0}, bad_sin{0}, bad_cos{0}, bad_atan{0}, bad_asin{0}, bad_acos{0};
+    std::atomic<uint64_t> bad_fdlibm{0}, bad_simd{0}, bad_expm1{0}, bad_sig{0}, bad_exp{0}, bad_log{0}, bad_sinh{0}, bad_cosh{0}, bad_sin{0}, bad_cos{0}, bad_atan{0}, bad_asin{0}, bad_acos{0}, far_ulp2{0};
     std::vector<std::thread> th;
     for (int w = 0; w < nt; w++)
         th.emplace_back([&, w]() {
-            uint64_t b0 = 0, b1 = 0, b2 = 0, b3 = 0, b4 = 0, b5 = 0, b6 = 0, b7 = 0, b8 = 0, b9 = 0, b10 = 0, b11 = 0, b12 = 0;
+            uint64_t b0 = 0, b1 = 0, b2 = 0, b3 = 0, b4 = 0, b5 = 0, b6 = 0, b7 = 0, b8 = 0, b9 = 0, b10 = 0, b11 = 0, b12 = 0, b13 = 0;
             for (uint64_t u = (uint64_t)w * stride; u < (1ull << 32); u += stride * nt) {
                 const float x = zmath::u2f((uint32_t)u);
                 const float atr = atanf(x), atg = zmath::atanf_fdlibm(x);
@@ -45,11 +45,17 @@ int main(int argc, char **argv)
                 const bool nan = ref != ref;
                 if (nan ? !(a != a) : zmath::f2u(a) != zmath::f2u(ref)) b0++;
                 if (nan ? !(s != s) : zmath::f2u(s) != zmath::f2u(ref)) b1++;
+                // the variant that is allowed 2 units in the last place: count what is further away
+                const float q = zmath::tanhf_ulp2(x);
+                if (nan ? !(q != q)
+                        : ((q < 0) != (ref < 0) && q != ref) ||
+                              (zmath::f2u(q) > zmath::f2u(ref) ? zmath::f2u(q) - zmath::f2u(ref) : zmath::f2u(ref) - zmath::f2u(q)) > 2)
+                    b13++;
                 if (fabsf(x) < 44.0f && zmath::f2u(zmath::expm1f_fdlibm(x)) != zmath::f2u(expm1f(x))) b2++;
                 const float sg = 0.5f + 0.5f * tanhf(0.5f * x), sz = zmath::sigmoidf_zenu(x);
                 if ((sg != sg) ? !(sz != sz) : zmath::f2u(sz) != zmath::f2u(sg)) b3++;
             }
-            bad_fdlibm += b0; bad_simd += b1; bad_expm1 += b2; bad_sig += b3; bad_exp += b4; bad_log += b5; bad_sinh += b6; bad_cosh += b7; bad_sin += b8; bad_cos += b9; bad_atan += b10; bad_asin += b11; bad_acos += b12;
+            bad_fdlibm += b0; bad_simd += b1; bad_expm1 += b2; bad_sig += b3; bad_exp += b4; bad_log += b5; bad_sinh += b6; bad_cosh += b7; bad_sin += b8; bad_cos += b9; bad_atan += b10; bad_asin += b11; bad_acos += b12; far_ulp2 += b13;
         });
     for (auto &t : th) t.join();
     // double precision: every stride-th value of the HIGH word (sign, exponent, 20 mantissa bits) with
@@ -127,5 +133,6 @@ int main(int argc, char **argv)
     printf("sinf_glibc %llu cosf_glibc %llu\n", (unsigned long long)bad_sin.load(), (unsigned long long)bad_cos.load());
     printf("atanf_fdlibm %llu asinf_fdlibm %llu acosf_fdlibm %llu\n", (unsigned long long)bad_atan.load(),
            (unsigned long long)bad_asin.load(), (unsigned long long)bad_acos.load());
-    return (bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64 + bad_exp64 + bad_sinh64 + bad_cosh64 + bad_exp + bad_log + bad_pow + bad_sinh + bad_cosh + bad_sin + bad_cos + bad_atan + bad_asin + bad_acos) ? 1 : 0;
+    printf("tanhf_ulp2_beyond_2ulp %llu\n", (unsigned long long)far_ulp2.load());
+    return (far_ulp2 + bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64 + bad_exp64 + bad_sinh64 + bad_cosh64 + bad_exp + bad_log + bad_pow + bad_sinh + bad_cosh + bad_sin + bad_cos + bad_atan + bad_asin + bad_acos) ? 1 : 0;
 }

@@ -6,11 +6,15 @@ Bars (written where they are used):
   f32 exp, log, powf, sinh, cosh, sin, cos, asin, acos, atan; f64 exp, sinh, cosh; tanh, sigmoid in f32 and f64
       (the host libm's algorithms, restated) .......................... bit-exact (bar: <= 2 ulp)
   f64 log, powf (device math library) ................................. <= 2 ulp
+  tanh_ulp2 (f32 evaluated in f64, not in the reference) .............. <= 2 ulp
   sums ................................................................ |gpu - cpu| <= 1e-5 (f32) /
       1e-12 (f64) times max(|cpu|, sum|x| / sqrt(n)); the second term is the typical magnitude
       of a sum of n such terms, so a result that cancels to ~0 is not held to a relative bar
       the sequential CPU sum itself cannot meet.
 """
+import os
+import subprocess
+
 import numpy as np
 import pytest
 
@@ -259,6 +263,44 @@ def test_tanh_sigmoid_dense_sweep(hip):
         ok = ~np.isnan(exp)
         assert np.array_equal(np.isnan(got), np.isnan(exp)), name
         assert max_ulp(got[ok], exp[ok]) == 0, name
+
+
+def test_tanh_ulp2_variant(hip):
+    """ZENU_TANH_ULP2 (no counterpart in the reference): never more than 2 ulp from the host tanhf,
+    the tolerance the transcendental functions are allowed; checked on every 64th f32 bit pattern and
+    the special values (the host build of the same function is checked on the same stride, and was
+    on all 2^32, in test_host_native.py); signs of zero and NaN positions as tanhf; views take the
+    same route as every unary operator; the f64 form is plain tanh."""
+    bits = np.arange(0, 1 << 32, 64, dtype=np.uint64).astype(np.uint32)
+    special = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1e-30, 1.1754944e-38, 0.17, 0.1733, 0.55,
+                        1.0, 9.01, 9.011, 19.9, 20.0, 20.1, 88.0, 3e38, -3e38], dtype=np.float32)
+    x = np.concatenate([bits.view(np.float32), special])
+    exp = np.empty_like(x)
+    with np.errstate(all="ignore"):
+        zo.unary(zo.TANH, exp, x)
+    got = hip.Matrix.from_numpy(x).tanh_ulp2().to_numpy()
+    assert np.array_equal(np.isnan(got), np.isnan(exp))
+    ok = ~np.isnan(exp)
+    assert np.array_equal(np.signbit(got[ok]), np.signbit(exp[ok]))
+    u = max_ulp(got[ok], exp[ok])
+    print(f"tanh_ulp2: max ulp vs libm = {u}; equal on {np.mean(got[ok] == exp[ok]):.4f} of the points", flush=True)
+    assert u <= 2
+    # only IEEE operations: the kernel returns the bits of the same source compiled for the host
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "native", "bin", "zmath_host_eval")
+    if not os.path.exists(exe):
+        pytest.skip("tests/native/bin/zmath_host_eval is not built (run __graft_entry__.build())")
+    host = np.frombuffer(subprocess.run([exe, "tanh_ulp2"], input=x.tobytes(), capture_output=True, check=True).stdout,
+                         dtype=np.float32)
+    assert np.array_equal(host.view(np.uint32)[ok], got.view(np.uint32)[ok])
+    r = rng(12)
+    a = r.standard_normal((130, 70)).astype(np.float32) * np.float32(3)
+    e2 = np.empty((70, 130), dtype=np.float32)
+    zo.unary(zo.TANH, e2, np.ascontiguousarray(a.T))
+    g2 = hip.Matrix.from_numpy(a).transpose().tanh_ulp2().to_numpy()
+    assert g2.shape == (70, 130) and max_ulp(g2, e2) <= 2
+    d = r.standard_normal(1000)
+    D = hip.Matrix.from_numpy(d)
+    assert np.array_equal(D.tanh_ulp2().to_numpy(), D.tanh().to_numpy())
 
 
 def test_unary_f64(hip):

@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libzenu_hip.so")
 MAX_DIM = 6
 F32, F64 = 0, 1
 ADD, SUB, MUL, DIV = 0, 1, 2, 3
-(EXP, LOG, TANH, SQRT, ABS, SIN, COS, TAN, ASIN, ACOS, ATAN, SINH, COSH, SIGMOID) = range(14)
+(EXP, LOG, TANH, SQRT, ABS, SIN, COS, TAN, ASIN, ACOS, ATAN, SINH, COSH, SIGMOID, TANH_ULP2) = range(15)
 
 OK, ERR_RANK, ERR_SHAPE, ERR_AXIS, ERR_ARG, ERR_HIP, ERR_OOM, ERR_UNSUPPORTED, ERR_NOT_OWNED = range(9)
 

@@ -22,6 +22,9 @@ template <typename T> int unary_t(int fn, const zenu_tensor_t &to, const zenu_te
     case ZENU_SQRT: return run1<T>(to, in, UnaryF<T, ZENU_SQRT>(), s);
     case ZENU_ABS: return run1<T>(to, in, UnaryF<T, ZENU_ABS>(), s);
     case ZENU_SIGMOID: return run1<T>(to, in, UnaryF<T, ZENU_SIGMOID>(), s);
+    case ZENU_TANH_ULP2:
+        if constexpr (sizeof(T) == 4) return run1<T>(to, in, TanhUlp2F(), s);
+        else return run1<T>(to, in, UnaryF<T, ZENU_TANH>(), s);
     default: return unary_trig(ZenuDType<T>::value, fn, to, in, s);   // ew_unary_trig.hip
     }
 }
