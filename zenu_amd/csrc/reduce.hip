@@ -438,6 +438,12 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(RedParams<T> p)
 // splits; with splits > 1 partials are stored as [split][output] (coalesced) and the last
 // workgroup of a column tile to finish folds that tile's partials, split 0 first.
 
+// Loops over a thread's columns run over all VEC of them with a predicate.  A loop with the
+// run-time bound `ncol` indexes the accumulator array dynamically; the compiler then moves the
+// array to LDS and, to find each thread's slot, reads the workgroup size from the dispatch packet,
+// which sits in host memory: 2-10 us before the first load (measured on the arg-max kernel).
+#define ZENU_FOR_COLS(j) _Pragma("unroll") for (int j = 0; j < VEC; j++) if (j < ncol)
+
 template <typename T, typename Tr, int VEC, bool NT>
 __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int64_t col_tiles, int tx_shift)
 {
@@ -495,10 +501,10 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int
     } else if (ncol > 0) {
         for (int64_t b = split * chunk; b < R; b += p.splits * chunk)
             for (int64_t r = b + ty; r < R && r < b + chunk; r += ty_n)
-                for (int j = 0; j < ncol; j++) acc[j] = Tr::update(acc[j], src[r * p.elem_stride + j], r);
+                ZENU_FOR_COLS(j) acc[j] = Tr::update(acc[j], src[r * p.elem_stride + j], r);
     }
     if (split == 0 && ty == 0)
-        for (int j = 0; j < ncol; j++) acc[j] = Tr::first(acc[j], src[j]);
+        ZENU_FOR_COLS(j) acc[j] = Tr::first(acc[j], src[j]);
 
     // combine the ty lanes in fixed order
     if (ty_n > 1) {
@@ -517,11 +523,11 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int
     const int64_t o0 = q * p.inner + c;
     if (p.splits == 1) {
         if (ty == 0)
-            for (int j = 0; j < ncol; j++) emit_final<T, Tr>(p, o0 + j, acc[j]);
+            ZENU_FOR_COLS(j) emit_final<T, Tr>(p, o0 + j, acc[j]);
         return;
     }
     if (ty == 0)
-        for (int j = 0; j < ncol; j++) emit_partial<T, Tr>(p, (int64_t)split * p.nout + o0 + j, acc[j]);
+        ZENU_FOR_COLS(j) emit_partial<T, Tr>(p, (int64_t)split * p.nout + o0 + j, acc[j]);
     if (!arrive_last(p.counters + group * p.cstride, split, p.splits, p.fan)) return;
     // fold this column tile: row lane ty takes splits ty, ty + ty_n, ...; then the fixed LDS order
 #pragma unroll
@@ -557,7 +563,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int
         }
     }
     if (ty == 0)
-        for (int j = 0; j < ncol; j++) emit_final<T, Tr>(p, o0 + j, acc[j]);
+        ZENU_FOR_COLS(j) emit_final<T, Tr>(p, o0 + j, acc[j]);
     if (threadIdx.x == 0) store_agent(p.counters + group * p.cstride, 0);
 }
 
