@@ -511,12 +511,10 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int
 #pragma unroll
         for (int j = 0; j < VEC; j++) lds[j * kBlock + threadIdx.x] = acc[j];   // [vector element][thread]: consecutive lanes, consecutive banks
         __syncthreads();
-        if (ty == 0) {
+        if (ty == 0) {   // row lane by row lane, the VEC columns side by side: ty_n - 1 dependent LDS round trips, not VEC times that
+            for (int w = 1; w < ty_n; w++) {
 #pragma unroll
-            for (int j = 0; j < VEC; j++) {
-                A r = lds[j * kBlock + tx];
-                for (int w = 1; w < ty_n; w++) r = Tr::merge(r, lds[j * kBlock + w * tx_n + tx]);
-                acc[j] = r;
+                for (int j = 0; j < VEC; j++) acc[j] = Tr::merge(acc[j], lds[j * kBlock + w * tx_n + tx]);
             }
         }
     }
@@ -553,12 +551,10 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int
 #pragma unroll
         for (int j = 0; j < VEC; j++) lds[j * kBlock + threadIdx.x] = acc[j];   // [vector element][thread]: consecutive lanes, consecutive banks
         __syncthreads();
-        if (ty == 0) {
+        if (ty == 0) {   // row lane by row lane, the VEC columns side by side: ty_n - 1 dependent LDS round trips, not VEC times that
+            for (int w = 1; w < ty_n; w++) {
 #pragma unroll
-            for (int j = 0; j < VEC; j++) {
-                A r = lds[j * kBlock + tx];
-                for (int w = 1; w < ty_n; w++) r = Tr::merge(r, lds[j * kBlock + w * tx_n + tx]);
-                acc[j] = r;
+                for (int j = 0; j < VEC; j++) acc[j] = Tr::merge(acc[j], lds[j * kBlock + w * tx_n + tx]);
             }
         }
     }
