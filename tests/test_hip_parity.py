@@ -448,6 +448,43 @@ def test_strided_broadcast_binary(hip, idx, dt):
         assert_bits(BIG.to_numpy(), big, f"strided destination case {idx}")
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_one_operand_periodic(hip, dt):
+    """a contiguous operand with one that varies along a single dim (a channel bias on [N,C,H,W], a row
+    or a column on a matrix, a per-sample scalar): the flat kernel that reads y[(i / inner) % mid], in its
+    three forms (y as vectors; one y per vector; a vector spanning two y), with the periodic operand
+    on either side of a non-commutative operator, sizes that end inside a vector or a tile, and in place"""
+    r = rng(77)
+    cases = [((5, 8, 6, 6), (1, 8, 1, 1)),      # inner 36: one y per vector
+             ((3, 5, 7, 7), (1, 5, 1, 1)),      # inner 49: vectors span two channels; 735 elements, ragged end
+             ((4, 6, 5), (1, 6, 1)),            # inner 5
+             ((37, 64), (1, 64)),               # a row: y read as vectors
+             ((37, 64), (37, 1)),               # a column: inner 64
+             ((129, 1030), (1, 1030)),          # row length not a multiple of 4 (f32): vectors span two rows of y
+             ((700, 3), (1, 3)),                # inner 1, period 3: handled by the general kernels
+             ((6, 2, 3), (6, 1, 1)),            # per-sample scalar, inner 6
+             ((2, 4100, 12), (1, 4100, 1))]     # more than one tile
+    for shape, yshape in cases:
+        x = r.standard_normal(shape).astype(dt)
+        y = (r.standard_normal(yshape) + 3).astype(dt)
+        X, Y = hip.Matrix.from_numpy(x), hip.Matrix.from_numpy(y)
+        for name, op in (("sub", zo.SUB), ("div", zo.DIV)):
+            exp = np.empty(shape, dtype=dt)
+            zo.binary_array(op, exp, x, y)
+            out = hip.Matrix.alloc(shape, dt)
+            getattr(out, f"{name}_array")(X, Y)
+            assert_bits(out.to_numpy(), exp, f"{name} {shape} {yshape}")
+            assert_bits(exp, {"sub": np.subtract, "div": np.divide}[name](x, y), "oracle vs numpy broadcasting")
+            zo.binary_array(op, exp, y, x)                # periodic operand on the left
+            getattr(out, f"{name}_array")(Y, X)
+            assert_bits(out.to_numpy(), exp, f"{name} {yshape} {shape}")
+        X2 = hip.Matrix.from_numpy(x)
+        X2.add_assign(Y)                                  # in place: the output aliases the full operand
+        exp = x.copy()
+        zo.binary_assign(zo.ADD, exp, y)
+        assert_bits(X2.to_numpy(), exp, f"add_assign {shape} {yshape}")
+
+
 def test_copy_transpose_large(hip):
     r = rng(12)
     a = r.standard_normal((1000, 777)).astype(np.float32)
