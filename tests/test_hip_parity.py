@@ -478,6 +478,17 @@ def test_one_operand_periodic(hip, dt):
             zo.binary_array(op, exp, y, x)                # periodic operand on the left
             getattr(out, f"{name}_array")(Y, X)
             assert_bits(out.to_numpy(), exp, f"{name} {yshape} {shape}")
+        out = hip.Matrix.alloc(shape, dt)
+        exp = np.empty(shape, dtype=dt)
+        try:                                              # broadcast.rs accepts trailing-dim sources only
+            zo.broadcast(exp, y)
+        except zo.OracleError:
+            with pytest.raises(hip.ZenuHipError):
+                out.broadcast(Y)
+        else:
+            out.broadcast(Y)                              # no full-size input at all: a lone store stream
+            assert_bits(out.to_numpy(), exp, f"broadcast {yshape} -> {shape}")
+            assert_bits(exp, np.broadcast_to(y, shape).copy(), "oracle vs numpy broadcasting")
         X2 = hip.Matrix.from_numpy(x)
         X2.add_assign(Y)                                  # in place: the output aliases the full operand
         exp = x.copy()

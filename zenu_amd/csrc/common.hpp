@@ -62,6 +62,7 @@ zenu_tensor_t default_view(void *ptr, int ndim, const int64_t *shape);
 // zenu-matrix/src/with_clousers.rs:87-107,155-178.
 int check_binary(const zenu_tensor_t &to, const zenu_tensor_t &lhs, const zenu_tensor_t &rhs);
 int check_binary_assign(const zenu_tensor_t &to, const zenu_tensor_t &rhs);
+int check_broadcast(const zenu_tensor_t &to, const zenu_tensor_t &source);
 
 // An elementwise problem over `nops` operands (operand 0 is the output) sharing one iteration
 // space.  Input strides are already broadcast-expanded (0 on broadcast dims) and aligned to the

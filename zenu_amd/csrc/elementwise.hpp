@@ -278,7 +278,8 @@ __global__ __launch_bounds__(ContigShape<F>::kBlock) void ew_contig_kernel(T *ou
 // The output and one input are contiguous and of full size; the other input varies along ONE of the
 // (collapsed) dims only, where it is contiguous: a bias [1,C,1,1] on [N,C,H,W], a row [1,n] on
 // [m,n], a column [m,1] on [m,n].  Flat index i reads y[(i / inner) % mid].  Indices are 32-bit
-// (checked at launch).  MODE 0: inner == 1 and mid % VEC == 0, y is read as vectors; MODE 1:
+// (checked at launch).  With a one-input functor there is no x: the output is f(y) spread over the
+// other dims (broadcast of a row, a column, a bias).  MODE 0: inner == 1 and mid % VEC == 0, y is read as vectors; MODE 1:
 // inner % VEC == 0, one y per vector; MODE 2: inner >= VEC, a vector spans at most two y.
 
 template <typename T, int VEC, bool NT, typename F, bool Y_FIRST, int MODE, int kBlock, int kUnroll>
@@ -307,8 +308,9 @@ __global__ __launch_bounds__(kBlock) void ew_periodic_kernel(T *out, const T *x,
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             const uint32_t i0 = base + (uint32_t)(u * kBlock + threadIdx.x) * VEC;
-            xv[u] = load_pack<T, VEC, NT>(x + i0);
             yv[u] = y_of(i0);
+            if constexpr (F::NIN == 2) xv[u] = load_pack<T, VEC, NT>(x + i0);
+            else xv[u] = yv[u];
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
@@ -322,7 +324,8 @@ __global__ __launch_bounds__(kBlock) void ew_periodic_kernel(T *out, const T *x,
             for (int j = 0; j < VEC; j++) {
                 const uint64_t i = i0 + j;
                 if (i < n) {
-                    const T xs = x[i], ys = y[((uint32_t)i / inner) % mid];
+                    const T ys = y[((uint32_t)i / inner) % mid];
+                    const T xs = (F::NIN == 2) ? x[i] : ys;
                     out[i] = Y_FIRST ? f(ys, xs) : f(xs, ys);
                 }
             }
@@ -648,7 +651,7 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
     }
 
     // flat with one periodic operand (bias over channels, a row or a column over a matrix)
-    if constexpr (F::NIN == 2) {
+    {
         if (p.numel < ((int64_t)1 << 32) - 65536 && aligned16(out)) {
             auto flat = [&](int o) {
                 int64_t want = 1;
@@ -668,10 +671,12 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
                 return m;
             };
             int yo = 0, m = -1;
-            if (flat(0) && flat(1) && (m = period_dim(2)) >= 0) yo = 2;
+            if (nin == 1) {
+                if (flat(0) && !flat(1) && (m = period_dim(1)) >= 0) yo = 1;
+            } else if (flat(0) && flat(1) && (m = period_dim(2)) >= 0) yo = 2;
             else if (flat(0) && flat(2) && (m = period_dim(1)) >= 0) yo = 1;
             if (yo) {
-                const T *x = yo == 2 ? a : b, *y = yo == 2 ? b : a;
+                const T *x = yo == 2 ? a : b, *y = yo == 2 ? b : a;   // one input: x == y == a, x is not read
                 int64_t inner = 1;
                 for (int d = m + 1; d < p.ndim; d++) inner *= p.shape[d];
                 const int64_t mid = p.shape[m];
@@ -687,7 +692,8 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
                     auto go = [&](auto yfirst_c, auto mode_c) {
                         constexpr bool YF = decltype(yfirst_c)::value;
                         constexpr int MODE = decltype(mode_c)::value;
-                        constexpr bool small = MODE == 0 && !IsValuBound<F>::value;
+                        // a lone store stream (one-input functor) keeps the larger shape, like the fill kernel
+                        constexpr bool small = MODE == 0 && !IsValuBound<F>::value && F::NIN == 2;
                         constexpr int B = small ? ZENU_EW1_BLOCK : 256, U = small ? ZENU_EW1_UNROLL : 2;
                         const int64_t tile = (int64_t)B * VEC * U;
                         const unsigned grid = (unsigned)((p.numel + tile - 1) / tile);

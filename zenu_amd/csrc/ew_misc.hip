@@ -50,7 +50,7 @@ int zenu_hip_broadcast(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *
 {
     int rc = check2(to, source);
     if (!rc) rc = ensure_init();
-    if (!rc) rc = check_binary_assign(*to, *source);   // is_include || is_include_bradcast, broadcast.rs:13-17
+    if (!rc) rc = check_broadcast(*to, *source);   // broadcast.rs:11-43: the test at :13-17 and what its recursion then requires
     if (rc) return rc;
     if (dtype == ZENU_F32) return run1<float>(*to, *source, CopyF<float>(), as_stream(stream));
     if (dtype == ZENU_F64) return run1<double>(*to, *source, CopyF<double>(), as_stream(stream));

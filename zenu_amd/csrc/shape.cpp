@@ -111,6 +111,35 @@ int check_binary_assign(const zenu_tensor_t &to, const zenu_tensor_t &rhs)
     return ZENU_OK;
 }
 
+// Matrix::broadcast, broadcast.rs:11-43, walked on shapes only: the legality test at every level of
+// its recursion, the leading size-1 axes of the source it drops, and the shape equality its final
+// copy_from demands.  What the reference would panic on is an error here: a source such as [1,C,1,1]
+// or a column [m,1] passes the first test but fails inside the recursion.
+static int broadcast_walk(const int64_t *to, int nt, const int64_t *src, int ns)
+{
+    zenu_tensor_t a{}, b{};
+    a.ndim = nt;
+    b.ndim = ns;
+    for (int i = 0; i < nt; i++) a.shape[i] = to[i];
+    for (int i = 0; i < ns; i++) b.shape[i] = src[i];
+    if (!(dims_include(a, b) || dims_include_broadcast(a, b))) return ZENU_ERR_SHAPE;
+    if (same_shape(a, b)) return ZENU_OK;
+    if (ns > 0 && src[0] == 1) return broadcast_walk(to, nt, src + 1, ns - 1);
+    if (nt == 0) return ZENU_ERR_RANK;
+    if (to[0] == 0) return ZENU_OK;                       // no iteration of the loop over the leading axis
+    if (nt - ns == 1) {                                   // copy_from(&source) on each index of the leading axis
+        for (int i = 0; i < ns; i++)
+            if (to[1 + i] != src[i]) return ZENU_ERR_SHAPE;
+        return ZENU_OK;
+    }
+    return broadcast_walk(to + 1, nt - 1, src, ns);
+}
+
+int check_broadcast(const zenu_tensor_t &to, const zenu_tensor_t &source)
+{
+    return broadcast_walk(to.shape, to.ndim, source.shape, source.ndim);
+}
+
 void ew_set_operand(EwProblem &p, int slot, const zenu_tensor_t &t, int out_ndim,
                     const int64_t *out_shape)
 {
