@@ -633,20 +633,19 @@ ZM_HD float atanf_fdlibm(float x)
         if (ix > 0x7f800000u) return x + x;              // NaN
         return neg ? -hi3 - lo3 : hi3 + lo3;
     }
-    bool reduced = false;
+    // The four argument reductions are one division each in the sources; here the numerator and
+    // denominator are selected first, so a wavefront with arguments in several ranges divides once.
+    const bool reduced = ix >= 0x3ee00000u;              // |x| >= 0.4375
+    if (!reduced && ix < 0x31000000u) return x;          // |x| < 2^-29
     float h = 0.0f, l = 0.0f;
-    if (ix < 0x3ee00000u) {                              // |x| < 0.4375
-        if (ix < 0x31000000u) return x;                  // |x| < 2^-29
-    } else {
-        reduced = true;
-        x = u2f(ix);
-        if (ix < 0x3f980000u) {                          // |x| < 1.1875
-            if (ix < 0x3f300000u) { h = hi0; l = lo0; x = (2.0f * x - one) / (2.0f + x); }
-            else                  { h = hi1; l = lo1; x = (x - one) / (x + one); }
-        } else {
-            if (ix < 0x401c0000u) { h = hi2; l = lo2; x = (x - 1.5f) / (one + 1.5f * x); }
-            else                  { h = hi3; l = lo3; x = -1.0f / x; }
-        }
+    if (reduced) {
+        const float ax = u2f(ix);
+        const bool r0 = ix < 0x3f300000u, r1 = ix < 0x3f980000u, r2 = ix < 0x401c0000u;   // < 0.6875, < 1.1875, < 2.4375
+        const float num = r0 ? 2.0f * ax - one : r1 ? ax - one : r2 ? ax - 1.5f : -1.0f;
+        const float den = r0 ? 2.0f + ax : r1 ? ax + one : r2 ? one + 1.5f * ax : ax;
+        h = r0 ? hi0 : r1 ? hi1 : r2 ? hi2 : hi3;
+        l = r0 ? lo0 : r1 ? lo1 : r2 ? lo2 : lo3;
+        x = num / den;
     }
     const float z = x * x;
     const float w = z * z;
@@ -667,15 +666,13 @@ ZM_HD float asinf_fdlibm(float x)
     const uint32_t ix = hx & 0x7fffffffu;
     if (ix == 0x3f800000u) return x * pio2_hi + x * pio2_lo;     // asin(+-1) = +-pi/2
     if (ix > 0x3f800000u) return (x - x) / (x - x);              // |x| > 1, NaN
-    if (ix < 0x3f000000u) {                              // |x| < 0.5
-        if (ix < 0x32000000u) return x;                  // |x| < 2^-27
-        const float t = x * x;
-        const float w = t * (p0 + t * (p1 + t * (p2 + t * (p3 + t * p4))));
-        return x + x * w;
-    }
+    // both ranges evaluate the same polynomial, of x^2 below 0.5 and of (1 - |x|) / 2 above: once here
+    const bool small = ix < 0x3f000000u;                 // |x| < 0.5
+    if (small && ix < 0x32000000u) return x;             // |x| < 2^-27
     float w = one - u2f(ix);
-    float t = w * 0.5f;
+    float t = small ? x * x : w * 0.5f;
     float p = t * (p0 + t * (p1 + t * (p2 + t * (p3 + t * p4))));
+    if (small) return x + x * p;
     const float s = sqrtf(t);
     if (ix >= 0x3F79999Au) {                             // |x| > 0.975
         t = pio2_hi - (2.0f * (s + s * p) - pio2_lo);
@@ -701,30 +698,22 @@ ZM_HD float acosf_fdlibm(float x)
     const bool neg = (hx >> 31) != 0;
     if (ix == 0x3f800000u) return neg ? pi + 2.0f * pio2_lo : 0.0f;   // acos(-1) = pi, acos(1) = 0
     if (ix > 0x3f800000u) return (x - x) / (x - x);                   // |x| > 1, NaN
-    if (ix < 0x3f000000u) {                              // |x| < 0.5
-        if (ix <= 0x23000000u) return pio2_hi + pio2_lo; // |x| < 2^-57
-        const float z = x * x;
-        const float p = z * (pS0 + z * (pS1 + z * (pS2 + z * (pS3 + z * (pS4 + z * pS5)))));
-        const float q = one + z * (qS1 + z * (qS2 + z * (qS3 + z * qS4)));
-        const float r = p / q;
-        return pio2_hi - (x - (pio2_lo - x * r));
-    }
-    if (neg) {                                           // x < -0.5
-        const float z = (one + x) * 0.5f;
-        const float p = z * (pS0 + z * (pS1 + z * (pS2 + z * (pS3 + z * (pS4 + z * pS5)))));
-        const float q = one + z * (qS1 + z * (qS2 + z * (qS3 + z * qS4)));
-        const float s = sqrtf(z);
-        const float r = p / q;
-        const float w = r * s - pio2_lo;
-        return pi - 2.0f * (s + w);
-    }
-    const float z = (one - x) * 0.5f;                    // x > 0.5
-    const float s = sqrtf(z);
-    const float df = u2f(f2u(s) & 0xfffff000u);
-    const float c = (z - df * df) / (s + df);
+    // the three ranges evaluate the same rational function p(z) / q(z), of x^2, (1 + x) / 2 or
+    // (1 - x) / 2: once here, whatever mix of ranges a wavefront holds
+    const bool small = ix < 0x3f000000u;                 // |x| < 0.5
+    if (small && ix <= 0x23000000u) return pio2_hi + pio2_lo;   // |x| < 2^-57
+    const float z = small ? x * x : (neg ? (one + x) * 0.5f : (one - x) * 0.5f);
     const float p = z * (pS0 + z * (pS1 + z * (pS2 + z * (pS3 + z * (pS4 + z * pS5)))));
     const float q = one + z * (qS1 + z * (qS2 + z * (qS3 + z * qS4)));
     const float r = p / q;
+    if (small) return pio2_hi - (x - (pio2_lo - x * r));
+    const float s = sqrtf(z);
+    if (neg) {                                           // x < -0.5
+        const float w = r * s - pio2_lo;
+        return pi - 2.0f * (s + w);
+    }
+    const float df = u2f(f2u(s) & 0xfffff000u);          // x > 0.5
+    const float c = (z - df * df) / (s + df);
     const float w = r * s + c;
     return 2.0f * (df + w);
 }
