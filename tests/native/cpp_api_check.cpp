@@ -155,6 +155,7 @@ static void unary_tables()    // zenu-cuda/src/kernel/mod.rs:1015-1241, 1e-6
     M b = M::from_vec({1, 2, 3, 4}, {4});
     REQUIRE(close(b.log(), {0.0, 0.693147181, 1.098612289, 1.386294361}, 1e-6));
     REQUIRE(close(a.tanh(), {0.0, 0.761594156, 0.96402758, 0.995054754}, 1e-6));
+    REQUIRE(close(a.tanh_ulp2(), {0.0, 0.761594156, 0.96402758, 0.995054754}, 1e-6));   // the 2-ulp variant, same table
     REQUIRE(close(b.sqrt(), {1.0, 1.414213562, 1.732050808, 2.0}, 1e-6));
     M c = M::from_vec({-1, 2, -3, 4}, {4});
     REQUIRE(eq(c.abs(), {1, 2, 3, 4}));
