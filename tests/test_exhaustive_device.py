@@ -1,0 +1,101 @@
+"""Every f32 bit pattern through the kernels whose results are meant to be the host libm's bits.
+
+Opt-in (ZENU_EXHAUSTIVE=1): 2^32 arguments per function take a few minutes of host time for the
+oracle even on 16 threads, too long for the default suite, which checks every 64th pattern on the
+device (test_hip_parity.py) and every 31st in the host build of the same source
+(test_host_native.py).  Run as
+    ZENU_EXHAUSTIVE=1 python -u -m pytest tests/test_exhaustive_device.py -m gpu -x -s --timeout 3000
+"""
+import os
+from concurrent.futures import ThreadPoolExecutor
+
+import numpy as np
+import pytest
+
+import zenu_oracle as zo
+
+pytestmark = [pytest.mark.gpu,
+              pytest.mark.skipif(os.environ.get("ZENU_EXHAUSTIVE") != "1", reason="opt-in: set ZENU_EXHAUSTIVE=1")]
+
+CHUNK = 1 << 26
+THREADS = 16
+
+# (Matrix method, oracle function id or None for the sigmoid composite, largest allowed distance in ulp)
+FUNCTIONS = [("tanh", zo.TANH, 0), ("sigmoid", None, 0), ("exp", zo.EXP, 0), ("log", zo.LOG, 0),
+             ("sinh", zo.SINH, 0), ("cosh", zo.COSH, 0), ("sin", zo.SIN, 0), ("cos", zo.COS, 0),
+             ("asin", zo.ASIN, 0), ("acos", zo.ACOS, 0), ("atan", zo.ATAN, 0), ("tanh_ulp2", zo.TANH, 2)]
+
+
+def oracle_chunk(fn, x, exponent=None):
+    """the oracle (the host libm behind the reference's CPU path) on a chunk, split over threads;
+    ctypes releases the interpreter lock during each call"""
+    out = np.empty_like(x)
+    step = x.size // THREADS
+
+    def part(i):
+        sl = slice(i * step, x.size if i == THREADS - 1 else (i + 1) * step)
+        if exponent is not None:
+            zo.powf(out[sl], x[sl], exponent)
+        elif fn is None:
+            zo.sigmoid(out[sl], x[sl])
+        else:
+            zo.unary(fn, out[sl], x[sl])
+    with ThreadPoolExecutor(THREADS) as pool:
+        list(pool.map(part, range(THREADS)))
+    return out
+
+
+def ordered(a):
+    i = a.view(np.int32).astype(np.int64)
+    return np.where(i < 0, np.int64(-2**31) - i, i)
+
+
+@pytest.mark.parametrize("name,fn,bar", FUNCTIONS)
+def test_all_f32_bit_patterns(hip, name, fn, bar):
+    worst, differing, total = 0, 0, 0
+    with np.errstate(all="ignore"):
+        for start in range(0, 1 << 32, CHUNK):
+            x = np.arange(start, start + CHUNK, dtype=np.uint64).astype(np.uint32).view(np.float32)
+            got = getattr(hip.Matrix.from_numpy(x), name)().to_numpy()
+            exp = oracle_chunk(fn, x)
+            nan = np.isnan(exp)
+            assert np.array_equal(np.isnan(got), nan), f"{name}: NaN positions differ in chunk {start:#x}"
+            ok = ~nan
+            if bar == 0:
+                bad = got.view(np.uint32)[ok] != exp.view(np.uint32)[ok]
+                if bad.any():
+                    i = np.flatnonzero(ok)[np.flatnonzero(bad)[0]]
+                    raise AssertionError(f"{name}: {int(bad.sum())} of {CHUNK} differ in chunk {start:#x}, first x = "
+                                         f"{x[i]!r} ({x.view(np.uint32)[i]:#010x}): got {got[i]!r}, libm {exp[i]!r}")
+            else:
+                d = np.abs(ordered(got[ok]) - ordered(exp[ok]))
+                worst = max(worst, int(d.max()))
+                differing += int((d > 0).sum())
+                assert worst <= bar, f"{name}: {worst} ulp in chunk {start:#x}"
+            total += int(ok.sum())
+            if start % (1 << 30) == 0:
+                print(f"[exhaustive] {name}: {start >> 26} of 64 chunks", flush=True)
+    print(f"[exhaustive] {name}: {total} arguments, largest distance {worst} ulp, {differing} differ", flush=True)
+
+
+@pytest.mark.parametrize("exponent", [2.0, 0.5, 2.5, -1.0, 3.0, -0.5, 1.0 / 3.0])
+def test_powf_all_bases(hip, exponent):
+    """powf(x, exponent) for every f32 base (negative bases, zeros, subnormals, infinities and NaN included)"""
+    total = 0
+    with np.errstate(all="ignore"):
+        for start in range(0, 1 << 32, CHUNK):
+            x = np.arange(start, start + CHUNK, dtype=np.uint64).astype(np.uint32).view(np.float32)
+            got = hip.Matrix.from_numpy(x).powf_array(exponent).to_numpy()
+            exp = oracle_chunk(None, x, exponent)
+            nan = np.isnan(exp)
+            assert np.array_equal(np.isnan(got), nan), f"powf {exponent}: NaN positions differ in chunk {start:#x}"
+            ok = ~nan
+            bad = got.view(np.uint32)[ok] != exp.view(np.uint32)[ok]
+            if bad.any():
+                i = np.flatnonzero(ok)[np.flatnonzero(bad)[0]]
+                raise AssertionError(f"powf {exponent}: {int(bad.sum())} differ in chunk {start:#x}, first x = {x[i]!r}: "
+                                     f"got {got[i]!r}, libm {exp[i]!r}")
+            total += int(ok.sum())
+            if start % (1 << 30) == 0:
+                print(f"[exhaustive] powf {exponent}: {start >> 26} of 64 chunks", flush=True)
+    print(f"[exhaustive] powf(x, {exponent}): {total} bases, 0 differ", flush=True)
