@@ -99,3 +99,31 @@ def test_powf_all_bases(hip, exponent):
             if start % (1 << 30) == 0:
                 print(f"[exhaustive] powf {exponent}: {start >> 26} of 64 chunks", flush=True)
     print(f"[exhaustive] powf(x, {exponent}): {total} bases, 0 differ", flush=True)
+
+
+@pytest.mark.parametrize("name,fn", [("tanh", zo.TANH), ("sigmoid", None), ("exp", zo.EXP), ("sinh", zo.SINH),
+                                     ("cosh", zo.COSH)])
+def test_f64_every_fourth_high_word(hip, name, fn):
+    """f64 cannot be exhausted: every 4th value of the high word (sign, exponent, 20 mantissa bits) with a
+    pseudo-random low word, 2^30 arguments per function, must give the host libm's bits"""
+    total = 0
+    n = 1 << 25
+    with np.errstate(all="ignore"):
+        for c in range(32):
+            hi = (np.arange(c * n, (c + 1) * n, dtype=np.uint64) * 4 + (c & 3)) & 0xffffffff
+            lo = (hi * np.uint64(0x9E3779B97F4A7C15) >> np.uint64(29)) & np.uint64(0xffffffff)
+            x = ((hi << np.uint64(32)) | lo).view(np.float64)
+            got = getattr(hip.Matrix.from_numpy(x), name)().to_numpy()
+            exp = oracle_chunk(fn, x)
+            nan = np.isnan(exp)
+            assert np.array_equal(np.isnan(got), nan), f"{name} f64: NaN positions differ in chunk {c}"
+            ok = ~nan
+            bad = got.view(np.uint64)[ok] != exp.view(np.uint64)[ok]
+            if bad.any():
+                i = np.flatnonzero(ok)[np.flatnonzero(bad)[0]]
+                raise AssertionError(f"{name} f64: {int(bad.sum())} differ in chunk {c}, first x = {x[i]!r} "
+                                     f"({x.view(np.uint64)[i]:#018x}): got {got[i]!r}, libm {exp[i]!r}")
+            total += int(ok.sum())
+            if c % 8 == 0:
+                print(f"[exhaustive] {name} f64: {c} of 32 chunks", flush=True)
+    print(f"[exhaustive] {name} f64: {total} arguments, 0 differ", flush=True)
