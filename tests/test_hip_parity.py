@@ -496,6 +496,106 @@ def test_one_operand_periodic(hip, dt):
         assert_bits(X2.to_numpy(), exp, f"add_assign {shape} {yshape}")
 
 
+def random_view(r, shape, dt):
+    """a numpy view of the given shape over a larger base: random storage order (a permutation of the
+    dims), a random step (1 or 2) and offset per dim; small integer values, so sums and products are exact"""
+    nd = len(shape)
+    perm = [int(i) for i in r.permutation(nd)] if nd else []
+    step = [int(v) for v in r.integers(1, 3, size=nd)]
+    off = [int(v) for v in r.integers(0, 2, size=nd)]
+    full = [shape[d] * step[d] + off[d] + int(r.integers(0, 2)) for d in range(nd)]
+    base = np.asarray(r.integers(-4, 5, size=[full[d] for d in perm])).astype(dt)
+    if nd == 0:
+        return base.reshape(())
+    inv = [perm.index(d) for d in range(nd)]
+    v = base.transpose(inv)
+    return v[tuple(slice(off[d], off[d] + shape[d] * step[d], step[d]) for d in range(nd))]
+
+
+def random_shape(r):
+    nd = int(r.integers(0, 5))
+    big = int(r.integers(0, nd)) if nd and r.random() < 0.5 else -1
+    return tuple(int(r.integers(60, 140)) if d == big else int(r.integers(1, 8)) for d in range(nd))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_views_fuzz(hip, seed):
+    """seeded random shapes (0-4 dims, one of them sometimes 60-140 long), random strided / permuted
+    views for every operand and destination, random broadcast patterns: binary operators out of place
+    and in place, exp, copy_from, sum / max / arg-max along a random axis.  Bit-exact against the
+    oracle (integer-valued data make the sums exact); where the oracle refuses a combination, the
+    library must refuse it too."""
+    r = rng(1000 + seed)
+    ops = (("add", zo.ADD), ("sub", zo.SUB), ("mul", zo.MUL), ("div", zo.DIV))
+    for case in range(80):
+        dt = np.float32 if r.random() < 0.7 else np.float64
+        shape = random_shape(r)
+        nd = len(shape)
+        # the other operand: same rank with some dims 1, or fewer (trailing) dims, sometimes with a 1
+        if nd and r.random() < 0.5:
+            oshape = tuple(1 if r.random() < 0.4 else s for s in shape)
+        else:
+            k = int(r.integers(0, nd + 1))
+            oshape = tuple(shape[nd - k:])
+            if k and r.random() < 0.2:
+                oshape = tuple(1 if i == int(r.integers(0, k)) else s_ for i, s_ in enumerate(oshape))
+        a, b = random_view(r, shape, dt), random_view(r, oshape, dt)
+        A, B = dev_view(hip, root_of(a), a), dev_view(hip, root_of(b), b)
+        name, op = ops[int(r.integers(0, 4))]
+        swap = r.random() < 0.3
+        lhs, rhs, L, R = (b, a, B, A) if swap else (a, b, A, B)
+        what = f"seed {seed} case {case}: {name} {lhs.shape}{lhs.strides} {rhs.shape}{rhs.strides} {np.dtype(dt).name}"
+        print(what, flush=True)
+        dst = random_view(r, shape, dt)
+        D = dev_view(hip, root_of(dst), dst)
+        with np.errstate(all="ignore"):
+            try:
+                zo.binary_array(op, dst, lhs, rhs)
+            except zo.OracleError:
+                with pytest.raises(hip.ZenuHipError):
+                    getattr(D, f"{name}_array")(L, R)
+            else:
+                getattr(D, f"{name}_array")(L, R)
+                got, exp = D.to_numpy(), np.array(dst, order="C")
+                nan = np.isnan(exp)
+                assert np.array_equal(np.isnan(got), nan), what
+                assert_bits(got[~nan], exp[~nan], what)
+            # in place: a op= b
+            a2 = a.copy()
+            A2 = hip.Matrix.from_numpy(a2)
+            try:
+                zo.binary_assign(op, a2, b)
+            except zo.OracleError:
+                with pytest.raises(hip.ZenuHipError):
+                    getattr(A2, f"{name}_assign")(B)
+            else:
+                getattr(A2, f"{name}_assign")(B)
+                got = A2.to_numpy()
+                nan = np.isnan(a2)
+                assert np.array_equal(np.isnan(got), nan), what + " (assign)"
+                assert_bits(got[~nan], a2[~nan], what + " (assign)")
+        # exp and copy between two views
+        dst2 = random_view(r, shape, dt)
+        D2 = dev_view(hip, root_of(dst2), dst2)
+        D2.exp_array(A)
+        zo.unary(zo.EXP, dst2, a)
+        assert_bits(D2.to_numpy(), np.array(dst2, order="C"), what + " (exp)")
+        D2.copy_from(A)
+        zo.copy_from(dst2, a)
+        assert_bits(D2.to_numpy(), np.array(dst2, order="C"), what + " (copy)")
+        # reductions along a random axis of the view
+        if nd:
+            axis = int(r.integers(0, nd))
+            assert_bits(A.sum(axis).to_numpy(), zo.sum_axis(a, axis), what + f" (sum axis {axis})")
+            assert_bits(A.max_axis(axis).to_numpy(), zo.max_axis(a, axis), what + f" (max axis {axis})")
+            assert A.max_axis_idx_ravel(axis) == [int(i) for i in zo.max_axis_idx_ravel(a, axis)], what + " (arg-max)"
+            total = hip.Matrix.zeros((), dt)
+            exp_total = np.zeros((), dtype=dt)
+            zo.sum_to(a, exp_total)
+            hip.sum_to(A, total)
+            assert_bits(total.to_numpy(), exp_total, what + " (sum_to scalar)")
+
+
 def test_copy_transpose_large(hip):
     r = rng(12)
     a = r.standard_normal((1000, 777)).astype(np.float32)
