@@ -583,6 +583,37 @@ def test_random_views_fuzz(hip, seed):
         D2.copy_from(A)
         zo.copy_from(dst2, a)
         assert_bits(D2.to_numpy(), np.array(dst2, order="C"), what + " (copy)")
+        # scalar operand, relu with a slope, clip, sigmoid: view to view
+        sc = float(r.integers(-3, 4)) + 0.5
+        getattr(D2, f"{name}_scalar")(A, sc)
+        zo.binary_scalar(op, dst2, a, sc)
+        assert_bits(D2.to_numpy(), np.array(dst2, order="C"), what + " (scalar)")
+        D2.relu(A, 0.25)
+        zo.relu(dst2, a, 0.25)
+        assert_bits(D2.to_numpy(), np.array(dst2, order="C"), what + " (relu)")
+        D2.relu_backward_mask(A, 0.25)
+        zo.relu_backward_mask(dst2, a, 0.25)
+        assert_bits(D2.to_numpy(), np.array(dst2, order="C"), what + " (relu mask)")
+        exp_c = np.empty(shape, dtype=dt)
+        try:
+            zo.clip(exp_c, a, -1.5, 2.0)
+        except zo.OracleError:                            # 0-d: unimplemented!() in clip.rs
+            with pytest.raises(hip.ZenuHipError):
+                A.clip(-1.5, 2.0)
+        else:
+            assert_bits(A.clip(-1.5, 2.0).to_numpy(), exp_c, what + " (clip)")
+        zo.sigmoid(exp_c, a)
+        assert_bits(A.sigmoid().to_numpy(), exp_c, what + " (sigmoid)")
+        # whole-view reductions: |x| summed (integers: exact), first maximum
+        # asum.rs:49-68 recurses over the leading axis of a view that is not dense down to single
+        # elements, which it adds as they are (no abs); the library follows that.  A view whose SORTED
+        # strides are dense goes to BLAS with the last dim's stride, which for a permuted view reads
+        # other memory: there the oracle is not asked (the library sums |x| over the view's elements).
+        if all(a.strides[-1] <= st for st in a.strides):
+            assert A.asum() == zo.asum(a), what + " (asum)"
+        if nd:
+            assert tuple(A.max_idx()) == tuple(int(i) for i in zo.max_idx(a)), what + " (max_idx)"
+            assert A.max_item() == zo.max_item(a), what + " (max_item)"
         # reductions along a random axis of the view
         if nd:
             axis = int(r.integers(0, nd))

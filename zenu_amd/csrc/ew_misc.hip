@@ -89,6 +89,7 @@ int zenu_hip_clip(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *other
     if (!rc) rc = ensure_init();
     if (rc) return rc;
     if (!same_shape(*to, *other)) return ZENU_ERR_SHAPE;
+    if (to->ndim == 0) return ZENU_ERR_RANK;   // clip.rs:213-214: a 0-d input is unimplemented!() in the reference
     if (dtype == ZENU_F32) { ClipF<float> f; f.lo = (float)min; f.hi = (float)max; return run1<float>(*to, *other, f, as_stream(stream)); }
     if (dtype == ZENU_F64) { ClipF<double> f; f.lo = min; f.hi = max; return run1<double>(*to, *other, f, as_stream(stream)); }
     return ZENU_ERR_ARG;
@@ -101,6 +102,7 @@ int zenu_hip_clip_backward_mask(int dtype, const zenu_tensor_t *mask, const zenu
     if (!rc) rc = ensure_init();
     if (rc) return rc;
     if (!same_shape(*mask, *other)) return ZENU_ERR_SHAPE;
+    if (mask->ndim == 0) return ZENU_ERR_RANK;   // clip.rs:251-252, as above
     if (dtype == ZENU_F32) { ClipMaskF<float> f; f.lo = (float)min; f.hi = (float)max; return run1<float>(*mask, *other, f, as_stream(stream)); }
     if (dtype == ZENU_F64) { ClipMaskF<double> f; f.lo = min; f.hi = max; return run1<double>(*mask, *other, f, as_stream(stream)); }
     return ZENU_ERR_ARG;
