@@ -518,7 +518,7 @@ def random_shape(r):
     return tuple(int(r.integers(60, 140)) if d == big else int(r.integers(1, 8)) for d in range(nd))
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(int(os.environ.get("ZENU_FUZZ_SEEDS", "12"))))   # more seeds on request
 def test_random_views_fuzz(hip, seed):
     """seeded random shapes (0-4 dims, one of them sometimes 60-140 long), random strided / permuted
     views for every operand and destination, random broadcast patterns: binary operators out of place
