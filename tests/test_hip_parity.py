@@ -853,6 +853,53 @@ def test_c3_adamw(hip, n, dt):
         assert_bits(G.to_numpy(), g, "g untouched")
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_optimizer_fuzz(hip, seed):
+    """seeded random sizes (1 .. 70 000, mostly not multiples of the vector width), pointers 0-3 elements
+    into their buffers (unaligned), random hyper-parameters and step numbers, Adam / AdamW (as weight
+    or as bias) / SGD in f32 and f64: bit-exact against the oracle's operator-by-operator updates, and
+    nothing outside [offset, offset + n) changes"""
+    from zenu_amd import _lib
+    from zenu_amd._lib import check
+    r = rng(500 + seed)
+    l = hip.lib()
+    for case in range(25):
+        dt = np.float32 if r.random() < 0.6 else np.float64
+        code = _lib.F32 if dt == np.float32 else _lib.F64
+        f = np.dtype(dt).type
+        n = int(r.integers(1, 70000)) if r.random() < 0.7 else int(r.integers(1, 40))
+        pad = 8
+        offs = [int(v) for v in r.integers(0, 4, size=4)]
+        bufs = [(r.standard_normal(n + pad) * sc).astype(dt) for sc in (0.02, 1e-3, 1e-4, 1e-6)]
+        bufs[3] = np.abs(bufs[3])
+        dev = [hip.Matrix.from_numpy(b) for b in bufs]
+        isz = np.dtype(dt).itemsize
+        ptr = [d.as_ptr() + o * isz for d, o in zip(dev, offs)]
+        seg = [np.ascontiguousarray(b[o:o + n]) for b, o in zip(bufs, offs)]
+        lr, b1, b2 = f(10.0 ** r.uniform(-4, -1)), f(r.uniform(0.5, 0.99)), f(r.uniform(0.9, 0.9999))
+        eps, wd, step = f(10.0 ** r.uniform(-10, -6)), f(r.uniform(0, 0.1)), int(r.integers(1, 2000))
+        kind = int(r.integers(0, 4))
+        what = f"seed {seed} case {case}: kind {kind} n {n} offs {offs} {np.dtype(dt).name} step {step}"
+        print(what, flush=True)
+        pe, ge, me, ve = (x.copy() for x in seg)
+        if kind == 0:
+            zo.adam_update(pe, ge, me, ve, lr, b1, b2, eps, f(step))
+            check(l.zenu_hip_adam_step(code, ptr[0], ptr[1], ptr[2], ptr[3], n, float(lr), float(b1), float(b2), float(eps),
+                                       float(step), None), "adam")
+        elif kind in (1, 2):
+            decay = kind == 1
+            zo.adamw_update(pe, ge, me, ve, lr, b1, b2, eps, wd, decay, f(step))
+            check(l.zenu_hip_adamw_step(code, ptr[0], ptr[1], ptr[2], ptr[3], n, float(lr), float(b1), float(b2), float(eps),
+                                        float(wd), 1 if decay else 0, float(step), None), "adamw")
+        else:
+            zo.sgd_update(pe, ge, lr)
+            check(l.zenu_hip_sgd_step(code, ptr[0], ptr[1], n, float(lr), None), "sgd")
+        for b, o, e, d, nm in zip(bufs, offs, (pe, ge, me, ve), dev, "pgmv"):
+            exp = b.copy()
+            exp[o:o + n] = e
+            assert_bits(d.to_numpy(), exp, what + f" ({nm})")
+
+
 def test_sgd(hip):
     from zenu_amd import _lib
     from zenu_amd._lib import check
