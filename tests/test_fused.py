@@ -87,6 +87,49 @@ def test_softmax_forward_backward(hip, dtype, shape, axis):
         assert np.max(np.abs(g.astype(np.float64) - gref)) <= (1e-5 if dtype == np.float32 else 1e-12) * scale
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_fused_fuzz(hip, seed):
+    """seeded random shapes (1-4 dims, the softmax axis 1 .. 1500 long), random axis, f32 / f64:
+    softmax and its backward against the op-by-op chains with the bars of test_softmax_forward_backward,
+    bias add + ReLU (bit-exact), and for 2-d shapes the cross-entropy loss and its backward"""
+    r = np.random.default_rng(900 + seed)
+    for case in range(25):
+        dtype = np.float32 if r.random() < 0.6 else np.float64
+        nd = int(r.integers(1, 5))
+        axis = int(r.integers(0, nd))
+        shape = tuple(int(r.integers(1, 1500)) if d == axis and r.random() < 0.6 else int(r.integers(1, 9)) for d in range(nd))
+        print(f"[fuzz] seed {seed} case {case}: {shape} axis {axis} {np.dtype(dtype).name}", flush=True)
+        x = (r.standard_normal(shape) * 3).astype(dtype)
+        gy = r.standard_normal(shape).astype(dtype)
+        R, inner = shape[axis], int(np.prod(shape[axis + 1:]))
+        in_order = R <= 64 or inner > 1
+        tol = (2e-6 if dtype == np.float32 else 1e-14) if in_order else (1e-5 if dtype == np.float32 else 1e-12)
+        ref = CpuMatrix.zeros(shape, dtype)
+        ref.softmax_assign(CpuMatrix.from_numpy(x), axis)
+        out = hip.Matrix.zeros(shape, dtype)
+        out.softmax_assign(hip.Matrix.from_numpy(x), axis)
+        y = out.to_numpy()
+        assert rel_err(y, ref.a) <= tol
+        if in_order:
+            assert bits_equal(y, ref.a)
+        gref = cpu_matrix.softmax_backward(CpuMatrix.from_numpy(y), CpuMatrix.from_numpy(gy), axis).a
+        g = hip.softmax_backward(hip.Matrix.from_numpy(y), hip.Matrix.from_numpy(gy), axis).to_numpy()
+        if in_order:
+            assert bits_equal(g, gref)
+        else:
+            assert np.max(np.abs(g.astype(np.float64) - gref)) <= (1e-5 if dtype == np.float32 else 1e-12) * max(np.max(np.abs(gref)), 1e-30)
+        if nd >= 2:
+            # bias over the last dim, added and rectified: arithmetic only, bit-exact
+            bias = r.standard_normal(shape[-1]).astype(dtype)
+            alpha = float(r.choice([0.0, 0.2]))
+            cref = CpuMatrix.zeros(shape, dtype)
+            cpre = CpuMatrix.zeros(shape, dtype)
+            cref.bias_add_relu(CpuMatrix.from_numpy(x), CpuMatrix.from_numpy(bias), alpha, cpre)
+            act, pre = hip.Matrix.zeros(shape, dtype), hip.Matrix.zeros(shape, dtype)
+            act.bias_add_relu(hip.Matrix.from_numpy(x), hip.Matrix.from_numpy(bias), alpha, pre)
+            assert bits_equal(act.to_numpy(), cref.a) and bits_equal(pre.to_numpy(), cpre.a)
+
+
 def test_softmax_strided_views(hip):
     """transposed source and sliced destination go through contiguous staging"""
     r = np.random.default_rng(5)
