@@ -900,6 +900,59 @@ def test_optimizer_fuzz(hip, seed):
             assert_bits(d.to_numpy(), exp, what + f" ({nm})")
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_error_parity_fuzz(hip, seed):
+    """random pairs of small shapes, most of them NOT compatible: for copy_from, broadcast, relu, exp,
+    powf, sum_to and the in-place operators the library must refuse exactly what the oracle (the
+    reference's checks and recursions, restated) refuses, and agree bit for bit on what it accepts"""
+    from cpu_matrix import CpuMatrix
+    import cpu_matrix
+    r = rng(2000 + seed)
+
+    def shp():
+        nd = int(r.integers(0, 4))
+        return tuple(int(r.choice([1, 2, 3])) for _ in range(nd))
+
+    def both(what, fn_cpu, fn_hip, result_cpu, result_hip):
+        try:
+            fn_cpu()
+            ok = True
+        except (zo.OracleError, AssertionError):
+            ok = False
+        if not ok:
+            with pytest.raises(hip.ZenuHipError):
+                fn_hip()
+            return 0
+        fn_hip()
+        assert_bits(result_hip(), result_cpu(), what)
+        return 1
+
+    accepted = 0
+    for case in range(150):
+        sa, sb = shp(), shp()
+        if r.random() < 0.3:
+            sb = sa[len(sa) - int(r.integers(0, len(sa) + 1)):]       # a trailing part: often legal
+        a = r.integers(-4, 5, size=sa).astype(np.float32).reshape(sa)
+        b = r.integers(1, 5, size=sb).astype(np.float32).reshape(sb)
+        what = f"seed {seed} case {case}: {sa} <- {sb}"
+        print(what, flush=True)
+        for name in ("copy_from", "broadcast", "add_assign", "div_assign"):
+            ca, cb = CpuMatrix.from_numpy(a), CpuMatrix.from_numpy(b)
+            ha, hb = hip.Matrix.from_numpy(a), hip.Matrix.from_numpy(b)
+            accepted += both(f"{what} {name}", lambda: getattr(ca, name)(cb), lambda: getattr(ha, name)(hb),
+                             lambda: ca.a, lambda: ha.to_numpy())
+        for name, args in (("relu", (0.1,)), ("exp_array", ()), ("powf", (2.0,))):
+            ca, cb = CpuMatrix.from_numpy(a), CpuMatrix.from_numpy(b)
+            ha, hb = hip.Matrix.from_numpy(a), hip.Matrix.from_numpy(b)
+            accepted += both(f"{what} {name}", lambda: getattr(ca, name)(cb, *args), lambda: getattr(ha, name)(hb, *args),
+                             lambda: ca.a, lambda: ha.to_numpy())
+        ca, cb = CpuMatrix.from_numpy(a), CpuMatrix.from_numpy(b)
+        ha, hb = hip.Matrix.from_numpy(a), hip.Matrix.from_numpy(b)
+        accepted += both(f"{what} sum_to", lambda: cpu_matrix.sum_to(ca, cb), lambda: hip.sum_to(ha, hb),
+                         lambda: cb.a, lambda: hb.to_numpy())
+    assert accepted > 100    # the generator does produce legal combinations too
+
+
 def test_sgd(hip):
     from zenu_amd import _lib
     from zenu_amd._lib import check
