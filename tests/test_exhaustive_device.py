@@ -105,13 +105,16 @@ def test_powf_all_bases(hip, exponent):
                                      ("cosh", zo.COSH)])
 def test_f64_every_fourth_high_word(hip, name, fn):
     """f64 cannot be exhausted: every 4th value of the high word (sign, exponent, 20 mantissa bits) with a
-    pseudo-random low word, 2^30 arguments per function, must give the host libm's bits"""
+    pseudo-random low word, 2^30 arguments per function (ZENU_EXHAUSTIVE_F64_LOG2=33: eight times as many,
+    with other low words), must give the host libm's bits"""
     total = 0
     n = 1 << 25
+    passes = 1 << max(0, int(os.environ.get("ZENU_EXHAUSTIVE_F64_LOG2", "30")) - 30)   # more low words on request
     with np.errstate(all="ignore"):
-        for c in range(32):
-            hi = (np.arange(c * n, (c + 1) * n, dtype=np.uint64) * 4 + (c & 3)) & 0xffffffff
-            lo = (hi * np.uint64(0x9E3779B97F4A7C15) >> np.uint64(29)) & np.uint64(0xffffffff)
+        for c in range(32 * passes):
+            rep, c = divmod(c, 32)
+            hi = (np.arange(c * n, (c + 1) * n, dtype=np.uint64) * 4 + ((c + rep) & 3)) & 0xffffffff
+            lo = ((hi + np.uint64(rep)) * np.uint64(0x9E3779B97F4A7C15 + 2 * rep) >> np.uint64(29)) & np.uint64(0xffffffff)
             x = ((hi << np.uint64(32)) | lo).view(np.float64)
             got = getattr(hip.Matrix.from_numpy(x), name)().to_numpy()
             exp = oracle_chunk(fn, x)
@@ -125,5 +128,5 @@ def test_f64_every_fourth_high_word(hip, name, fn):
                                      f"({x.view(np.uint64)[i]:#018x}): got {got[i]!r}, libm {exp[i]!r}")
             total += int(ok.sum())
             if c % 8 == 0:
-                print(f"[exhaustive] {name} f64: {c} of 32 chunks", flush=True)
+                print(f"[exhaustive] {name} f64: pass {rep}, {c} of 32 chunks", flush=True)
     print(f"[exhaustive] {name} f64: {total} arguments, 0 differ", flush=True)
