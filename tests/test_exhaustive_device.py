@@ -130,3 +130,44 @@ def test_f64_every_fourth_high_word(hip, name, fn):
             if c % 8 == 0:
                 print(f"[exhaustive] {name} f64: pass {rep}, {c} of 32 chunks", flush=True)
     print(f"[exhaustive] {name} f64: {total} arguments, 0 differ", flush=True)
+
+
+def test_beyond_2_31_and_2_32_elements(hip):
+    """index arithmetic past 32 bits: tensors of 2^31 + 4099 and of 65537 x 65540 (> 2^32) f32 elements, built
+    and checked on the device (only small slices come back): fills, scalar and row-broadcast operators,
+    out-of-place multiply, first-maximum search, sums along both axes and over everything"""
+    M = hip.Matrix
+    n = (1 << 31) + 4099
+    A = M.zeros((n,))
+    A.add_scalar_assign(1.0)
+    A.slice(slice(n - 1, n)).copy_from(M.from_numpy(np.array([5.0], dtype=np.float32)))
+    A.slice(slice(n - 3000, n - 2999)).copy_from(M.from_numpy(np.array([5.0], dtype=np.float32)))
+    with pytest.raises(hip.ZenuHipError):                 # positions are tracked in 32 bits: a reduced length of
+        A.max_idx()                                       # 2^31 - 1 or more is refused, never answered wrongly
+    V = M(A.buf, A.offset + 4099, (2, 1 << 30), (1 << 30, 1), A.dtype)   # the last 2^31 elements as two rows
+    assert V.max_axis_idx_ravel(1) == [0, (1 << 30) - 3000]   # the first of the two maxima of the second row
+    B = A * 2.0
+    head, tail = B.slice(slice(0, 8)).to_numpy(), B.slice(slice(n - 8, n)).to_numpy()
+    assert np.array_equal(head, np.full(8, 2.0, np.float32))
+    assert np.array_equal(tail, np.array([2.0] * 7 + [10.0], dtype=np.float32))
+    total = float(A.sum(0).to_numpy())
+    assert abs(total - (n + 8.0)) <= 1e-5 * n
+    print("[exhaustive] 2^31 + 4099 elements: ok", flush=True)
+    del A, B
+
+    rows, cols = 65537, 65540                             # 4 295 295 980 elements, 16 GiB
+    X = M.zeros((rows, cols))
+    X.add_scalar_assign(1.0)
+    row = M.from_numpy(np.arange(cols, dtype=np.float32).reshape(1, cols) % 7)
+    X.add_assign(row)                                     # too long for the 32-bit flat kernel: the row kernel
+    exp_row = (np.arange(cols) % 7 + 1).astype(np.float32)
+    for r0 in (0, 1, rows // 2, rows - 1):
+        assert np.array_equal(X.slice(slice(r0, r0 + 1)).to_numpy()[0], exp_row), r0
+    s0 = X.sum(0).to_numpy()                              # over the rows: each column sums to rows * value
+    assert np.allclose(s0, exp_row.astype(np.float64) * rows, rtol=1e-5)
+    s1 = X.sum(1).to_numpy()
+    assert np.allclose(s1, float(exp_row.astype(np.float64).sum()), rtol=1e-5)
+    X.slice(slice(rows - 1, rows), slice(cols - 1, cols)).copy_from(M.from_numpy(np.array([[100.0]], dtype=np.float32)))
+    idx = X.max_axis_idx_ravel(1)                         # per row; the last row's maximum sits past 2^32 elements
+    assert idx[-1] == cols - 1 and idx[0] == 6
+    print("[exhaustive] 65537 x 65540 elements: ok", flush=True)
