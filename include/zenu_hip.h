@@ -100,6 +100,23 @@ int zenu_hip_device_synchronize(void);
  * Honours ZENU_USE_MEMPOOL=0 (zenu-matrix/src/lib.rs:36): every call goes to hipMalloc/hipFree. */
 int zenu_hip_malloc(void **ptr_dev, size_t bytes, zenu_stream_t stream);
 int zenu_hip_free(void *ptr_dev, zenu_stream_t stream);
+/* Stream capture (HIP graphs).  Kernels recorded into a graph keep the addresses they were
+ * recorded with and use them again on every replay.  Every block that zenu_hip_malloc hands out
+ * while `stream` is capturing -- the library's own scratch (reduction partials, staging copies,
+ * the temporaries of zenu_hip_sum_to) as well as the caller's tensors -- is therefore kept out of
+ * ordinary requests when it is freed, during the capture or later: only later captures on the
+ * same stream may reuse it (graphs recorded on one stream share scratch and must not be
+ * replayed concurrently with each other).  After destroying the graphs, call
+ * zenu_hip_release_captured(stream) to return those blocks to the pool; zenu_hip_stream_destroy
+ * does the same.  A request the pool cannot serve from its cache during a capture goes to
+ * hipMalloc, which only the relaxed capture mode tolerates: run the sequence once eagerly on the
+ * stream first.  A split reduction on a stream that the library did not create needs its counter
+ * ring before the capture starts (any eager reduction on that stream creates it); while
+ * capturing, such a call returns ZENU_ERR_UNSUPPORTED instead of blocking.  A captured graph
+ * owns a fixed range of its capture stream's counter ring: replay it on that stream, or at
+ * least never concurrently with reductions running on that stream.
+ * No counterpart in the reference (it never captures). */
+int zenu_hip_release_captured(zenu_stream_t stream);
 /* Return all cached (free) blocks to the driver. */
 int zenu_hip_mempool_trim(void);
 typedef struct zenu_mempool_stats {

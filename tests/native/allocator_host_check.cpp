@@ -155,6 +155,46 @@ int main()
         CHECK(a.free(nullptr, S1) == 0, "null is a no-op");
         printf("ok not_owned\n");
     }
+    {   // blocks a capturing stream took from the pool stay with that stream's graphs
+        FakeBackend be; CachingAllocator a(&be);
+        void *w, *t1, *t2, *e, *out;
+        a.malloc(&w, 64u << 20, S1); a.free(w, S1);                  // rehearsal: the pool holds the block
+        CHECK(a.malloc(&t1, 64u << 20, S1, true) == 0 && t1 == w, "capture takes the cached block");
+        CHECK(a.free(t1, S1) == 0, "free during capture");
+        CHECK(a.bytes_captured() == (64u << 20), "held back for the graph");
+        CHECK(a.malloc(&t2, 64u << 20, S1, true) == 0 && t2 == w, "reused inside the capture (recorded order)");
+        a.free(t2, S1);
+        CHECK(a.malloc(&out, 4096, S1, true) == 0, "an output allocated during the capture");
+        // capture over: an ordinary request must not get the block the recorded kernels write
+        CHECK(a.malloc(&e, 64u << 20, S1) == 0 && e != w, "eager request gets other memory");
+        CHECK(a.stats().n_driver_allocs == 3, "a new segment for the eager tensor");
+        void *e2; CHECK(a.malloc(&e2, 64u << 20, S2) == 0 && e2 != w, "other streams neither");
+        a.free(e2, S2);
+        a.free(out, S2);                                             // freed eagerly, on another stream: still the graph's
+        void *o2; CHECK(a.malloc(&o2, 4096, S1) == 0 && o2 != out, "captured output not handed out eagerly");
+        a.free(o2, S1);
+        a.trim();
+        CHECK(a.bytes_captured() >= (64u << 20), "trim leaves the graph's blocks alone");
+        AllocStats st = a.stats();
+        CHECK(st.bytes_reserved == st.bytes_in_use + st.bytes_cached, "accounting with captured blocks");
+        a.release_captured(S1);                                      // graphs destroyed
+        CHECK(a.bytes_captured() == 0, "released");
+        void *r; CHECK(a.malloc(&r, 64u << 20, S1) == 0 && r == w, "ordinary again after release");
+        a.free(r, S1); a.free(e, S1);
+        a.trim();
+        CHECK(be.live.empty(), "everything returns to the driver");
+        // a live captured block at release time becomes ordinary when it is freed later
+        void *l; a.malloc(&l, 8192, S1, true);
+        a.release_captured(S1);
+        a.free(l, S1);
+        CHECK(a.bytes_captured() == 0, "live block released with its stream");
+        // retiring the stream releases too
+        void *m; a.malloc(&m, 8192, S2, true); a.free(m, S2);
+        CHECK(a.bytes_captured() > 0, "held");
+        a.retire_stream(S2);
+        CHECK(a.bytes_captured() == 0, "retire releases");
+        printf("ok capture_blocks\n");
+    }
     {   // randomized stress against a shadow model: no overlap, accounting consistent
         FakeBackend be; CachingAllocator a(&be);
         struct L { char *p; size_t n; void *s; };
@@ -165,7 +205,7 @@ int main()
             if (live.empty() || rnd() % 3) {
                 size_t n = (rnd() % 4 == 0) ? (size_t)(rnd() % (32u << 20)) + 1 : (size_t)(rnd() % 70000) + 1;
                 void *s = (rnd() & 1) ? S1 : S2, *p;
-                CHECK(a.malloc(&p, n, s) == 0, "stress alloc");
+                CHECK(a.malloc(&p, n, s, rnd() % 5 == 0) == 0, "stress alloc");
                 for (auto &l : live) CHECK((char *)p + n <= l.p || l.p + l.n <= (char *)p, "no overlap");
                 live.push_back({(char *)p, n, s});
             } else {
@@ -173,11 +213,14 @@ int main()
                 CHECK(a.free(live[i].p, live[i].s) == 0, "stress free");
                 live[i] = live.back(); live.pop_back();
             }
+            if (it % 997 == 0) a.release_captured((rnd() & 1) ? S1 : S2);
+            if (it % 4001 == 0) a.trim();
             AllocStats st = a.stats();
             CHECK(st.bytes_reserved == st.bytes_in_use + st.bytes_cached, "reserved = in use + cached");
         }
         for (auto &l : live) a.free(l.p, l.s);
         CHECK(a.stats().bytes_in_use == 0, "all returned");
+        a.release_captured(S1); a.release_captured(S2);
         a.trim();
         CHECK(be.live.empty(), "trim frees everything when nothing is live");
         printf("ok stress\n");

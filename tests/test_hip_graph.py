@@ -3,10 +3,11 @@
 What a capturing caller relies on: no entry point synchronises or calls the driver's allocator
 when the caching pool can serve the request (rehearsal runs make every request a hit), zero fills
 are kernels (no memset nodes), the arrival counters of the split reductions are back at zero after
-every run, and scratch taken from the pool during the capture stays valid for replays on the same
-stream.  The graph is replayed several times with new inputs, eager work on the same stream and
-synchronisations in between, and every replay is compared bit for bit with the eager sequence on
-the same inputs.
+every run, and memory taken from the pool during the capture -- the library's scratch as well as
+tensors the sequence allocates and drops -- stays out of ordinary requests afterwards, so tensors
+allocated after the capture survive every replay.  The graph is replayed several times with new
+inputs, eager work on the same stream and synchronisations in between, and every replay is compared
+bit for bit with the eager sequence on the same inputs.
 """
 import ctypes as C
 
@@ -96,6 +97,17 @@ def test_library_calls_in_a_captured_graph(hip):
         assert rc == 0
         assert rt.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
         keep = dict(outs)                                        # the captured outputs' buffers
+        # tensors allocated AFTER the capture, of every size the sequence used for scratch and
+        # temporaries: the recorded kernels still write those addresses on each replay, so none of
+        # these may have been given one of them
+        sentinel_shapes = [(rows, cols), (rows, cols), (rows, cols), (cols,), (rows,), (), (512, cols), (64, cols),
+                           (8, cols), (2 * rows,), (4 * rows,), (130,), (rows * 4,), (cols * 16,), (1 << 20,), (1 << 18,)]
+        sentinels = []
+        for k, shp in enumerate(sentinel_shapes * 2):
+            v = np.full(shp, 1000.0 + k, dtype=np.float32)
+            sentinels.append((v, M.from_numpy(v)))
+        st0 = _lib.MempoolStats()
+        _lib.check(l.zenu_hip_mempool_stats(C.byref(st0)), "stats")
         for i, inp in enumerate(inputs):
             reset(inp)
             opt.step = 1                                         # frozen in the graph as a kernel argument
@@ -109,7 +121,19 @@ def test_library_calls_in_a_captured_graph(hip):
             z = x.exp().max_axis(1)
             del y, z
             hip.synchronize()
-        del keep
+            for v, S in sentinels:
+                assert np.array_equal(S.to_numpy(), v), ("a tensor allocated after the capture was overwritten by replay", i, v.shape)
+        del keep, sentinels
+        hip.synchronize()
+        rt.hipGraphExecDestroy(gexec)
+        rt.hipGraphDestroy(graph)
+        gexec, graph = C.c_void_p(), C.c_void_p()
+        _lib.check(l.zenu_hip_release_captured(stream), "release_captured")   # the graph is gone: blocks are ordinary again
+        big = [M.alloc((rows, cols)) for _ in range(8)]
+        st1 = _lib.MempoolStats()
+        _lib.check(l.zenu_hip_mempool_stats(C.byref(st1)), "stats")
+        assert st1.bytes_reserved == st1.bytes_in_use + st1.bytes_cached
+        del big
     finally:
         hip.synchronize()
         if gexec:

@@ -347,6 +347,145 @@ def test_unary_f64(hip):
     del X, W, W2
 
 
+# ---- the functions that come from the device math library: f32 / f64 tan, f64 sin ... atan, log, powf ---------------
+# Bar: <= 2 ulp against the oracle (which calls the host libm, as Rust's f32::tan / f64::sin ... do:
+# zenu-matrix/src/operation/basic_operations.rs:441-453; device side of the reference:
+# zenu-cuda-kernel-sys/kernel/array_scalar.cu:212-290, literal tables zenu-cuda/src/kernel/mod.rs:1015-1241).
+
+_TRIG_F64 = (("sin", zo.SIN), ("cos", zo.COS), ("tan", zo.TAN), ("asin", zo.ASIN), ("acos", zo.ACOS), ("atan", zo.ATAN))
+
+
+def _trig_special(dt):
+    """+-0, +-inf, NaN, subnormals, the smallest and largest normals, arguments next to multiples of
+    pi/2 (where tan has its poles and sin / cos their zeros) and large arguments (|x| > 2^20, up to the
+    top of the range: the multi-word reduction by pi/2)"""
+    dt = np.dtype(dt)
+    fi = np.finfo(dt)
+    k = np.array([1, 2, 3, 4, 5, 7, 10, 100, 1000, 12345, 1 << 20, (1 << 24) + 1], dtype=np.float64)
+    near = (k * (np.pi / 2)).astype(dt)
+    near = np.concatenate([near, np.nextafter(near, dt.type(np.inf)), np.nextafter(near, dt.type(-np.inf)), -near])
+    big = np.array([2.0 ** 20 + 0.5, 2.0 ** 21 + 1.25, 1e7, 3.3e7, 1e9, 1e15, 2.0 ** 60, 1e22, 1e30, 1e38], dtype=dt)
+    if dt == np.float64:
+        big = np.concatenate([big, np.array([1e100, 1e200, 1e300, fi.max])])
+    edge = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, fi.tiny, -fi.tiny, fi.smallest_subnormal,
+                     -fi.smallest_subnormal, fi.tiny / 4, fi.max, -fi.max, 1.0, -1.0, 0.5, -0.5,
+                     1 - fi.epsneg, -(1 - fi.epsneg), 1 + fi.eps, 0.99, -0.99, 1e-8, -1e-8, 1e-4, 0.7853981633974483,
+                     1.5707963267948966, 3.141592653589793, 6.283185307179586], dtype=dt)
+    return np.concatenate([edge, near, big, -big])
+
+
+def _check_device_libm(hip, name, fn, x, bar=2, what=""):
+    exp = np.empty_like(x)
+    with np.errstate(all="ignore"):
+        zo.unary(fn, exp, x)
+    got = getattr(hip.Matrix.from_numpy(x), name)().to_numpy()
+    assert np.array_equal(np.isnan(got), np.isnan(exp)), (name, what, "NaN positions")
+    ok = ~np.isnan(exp)
+    u = max_ulp(got[ok], exp[ok]) if ok.any() else 0
+    if u > bar:
+        d = np.abs(ordered(got[ok]) - ordered(exp[ok]))
+        i = int(np.argmax(d))
+        raise AssertionError(f"{name} {x.dtype} {what}: {u} ulp at x={x[ok].reshape(-1)[i]!r}: "
+                             f"got {got[ok].reshape(-1)[i]!r} exp {exp[ok].reshape(-1)[i]!r}")
+    # where the result is zero or infinite its sign is the host's
+    z = ok & ((exp == 0) | np.isinf(exp))
+    assert np.array_equal(np.signbit(got[z]), np.signbit(exp[z])), (name, what, "sign of 0 / inf")
+    return u
+
+
+def test_tan_f32_device_libm(hip, c1):
+    """f32 tan on the C1 tensor, on special values and on a strided view: <= 2 ulp"""
+    u = _check_device_libm(hip, "tan", zo.TAN, c1["a"], what="c1")
+    print(f"[c1] tan f32: max ulp vs libm = {u}", flush=True)
+    r = rng(31)
+    wide = np.concatenate([_trig_special(np.float32),
+                           (r.standard_normal(400000) * 10.0).astype(np.float32),
+                           (r.uniform(-1, 1, 400000) * 2.0 ** 22).astype(np.float32),
+                           (r.uniform(-1, 1, 200000) * 1e30).astype(np.float32),
+                           (r.uniform(-1, 1, 100000) * 1e-3).astype(np.float32)])
+    u = _check_device_libm(hip, "tan", zo.TAN, wide, what="wide")
+    print(f"tan f32 wide: max ulp vs libm = {u}", flush=True)
+    # every 1024th bit pattern (4 M arguments over the whole range)
+    bits = np.arange(0, 1 << 32, 1024, dtype=np.uint64).astype(np.uint32)
+    u = _check_device_libm(hip, "tan", zo.TAN, bits.view(np.float32), what="sweep")
+    print(f"tan f32 sweep: max ulp vs libm = {u}", flush=True)
+    # a strided view (transposed and column-sliced): same function through the other kernels
+    a = (r.standard_normal((300, 200)) * 3).astype(np.float32)
+    V = hip.Matrix.from_numpy(a).transpose().slice(slice(0, 200, 3), slice(1, 300, 2))
+    v = np.ascontiguousarray(a.T[0:200:3, 1:300:2])
+    exp = np.empty_like(v)
+    zo.unary(zo.TAN, exp, v)
+    got = V.tan().to_numpy()
+    assert got.shape == v.shape and max_ulp(got, exp) <= 2
+    got2 = hip.Matrix.alloc(v.shape)
+    got2.tan_array(V)
+    assert max_ulp(got2.to_numpy(), exp) <= 2
+
+
+@pytest.mark.parametrize("name,fn", _TRIG_F64, ids=[n for n, _ in _TRIG_F64])
+def test_trig_f64_device_libm(hip, c1, name, fn):
+    """f64 sin, cos, tan, asin, acos, atan: the C1 tensor in f64 ([4096,4096], seed 1; asin / acos on
+    values clipped to +-0.99), special values, wide ranges and a strided view: <= 2 ulp"""
+    x = c1["a"].astype(np.float64)
+    r = rng(32)
+    x += r.standard_normal(x.shape) * 2.0 ** -30          # low words that are not zero
+    inverse = name in ("asin", "acos")
+    if inverse:
+        x = np.clip(x, -0.99, 0.99)
+    u = _check_device_libm(hip, name, fn, x, what="c1")
+    print(f"[c1] {name} f64: max ulp vs libm = {u}", flush=True)
+    sp = _trig_special(np.float64)
+    if inverse:
+        wide = np.concatenate([sp, r.uniform(-1, 1, 600000), 1 - np.abs(r.standard_normal(200000)) * 1e-6,
+                               -1 + np.abs(r.standard_normal(200000)) * 1e-9, r.uniform(-1, 1, 100000) * 1e-9,
+                               r.uniform(0.49, 0.51, 100000), r.uniform(-1.01, 1.01, 1000)])
+    elif name == "atan":
+        wide = np.concatenate([sp, r.standard_normal(400000) * 10, r.uniform(-1, 1, 200000) * 1e-6,
+                               np.exp(r.uniform(-700, 700, 400000)) * r.choice([-1.0, 1.0], 400000),
+                               r.uniform(0.4, 2.5, 200000)])
+    else:
+        wide = np.concatenate([sp, r.standard_normal(400000) * 10, r.uniform(-1, 1, 400000) * 2.0 ** 22,
+                               r.uniform(-1, 1, 200000) * 1e15, r.uniform(-1, 1, 100000) * 1e-3,
+                               np.exp(r.uniform(0, 700, 300000)) * r.choice([-1.0, 1.0], 300000),
+                               (np.arange(1, 100001) * (np.pi / 2))])
+    u = _check_device_libm(hip, name, fn, wide, what="wide")
+    print(f"{name} f64 wide: max ulp vs libm = {u}", flush=True)
+    a = r.standard_normal((300, 200)) * (0.4 if inverse else 3)
+    if inverse:
+        a = np.clip(a, -1, 1)
+    V = hip.Matrix.from_numpy(a).transpose().slice(slice(0, 200, 3), slice(1, 300, 2))
+    v = np.ascontiguousarray(a.T[0:200:3, 1:300:2])
+    exp = np.empty_like(v)
+    zo.unary(fn, exp, v)
+    got = getattr(V, name)().to_numpy()
+    assert got.shape == v.shape and max_ulp(got, exp) <= 2
+
+
+def test_log_powf_f64_device_libm(hip, c1):
+    """f64 log and powf at C1 size and on wide ranges: <= 2 ulp"""
+    r = rng(33)
+    x = np.abs(c1["a"].astype(np.float64) + r.standard_normal(c1["a"].shape) * 2.0 ** -30) + 1e-12
+    u = _check_device_libm(hip, "log", zo.LOG, x, what="c1")
+    print(f"[c1] log f64: max ulp vs libm = {u}", flush=True)
+    fi = np.finfo(np.float64)
+    wide = np.concatenate([np.exp(r.uniform(-745, 709, 500000)), r.uniform(0.5, 2.0, 400000), 1 + r.standard_normal(200000) * 1e-9,
+                           np.array([0.0, -0.0, 1.0, np.inf, -1.0, np.nan, fi.tiny, fi.smallest_subnormal, fi.max,
+                                     fi.tiny / 1024, 1 - fi.epsneg, 1 + fi.eps])])
+    u = _check_device_libm(hip, "log", zo.LOG, wide, what="wide")
+    print(f"log f64 wide: max ulp vs libm = {u}", flush=True)
+    base = np.concatenate([np.abs(r.standard_normal(300000)) * 3 + 1e-3, np.exp(r.uniform(-300, 300, 100000)),
+                           -np.abs(r.standard_normal(50000)) * 3, np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan])])
+    B = hip.Matrix.from_numpy(base)
+    for y in (2.0, 0.5, 2.5, -1.0, 3.0, -0.5, 1.0 / 3.0, 0.0, 1.0, -2.0, 10.25, 1e-3, 55.0, -3.0):
+        exp = np.empty_like(base)
+        with np.errstate(all="ignore"):
+            zo.powf(exp, base, y)
+        got = B.powf_array(y).to_numpy()
+        assert np.array_equal(np.isnan(got), np.isnan(exp)), ("powf", y)
+        ok = ~np.isnan(exp)
+        assert max_ulp(got[ok], exp[ok]) <= 2, ("powf", y, max_ulp(got[ok], exp[ok]))
+
+
 def test_powf(hip):
     """powf (zenu-matrix/src/device/cpu/basic_operations.rs pow: `x.powf(scalar)` per element):
     f32 has the host libm's bits for every exponent class -- integer, half-integer, negative,
@@ -1263,5 +1402,54 @@ def test_split_reductions_on_two_streams(hip):
         hip.synchronize()
         hip.set_stream(old)
         _lib.check(l.zenu_hip_stream_synchronize(s2), "sync")
+    _lib.check(l.zenu_hip_stream_destroy(s1), "destroy")
+    _lib.check(l.zenu_hip_stream_destroy(s2), "destroy")
+
+
+def test_split_reduction_handoff_repeatable(hip):
+    """200 back-to-back split reductions (cross-workgroup hand-off: partials stored, arrival counter,
+    last arriver folds) alternating between two streams and between four different inputs that
+    reuse the same scratch blocks: a partial read before it has landed would be the previous
+    launch's, i.e. another input's.  Every result must equal the first result of its input bit for
+    bit; stops at the first mismatch."""
+    import ctypes as C
+    from zenu_amd import _lib
+    l = hip.lib()
+    r = rng(77)
+    xs = [r.standard_normal((2048, 2048)).astype(np.float32) * np.float32(1 + k) for k in range(4)]
+    Xs = [hip.Matrix.from_numpy(x) for x in xs]
+    hip.synchronize()
+    s1, s2 = C.c_void_p(), C.c_void_p()
+    _lib.check(l.zenu_hip_stream_create(C.byref(s1)), "stream")
+    _lib.check(l.zenu_hip_stream_create(C.byref(s2)), "stream")
+    old = hip.get_stream()
+    try:
+        first = {}
+        outs = []
+        for i in range(200):
+            hip.set_stream(s1 if i % 2 == 0 else s2)
+            k = (i // 2 + i) % 4
+            X = Xs[k]
+            outs.append((k, X.sum_all(), X.sum(0), X.max_axis(0), X.transpose().sum(0)))
+        for s in (s1, s2):
+            _lib.check(l.zenu_hip_stream_synchronize(s), "sync")
+        hip.set_stream(s1)
+        for i, (k, *res) in enumerate(outs):
+            got = [t.to_numpy().copy() for t in res]
+            if k not in first:
+                first[k] = got
+                x = xs[k]
+                assert_sum_close(got[0], np.float32(x.sum(dtype=np.float64)), x, None, "sum_all")
+                assert_bits(got[2], x.max(0), "max axis 0")
+                continue
+            for name, a, b in zip(("sum_all", "sum axis 0", "max axis 0", "sum axis 1 of the transposed view"), got, first[k]):
+                assert bits_equal(a, b), f"launch {i} (input {k}): {name} differs from the first result"
+        del outs, res, got
+    finally:
+        hip.set_stream(s1)
+        hip.synchronize()
+        hip.set_stream(old)
+        _lib.check(l.zenu_hip_stream_synchronize(s2), "sync")
+    del Xs, X
     _lib.check(l.zenu_hip_stream_destroy(s1), "destroy")
     _lib.check(l.zenu_hip_stream_destroy(s2), "destroy")

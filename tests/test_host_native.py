@@ -18,12 +18,13 @@ def build(src, out, extra=()):
 def test_allocator_bookkeeping(tmp_path):
     """mirrors zenu-matrix/src/memory_pool/test.rs:51-422 (mock device) for the new allocator:
     size classes, same-stream and cross-stream reuse, split/merge, OOM -> trim -> retry, foreign
-    pointers, and a randomized stress run against a shadow model"""
+    pointers, blocks taken during a stream capture staying out of ordinary requests until released,
+    and a randomized stress run against a shadow model"""
     exe = build("allocator_host_check.cpp", str(tmp_path / "alloc_check"))
     out = subprocess.run([exe], capture_output=True, text=True)
     assert out.returncode == 0, out.stdout + out.stderr
     for name in ("size_classes", "same_stream_reuse", "cross_stream_reuse", "retire_stream", "split_merge_trim", "oom_retry",
-                 "injected_failure", "not_owned", "stress"):
+                 "injected_failure", "not_owned", "capture_blocks", "stress"):
         assert f"ok {name}" in out.stdout
 
 

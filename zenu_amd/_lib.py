@@ -52,6 +52,7 @@ SIGNATURES = {
     "zenu_hip_device_synchronize": [],
     "zenu_hip_malloc": [C.POINTER(_vp), _sz, _vp],
     "zenu_hip_free": [_vp, _vp],
+    "zenu_hip_release_captured": [_vp],
     "zenu_hip_mempool_trim": [],
     "zenu_hip_mempool_stats": [C.POINTER(MempoolStats)],
     "zenu_hip_raw_malloc": [C.POINTER(_vp), _sz],

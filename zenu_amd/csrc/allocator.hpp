@@ -19,6 +19,13 @@
 //     (the flow memory_pool/mod.rs:9-20 describes), then report ZENU_ERR_OOM.
 //   * free() of a pointer the pool does not know returns ZENU_ERR_NOT_OWNED so the caller can
 //     fall back to a raw free (device/mod.rs:34-45).
+//   * Stream capture.  A kernel recorded into a graph keeps the addresses it was recorded with
+//     and writes them again on every replay, long after the capture's own frees.  A block that a
+//     capturing stream takes from the pool is therefore marked; whenever it is freed (during
+//     the capture or later) it goes to a list that only later captures on the same stream may
+//     draw from (inside one capture the recorded order makes reuse safe), never to an ordinary
+//     request.  release_captured(stream) -- or retiring the stream -- returns those blocks to
+//     the ordinary lists once the caller has destroyed the graphs.
 //
 // The device is reached only through `Backend`, so the bookkeeping is testable on the host
 // with a fake backend (as memory_pool/test.rs:18-49 does with MockDeviceBase).
@@ -64,7 +71,8 @@ public:
     explicit CachingAllocator(AllocBackend *backend) : be_(backend) {}
     ~CachingAllocator() { release_all(); }
 
-    int malloc(void **out, size_t bytes, void *stream)
+    // `capturing`: `stream` is recording a graph (the caller asks the runtime)
+    int malloc(void **out, size_t bytes, void *stream, bool capturing = false)
     {
         if (!out) return kErrArg;
         *out = nullptr;
@@ -74,8 +82,11 @@ public:
         const size_t size = round_size(bytes);
         const bool small = size <= kSmallLimit;
 
-        Block *b = take_free_block(size, small, stream, /*other_streams=*/false);
-        if (!b) b = take_free_block(size, small, stream, /*other_streams=*/true);
+        Block *b = nullptr;
+        if (capturing) b = take_free_block(size, small, stream, /*other_streams=*/false, /*captured=*/true);
+        if (!b) b = take_free_block(size, small, stream, /*other_streams=*/false);
+        // a block of another stream comes with an event wait, which a capture would record: not then
+        if (!b && !capturing) b = take_free_block(size, small, stream, /*other_streams=*/true);
         if (b) {
             stats_.n_cache_hits++;
         } else {
@@ -107,6 +118,8 @@ public:
             r->size = b->size - size;
             r->small = b->small;
             r->stream = stream;
+            r->captured = b->captured;
+            r->capture_stream = b->capture_stream;
             r->prev = b;
             r->next = b->next;
             if (b->next) b->next->prev = r;
@@ -116,6 +129,10 @@ public:
         }
         b->allocated = true;
         b->stream = stream;
+        if (capturing) {
+            b->captured = true;
+            b->capture_stream = stream;
+        }
         live_[b->ptr] = b;
         stats_.bytes_in_use += b->size;
         *out = b->ptr;
@@ -132,6 +149,7 @@ public:
         live_.erase(it);
         stats_.bytes_in_use -= b->size;
         b->allocated = false;
+        if (b->captured) stream = b->capture_stream;   // stays with the graphs of the stream that recorded it
         if (retired_.count(stream)) stream = nullptr;  // freed after its stream was destroyed (and synchronised)
         b->stream = stream;  // the last stream to use the block: stream-ordered free
         // merge with free neighbours that belong to the same stream
@@ -150,15 +168,35 @@ public:
         return kOk;
     }
 
+    // The graphs recorded on `stream` are gone: the blocks their captures took from the pool become
+    // ordinary blocks again (free ones now, live ones when they are freed).
+    void release_captured(void *stream)
+    {
+        std::lock_guard<std::mutex> g(mu_);
+        release_captured_locked(stream);
+    }
+
+    // bytes held back for the graphs of all streams (free blocks only)
+    uint64_t bytes_captured()
+    {
+        std::lock_guard<std::mutex> g(mu_);
+        uint64_t n = 0;
+        for (auto &kv : free_)
+            if (kv.first.captured)
+                for (Block *b : kv.second) n += b->size;
+        return n;
+    }
+
     // `stream` is about to be destroyed and has been synchronised: its cached blocks are idle,
     // so they move to the null stream's lists (nobody may order work after a dead stream).
     void retire_stream(void *stream)
     {
         if (!stream) return;
         std::lock_guard<std::mutex> g(mu_);
+        release_captured_locked(stream);
         retired_.insert(stream);
         for (int small = 0; small < 2; small++) {
-            auto it = free_.find(PoolKey{stream, small != 0});
+            auto it = free_.find(PoolKey{stream, small != 0, false});
             if (it == free_.end()) continue;
             std::vector<Block *> blocks(it->second.begin(), it->second.end());
             free_.erase(it);
@@ -209,6 +247,8 @@ private:
         bool small = false;
         bool allocated = false;
         bool segment_head = false;  // first block of a driver allocation
+        bool captured = false;      // taken from the pool by a capturing stream: recorded kernels hold its address
+        void *capture_stream = nullptr;
         void *stream = nullptr;
         Block *prev = nullptr, *next = nullptr;  // neighbours inside the segment
     };
@@ -223,33 +263,36 @@ private:
     struct PoolKey {
         void *stream;
         bool small;
+        bool captured;
         bool operator<(const PoolKey &o) const
         {
             if (stream != o.stream) return stream < o.stream;
-            return small < o.small;
+            if (small != o.small) return small < o.small;
+            return captured < o.captured;
         }
     };
 
     void insert_free(Block *b)
     {
-        free_[PoolKey{b->stream, b->small}].insert(b);
+        free_[PoolKey{b->stream, b->small, b->captured}].insert(b);
         stats_.bytes_cached += b->size;
     }
     void erase_free(Block *b)
     {
-        auto it = free_.find(PoolKey{b->stream, b->small});
+        auto it = free_.find(PoolKey{b->stream, b->small, b->captured});
         if (it != free_.end()) it->second.erase(b);
         stats_.bytes_cached -= b->size;
     }
 
-    // best fit in one stream's list (other_streams=false) or any other stream's (true)
-    Block *take_free_block(size_t size, bool small, void *stream, bool other_streams)
+    // best fit in one stream's list (other_streams=false) or any other stream's (true); `captured`
+    // selects the blocks held back for the stream's graphs instead of the ordinary ones
+    Block *take_free_block(size_t size, bool small, void *stream, bool other_streams, bool captured = false)
     {
         Block key;
         key.size = size;
         key.ptr = nullptr;
         for (auto &kv : free_) {
-            if (kv.first.small != small) continue;
+            if (kv.first.small != small || kv.first.captured != captured) continue;
             if ((kv.first.stream == stream) == other_streams) continue;
             FreeSet &fs = kv.second;
             auto it = fs.lower_bound(&key);
@@ -269,7 +312,7 @@ private:
 
     Block *try_merge(Block *b, Block *nb)
     {
-        if (!nb || nb->allocated || nb->stream != b->stream) return b;
+        if (!nb || nb->allocated || nb->stream != b->stream || nb->captured != b->captured) return b;
         erase_free(nb);
         if (nb == b->prev) {
             nb->size += b->size;
@@ -285,20 +328,50 @@ private:
         return b;
     }
 
+    void release_captured_locked(void *stream)
+    {
+        for (int small = 0; small < 2; small++) {
+            auto it = free_.find(PoolKey{stream, small != 0, true});
+            if (it == free_.end()) continue;
+            std::vector<Block *> blocks(it->second.begin(), it->second.end());
+            free_.erase(it);
+            for (Block *b : blocks) {
+                stats_.bytes_cached -= b->size;
+                b->captured = false;
+                b->capture_stream = nullptr;
+                b = try_merge(b, b->prev);
+                b = try_merge(b, b->next);
+                insert_free(b);
+            }
+        }
+        for (auto &kv : live_)
+            if (kv.second->captured && kv.second->capture_stream == stream) {
+                kv.second->captured = false;
+                kv.second->capture_stream = nullptr;
+            }
+    }
+
     // Only after device_synchronize(): nothing is in flight, so free neighbours can be joined
-    // whatever stream they were freed on.
+    // whatever stream they were freed on.  Blocks held back for graphs stay as they are.
     void coalesce_across_streams()
     {
         std::vector<Block *> all;
-        for (auto &kv : free_)
-            for (Block *b : kv.second) all.push_back(b);
-        free_.clear();
-        stats_.bytes_cached = 0;
+        for (auto it = free_.begin(); it != free_.end();) {
+            if (it->first.captured) {
+                ++it;
+                continue;
+            }
+            for (Block *b : it->second) {
+                all.push_back(b);
+                stats_.bytes_cached -= b->size;
+            }
+            it = free_.erase(it);
+        }
         std::set<Block *> dead;
         for (Block *b : all) {
             if (dead.count(b)) continue;
-            if (b->prev && !b->prev->allocated) continue;  // not the head of its free run
-            while (b->next && !b->next->allocated) {
+            if (b->prev && !b->prev->allocated && !b->prev->captured) continue;  // not the head of its free run
+            while (b->next && !b->next->allocated && !b->next->captured) {
                 Block *n = b->next;
                 b->size += n->size;
                 b->next = n->next;
@@ -316,6 +389,7 @@ private:
     {
         coalesce_across_streams();
         for (auto &kv : free_) {
+            if (kv.first.captured) continue;   // recorded kernels still hold these addresses
             FreeSet &fs = kv.second;
             for (auto it = fs.begin(); it != fs.end();) {
                 Block *b = *it;

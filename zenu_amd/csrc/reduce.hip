@@ -228,9 +228,13 @@ __device__ __forceinline__ void emit_final(const RedParams<T> &p, int64_t o, typ
 // partials travel with device-scope (write-through / L2-bypassing) accesses instead of a
 // device-scope fence: a release fence would write back and invalidate the whole L2 in every
 // workgroup (measured: 20x slower).  Order of events in a producer: device-scope stores of the
-// partials, wait until they are acknowledged (workgroup-scope release = s_waitcnt), barrier, then
-// one device-scope atomic increment by thread 0.  The consumer (the workgroup that reads
-// expected-1 from the counter) loads the partials with device-scope loads.
+// partials (write-through: they go to memory, not to this XCD's L2); every thread then waits
+// until its own vector-memory operations are acknowledged (an explicit s_waitcnt vmcnt(0): a
+// workgroup-scope release fence only waits for LDS and scalar traffic and would let the counter
+// overtake the partials); barrier; one device-scope atomic increment by thread 0.  A store that
+// has been acknowledged at device scope has reached the point every XCD reads through, so the
+// consumer (the workgroup that reads expected-1 from the counter) sees it with device-scope
+// loads, which it issues only after that atomic has returned.
 template <typename U> __device__ __forceinline__ void store_agent(U *p, U v)
 {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -283,7 +287,9 @@ __device__ __forceinline__ typename Tr::Acc load_partial(const RedParams<T> &p, 
 __device__ __forceinline__ bool arrive_last(int *c, int split, int splits, int fan)
 {
     __shared__ int s_last;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // this thread's partial stores are acknowledged
+    // every thread: all of my vector-memory stores (the partials) are acknowledged before the
+    // barrier lets thread 0 announce this workgroup
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
         bool last;

@@ -63,10 +63,24 @@ struct State {
 State g_state;
 std::mutex g_init_mu;
 
+// is `stream` recording a graph?  (the null stream never is)
+bool stream_is_capturing(hipStream_t stream)
+{
+    if (!stream) return false;
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return st != hipStreamCaptureStatusNone;
+}
+
 // allocate and clear the ring of `stream` (blocking; at init, at stream creation, or at the first
-// split reduction on a stream the library did not create)
+// split reduction on a stream the library did not create).  Not while that stream records a
+// graph: the blocking calls would invalidate the capture.
 int *make_ring(hipStream_t stream)
 {
+    if (stream_is_capturing(stream)) return nullptr;
     int *base = nullptr;
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&base), kNumCounters * sizeof(int));
     if (e == hipSuccess) e = hipMemset(base, 0, kNumCounters * sizeof(int));
@@ -271,7 +285,7 @@ int zenu_hip_malloc(void **ptr_dev, size_t bytes, zenu_stream_t stream)
         if (g_state.backend.raw_alloc(ptr_dev, bytes ? bytes : 1) != 0) return ZENU_ERR_OOM;
         return ZENU_OK;
     }
-    return g_state.pool->malloc(ptr_dev, bytes, stream);
+    return g_state.pool->malloc(ptr_dev, bytes, stream, stream_is_capturing(as_stream(stream)));
 }
 
 int zenu_hip_free(void *ptr_dev, zenu_stream_t stream)
@@ -284,6 +298,15 @@ int zenu_hip_free(void *ptr_dev, zenu_stream_t stream)
         return ZENU_OK;
     }
     return g_state.pool->free(ptr_dev, stream);
+}
+
+int zenu_hip_release_captured(zenu_stream_t stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (stream_is_capturing(as_stream(stream))) return ZENU_ERR_ARG;
+    if (g_state.pool) g_state.pool->release_captured(stream);
+    return ZENU_OK;
 }
 
 int zenu_hip_mempool_trim(void)
