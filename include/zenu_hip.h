@@ -39,7 +39,9 @@ typedef enum {
     ZENU_ERR_HIP = 5,         /* a HIP runtime call failed: see zenu_hip_last_hip_error */
     ZENU_ERR_OOM = 6,         /* device allocation failed even after trimming the cache */
     ZENU_ERR_UNSUPPORTED = 7, /* valid request this build has no kernel for  */
-    ZENU_ERR_NOT_OWNED = 8    /* zenu_hip_free: pointer unknown to the pool (MemPoolFreeError) */
+    ZENU_ERR_NOT_OWNED = 8,   /* zenu_hip_free: pointer unknown to the pool (MemPoolFreeError) */
+    ZENU_ERR_NOT_INIT = 9,    /* an entry point that may not allocate was called before zenu_hip_init */
+    ZENU_ERR_SCRATCH_LIMIT = 10 /* zenu_hip_sum_axis_noalloc: the request needs more than its static scratch */
 } zenu_status_t;
 
 typedef enum { ZENU_F32 = 0, ZENU_F64 = 1 } zenu_dtype_t;
@@ -224,6 +226,26 @@ int zenu_hip_broadcast(int dtype, const zenu_tensor_t *to, const zenu_tensor_t *
  * (zenu-matrix/src/operation/sum.rs:9-32).  out may be strided. */
 int zenu_hip_sum_axis(int dtype, const zenu_tensor_t *out, const zenu_tensor_t *src, int axis,
                       zenu_stream_t stream);
+/* zenu_hip_sum_axis for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same result as
+ * zenu_hip_sum_axis, bit for bit (same kernels, same launch geometry), but the call allocates
+ * nothing, neither from the driver nor from the caching pool: the arrival counters and partial
+ * results of a split reduction and the contiguous staging of a strided destination live in a
+ * static device array of 1 040 KiB (16 KiB of counters, 512 KiB of partials, 512 KiB of staging)
+ * that the device holds until the process ends.  Limits:
+ *   - zenu_hip_init must have run (ZENU_ERR_NOT_INIT otherwise: initialising allocates);
+ *   - a source view that zenu_hip_sum_axis would first copy to a contiguous buffer (kept dims
+ *     that are neither one uniform stride chain nor a unit-stride run) is refused with
+ *     ZENU_ERR_UNSUPPORTED;
+ *   - outputs x splits x element size > 512 KiB, more than 4096 counters, or a strided
+ *     destination of more than 512 KiB are refused with ZENU_ERR_SCRATCH_LIMIT (a contiguous
+ *     destination has no size limit; with 256 compute units no split reduction exceeds 512 KiB
+ *     of partials).
+ * Every call on the device shares the one array: calls that overlap in time (different streams,
+ * or graph replays running concurrently) race and give wrong results; calls ordered on one stream
+ * are safe. */
+int zenu_hip_sum_axis_noalloc(int dtype, const zenu_tensor_t *out, const zenu_tensor_t *src, int axis,
+                              zenu_stream_t stream);
 /* *out_dev = sum of every element (sum_to(x, []), sum.rs:35-94). */
 int zenu_hip_sum_all(int dtype, void *out_dev, const zenu_tensor_t *src, zenu_stream_t stream);
 /* target = sum_to(src) for any legal target shape (sum.rs:35-94). */

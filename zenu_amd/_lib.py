@@ -14,7 +14,8 @@ F32, F64 = 0, 1
 ADD, SUB, MUL, DIV = 0, 1, 2, 3
 (EXP, LOG, TANH, SQRT, ABS, SIN, COS, TAN, ASIN, ACOS, ATAN, SINH, COSH, SIGMOID, TANH_ULP2) = range(15)
 
-OK, ERR_RANK, ERR_SHAPE, ERR_AXIS, ERR_ARG, ERR_HIP, ERR_OOM, ERR_UNSUPPORTED, ERR_NOT_OWNED = range(9)
+(OK, ERR_RANK, ERR_SHAPE, ERR_AXIS, ERR_ARG, ERR_HIP, ERR_OOM, ERR_UNSUPPORTED, ERR_NOT_OWNED, ERR_NOT_INIT,
+ ERR_SCRATCH_LIMIT) = range(11)
 
 
 class Tensor(C.Structure):
@@ -85,6 +86,7 @@ SIGNATURES = {
     "zenu_hip_softmax_cross_entropy_backward": [_i, _TP, _TP, _TP, _TP, _vp],
     "zenu_hip_bias_add_relu": [_i, _TP, _TP, _TP, _TP, _d, _vp],
     "zenu_hip_sum_axis": [_i, _TP, _TP, _i, _vp],
+    "zenu_hip_sum_axis_noalloc": [_i, _TP, _TP, _i, _vp],
     "zenu_hip_sum_all": [_i, _vp, _TP, _vp],
     "zenu_hip_sum_to": [_i, _TP, _TP, _vp],
     "zenu_hip_max_axis": [_i, _TP, _TP, _i, _vp],

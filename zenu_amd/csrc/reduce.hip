@@ -39,8 +39,33 @@ namespace zenu {
 
 // `n` consecutive arrival counters (zero at rest) from the ring of `stream`, or nullptr
 int *reserve_counters(int64_t n, hipStream_t stream);
+bool library_ready();
 
 namespace {
+
+// ---- static scratch of the allocation-free entry point (zenu_hip_sum_axis_noalloc) -------------------
+// Counters, partials and the staging of a strided destination for callers that may not allocate.
+// Held by the device from the moment the library's code object is loaded until the process ends.
+// In host code the array's name is only a stand-in: its device address comes from
+// hipGetSymbolAddress (init_static_scratch, called once by the library's init with the device
+// current) and that pointer is what kernels and fills get.
+constexpr size_t kScratchCounters = 4096;                       // arrival counters (ints)
+constexpr size_t kScratchCounterBytes = kScratchCounters * sizeof(int);
+constexpr size_t kScratchPartialBytes = 512u << 10;             // partial results of a split reduction
+constexpr size_t kScratchStageBytes = 512u << 10;               // contiguous result of a strided destination
+constexpr size_t kScratchBytes = kScratchCounterBytes + kScratchPartialBytes + kScratchStageBytes;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+unsigned char *g_scratch_ptr = nullptr;   // device address of `scratch` (one device per process)
+
+// where a reduction finds its cross-workgroup memory when it may not allocate
+struct FixedScratch {
+    int *counters;
+    int64_t n_counters;
+    void *partials;
+    size_t partial_bytes;
+    void *stage;
+    size_t stage_bytes;
+};
 
 constexpr int kBlock = 256;
 constexpr int kWave = 64;
@@ -647,7 +672,8 @@ int launch_cols(const RedParams<T> &p, hipStream_t s)
 // r < R; the inner run has unit stride) into contiguous outputs of outer*inner elements.
 template <typename T, typename Tr>
 int reduce_strided(const T *src, int64_t outer, int64_t R, int64_t inner, int64_t outer_stride,
-                   int64_t elem_stride, T *out_val, int64_t *out_idx, hipStream_t s)
+                   int64_t elem_stride, T *out_val, int64_t *out_idx, hipStream_t s,
+                   const FixedScratch *fixed = nullptr)
 {
     constexpr int VEC = VecOf<T>::N;
     const int64_t nout = outer * inner;
@@ -716,6 +742,28 @@ int reduce_strided(const T *src, int64_t outer, int64_t R, int64_t inner, int64_
         fan = 8;   // measured on 512 splits: 2 / 4 / 8 / 16 / 23 (= sqrt) / 64 / flat -> 23.6 / 22.9 / 22.8 / 23.4 / 24.3 / 25.0 / 25.0 us
         cstride = 1 + (int)((splits + fan - 1) / fan);
     }
+    const size_t key_bytes = ((size_t)nout * splits * sizeof(T) + 255) / 256 * 256;
+    const size_t idx_bytes = Tr::kHasIdx ? (size_t)nout * splits * sizeof(int32_t) : 0;
+    if (fixed) {
+        // the caller may not allocate: counters and partials live in the static scratch, which
+        // every such call on the device shares and which keeps the last call's contents
+        if (groups * cstride > fixed->n_counters) {
+            fan = (int)splits;
+            cstride = 1;
+        }
+        if (groups * cstride > fixed->n_counters || key_bytes + idx_bytes > fixed->partial_bytes)
+            return ZENU_ERR_SCRATCH_LIMIT;
+        // counters must start at zero; a fill kernel, not a memset node, so the call can be captured
+        int rc = zenu_hip_memset_zero(fixed->counters, (size_t)(groups * cstride) * sizeof(int),
+                                      reinterpret_cast<zenu_stream_t>(s));
+        if (rc) return rc;
+        p.fan = fan;
+        p.cstride = cstride;
+        p.part_key = static_cast<T *>(fixed->partials);
+        p.part_idx = Tr::kHasIdx ? reinterpret_cast<int32_t *>(static_cast<char *>(fixed->partials) + key_bytes) : nullptr;
+        p.counters = fixed->counters;
+        return use_cols ? launch_cols<T, Tr>(p, s) : launch_rows<T, Tr>(p, s);
+    }
     int *counters = reserve_counters(groups * cstride, s);
     if (!counters && cstride > 1) {   // too many groups for trees: flat counters
         fan = (int)splits;
@@ -725,8 +773,6 @@ int reduce_strided(const T *src, int64_t outer, int64_t R, int64_t inner, int64_
     if (!counters) return ZENU_ERR_UNSUPPORTED;
     p.fan = fan;
     p.cstride = cstride;
-    const size_t key_bytes = ((size_t)nout * splits * sizeof(T) + 255) / 256 * 256;
-    const size_t idx_bytes = Tr::kHasIdx ? (size_t)nout * splits * sizeof(int32_t) : 0;
     Workspace ws(key_bytes + idx_bytes, s);
     if (ws.status) return ws.status;
     p.part_key = static_cast<T *>(ws.ptr);
@@ -811,7 +857,7 @@ StridedMap map_strided(const zenu_tensor_t &src, int axis)
 
 template <typename T>
 int reduce_axis_t(int kind, int dtype, const zenu_tensor_t *out, int64_t *out_idx,
-                  const zenu_tensor_t &src, int axis, hipStream_t s)
+                  const zenu_tensor_t &src, int axis, hipStream_t s, const FixedScratch *fixed = nullptr)
 {
     const int64_t n = num_elm(src);
     int64_t outer = 1, inner = 1;
@@ -826,6 +872,7 @@ int reduce_axis_t(int kind, int dtype, const zenu_tensor_t *out, int64_t *out_id
     // else goes through a contiguous copy first (to_default_stride, as max.rs:49 does).
     StridedMap map = map_strided(src, axis);
     const T *sp = static_cast<const T *>(src.ptr);
+    if (fixed && !map.ok) return ZENU_ERR_UNSUPPORTED;   // would need a copy of the whole source
     Workspace wsrc(map.ok ? 0 : (size_t)n * sizeof(T), s);
     if (!map.ok) {
         if (wsrc.status) return wsrc.status;
@@ -842,10 +889,15 @@ int reduce_axis_t(int kind, int dtype, const zenu_tensor_t *out, int64_t *out_id
     // contiguous destination, or a temporary that is copied out afterwards
     T *ov = nullptr;
     bool need_copy = false;
-    Workspace wout((out && !is_default_stride_strict(*out)) ? (size_t)(nout ? nout : 1) * sizeof(T) : 0, s);
+    const bool stage_out = out && !is_default_stride_strict(*out);
+    if (fixed && stage_out && (size_t)nout * sizeof(T) > fixed->stage_bytes) return ZENU_ERR_SCRATCH_LIMIT;
+    Workspace wout((stage_out && !fixed) ? (size_t)(nout ? nout : 1) * sizeof(T) : 0, s);
     if (out) {
-        if (is_default_stride_strict(*out)) {
+        if (!stage_out) {
             ov = static_cast<T *>(out->ptr);
+        } else if (fixed) {
+            ov = static_cast<T *>(fixed->stage);
+            need_copy = true;
         } else {
             if (wout.status) return wout.status;
             ov = static_cast<T *>(wout.ptr);
@@ -853,9 +905,9 @@ int reduce_axis_t(int kind, int dtype, const zenu_tensor_t *out, int64_t *out_id
         }
     }
     int rc;
-    if (kind == kSum) rc = reduce_strided<T, SumTr<T>>(sp, map.outer, R, map.inner, map.outer_stride, map.elem_stride, ov, nullptr, s);
-    else if (kind == kAsum) rc = reduce_strided<T, AsumTr<T>>(sp, map.outer, R, map.inner, map.outer_stride, map.elem_stride, ov, nullptr, s);
-    else rc = reduce_strided<T, ArgmaxTr<T>>(sp, map.outer, R, map.inner, map.outer_stride, map.elem_stride, ov, out_idx, s);
+    if (kind == kSum) rc = reduce_strided<T, SumTr<T>>(sp, map.outer, R, map.inner, map.outer_stride, map.elem_stride, ov, nullptr, s, fixed);
+    else if (kind == kAsum) rc = reduce_strided<T, AsumTr<T>>(sp, map.outer, R, map.inner, map.outer_stride, map.elem_stride, ov, nullptr, s, fixed);
+    else rc = reduce_strided<T, ArgmaxTr<T>>(sp, map.outer, R, map.inner, map.outer_stride, map.elem_stride, ov, out_idx, s, fixed);
     if (rc) return rc;
     if (need_copy) {
         zenu_tensor_t tmp = default_view(ov, out->ndim, out->shape);
@@ -865,16 +917,16 @@ int reduce_axis_t(int kind, int dtype, const zenu_tensor_t *out, int64_t *out_id
 }
 
 int reduce_axis(int kind, int dtype, const zenu_tensor_t *out, int64_t *out_idx, const zenu_tensor_t *src,
-                int axis, hipStream_t s)
+                int axis, hipStream_t s, const FixedScratch *fixed = nullptr)
 {
     int rc = validate_tensor(src);
     if (!rc && out) rc = validate_tensor(out);
-    if (!rc) rc = ensure_init();
+    if (!rc) rc = fixed ? ZENU_OK : ensure_init();   // the allocation-free caller has checked that init ran
     if (rc) return rc;
     if (axis < 0 || axis >= src->ndim) return ZENU_ERR_AXIS;
     if (out && !reduced_shape_ok(*out, *src, axis)) return ZENU_ERR_SHAPE;
-    if (dtype == ZENU_F32) return reduce_axis_t<float>(kind, dtype, out, out_idx, *src, axis, s);
-    if (dtype == ZENU_F64) return reduce_axis_t<double>(kind, dtype, out, out_idx, *src, axis, s);
+    if (dtype == ZENU_F32) return reduce_axis_t<float>(kind, dtype, out, out_idx, *src, axis, s, fixed);
+    if (dtype == ZENU_F64) return reduce_axis_t<double>(kind, dtype, out, out_idx, *src, axis, s, fixed);
     return ZENU_ERR_ARG;
 }
 
@@ -915,11 +967,41 @@ int reduce_all(int kind, int dtype, void *out_val, int64_t *out_idx, const zenu_
 }
 
 }  // namespace
+
+// Called once by the library's init, with its device current: the device address of the static
+// scratch.  Each device holds its own copy of the array at its own address; the library drives
+// one device per process, so one pointer is kept.
+int init_static_scratch()
+{
+    if (g_scratch_ptr) return ZENU_OK;
+    void *p = nullptr;
+    ZENU_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return ZENU_ERR_HIP;
+    g_scratch_ptr = static_cast<unsigned char *>(p);
+    return ZENU_OK;
+}
+
 }  // namespace zenu
 
 using namespace zenu;
 
 extern "C" {
+
+int zenu_hip_sum_axis_noalloc(int dtype, const zenu_tensor_t *out, const zenu_tensor_t *src, int axis,
+                              zenu_stream_t stream)
+{
+    if (!out) return ZENU_ERR_ARG;
+    // initialising the library allocates (pool, counter rings): not from here
+    if (!library_ready() || !g_scratch_ptr) return ZENU_ERR_NOT_INIT;
+    FixedScratch fx;
+    fx.counters = reinterpret_cast<int *>(g_scratch_ptr);
+    fx.n_counters = (int64_t)kScratchCounters;
+    fx.partials = g_scratch_ptr + kScratchCounterBytes;
+    fx.partial_bytes = kScratchPartialBytes;
+    fx.stage = g_scratch_ptr + kScratchCounterBytes + kScratchPartialBytes;
+    fx.stage_bytes = kScratchStageBytes;
+    return reduce_axis(kSum, dtype, out, nullptr, src, axis, as_stream(stream), &fx);
+}
 
 int zenu_hip_sum_axis(int dtype, const zenu_tensor_t *out, const zenu_tensor_t *src, int axis,
                       zenu_stream_t stream)

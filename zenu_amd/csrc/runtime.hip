@@ -15,6 +15,8 @@
 
 namespace zenu {
 
+int init_static_scratch();   // reduce.hip
+
 static thread_local hipError_t tl_last_hip_error = hipSuccess;
 void set_last_hip_error(hipError_t e) { tl_last_hip_error = e; }
 
@@ -127,6 +129,8 @@ int init_locked(int device)
     g_state.info.lds_per_block = prop.sharedMemPerBlock;
     const char *env = getenv("ZENU_USE_MEMPOOL");  // zenu-matrix/src/lib.rs:36, default "1"
     g_state.use_pool = !(env && strcmp(env, "0") == 0);
+    int rc = init_static_scratch();
+    if (rc) return rc;
     g_state.pool = new CachingAllocator(&g_state.backend);
     g_state.ready = true;
     return make_ring(nullptr) ? ZENU_OK : ZENU_ERR_HIP;   // the null stream's ring; created streams get theirs at creation
@@ -149,6 +153,7 @@ __global__ __launch_bounds__(kFillBlock) void fill_zero_kernel(uint4 *dst16, siz
 }  // namespace
 
 const DeviceInfo &device_info() { return g_state.info; }
+bool library_ready() { return g_state.ready; }
 
 // Consecutive launches on a stream take consecutive ranges of that stream's ring; a range is reused
 // by a later launch of the same stream, which runs after the earlier one.  Every kernel leaves
@@ -228,6 +233,8 @@ const char *zenu_hip_status_string(int status)
     case ZENU_ERR_OOM: return "out of device memory";
     case ZENU_ERR_UNSUPPORTED: return "unsupported";
     case ZENU_ERR_NOT_OWNED: return "pointer not owned by the memory pool";
+    case ZENU_ERR_NOT_INIT: return "zenu_hip_init has not run (this entry point may not initialise the library: that allocates)";
+    case ZENU_ERR_SCRATCH_LIMIT: return "request needs more than the static scratch of the allocation-free entry point";
     default: return "unknown status";
     }
 }
