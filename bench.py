@@ -223,8 +223,7 @@ def build_ops(z, workload, stream):
         n = x.size
         sets = [(M.from_numpy(x), M.from_numpy(t), M.alloc(shape), M.alloc(shape), M.from_numpy(bias), M.alloc([]))
                 for _ in range(nsets(4 * 4 * n))]
-        sys.path.insert(0, os.path.join(ROOT, "tests"))
-        import cpu_matrix
+        import cpu_matrix   # oracle/: the CPU chains behind the cpu_fn legs
         cx, ct, cb = (cpu_matrix.CpuMatrix.from_numpy(v) for v in (x, t, bias))
         co = cpu_matrix.CpuMatrix.zeros(shape)
 
@@ -357,31 +356,36 @@ def build_ops(z, workload, stream):
     return ops
 
 
-def run_c4(z, args, sync):
+def measure_c4(z, args, sync, steps=None):
     """configs[4]: the MLP training step (batch 256, 784-512-512-10, softmax-CE, backward, Adam) as
-    ZeNu's op sequence; GEMM on rocBLAS, everything else on this library.  Reports the wall time of
-    a step and, from one event-instrumented step, the time per kernel family."""
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    import mlp_devices
-    import mlp_step
+    ZeNu's op sequence; GEMM on rocBLAS, everything else on this library.  Returns the wall time of
+    a step for each way of issuing it and, from one event-instrumented step, the time per kernel
+    family."""
+    from harness import hip_dev, mlp_step
     x, t, params = mlp_step.make_inputs()
+    steps = steps or args.steps
+
+    class A:      # what the helpers read
+        pass
+    a = A()
+    a.steps, a.warmup = steps, args.warmup
 
     def measure(fused):
-        dev = mlp_devices.HipDev(z, timed=False)
+        dev = hip_dev.HipDev(z, timed=False)
         st = mlp_step.MlpStep(dev, x, t, params, fused=fused)
-        for _ in range(max(args.warmup, 3)):
+        for _ in range(max(a.warmup, 3)):
             st.step()
         sync()
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             st.step()
         sync()
-        ms = (time.perf_counter() - t0) / args.steps * 1e3
+        ms = (time.perf_counter() - t0) / steps * 1e3
         dev.__init__(z, timed=True)
         dev.begin()
         st.step()
         br = {k: round(v, 1) for k, v in dev.breakdown().items()}
-        return ms, br, capture_and_replay_c4(z, st, args, sync)
+        return ms, br, capture_and_replay_c4(z, st, a, sync)
 
     ms, br, graph = measure(False)
     fms, fbr, fgraph = measure(True)
@@ -389,10 +393,11 @@ def run_c4(z, args, sync):
                      "forward / backward, ReLU backward)",
              "ms_per_step": round(fms, 4), "steps_per_s": round(1e3 / fms, 1),
              "breakdown_us_one_instrumented_step": fbr, "hip_graph_replay": fgraph}
-    compiled = compiled_host_c4(x, t, params, args)
+    compiled = compiled_host_c4(x, t, params, a)
     cpu = None
     if not args.no_cpu_baseline:
-        cst = mlp_step.MlpStep(mlp_devices.CpuDev(), x, t, params)
+        import cpu_dev      # oracle/: the CPU leg of the same step
+        cst = mlp_step.MlpStep(cpu_dev.CpuDev(), x, t, params)
         cst.step()
         t1 = time.perf_counter()
         n = 3
@@ -404,24 +409,62 @@ def run_c4(z, args, sync):
     head_ms, host = ms, "python mirror (ctypes)"
     if isinstance(compiled.get("ops"), dict) and "ms_per_step" in compiled["ops"]:
         head_ms, host = compiled["ops"]["ms_per_step"], "compiled host (C++ API)"
+    return dict(head_ms=head_ms, host=host, ms=ms, breakdown=br, graph=graph, fused=fused, compiled=compiled, cpu=cpu)
+
+
+C4_WORKLOAD = "configs[4]: batch 256, Linear 784-512-ReLU-512-ReLU-10, softmax-CE, Adam"
+
+
+def run_c4(z, args, sync):
+    """--workload c4: the MLP step as the headline of its own JSON line"""
+    r = measure_c4(z, args, sync)
     print(json.dumps({
-        "metric": "MLP training step (configs[4]): steps/s; time per kernel family", "value": round(1e3 / head_ms, 1),
-        "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(head_ms, 4),
-        "host": host, "python_mirror_ms_per_step": round(ms, 4),
+        "metric": "MLP training step (configs[4]): steps/s; time per kernel family", "value": round(1e3 / r["head_ms"], 1),
+        "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(r["head_ms"], 4),
+        "host": r["host"], "python_mirror_ms_per_step": round(r["ms"], 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "configs[4]: batch 256, Linear 784-512-ReLU-512-ReLU-10, softmax-CE, Adam"},
-        "breakdown_us_one_instrumented_step": br, "hip_graph_replay": graph, "fused_entry_points": fused,
-        "compiled_host": compiled, "cpu_baseline": cpu}))
+        "config": {"workload": C4_WORKLOAD},
+        "breakdown_us_one_instrumented_step": r["breakdown"], "hip_graph_replay": r["graph"], "fused_entry_points": r["fused"],
+        "compiled_host": r["compiled"], "cpu_baseline": r["cpu"]}))
+
+
+def c4_summary(z, args, sync):
+    """configs[4] for the default line: never `value`, never `roofline`; an object of its own"""
+    try:
+        r = measure_c4(z, args, sync, steps=max(args.steps, 50))
+    except Exception as e:      # the configs[0..3] figures stand on their own
+        return {"workload": C4_WORKLOAD, "error": repr(e)}
+    comp = r["compiled"]
+
+    def ms_of(key):
+        v = comp.get(key) if isinstance(comp, dict) else None
+        return v.get("ms_per_step") if isinstance(v, dict) else None
+    return {
+        "workload": C4_WORKLOAD, "dtype": "f32", "unit": "ms per training step",
+        "eager_compiled_host_ms_per_step": ms_of("ops"),
+        "fused_compiled_host_ms_per_step": ms_of("fused"),
+        "fused_transposed_views_compiled_host_ms_per_step": ms_of("lean"),
+        "eager_python_mirror_ms_per_step": round(r["ms"], 4),
+        "fused_python_mirror_ms_per_step": r["fused"]["ms_per_step"],
+        "eager_hip_graph_replay": r["graph"], "fused_hip_graph_replay": r["fused"]["hip_graph_replay"],
+        "kernel_family_us_eager_step": r["breakdown"],
+        "kernel_family_us_fused_step": r["fused"]["breakdown_us_one_instrumented_step"],
+        "launches_per_step": {"eager": 62, "fused": 37, "fused_transposed_views": 20},
+        "compiled_host_error": comp.get("error") if isinstance(comp, dict) else None,
+        "cpu_baseline": r["cpu"],
+        "note": "GEMMs on rocBLAS; gemm is one family of the breakdown, every other family is this library; "
+                "event-instrumented steps include one event record per op",
+    }
 
 
 def compiled_host_c4(x, t, params, args):
-    """The same step issued eagerly from a C++ host (tests/native/mlp_step_bench.cpp, built by
+    """The same step issued eagerly from a C++ host (harness/native/mlp_step_bench.cpp, built by
     __graft_entry__.build()): wall time per step without the Python mirror's per-call cost."""
     import subprocess
     import tempfile
-    exe = os.path.join(ROOT, "tests", "native", "bin", "mlp_step_bench")
+    exe = os.path.join(ROOT, "harness", "native", "bin", "mlp_step_bench")
     if not os.path.exists(exe):
-        return {"error": "tests/native/bin/mlp_step_bench is not built"}
+        return {"error": "harness/native/bin/mlp_step_bench is not built"}
     with tempfile.TemporaryDirectory() as d:
         path = os.path.join(d, "inputs.bin")
         with open(path, "wb") as f:
@@ -637,6 +680,14 @@ def main():
                           f"host has {os.cpu_count()} logical CPUs")
         log(f"[cpu] one step on the CPU oracle: {cpu_s:.2f} s = {cpu['value']} GB/s")
 
+    # ---- configs[4], the MLP training step: its own object on the default line ---------------------------
+    c4 = None
+    if args.workload == "suite":
+        t0 = time.time()
+        c4 = c4_summary(z, args, sync)
+        log(f"[c4] MLP step measured in {time.time() - t0:.1f} s: "
+            f"{c4.get('eager_compiled_host_ms_per_step')} ms eager, {c4.get('fused_compiled_host_ms_per_step')} ms fused")
+
     out = {
         "metric": "achieved HBM GB/s (% of MI355X peak) per op; Adam step params/sec",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -648,10 +699,10 @@ def main():
                                 "scaling": "copy, add, sums and tanh on 64 MiB, 256 MiB and 1 GiB f32 tensors (not a BASELINE config)",
                                 "next": "strided copy, broadcast, the remaining unary functions, powf, asum and sum_to on [4096,4096] f32 "
                                         "(not a BASELINE config)"}[args.workload],
-                   "ops_per_step": len(ops), "algorithmic_bytes_per_step": step_bytes},
+                   "ops_per_step": len(table), "algorithmic_bytes_per_step": step_bytes},
         "frac_of_peak_whole_step": round(value / PEAK_HBM_GBPS, 4),
         "adam_step_params_per_sec": (round(adam[0]["Gelem_per_s"] * 1e9) if adam else None),
-        "roofline": roofline, "cpu_baseline": cpu, "ops": table,
+        "roofline": roofline, "cpu_baseline": cpu, "c4": c4, "ops": table,
         "timing": f"HIP events on the launch stream; per op {args.op_reps} back-to-back launches after 10 warm-up launches: "
                   "us = batch mean, us_bracketed_* = per-launch event pairs (each includes one event record)",
     }

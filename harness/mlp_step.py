@@ -1,7 +1,7 @@
 """BASELINE config[4]: one training step of the MNIST-shaped MLP (Linear 784-512-ReLU-512-ReLU-10,
 softmax cross-entropy, backward, one Adam step), replayed as the sequence of zenu-matrix ops that
 ZeNu's autograd issues, written once against the Matrix API and run on either device (CpuMatrix =
-oracle, zenu_amd.Matrix = HIP).  Used by tests/test_mlp_step.py and bench.py --workload c4.
+oracle, zenu_amd.Matrix = HIP).  Used by tests/test_mlp_step.py and bench.py.
 
 Op sequence followed (reference file:line):
   Linear::call            transpose(W) materialised, matmul, + bias     zenu-layer/src/layers/linear.rs:23-32,

@@ -8,8 +8,8 @@ tensor's largest magnitude."""
 import numpy as np
 import pytest
 
-import mlp_devices
-import mlp_step
+import cpu_dev
+from harness import hip_dev, mlp_step
 
 
 def rel(a, b):
@@ -19,7 +19,7 @@ def rel(a, b):
 def test_cpu_step_matches_plain_numpy():
     """pins the op sequence itself: the oracle-run step equals a direct numpy forward/backward"""
     x, t, params = mlp_step.make_inputs()
-    cpu = mlp_step.MlpStep(mlp_devices.CpuDev(), x, t, params)
+    cpu = mlp_step.MlpStep(cpu_dev.CpuDev(), x, t, params)
     loss, grads = cpu.step()
     W1, b1, W2, b2, W3, b3 = (params[f"linear{i}.{n}"].astype(np.float64) for i in (1, 2, 3) for n in ("weight", "bias"))
     xd, td = x.astype(np.float64), t.astype(np.float64)
@@ -42,8 +42,8 @@ def test_cpu_step_matches_plain_numpy():
 def test_cpu_fused_spelling_is_the_same_chain():
     """on the CPU device the fused names are the op-by-op chains: identical bits"""
     x, t, params = mlp_step.make_inputs()
-    a = mlp_step.MlpStep(mlp_devices.CpuDev(), x, t, params)
-    b = mlp_step.MlpStep(mlp_devices.CpuDev(), x, t, params, fused=True)
+    a = mlp_step.MlpStep(cpu_dev.CpuDev(), x, t, params)
+    b = mlp_step.MlpStep(cpu_dev.CpuDev(), x, t, params, fused=True)
     la, ga = a.step()
     lb, gb = b.step()
     assert np.array_equal(la.to_numpy(), lb.to_numpy())
@@ -57,7 +57,7 @@ def test_hip_fused_step_matches_hip_step(hip):
     """fused entry points against the op sequence on the same device and the same GEMMs: they differ
     only in summation order (softmax denominators over 10 classes, the loss), far below 1e-5"""
     x, t, params = mlp_step.make_inputs()
-    dev = mlp_devices.HipDev(hip)
+    dev = hip_dev.HipDev(hip)
     a = mlp_step.MlpStep(dev, x, t, params)
     b = mlp_step.MlpStep(dev, x, t, params, fused=True)
     for step in range(3):
@@ -71,7 +71,7 @@ def test_hip_fused_step_matches_hip_step(hip):
 
 
 def write_inputs(path, x, t, params):
-    """raw f32 in the order tests/native/mlp_step_bench.cpp reads"""
+    """raw f32 in the order harness/native/mlp_step_bench.cpp reads"""
     with open(path, "wb") as f:
         for a in [x, t] + [params[f"linear{i}.{n}"] for i in (1, 2, 3) for n in ("weight", "bias")]:
             f.write(np.ascontiguousarray(a, dtype=np.float32).tobytes())
@@ -83,9 +83,9 @@ def test_compiled_host_step_matches_python_host(hip, tmp_path):
     the losses of the first steps agree to rounding noise of the launch-order-independent kernels"""
     import os
     import subprocess
-    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "tests", "native", "bin", "mlp_step_bench")
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "harness", "native", "bin", "mlp_step_bench")
     if not os.path.exists(exe):
-        pytest.skip("tests/native/bin/mlp_step_bench is not built (run __graft_entry__.build())")
+        pytest.skip("harness/native/bin/mlp_step_bench is not built (run __graft_entry__.build())")
     x, t, params = mlp_step.make_inputs()
     write_inputs(tmp_path / "inputs.bin", x, t, params)
     out = subprocess.run([exe, "--inputs", str(tmp_path / "inputs.bin"), "--dump-loss", "3", "--steps", "2", "--warmup", "0"],
@@ -93,7 +93,7 @@ def test_compiled_host_step_matches_python_host(hip, tmp_path):
     print(out.stdout, flush=True)
     assert out.returncode == 0, out.stdout + out.stderr
     got = {(l.split()[0], int(l.split()[2])): float(l.split()[3]) for l in out.stdout.splitlines() if " loss " in l}
-    dev = mlp_devices.HipDev(hip)
+    dev = hip_dev.HipDev(hip)
     for fused in (False, True):
         st = mlp_step.MlpStep(dev, x, t, params, fused=fused)
         for step in (1, 2, 3):
@@ -109,8 +109,8 @@ def test_compiled_host_step_matches_python_host(hip, tmp_path):
 def test_hip_step_matches_cpu_step(hip):
     import zenu_oracle as zo
     x, t, params = mlp_step.make_inputs()
-    cpu = mlp_step.MlpStep(mlp_devices.CpuDev(), x, t, params)
-    dev = mlp_devices.HipDev(hip)
+    cpu = mlp_step.MlpStep(cpu_dev.CpuDev(), x, t, params)
+    dev = hip_dev.HipDev(hip)
     gpu = mlp_step.MlpStep(dev, x, t, params)
     losses = []
     for step in range(1, 4):
