@@ -19,8 +19,9 @@
 //            128-bit loads in 128-byte segments, turned through LDS (pitch 65 words, eight lanes
 //            per segment: no bank conflicts in either direction, checked with the hardware
 //            counter), and every HBM access stays coalesced.                        [HBM bound]
-//   generic: anything else (strided output, gathers): one element per thread, index arithmetic
-//            per element.
+//   strided: anything else (a strided destination, gathers, views without a unit-stride dim):
+//            lanes along the innermost dim whatever its stride, the outer index decomposed once
+//            per thread, four elements per thread with the loads issued first.
 //
 // Arithmetic is plain IEEE with contraction off; + - * / sqrt are correctly rounded on gfx950,
 // so results are bit-identical to the CPU loops of basic_operations.rs:93-181.
@@ -583,25 +584,54 @@ __global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, con
     }
 }
 
-// ---- kernel 4: generic -----------------------------------------------------------------------------
+// ---- kernel 4: strided rows (anything else) ----------------------------------------------------------
+// Operands whose innermost (collapsed) dim has any stride: a strided destination (out[:, ::2] = ...),
+// gathers (a[:, ::2] + b), views without a unit-stride dim.  The threads of a workgroup form
+// (ty rows) x (tx columns) with the columns along the innermost dim, so consecutive lanes touch
+// addresses one inner stride apart (as coalesced as the view allows); the outer index is
+// decomposed once per thread, not per element, and an element's offset is column * stride.
 
-struct GenericParams {
-    OuterDesc dims;  // all collapsed dims
-    int64_t numel;
+struct StridedRowsParams {
+    OuterDesc outer;
+    int64_t nrows, ncols;
+    int64_t inner[kMaxOperands];   // stride along the innermost dim per operand (any value)
+    int tx_shift;
+    int64_t col_tiles;
 };
 
-template <typename T, typename F>
-__global__ __launch_bounds__(kBlock) void ew_generic_kernel(T *out, const T *a, const T *b,
-                                                            GenericParams p, F f)
+template <typename T, typename F, int kUnroll>
+__global__ __launch_bounds__(kBlock) void ew_strided_rows_kernel(T *out, const T *a, const T *b,
+                                                                 StridedRowsParams p, F f)
 {
     f.init();
-    const int64_t step = (int64_t)gridDim.x * kBlock;
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < p.numel; i += step) {
-        int64_t oo, oa, ob;
-        decompose(p.dims, i, oo, oa, ob);
-        T x = a[oa];
-        T y = (F::NIN == 2) ? b[ob] : x;
-        out[oo] = f(x, y);
+    const int tx_n = 1 << p.tx_shift;
+    const int ty_n = kBlock >> p.tx_shift;
+    const int tx = threadIdx.x & (tx_n - 1);
+    const int ty = threadIdx.x >> p.tx_shift;
+    const uint32_t row_blk32 = blockIdx.x / (uint32_t)p.col_tiles;   // grid and col_tiles fit 32 bits (checked at launch)
+    const int64_t col_tile = blockIdx.x - row_blk32 * (uint32_t)p.col_tiles;
+    const int64_t row = (int64_t)row_blk32 * ty_n + ty;
+    if (row >= p.nrows) return;
+    int64_t oo, oa, ob;
+    decompose(p.outer, row, oo, oa, ob);
+    T *orow = out + oo;
+    const T *arow = a + oa;
+    const T *brow = (F::NIN == 2) ? b + ob : arow;
+    const int64_t so = p.inner[0], sa = p.inner[1], sb = p.inner[2];
+    const int64_t c0 = col_tile * ((int64_t)tx_n * kUnroll) + tx;
+    T x[kUnroll], y[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {          // all loads of the thread first
+        const int64_t c = c0 + (int64_t)u * tx_n;
+        if (c < p.ncols) {
+            x[u] = arow[c * sa];
+            y[u] = (F::NIN == 2) ? brow[c * sb] : x[u];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+        const int64_t c = c0 + (int64_t)u * tx_n;
+        if (c < p.ncols) orow[c * so] = f(x[u], y[u]);
     }
 }
 
@@ -842,19 +872,27 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
         }
     }
 
-    // generic
-    GenericParams gp;
-    gp.dims.nouter = p.ndim;
+    // strided rows: rows = everything but the innermost dim
+    StridedRowsParams sp;
+    sp.outer.nouter = p.ndim - 1;
     for (int d = 0; d < kMaxDim; d++) {
-        gp.dims.shape[d] = d < p.ndim ? p.shape[d] : 1;
+        sp.outer.shape[d] = d < p.ndim - 1 ? p.shape[d] : 1;
         for (int o = 0; o < kMaxOperands; o++)
-            gp.dims.stride[o][d] = (d < p.ndim && o < p.nops) ? p.stride[o][d] : 0;
+            sp.outer.stride[o][d] = (d < p.ndim - 1 && o < p.nops) ? p.stride[o][d] : 0;
     }
-    gp.numel = p.numel;
-    int64_t grid = (p.numel + kBlock - 1) / kBlock;
-    int64_t cap = (int64_t)device_info().num_cus * 32;
-    if (grid > cap) grid = cap;
-    ew_generic_kernel<T, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, gp, f);
+    sp.ncols = p.shape[last];
+    sp.nrows = p.numel / sp.ncols;
+    for (int o = 0; o < kMaxOperands; o++) sp.inner[o] = o < p.nops ? p.stride[o][last] : 0;
+    constexpr int kStridedUnroll = 4;
+    int shift = 0;
+    while ((1 << shift) < kBlock && ((int64_t)1 << shift) < sp.ncols) shift++;
+    sp.tx_shift = shift;
+    const int64_t cols_per_tile = ((int64_t)1 << shift) * kStridedUnroll;
+    sp.col_tiles = (sp.ncols + cols_per_tile - 1) / cols_per_tile;
+    const int64_t rows_per_blk = kBlock >> shift;
+    const int64_t grid = ((sp.nrows + rows_per_blk - 1) / rows_per_blk) * sp.col_tiles;
+    if (grid > 0x7fffffffLL || sp.col_tiles > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
+    ew_strided_rows_kernel<T, F, kStridedUnroll><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, sp, f);
     ZENU_LAUNCH_CHECK();
     return ZENU_OK;
 }

@@ -171,6 +171,25 @@ ZM_HD float tanhf_fdlibm(float x)
     return neg ? -z : z;
 }
 
+// Quotient a / b for the two divisions inside tanhf_simd.  On the device: reciprocal estimate,
+// product, one correction of the quotient by its exact remainder (4 instructions against the 11
+// of the IEEE sequence with its operand scaling and fix-up).  That sequence is not correctly
+// rounded for every pair of operands, but it is for every pair tanhf_simd feeds it (divisors in
+// [5, 7] and [1, 2^30], no overflow, no underflow of the remainder): the kernel's results equal
+// the host library's on all 2^32 arguments (tests/test_exhaustive_device.py).  The host build
+// divides; it checks everything but this sequence.
+ZM_HD float div_tanh(float a, float b)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    const float r = __builtin_amdgcn_rcpf(b);
+    const float q = a * r;
+    const float rem = __builtin_fmaf(-b, q, a);
+    return __builtin_fmaf(rem, r, q);
+#else
+    return a / b;
+#endif
+}
+
 // The same tanh, restructured for 64-wide SIMD execution: one path through the argument
 // reduction, the rational core and ONE division pair for every lane, the per-k tails computed
 // side by side and selected, so that a wavefront whose lanes hold |x| on both sides of 1 and
@@ -178,6 +197,21 @@ ZM_HD float tanhf_fdlibm(float x)
 // arithmetic operation that reaches the result is the one tanhf_fdlibm performs, on the same
 // operands, so the bits are identical; this is checked over every f32 bit pattern against
 // tanhf_fdlibm and the host libm (tests/native/zmath_host_check.cpp).
+//
+// The kernel is bound by its vector instructions (about 0.4 us per instruction and element on
+// 2^24 elements), so the count is what matters.  What was removed without changing a bit:
+//   * hi = a - k*ln2_hi is one fused multiply-add: k*ln2_hi is exact (ln2_hi ends in 7 zero bits,
+//     |k| < 64), so fusing does not change the rounding;
+//   * the special cases |a| < 2^-25 (expm1 returns a) and |x| < 2^-55 (tanh returns x*(1+x)) need
+//     no select: the k = 0 formula returns a there (its correction term is below half a unit in
+//     the last place), and -a/(a+2) is then |x| exactly;
+//   * k == -1: 0.5*(xr - e1) - 0.5 = -0.5*(e1 - xr) - 0.5 shares e1 - xr with the other tails;
+//   * k <= -2 and 2 <= k < 23 are one formula, A - (e1 - xr) scaled by 2^k, with A = 1 (and a
+//     final - 1) or A = 1 - 2^-k;
+//   * |x| >= 9.02: 2/(expm1(2|x|) + 2) is below 2^-25 and vanishes against 1, so any large em1
+//     gives the result 1 (fdlibm takes its k > 56 tail and its |x| >= 22 exit for this);
+//     everything rare (k >= 23, i.e. |x| >= 7.8, and non-finite x) sits behind one test;
+//   * the sign goes back with one bit operation.
 ZM_HD float tanhf_simd(float x)
 {
     const float one = 1.0f, two = 2.0f;
@@ -186,24 +220,20 @@ ZM_HD float tanhf_simd(float x)
                 Q4 = u2f(0x36867e54u), Q5 = u2f(0xb457edbbu);
     const uint32_t jx = f2u(x);
     const uint32_t ix = jx & 0x7fffffffu;
-    const bool neg = (jx >> 31) != 0;
-
-    if (ix >= 0x41b00000u) {                 // |x| >= 22, inf, NaN (rare)
-        if (ix >= 0x7f800000u) return neg ? one / x - one : one / x + one;
-        return neg ? -one : one;             // 1 - tiny rounds to 1
-    }
-    if (ix < 0x24000000u) return ix == 0 ? x : x * (one + x);   // |x| < 2^-55
-
     const float ax = u2f(ix);
     const bool big = ix >= 0x3f800000u;      // |x| >= 1: expm1(+2|x|), else expm1(-2|x|)
-    const float a = big ? two * ax : -two * ax;
-    const uint32_t ha = f2u(a) & 0x7fffffffu;
+    const float a2 = ax + ax;
+    const float a = big ? a2 : -a2;
 
-    // expm1(a), a in (-2, 0) or [2, 44): k = round(a / ln2) when |a| > 0.5 ln2, else 0
+    // expm1(a), a in (-2, 0] or [2, 44): k = round(a / ln2) when |a| > 0.5 ln2, else 0
     int32_t k = (int32_t)(invln2 * a + (big ? 0.5f : -0.5f));
-    k = (ha > 0x3eb17218u) ? k : 0;
+    k = (f2u(a2) > 0x3eb17218u) ? k : 0;
     const float tk = (float)k;
-    const float hi = a - tk * ln2_hi;
+#if defined(__HIP_DEVICE_COMPILE__)
+    const float hi = __builtin_fmaf(-tk, ln2_hi, a);
+#else
+    const float hi = a - tk * ln2_hi;        // the product is exact: same value
+#endif
     const float lo = tk * ln2_lo;
     const float xr = hi - lo;
     const float c = (hi - xr) - lo;
@@ -211,39 +241,35 @@ ZM_HD float tanhf_simd(float x)
     const float hfx = 0.5f * xr;
     const float hxs = xr * hfx;
     const float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
-    float t = 3.0f - r1 * hfx;
-    const float e = hxs * ((r1 - t) / (6.0f - xr * t));
+    const float t = 3.0f - r1 * hfx;
+    const float e = hxs * div_tanh(r1 - t, 6.0f - xr * t);
 
-    float em1;                               // expm1(a)
-    if (ha < 0x33000000u) {
-        em1 = a;                             // |a| < 2^-25
-    } else if (k == 0) {
-        em1 = xr - (xr * e - hxs);
-    } else {
-        float e1 = (xr * (e - c) - c);
-        e1 -= hxs;
-        if (k == -1) {
-            em1 = 0.5f * (xr - e1) - 0.5f;
-        } else if (k <= -2 || k > 56) {
-            float y = one - (e1 - xr);
-            y = u2f(f2u(y) + ((uint32_t)k << 23));
-            em1 = y - one;
-        } else if (k < 23) {                 // 2 <= k < 23 here (k == 1 needs |a| < 1.5 ln2 < 2)
-            const float tt = u2f(0x3f800000u - (0x1000000u >> k));
-            float y = tt - (e1 - xr);
-            em1 = u2f(f2u(y) + ((uint32_t)k << 23));
-        } else {
-            const float tt = u2f((uint32_t)(0x7f - k) << 23);
-            float y = xr - (e1 + tt);
-            y += one;
-            em1 = u2f(f2u(y) + ((uint32_t)k << 23));
+    const float m0 = xr - (xr * e - hxs);                // k == 0
+    float e1 = xr * (e - c) - c;
+    e1 -= hxs;
+    const float d = e1 - xr;
+    const float mneg1 = -0.5f * d - 0.5f;                // k == -1
+    const bool kpos = k >= 2;                            // 2 <= k < 23: (1 - 2^-k) - d, scaled; k <= -2: (1 - d) scaled, - 1
+    const float tt = u2f(0x3f800000u - (0x1000000u >> (k & 31)));
+    const float y = (kpos ? tt : one) - d;
+    const float ys = u2f(f2u(y) + ((uint32_t)k << 23));
+    float em1 = kpos ? ys : ys - one;
+    em1 = (k == -1) ? mneg1 : em1;
+    em1 = (k == 0) ? m0 : em1;
+    if (ix >= 0x40f00000u) {                             // |x| >= 7.5 (rare)
+        if (k >= 23) {                                   // 2^-k no longer fits next to 1
+            const float t2 = u2f((uint32_t)(0x7f - k) << 23);
+            float y2 = xr - (e1 + t2);
+            y2 += one;
+            em1 = u2f(f2u(y2) + ((uint32_t)k << 23));
         }
+        if (ix >= 0x411051ecu) em1 = u2f(0x4e800000u);   // |x| >= 9.02: the result is 1 for any large em1
+        if (ix > 0x7f800000u) em1 = x;                   // NaN stays NaN
     }
     // |x| >= 1: 1 - 2/(t+2);  |x| < 1: -t/(t+2) = -(t/(t+2))
-    const float num = big ? two : em1;
-    const float q = num / (em1 + two);
+    const float q = div_tanh(big ? two : em1, em1 + two);
     const float z = big ? one - q : -q;
-    return neg ? -z : z;
+    return u2f((f2u(z) & 0x7fffffffu) | (jx & 0x80000000u));
 }
 
 // ---- f32 exp and log: the table-driven routines glibc ships since 2.27 (from ARM's optimized routines) ----
