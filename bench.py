@@ -291,6 +291,25 @@ def build_ops(z, workload, stream):
             ops.append(Op(name, "next", "f32", 2 * nb, n * n,
                           mk(lambda A, P, U, R, O, V, S, fn=fn, src=src: (lambda d=O.desc(), s_=(A, P, U)[src].desc(): check(l.zenu_hip_unary(fn, _lib.F32, ref(d), ref(s_), stream), "unary"))),
                           lambda fn=fn, host=host: zo.unary(fn, out_h, host)))
+        # views that none of the contiguous / row / tile kernels take: a strided destination, a gather, and a
+        # 4-d permuted copy (NCHW -> NHWC of [64,64,64,64], the tile kernel with two batch dims)
+        half = n // 2
+        ops.append(Op("out[:, ::2] = a[:, :half] + b[:, :half] (strided destination)", "next", "f32", 3 * nb // 2, n * half,
+                      mk(lambda A, P, U, R, O, V, S: (lambda d=O.slice(slice(None), slice(0, n, 2)).desc(), x=A.slice(slice(None), slice(0, half)).desc(),
+                                                             y=P.slice(slice(None), slice(0, half)).desc():
+                                                      check(l.zenu_hip_binary(_lib.ADD, _lib.F32, ref(d), ref(x), ref(y), stream), "strided dst"))),
+                      lambda: zo.binary_array(zo.ADD, out_h[:, ::2], a[:, :half], pos[:, :half])))
+        ops.append(Op("out[:, :half] = a[:, ::2] + b[:, :half] (gather)", "next", "f32", 3 * nb // 2, n * half,
+                      mk(lambda A, P, U, R, O, V, S: (lambda d=O.slice(slice(None), slice(0, half)).desc(), x=A.slice(slice(None), slice(0, n, 2)).desc(),
+                                                             y=P.slice(slice(None), slice(0, half)).desc():
+                                                      check(l.zenu_hip_binary(_lib.ADD, _lib.F32, ref(d), ref(x), ref(y), stream), "gather"))),
+                      lambda: zo.binary_array(zo.ADD, out_h[:, :half], a[:, ::2], pos[:, :half])))
+        a4 = a.reshape(64, 64, 64, 64)
+        o4 = out_h.reshape(64, 64, 64, 64)
+        ops.append(Op("4-d permuted copy NCHW -> NHWC [64,64,64,64]", "next", "f32", 2 * nb, n * n,
+                      mk(lambda A, P, U, R, O, V, S: (lambda d=O.reshape((64, 64, 64, 64)).desc(), s_=A.reshape((64, 64, 64, 64)).transpose_by_index([0, 2, 3, 1]).desc():
+                                                      check(l.zenu_hip_copy(_lib.F32, ref(d), ref(s_), stream), "permute"))),
+                      lambda: zo.copy_from(o4, a4.transpose(0, 2, 3, 1))))
         ops.append(Op("tanh, the <= 2 ulp variant (ZENU_TANH_ULP2)", "next", "f32", 2 * nb, n * n,
                       mk(lambda A, P, U, R, O, V, S: (lambda d=O.desc(), s_=A.desc(): check(l.zenu_hip_unary(_lib.TANH_ULP2, _lib.F32, ref(d), ref(s_), stream), "unary"))),
                       lambda: zo.unary(zo.TANH, out_h, a)))

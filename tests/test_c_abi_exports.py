@@ -52,3 +52,21 @@ def test_shape_errors_need_no_gpu():
     assert lib.zenu_hip_unary(_lib.EXP, _lib.F32, ctypes.byref(t), ctypes.byref(t), None) == _lib.ERR_ARG
     assert lib.zenu_hip_binary(_lib.ADD, _lib.F32, None, None, None, None) == _lib.ERR_ARG
     assert lib.zenu_hip_sgd_step(_lib.F32, None, None, -1, 0.1, None) == _lib.ERR_ARG
+
+
+def test_void_entry_points_leave_a_sticky_status():
+    """the reference-named functions return void; the first failure behind them stays readable per
+    thread until zenu_hip_last_status() clears it (host-side checks only: nothing is launched)"""
+    import zenu_amd
+    from zenu_amd import _lib
+    lib = zenu_amd.lib()
+    f = ctypes.POINTER(ctypes.c_float)
+    lib.array_exp_float.argtypes = [f, ctypes.c_int, ctypes.c_int, f, ctypes.c_int]
+    lib.array_exp_float.restype = None
+    lib.array_array_add_float.argtypes = [f, ctypes.c_int, f, ctypes.c_int, f, ctypes.c_int, ctypes.c_int]
+    lib.array_array_add_float.restype = None
+    assert lib.zenu_hip_last_status() == _lib.OK
+    lib.array_exp_float(None, -5, 1, None, 1)                 # a negative element count
+    lib.array_array_add_float(None, 1, None, 1, None, 1, -1)  # a second failure: the first one is kept
+    assert lib.zenu_hip_last_status() == _lib.ERR_ARG
+    assert lib.zenu_hip_last_status() == _lib.OK              # read once, then clear

@@ -47,6 +47,7 @@ SIGNATURES = {
     "zenu_hip_init": [_i],
     "zenu_hip_shutdown": [],
     "zenu_hip_last_hip_error": [],
+    "zenu_hip_last_status": [],
     "zenu_hip_stream_create": [C.POINTER(_vp)],
     "zenu_hip_stream_destroy": [_vp],
     "zenu_hip_stream_synchronize": [_vp],

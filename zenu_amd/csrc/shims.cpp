@@ -2,10 +2,18 @@
 // unchanged wrappers of zenu-cuda/src/kernel/mod.rs and kernel/activation.rs link against this
 // library.  Same names, same argument order, `int` sizes and element strides, launches on the
 // null stream, no return value (the reference's functions return void and check nothing).
-// Each one forwards to the N-d entry point with a 1-D strided view.
+// Each one forwards to the N-d entry point with a 1-D strided view.  A status that the void
+// signature cannot return is kept per thread: the first failure since the last call of
+// zenu_hip_last_status() stays there until that call reads and clears it.
 #include "common.hpp"
 
 namespace {
+
+thread_local int tl_sticky_status = ZENU_OK;
+inline void note(int rc)
+{
+    if (rc != ZENU_OK && tl_sticky_status == ZENU_OK) tl_sticky_status = rc;
+}
 
 zenu_tensor_t view1d(const void *p, int n, int stride)
 {
@@ -27,42 +35,42 @@ template <typename T>
 void aa(int op, T *a, int sa, T *b, int sb, T *c, int sc, int n)
 {
     zenu_tensor_t ta = view1d(a, n, sa), tb = view1d(b, n, sb), tc = view1d(c, n, sc);
-    (void)zenu_hip_binary(op, dtype_of<T>(), &tc, &ta, &tb, nullptr);
+    note(zenu_hip_binary(op, dtype_of<T>(), &tc, &ta, &tb, nullptr));
 }
 template <typename T> void aa_assign(int op, T *a, int sa, T *b, int sb, int n)
 {
     zenu_tensor_t ta = view1d(a, n, sa), tb = view1d(b, n, sb);
-    (void)zenu_hip_binary_assign(op, dtype_of<T>(), &ta, &tb, nullptr);
+    note(zenu_hip_binary_assign(op, dtype_of<T>(), &ta, &tb, nullptr));
 }
 template <typename T> void as(int op, T *a, int n, int sa, T s, T *out, int so)
 {
     zenu_tensor_t ta = view1d(a, n, sa), to = view1d(out, n, so);
-    (void)zenu_hip_binary_scalar(op, dtype_of<T>(), &to, &ta, (double)s, nullptr);
+    note(zenu_hip_binary_scalar(op, dtype_of<T>(), &to, &ta, (double)s, nullptr));
 }
 template <typename T> void as_assign(int op, T *a, int n, int sa, T s)
 {
     zenu_tensor_t ta = view1d(a, n, sa);
-    (void)zenu_hip_binary_scalar_assign(op, dtype_of<T>(), &ta, (double)s, nullptr);
+    note(zenu_hip_binary_scalar_assign(op, dtype_of<T>(), &ta, (double)s, nullptr));
 }
 template <typename T> void asp(int op, T *a, int n, int sa, T *s, T *out, int so)
 {
     zenu_tensor_t ta = view1d(a, n, sa), to = view1d(out, n, so);
-    (void)zenu_hip_binary_scalar_ptr(op, dtype_of<T>(), &to, &ta, s, nullptr);
+    note(zenu_hip_binary_scalar_ptr(op, dtype_of<T>(), &to, &ta, s, nullptr));
 }
 template <typename T> void asp_assign(int op, T *a, int n, int sa, T *s)
 {
     zenu_tensor_t ta = view1d(a, n, sa);
-    (void)zenu_hip_binary_scalar_assign_ptr(op, dtype_of<T>(), &ta, s, nullptr);
+    note(zenu_hip_binary_scalar_assign_ptr(op, dtype_of<T>(), &ta, s, nullptr));
 }
 template <typename T> void un(int fn, T *a, int n, int si, T *out, int so)
 {
     zenu_tensor_t ta = view1d(a, n, si), to = view1d(out, n, so);
-    (void)zenu_hip_unary(fn, dtype_of<T>(), &to, &ta, nullptr);
+    note(zenu_hip_unary(fn, dtype_of<T>(), &to, &ta, nullptr));
 }
 template <typename T> void un_assign(int fn, T *a, int n, int s)
 {
     zenu_tensor_t ta = view1d(a, n, s);
-    (void)zenu_hip_unary_assign(fn, dtype_of<T>(), &ta, nullptr);
+    note(zenu_hip_unary_assign(fn, dtype_of<T>(), &ta, nullptr));
 }
 
 zenu_tensor_t view3d(const void *p, int64_t d0, int64_t d1, int64_t d2, int64_t s0, int64_t s1, int64_t s2)
@@ -85,19 +93,19 @@ void conv_bias(const T *in, T *out, int cs, const T *bias, int C, int total)
     if (images > 0) {
         zenu_tensor_t ti = view3d(in, images, C, cs, image, cs, 1), to = view3d(out, images, C, cs, image, cs, 1);
         zenu_tensor_t tb = view3d(bias, 1, C, 1, C, 1, 1);
-        (void)zenu_hip_binary(ZENU_ADD, dtype_of<T>(), &to, &ti, &tb, nullptr);
+        note(zenu_hip_binary(ZENU_ADD, dtype_of<T>(), &to, &ti, &tb, nullptr));
     }
     int64_t done = images * image;
     const int64_t chans = (total - done) / cs;
     if (chans > 0) {
         zenu_tensor_t ti = view3d(in + done, 1, chans, cs, image, cs, 1), to = view3d(out + done, 1, chans, cs, image, cs, 1);
         zenu_tensor_t tb = view3d(bias, 1, chans, 1, C, 1, 1);
-        (void)zenu_hip_binary(ZENU_ADD, dtype_of<T>(), &to, &ti, &tb, nullptr);
+        note(zenu_hip_binary(ZENU_ADD, dtype_of<T>(), &to, &ti, &tb, nullptr));
         done += chans * cs;
     }
     if (done < total) {
         zenu_tensor_t ti = view1d(in + done, (int)(total - done), 1), to = view1d(out + done, (int)(total - done), 1);
-        (void)zenu_hip_binary_scalar_ptr(ZENU_ADD, dtype_of<T>(), &to, &ti, bias + chans, nullptr);
+        note(zenu_hip_binary_scalar_ptr(ZENU_ADD, dtype_of<T>(), &to, &ti, bias + chans, nullptr));
     }
 }
 
@@ -119,7 +127,7 @@ template <typename T> void conv_bias_bkwd(const T *dout, T *dbias, int N, int C,
         dst.shape[i] = (i == 1) ? C : 1;
         dst.stride[i] = (i == 0) ? C : 1;
     }
-    (void)zenu_hip_sum_to(dtype_of<T>(), &dst, &src, nullptr);
+    note(zenu_hip_sum_to(dtype_of<T>(), &dst, &src, nullptr));
 }
 
 template <typename T> void max_idx(T *a, int size, int stride, int *out)
@@ -127,17 +135,26 @@ template <typename T> void max_idx(T *a, int size, int stride, int *out)
     // `out` is host memory (zenu-cuda/src/kernel/mod.rs:570-588): blocking, like the reference
     zenu_tensor_t ta = view1d(a, size, stride);
     void *d = nullptr;
-    if (zenu_hip_malloc(&d, sizeof(int64_t), nullptr) != ZENU_OK) return;
+    int rc = zenu_hip_malloc(&d, sizeof(int64_t), nullptr);
+    if (rc != ZENU_OK) { note(rc); return; }
     int64_t h = 0;
-    if (zenu_hip_max_idx(dtype_of<T>(), static_cast<int64_t *>(d), nullptr, &ta, nullptr) == ZENU_OK &&
-        zenu_hip_memcpy_d2h(&h, d, sizeof h, nullptr) == ZENU_OK)
-        *out = (int)h;
-    (void)zenu_hip_free(d, nullptr);
+    rc = zenu_hip_max_idx(dtype_of<T>(), static_cast<int64_t *>(d), nullptr, &ta, nullptr);
+    if (rc == ZENU_OK) rc = zenu_hip_memcpy_d2h(&h, d, sizeof h, nullptr);
+    if (rc == ZENU_OK) *out = (int)h;
+    note(rc);
+    note(zenu_hip_free(d, nullptr));
 }
 
 }  // namespace
 
 extern "C" {
+
+int zenu_hip_last_status(void)
+{
+    const int rc = tl_sticky_status;
+    tl_sticky_status = ZENU_OK;
+    return rc;
+}
 
 #define ZENU_DEF_1D(T, S)                                                                                  \
     void array_array_add_##S(T *a, int sa, T *b, int sb, T *c, int sc, int n) { aa<T>(ZENU_ADD, a, sa, b, sb, c, sc, n); } \
@@ -193,32 +210,32 @@ extern "C" {
     void array_pow_##S(T *a, int n, int sa, T scalar, T *o, int so)                                        \
     {                                                                                                      \
         zenu_tensor_t ti = view1d(a, n, sa), to = view1d(o, n, so);                                        \
-        (void)zenu_hip_powf(dtype_of<T>(), &to, &ti, (double)scalar, nullptr);                             \
+        note(zenu_hip_powf(dtype_of<T>(), &to, &ti, (double)scalar, nullptr));                             \
     }                                                                                                      \
     void array_pow_assign_##S(T *a, int n, int s, T scalar)                                                \
     {                                                                                                      \
         zenu_tensor_t t = view1d(a, n, s);                                                                 \
-        (void)zenu_hip_powf(dtype_of<T>(), &t, &t, (double)scalar, nullptr);                               \
+        note(zenu_hip_powf(dtype_of<T>(), &t, &t, (double)scalar, nullptr));                               \
     }                                                                                                      \
     void array_clip_##S(T *in, T *out, int n, int si, int so, T lo, T hi)                                  \
     {                                                                                                      \
         zenu_tensor_t ti = view1d(in, n, si), to = view1d(out, n, so);                                     \
-        (void)zenu_hip_clip(dtype_of<T>(), &to, &ti, (double)lo, (double)hi, nullptr);                     \
+        note(zenu_hip_clip(dtype_of<T>(), &to, &ti, (double)lo, (double)hi, nullptr));                     \
     }                                                                                                      \
     void array_clip_assign_##S(T *a, int n, int s, T lo, T hi)                                             \
     {                                                                                                      \
         zenu_tensor_t t = view1d(a, n, s);                                                                 \
-        (void)zenu_hip_clip(dtype_of<T>(), &t, &t, (double)lo, (double)hi, nullptr);                       \
+        note(zenu_hip_clip(dtype_of<T>(), &t, &t, (double)lo, (double)hi, nullptr));                       \
     }                                                                                                      \
     void array_clip_backward_##S(T *in, T *mask, T hi, T lo, int n, int si, int sm)                        \
     {                                                                                                      \
         zenu_tensor_t ti = view1d(in, n, si), tm = view1d(mask, n, sm);                                    \
-        (void)zenu_hip_clip_backward_mask(dtype_of<T>(), &tm, &ti, (double)lo, (double)hi, nullptr);       \
+        note(zenu_hip_clip_backward_mask(dtype_of<T>(), &tm, &ti, (double)lo, (double)hi, nullptr));       \
     }                                                                                                      \
     void array_clip_backward_assign_##S(T *a, T hi, T lo, int n, int s)                                    \
     {                                                                                                      \
         zenu_tensor_t t = view1d(a, n, s);                                                                 \
-        (void)zenu_hip_clip_backward_mask(dtype_of<T>(), &t, &t, (double)lo, (double)hi, nullptr);         \
+        note(zenu_hip_clip_backward_mask(dtype_of<T>(), &t, &t, (double)lo, (double)hi, nullptr));         \
     }                                                                                                      \
     void conv_bias_add_##S(const T *in, T *out, int channel_stride, const T *bias, int bias_size, int total) \
     {                                                                                                      \
@@ -231,21 +248,21 @@ extern "C" {
     void relu_##S(T *in, T *out, T alpha, int n, int si, int so)                                           \
     {                                                                                                      \
         zenu_tensor_t ti = view1d(in, n, si), to = view1d(out, n, so);                                     \
-        (void)zenu_hip_relu(dtype_of<T>(), &to, &ti, (double)alpha, nullptr);                              \
+        note(zenu_hip_relu(dtype_of<T>(), &to, &ti, (double)alpha, nullptr));                              \
     }                                                                                                      \
     void relu_backward_mask_##S(T *in, T *mask, T alpha, int n, int si, int sm)                            \
     {                                                                                                      \
         zenu_tensor_t ti = view1d(in, n, si), tm = view1d(mask, n, sm);                                    \
-        (void)zenu_hip_relu_backward_mask(dtype_of<T>(), &tm, &ti, (double)alpha, nullptr);                \
+        note(zenu_hip_relu_backward_mask(dtype_of<T>(), &tm, &ti, (double)alpha, nullptr));                \
     }                                                                                                      \
     void array_max_idx_##S(T *a, int size, int stride, int *out) { max_idx<T>(a, size, stride, out); }     \
     void memory_access_##S(T *array, int offset, T *result)                                                \
     {                                                                                                      \
-        (void)zenu_hip_memcpy_d2h(result, array + offset, sizeof(T), nullptr);                             \
+        note(zenu_hip_memcpy_d2h(result, array + offset, sizeof(T), nullptr));                             \
     }                                                                                                      \
     void memory_set_##S(T *array, int offset, T value)                                                     \
     {                                                                                                      \
-        (void)zenu_hip_memcpy_h2d(array + offset, &value, sizeof(T), nullptr);                             \
+        note(zenu_hip_memcpy_h2d(array + offset, &value, sizeof(T), nullptr));                             \
     }
 
 ZENU_DEF_1D(float, float)
