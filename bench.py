@@ -173,7 +173,7 @@ def build_ops(z, workload, stream):
             return [fn(X.desc(), o0.desc(), o1.desc(), oi.as_ptr(), oa.as_ptr()) for X, o0, o1, oi, oa in sets]
         ops.append(Op(f"sum axis0 {dname}", "c2", dname, inb + 4096 * isz, x.size,
                       mk(lambda dx, d0, d1, pi, pa: (lambda: check(l.zenu_hip_sum_axis(dcode, ref(d0), ref(dx), 0, stream), "sum0"))),
-                      lambda: zo.sum_axis(x, 0)))
+                      lambda: zo.sum_axis(x, 0), kernel=f"reduce_cols_kernel<{'float' if dname == 'f32' else 'double'}, SumTr, {16 // isz}, true>"))
         ops.append(Op(f"sum axis1 {dname}", "c2", dname, inb + 8192 * isz, x.size,
                       mk(lambda dx, d0, d1, pi, pa: (lambda: check(l.zenu_hip_sum_axis(dcode, ref(d1), ref(dx), 1, stream), "sum1"))),
                       lambda: zo.sum_axis(x, 1)))
@@ -570,19 +570,54 @@ def capture_and_replay_c4(z, st, args, sync):
         return {"error": repr(e)}
 
 
+# ops whose HBM traffic was measured with rocprofv3 --pmc: op name -> (summary under profiles/, the
+# sources that define the op's kernel).  A summary records the hash of those sources at the time of
+# the counter run; if the kernel's sources have changed since, the figure is stale and not reported.
+TRAFFIC_PROFILES = {
+    "adamw 25M": ("adam_kernel_c3_adamw25M_pmc_traffic.txt",
+                  ("zenu_amd/csrc/optim.hip", "zenu_amd/csrc/vecmem.hpp", "zenu_amd/csrc/common.hpp")),
+    "sum axis0 f64": ("reduce_cols_kernel_c2_sum_axis0_f64_pmc_traffic.txt",
+                      ("zenu_amd/csrc/reduce.hip", "zenu_amd/csrc/vecmem.hpp", "zenu_amd/csrc/common.hpp")),
+}
+
+
+def kernel_sources_sha256(paths):
+    import hashlib
+    h = hashlib.sha256()
+    for rel in paths:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
 def measured_traffic(op):
-    """HBM bytes per launch of the op's kernel from the committed rocprofv3 --pmc summary
-    (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size), or None if not recorded."""
-    if op.config != "c3":
-        return None
-    path = os.path.join(ROOT, "profiles", "adam_kernel_c3_adamw25M_pmc_traffic.txt")
+    """(HBM bytes per launch of the op's kernel, note): FETCH_SIZE + WRITE_SIZE from the committed
+    rocprofv3 --pmc summary, each scaled by what the same counter reads for a copy kernel of known
+    size; (None, reason) when no summary exists or the kernel's sources have changed since it was made."""
+    if op.name not in TRAFFIC_PROFILES:
+        return None, "no counter run recorded for this op"
+    fname, sources = TRAFFIC_PROFILES[op.name]
+    fields = {}
     try:
-        for line in open(path):
-            if line.startswith("traffic_bytes_per_launch:"):
-                return int(line.split(":")[1])
+        for line in open(os.path.join(ROOT, "profiles", fname)):
+            if ":" in line:
+                k, v = line.split(":", 1)
+                fields[k.strip()] = v.strip()
     except OSError:
-        pass
-    return None
+        return None, f"profiles/{fname} is missing"
+    if "traffic_bytes_per_launch" not in fields:
+        return None, f"profiles/{fname} holds no traffic figure"
+    if fields.get("kernel_sources_sha256") != kernel_sources_sha256(sources):
+        return None, f"profiles/{fname} was made from other kernel sources ({', '.join(sources)} changed since): stale, not reported"
+    return int(fields["traffic_bytes_per_launch"]), f"profiles/{fname}"
+
+
+def roofline_of(row, op):
+    traffic, note = measured_traffic(op)
+    return dict(bound="hbm", achieved=row["GBps"], peak=PEAK_HBM_GBPS, unit="GB/s",
+                frac=round(row["GBps"] / PEAK_HBM_GBPS, 4), traffic=traffic, traffic_source=note,
+                kernel=op.kernel or row["op"], op=row["op"], algorithmic_bytes_per_launch=row["alg_bytes"],
+                avg_launch_us=row["us"])
 
 
 def main():
@@ -669,12 +704,11 @@ def main():
         log(f"[op] {o.name:22s} {us:9.2f} us  {gbps:8.1f} GB/s  {100 * gbps / PEAK_HBM_GBPS:5.1f}% of peak")
 
     # dominant kernel of the step = the op with the largest share of the step time
-    dom = max(table, key=lambda t: t["us"])
-    dom_op = [o for o in ops if o.name == dom["op"]][0]
-    roofline = dict(bound="hbm", achieved=dom["GBps"], peak=PEAK_HBM_GBPS, unit="GB/s",
-                    frac=round(dom["GBps"] / PEAK_HBM_GBPS, 4), traffic=measured_traffic(dom_op),
-                    kernel=dom_op.kernel or dom["op"], algorithmic_bytes_per_launch=dom["alg_bytes"],
-                    avg_launch_us=dom["us"])
+    by_time = sorted(table, key=lambda t: -t["us"])
+    dom = by_time[0]
+    roofline = roofline_of(dom, [o for o in ops if o.name == dom["op"]][0])
+    # the same figures for the second-largest op of the step
+    roofline_second = roofline_of(by_time[1], [o for o in ops if o.name == by_time[1]["op"]][0]) if len(by_time) > 1 else None
     adam = [t for t in table if t["config"] == "c3"]
 
     # ---- CPU baseline: the oracle, one thread, one pass of the same step -----------------------------------
@@ -721,7 +755,7 @@ def main():
                    "ops_per_step": len(table), "algorithmic_bytes_per_step": step_bytes},
         "frac_of_peak_whole_step": round(value / PEAK_HBM_GBPS, 4),
         "adam_step_params_per_sec": (round(adam[0]["Gelem_per_s"] * 1e9) if adam else None),
-        "roofline": roofline, "cpu_baseline": cpu, "c4": c4, "ops": table,
+        "roofline": roofline, "roofline_second_largest_op": roofline_second, "cpu_baseline": cpu, "c4": c4, "ops": table,
         "timing": f"HIP events on the launch stream; per op {args.op_reps} back-to-back launches after 10 warm-up launches: "
                   "us = batch mean, us_bracketed_* = per-launch event pairs (each includes one event record)",
     }

@@ -15,10 +15,11 @@
 //            outer index is decomposed once per thread, the inner dim is walked with 128-bit
 //            accesses; a broadcast row stays in L2.                                   [HBM bound]
 //   tile   : some input is contiguous along a different dim than the output (a transposed
-//            operand).  64x64 tiles: the transposed input is read along ITS contiguous dim with
-//            128-bit loads in 128-byte segments, turned through LDS (pitch 65 words, eight lanes
-//            per segment: no bank conflicts in either direction, checked with the hardware
-//            counter), and every HBM access stays coalesced.                        [HBM bound]
+//            operand).  64x64 tiles walked along diagonals, one thread per vector: the transposed
+//            input is read along ITS contiguous dim with 128-bit loads in 128-byte segments,
+//            turned through LDS (pitch 65 words, eight lanes per segment: no bank conflicts in
+//            either direction, checked with the hardware counter), and every HBM access stays
+//            coalesced.                                                               [HBM bound]
 //   strided: anything else (a strided destination, gathers, views without a unit-stride dim):
 //            lanes along the innermost dim whatever its stride, the outer index decomposed once
 //            per thread, four elements per thread with the loads issued first.
@@ -366,6 +367,25 @@ __device__ __forceinline__ void decompose(const OuterDesc &d, int64_t lin, int64
     }
 }
 
+// the same for an index that is known to fit 32 bits (then every dim does): no 64-bit division
+__device__ __forceinline__ void decompose32(const OuterDesc &d, uint32_t lin, int64_t &o0, int64_t &o1,
+                                            int64_t &o2)
+{
+    o0 = o1 = o2 = 0;
+    for (int k = d.nouter - 1; k >= 0; k--) {
+        uint32_t q = 0, r = lin;
+        if (k != 0) {
+            const uint32_t s32 = (uint32_t)d.shape[k];
+            q = lin / s32;
+            r = lin - q * s32;
+        }
+        o0 += (int64_t)r * d.stride[0][k];
+        o1 += (int64_t)r * d.stride[1][k];
+        o2 += (int64_t)r * d.stride[2][k];
+        lin = q;
+    }
+}
+
 // ---- kernel 2: rows (inner dim contiguous or broadcast) -------------------------------------------
 
 struct RowsParams {
@@ -446,8 +466,19 @@ __global__ __launch_bounds__(kBlock) void ew_rows_kernel(T *out, const T *a, con
 
 // ---- kernel 3: 64x64 tiles with an LDS turn for transposed inputs ----------------------------------
 
-// 64x64 tiles for f32 (16.6 KB of LDS per staged input), 32x32 for f64 (8.4 KB).
+// 64x64 tiles for f32 (16.6 KB of LDS per staged input), 32x32 for f64 (8.4 KB).  With one input
+// (a transposed or permuted copy, a unary op on such a view) one thread per 16-byte vector of the
+// tile (1024 / 512 threads): ONE vector per thread is the shape that streams one load and one
+// store stream fastest here, as for the contiguous kernels.  Transposed copy of [4096,4096] f32 in
+// a stand-alone probe, tiles walked along diagonals: 23.9 us, against 25.2 us with 256 threads and
+// four vectors each; 32x32 tiles with 256 threads copy as fast (24.1 us) but leave operands that
+// are not transposed with 128-byte row pieces.
 template <typename T> struct TileOf { static constexpr int N = sizeof(T) == 4 ? 64 : 32; };
+// With two inputs (three streams, a + b^T) four vectors per thread and operand at 256 threads keep
+// more bytes in flight per compute unit and win: 39.5 us against 41.1 us.
+template <typename T, typename F> struct TileThreads {
+    static constexpr int value = F::NIN == 1 ? TileOf<T>::N * TileOf<T>::N / VecOf<T>::N : 256;
+};
 
 struct TileParams {
     OuterDesc outer;      // batch dims (everything except the two tile dims)
@@ -457,15 +488,17 @@ struct TileParams {
     int64_t ldc[kMaxOperands];  // stride along C per operand (1 for out; 0/1 direct; ld for transposed)
     int trans_a, trans_b;       // input goes through LDS
     int vec_ok;                 // alignment allows 128-bit accesses on full tiles
+    int grid3d;                 // the grid is (tiles_c, tiles_r, nbatch); else linear, tiles_c fastest
     int64_t tiles_r, tiles_c;
 };
 
 template <typename T, bool NT, typename F>
-__global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, const T *b,
-                                                         TileParams p, F f)
+__global__ __launch_bounds__((TileThreads<T, F>::value)) void ew_tile_kernel(T *out, const T *a, const T *b,
+                                                                           TileParams p, F f)
 {
     constexpr int VEC = VecOf<T>::N;
     constexpr int kTile = TileOf<T>::N;
+    constexpr int kBlock = TileThreads<T, F>::value;   // shadows the engine-wide 256
     constexpr int kPitch = kTile + 1;
     // Eight lanes cover one 128-byte segment of a tile row; 32 segments per pass.  With eight (not
     // sixteen) lanes along the vector dim the 32 lanes that the LDS serves together -- eight
@@ -474,19 +507,35 @@ __global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, con
     // lanes per row alias pairwise (4 m and 4 (m + 8) share a bank) whatever the pitch.
     constexpr int VPS = 8;                  // vectors per segment
     constexpr int SEG = kTile / (VPS * VEC);// segments per tile row (2)
-    constexpr int RPP = kBlock / VPS;       // segments per pass (32)
-    static_assert(kTile % RPP == 0 && SEG >= 1, "tile geometry");
+    static_assert(SEG >= 1 && (kTile * SEG * VPS) % kBlock == 0, "tile geometry");
     __shared__ T lds_a[kTile * kPitch];
     __shared__ T lds_b[(F::NIN == 2) ? kTile * kPitch : 1];
     f.init();
 
-    int64_t blk = blockIdx.x;
-    const int64_t tc = blk % p.tiles_c;
-    blk /= p.tiles_c;
-    const int64_t tr = blk % p.tiles_r;
-    const int64_t batch = blk / p.tiles_r;
+    // Tiles are walked along diagonals: consecutive workgroups (which run together) differ in BOTH
+    // tile coordinates.  Walking a tile row, they would read (or, walking a tile column, write) row
+    // pieces whose addresses differ by multiples of the matrix pitch; with a power-of-two pitch those
+    // fall on the same few memory channels (transposed copy of [4096,4096]: 26.8 us row by row,
+    // 29.1 us column by column, 25.2 us diagonally with the same 64x64 tiles).
+    // The grid is (column tiles, row tiles, batch) when that fits the grid limits, so that no
+    // workgroup starts with a chain of integer divisions (in 64 bits they were most of this kernel's
+    // instructions); otherwise a linear grid below 2^31, decomposed in 32 bits.
+    uint32_t tc32, tr32, batch32;
+    if (p.grid3d) {
+        tc32 = blockIdx.x;
+        tr32 = blockIdx.y;
+        batch32 = blockIdx.z;
+    } else {
+        const uint32_t ntc = (uint32_t)p.tiles_c, ntr = (uint32_t)p.tiles_r;
+        const uint32_t q = blockIdx.x / ntc;
+        tc32 = blockIdx.x - q * ntc;
+        batch32 = q / ntr;
+        tr32 = q - batch32 * ntr;
+    }
+    tr32 = (tr32 + tc32) % (uint32_t)p.tiles_r;
+    const int64_t tc = tc32, tr = tr32;
     int64_t oo, oa, ob;
-    decompose(p.outer, batch, oo, oa, ob);
+    decompose32(p.outer, batch32, oo, oa, ob);
     const int64_t r0 = tr * kTile, c0 = tc * kTile;
     const int64_t nr = (p.R - r0 < kTile) ? p.R - r0 : kTile;
     const int64_t nc = (p.C - c0 < kTile) ? p.C - c0 : kTile;
@@ -501,17 +550,19 @@ __global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, con
         // All global loads of the tile are issued first -- the transposed inputs along R (their
         // contiguous dim), the others along C -- so both streams are in flight together; then the
         // transposed ones are turned through LDS.
-        constexpr int K = kTile * SEG / RPP;    // passes: the segments of a tile, 32 at a time
-        constexpr int PPS = kTile / RPP;        // passes per segment column
-        const int seg_v = (tid % VPS) * VEC;    // vector position inside the segment
-        const int lane_o = tid / VPS;           // position along the other dim, + (k % PPS) * RPP
+        // vector e = k * kBlock + tid of the tile: eight consecutive ones form a segment, the segments
+        // of one segment column follow each other along the other dim
+        constexpr int K = kTile * SEG * VPS / kBlock;   // vectors per thread and operand (1 or 4)
+        const int seg_v = (tid % VPS) * VEC;            // vector position inside the segment
+        auto other_of = [&](int k) { return ((k * kBlock + tid) / VPS) % kTile; };                  // position along the other dim
+        auto vec_of = [&](int k) { return seg_v + (((k * kBlock + tid) / VPS) / kTile) * VPS * VEC; };  // element position along the vector dim
         const bool ta = p.trans_a != 0;
         const bool tb = (F::NIN == 2) && p.trans_b != 0;
         Pack<T, VEC> xa[K], xb[K];
 #pragma unroll
         for (int k = 0; k < K; k++) {
-            const int o = lane_o + (k % PPS) * RPP;
-            const int lane_v = seg_v + (k / PPS) * VPS * VEC;
+            const int o = other_of(k);
+            const int lane_v = vec_of(k);
             if (ta) xa[k] = load_pack<T, VEC, NT>(abase + lane_v + (int64_t)o * p.ldc[1]);
             else if (p.ldc[1] == 0) xa[k] = splat<T, VEC>(abase[(int64_t)o * p.ldr[1]]);
             else xa[k] = load_pack<T, VEC, NT>(abase + (int64_t)o * p.ldr[1] + lane_v);
@@ -524,8 +575,8 @@ __global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, con
         if (ta || tb) {
 #pragma unroll
             for (int k = 0; k < K; k++) {
-                const int c = lane_o + (k % PPS) * RPP;  // the loaded vector holds rows lane_v.. of column c
-                const int lane_v = seg_v + (k / PPS) * VPS * VEC;
+                const int c = other_of(k);               // the loaded vector holds rows lane_v.. of column c
+                const int lane_v = vec_of(k);
 #pragma unroll
                 for (int j = 0; j < VEC; j++) {
                     if (ta) lds_a[(lane_v + j) * kPitch + c] = xa[k].v[j];
@@ -538,8 +589,8 @@ __global__ __launch_bounds__(kBlock) void ew_tile_kernel(T *out, const T *a, con
         }
 #pragma unroll
         for (int k = 0; k < K; k++) {
-            const int r = lane_o + (k % PPS) * RPP;
-            const int lane_v = seg_v + (k / PPS) * VPS * VEC;
+            const int r = other_of(k);
+            const int lane_v = vec_of(k);
             Pack<T, VEC> x = xa[k], y;
             if (ta) {
 #pragma unroll
@@ -599,7 +650,7 @@ struct StridedRowsParams {
     int64_t col_tiles;
 };
 
-template <typename T, typename F, int kUnroll>
+template <typename T, typename F, int kUnroll, bool NT>
 __global__ __launch_bounds__(kBlock) void ew_strided_rows_kernel(T *out, const T *a, const T *b,
                                                                  StridedRowsParams p, F f)
 {
@@ -624,14 +675,18 @@ __global__ __launch_bounds__(kBlock) void ew_strided_rows_kernel(T *out, const T
     for (int u = 0; u < kUnroll; u++) {          // all loads of the thread first
         const int64_t c = c0 + (int64_t)u * tx_n;
         if (c < p.ncols) {
-            x[u] = arow[c * sa];
-            y[u] = (F::NIN == 2) ? brow[c * sb] : x[u];
+            x[u] = load_pack<T, 1, NT>(arow + c * sa).v[0];
+            y[u] = (F::NIN == 2) ? load_pack<T, 1, NT>(brow + c * sb).v[0] : x[u];
         }
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
         const int64_t c = c0 + (int64_t)u * tx_n;
-        if (c < p.ncols) orow[c * so] = f(x[u], y[u]);
+        if (c < p.ncols) {
+            Pack<T, 1> r;
+            r.v[0] = f(x[u], y[u]);
+            store_pack<T, 1, NT>(orow + c * so, r);
+        }
     }
 }
 
@@ -865,8 +920,10 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
             tp.tiles_c = (tp.C + kTile - 1) / kTile;
             int64_t grid = tp.nbatch * tp.tiles_r * tp.tiles_c;
             if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-            if (nt) ew_tile_kernel<T, true, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, tp, f);
-            else    ew_tile_kernel<T, false, F><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, tp, f);
+            tp.grid3d = (tp.tiles_r <= 65535 && tp.nbatch <= 65535) ? 1 : 0;
+            const dim3 g = tp.grid3d ? dim3((unsigned)tp.tiles_c, (unsigned)tp.tiles_r, (unsigned)tp.nbatch) : dim3((unsigned)grid);
+            if (nt) ew_tile_kernel<T, true, F><<<g, TileThreads<T, F>::value, 0, stream>>>(out, a, b, tp, f);
+            else    ew_tile_kernel<T, false, F><<<g, TileThreads<T, F>::value, 0, stream>>>(out, a, b, tp, f);
             ZENU_LAUNCH_CHECK();
             return ZENU_OK;
         }
@@ -892,7 +949,13 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
     const int64_t rows_per_blk = kBlock >> shift;
     const int64_t grid = ((sp.nrows + rows_per_blk - 1) / rows_per_blk) * sp.col_tiles;
     if (grid > 0x7fffffffLL || sp.col_tiles > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-    ew_strided_rows_kernel<T, F, kStridedUnroll><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, sp, f);
+    // streaming hint only when every cache line an access touches is used up by the same wavefront
+    // (small inner strides); with large strides the neighbours of an element belong to other rows
+    bool snt = nt;
+    for (int o = 0; o <= nin; o++)
+        if (sp.inner[o] > 4) snt = false;
+    if (snt) ew_strided_rows_kernel<T, F, kStridedUnroll, true><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, sp, f);
+    else     ew_strided_rows_kernel<T, F, kStridedUnroll, false><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, sp, f);
     ZENU_LAUNCH_CHECK();
     return ZENU_OK;
 }

@@ -360,9 +360,9 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(RedParams<T> p)
     } else if (MODE == kBlockRow) {
         o = blockIdx.x;
         split = 0;
-    } else {
-        o = (int64_t)(blockIdx.x / (unsigned)nsplit);
-        split = (int)(blockIdx.x - (unsigned)o * (unsigned)nsplit);
+    } else {            // grid = (splits, outputs): no division at the start of a workgroup
+        o = blockIdx.y;
+        split = (int)blockIdx.x;
     }
     const bool active = o < p.nout;
     A acc[U];
@@ -476,7 +476,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(RedParams<T> p)
 #define ZENU_FOR_COLS(j) _Pragma("unroll") for (int j = 0; j < VEC; j++) if (j < ncol)
 
 template <typename T, typename Tr, int VEC, bool NT>
-__global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int64_t col_tiles, int tx_shift)
+__global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, uint32_t col_tiles, int tx_shift, int grid3d)
 {
     typedef typename Tr::Acc A;
     __shared__ A lds[kBlock * VEC];
@@ -485,14 +485,25 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, int
     const int tx = threadIdx.x & (tx_n - 1);
     const int ty = threadIdx.x >> tx_shift;
     // column tile fastest: workgroups that are dispatched together read adjacent pieces of the
-    // same source rows
-    int64_t blk = blockIdx.x;
-    const int64_t ct = blk % col_tiles;
-    blk /= col_tiles;
-    const int split = (int)(blk % p.splits);
-    const int64_t q = blk / p.splits;
+    // same source rows.  The grid is (column tiles, splits, outer) when that fits the grid limits:
+    // every workgroup of a launch starts at the same time, so a chain of integer divisions at the
+    // top of the kernel delays the whole launch; otherwise linear (below 2^31), in 32 bits.
+    uint32_t ct, split_u, q_u;
+    if (grid3d) {
+        ct = blockIdx.x;
+        split_u = blockIdx.y;
+        q_u = blockIdx.z;
+    } else {
+        uint32_t blk = blockIdx.x;
+        const uint32_t b1 = blk / col_tiles;
+        ct = blk - b1 * col_tiles;
+        q_u = b1 / (uint32_t)p.splits;
+        split_u = b1 - q_u * (uint32_t)p.splits;
+    }
+    const int split = (int)split_u;
+    const int64_t q = q_u;
     const int64_t group = q * col_tiles + ct;   // the workgroups that share these outputs
-    const int64_t c = (ct * tx_n + tx) * VEC;
+    const int64_t c = ((int64_t)ct * tx_n + tx) * VEC;
 
     A acc[VEC];
 #pragma unroll
@@ -619,9 +630,11 @@ int launch_rows(const RedParams<T> &p, hipStream_t s)
         int64_t grid = p.nout * p.splits;
         if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
         if (p.splits > 1) {
-            if (nt)       reduce_rows_kernel<T, Tr, VEC, kSplitRow, true, kSplitU><<<(unsigned)grid, kBlock, 0, s>>>(p);
-            else if (vec) reduce_rows_kernel<T, Tr, VEC, kSplitRow, false, kRowsU><<<(unsigned)grid, kBlock, 0, s>>>(p);
-            else          reduce_rows_kernel<T, Tr, 1, kSplitRow, false, kRowsU><<<(unsigned)grid, kBlock, 0, s>>>(p);
+            if (p.nout > 65535) return ZENU_ERR_UNSUPPORTED;   // never: rows are split only when there are few of them
+            const dim3 g((unsigned)p.splits, (unsigned)p.nout);
+            if (nt)       reduce_rows_kernel<T, Tr, VEC, kSplitRow, true, kSplitU><<<g, kBlock, 0, s>>>(p);
+            else if (vec) reduce_rows_kernel<T, Tr, VEC, kSplitRow, false, kRowsU><<<g, kBlock, 0, s>>>(p);
+            else          reduce_rows_kernel<T, Tr, 1, kSplitRow, false, kRowsU><<<g, kBlock, 0, s>>>(p);
         } else {
             if (nt)       reduce_rows_kernel<T, Tr, VEC, kBlockRow, true, kRowsU><<<(unsigned)grid, kBlock, 0, s>>>(p);
             else if (vec) reduce_rows_kernel<T, Tr, VEC, kBlockRow, false, kRowsU><<<(unsigned)grid, kBlock, 0, s>>>(p);
@@ -661,9 +674,12 @@ int launch_cols(const RedParams<T> &p, hipStream_t s)
     const int64_t outer = p.nout / p.inner;
     int64_t grid = outer * col_tiles * p.splits;
     if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-    if (nt)       reduce_cols_kernel<T, Tr, VEC, true><<<(unsigned)grid, kBlock, 0, s>>>(p, col_tiles, shift);
-    else if (vec) reduce_cols_kernel<T, Tr, VEC, false><<<(unsigned)grid, kBlock, 0, s>>>(p, col_tiles, shift);
-    else          reduce_cols_kernel<T, Tr, 1, false><<<(unsigned)grid, kBlock, 0, s>>>(p, col_tiles, shift);
+    const int g3 = (p.splits <= 65535 && outer <= 65535) ? 1 : 0;
+    const dim3 g = g3 ? dim3((unsigned)col_tiles, (unsigned)p.splits, (unsigned)outer) : dim3((unsigned)grid);
+    const uint32_t ctl = (uint32_t)col_tiles;
+    if (nt)       reduce_cols_kernel<T, Tr, VEC, true><<<g, kBlock, 0, s>>>(p, ctl, shift, g3);
+    else if (vec) reduce_cols_kernel<T, Tr, VEC, false><<<g, kBlock, 0, s>>>(p, ctl, shift, g3);
+    else          reduce_cols_kernel<T, Tr, 1, false><<<g, kBlock, 0, s>>>(p, ctl, shift, g3);
     ZENU_LAUNCH_CHECK();
     return ZENU_OK;
 }
