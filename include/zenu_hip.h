@@ -246,6 +246,12 @@ int zenu_hip_sum_axis(int dtype, const zenu_tensor_t *out, const zenu_tensor_t *
  * are safe. */
 int zenu_hip_sum_axis_noalloc(int dtype, const zenu_tensor_t *out, const zenu_tensor_t *src, int axis,
                               zenu_stream_t stream);
+/* Split reductions hand their partial results from many workgroups to one.  That workgroup polls
+ * for them; after `polls` fruitless polls (about a microsecond each; default 2^20) it computes the
+ * missing ones itself, so no launch ever depends on the order in which workgroups are dispatched.
+ * 0 makes every split reduction take that path at once: a switch for tests, results are the same
+ * bits either way.  No counterpart in the reference. */
+int zenu_hip_set_reduce_spin_limit(int polls);
 /* *out_dev = sum of every element (sum_to(x, []), sum.rs:35-94). */
 int zenu_hip_sum_all(int dtype, void *out_dev, const zenu_tensor_t *src, zenu_stream_t stream);
 /* target = sum_to(src) for any legal target shape (sum.rs:35-94). */

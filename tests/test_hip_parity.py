@@ -1453,3 +1453,41 @@ def test_split_reduction_handoff_repeatable(hip):
     del Xs, X
     _lib.check(l.zenu_hip_stream_destroy(s1), "destroy")
     _lib.check(l.zenu_hip_stream_destroy(s2), "destroy")
+
+
+def test_split_reductions_when_the_folding_workgroup_computes_everything_itself(hip):
+    """The workgroup that folds a split reduction polls for the other workgroups' partial results and,
+    after a bounded number of polls, computes the missing ones itself.  With the bound at 0 it takes
+    that path at once, for partials that have not landed yet; the results must be the bits of the
+    ordinary path (same partials, same merge order), in f32 and f64, for sums, asum, max and arg-max
+    over rows, columns and the whole tensor.  Forced from the host; every kernel still exits normally."""
+    from zenu_amd import _lib
+    l = hip.lib()
+    r = rng(91)
+
+    def run_all(X, x):
+        out = [X.sum_all().to_numpy().copy(), X.sum(0).to_numpy().copy(), X.max_axis(0).to_numpy().copy(),
+               np.array(X.max_axis_idx_ravel(0)), X.transpose().sum(0).to_numpy().copy(),
+               np.array(X.max_idx()), X.asum()]
+        big = X.reshape((4, x.size // 4))
+        out += [big.sum(1).to_numpy().copy(), big.max_axis(1).to_numpy().copy(), np.array(big.max_axis_idx_ravel(1))]
+        return out
+
+    for dt in (np.float32, np.float64):
+        x = r.standard_normal((3000, 1028)).astype(dt)
+        x[5, 7] = x[2000, 7] = x.max() + 1          # a tie across splits: the first index must win
+        X = hip.Matrix.from_numpy(x)
+        ref = run_all(X, x)
+        _lib.check(l.zenu_hip_set_reduce_spin_limit(0), "spin limit")
+        try:
+            for rep in range(3):
+                got = run_all(X, x)
+                for i, (a, b) in enumerate(zip(got, ref)):
+                    assert bits_equal(np.asarray(a), np.asarray(b)), (np.dtype(dt).name, rep, i)
+        finally:
+            _lib.check(l.zenu_hip_set_reduce_spin_limit(1 << 20), "spin limit")
+        assert ref[3][7] == 5 and tuple(ref[5]) == (5, 7)
+        assert_sum_close(ref[1], zo.sum_axis(x, 0), x, 0, "sum axis 0")
+        del X
+    assert l.zenu_hip_set_reduce_spin_limit(-1) == _lib.ERR_ARG
+

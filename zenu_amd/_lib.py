@@ -88,6 +88,7 @@ SIGNATURES = {
     "zenu_hip_bias_add_relu": [_i, _TP, _TP, _TP, _TP, _d, _vp],
     "zenu_hip_sum_axis": [_i, _TP, _TP, _i, _vp],
     "zenu_hip_sum_axis_noalloc": [_i, _TP, _TP, _i, _vp],
+    "zenu_hip_set_reduce_spin_limit": [_i],
     "zenu_hip_sum_all": [_i, _vp, _TP, _vp],
     "zenu_hip_sum_to": [_i, _TP, _TP, _vp],
     "zenu_hip_max_axis": [_i, _TP, _TP, _i, _vp],

@@ -39,6 +39,9 @@ namespace zenu {
 
 // `n` consecutive arrival counters (zero at rest) from the ring of `stream`, or nullptr
 int *reserve_counters(int64_t n, hipStream_t stream);
+// `nwords` tagged 64-bit words from the ring of `stream` and this launch's tag, or nullptr
+uint64_t *reserve_slots(int64_t nwords, hipStream_t stream, uint32_t *epoch);
+int reduce_spin_limit();
 bool library_ready();
 
 namespace {
@@ -73,6 +76,7 @@ constexpr int kWaves = kBlock / kWave;
 #ifndef ZENU_SPLIT_U
 #define ZENU_SPLIT_U 8
 #endif
+constexpr int kSlotBatch = 2;           // partial results a thread of the folding workgroup polls for at a time
 constexpr int kRowsU = 4;               // vectors in flight per lane, one workgroup or wavefront per row
 constexpr int kSplitU = ZENU_SPLIT_U;   // the same when workgroups share a row
 
@@ -230,6 +234,10 @@ template <typename T> struct RedParams {
     int *counters;
     int fan;                 // splits per leaf counter of the arrival tree
     int cstride;             // counters per group: 1 + number of leaves (1 when fan >= splits)
+    // the other cross-workgroup stage: tagged words (slots != null), see "hand-off through tagged words"
+    uint64_t *slots;
+    uint32_t epoch;          // this launch's tag, never zero
+    int spin_limit;          // polls before the folding workgroup computes what is missing itself
     // value gather for max: value = gsrc[q * g_outer_stride + c + idx * g_elem_stride]
     const T *gsrc;
     int64_t g_outer_stride, g_elem_stride;
@@ -301,6 +309,60 @@ __device__ __forceinline__ typename Tr::Acc load_partial(const RedParams<T> &p, 
     return Tr::from_partial(k, i);
 }
 
+// ---- hand-off through tagged words ---------------------------------------------------------------------
+// The faster of the two cross-workgroup stages (whole-tensor f32 sum of 128 MiB: 21.5 us against
+// 23.4 us with the counters; streaming alone takes 20.4 us).  The counters cost four dependent
+// device-scope round trips after the last workgroup has finished streaming (partial stored and
+// acknowledged, leaf counter, root counter, partials loaded).  Here a partial travels as 64-bit
+// words {tag, 32 bits of payload}, each stored with ONE device-scope store and valid by itself: the
+// tag is this launch's number on its stream (RedParams::epoch), which no word left in the ring by
+// an earlier launch carries.  The workgroup with the highest index of a group -- workgroups are
+// dispatched in index order, so the others are running or done when it starts -- folds: after its
+// own streaming it polls the group's words until every tag matches and merges in split order.
+// What is left on the critical path is one store in flight and one poll.
+// Nothing here depends on the dispatch order for correctness: after `spin_limit` fruitless polls
+// the folding workgroup computes the missing partials itself, exactly as their owners would, and
+// stores them; a late owner later stores the same bits again.  Nobody else ever waits.
+// Launches recorded into a graph would replay their tag, so they use the counters; so do requests
+// larger than half a stream's ring of words, the allocation-free entry point, and the column
+// kernel (see reduce_strided).
+
+template <typename T, typename Tr> struct SlotWords {
+    static constexpr int K = sizeof(T) / 4;                    // payload words of the key
+    static constexpr int W = K + (Tr::kHasIdx ? 1 : 0);        // plus the index
+};
+
+// word w of slot s lives at slots[w * nslots + s]: consecutive slots are consecutive words
+template <typename T, typename Tr>
+__device__ __forceinline__ void emit_slot(const RedParams<T> &p, int64_t nslots, int64_t s, typename Tr::Acc r)
+{
+    const T k = Tr::key(r);
+    uint32_t w[3];
+    __builtin_memcpy(w, &k, sizeof(T));
+    if (Tr::kHasIdx) w[SlotWords<T, Tr>::K] = (uint32_t)Tr::idx(r);
+    const uint64_t tag = (uint64_t)p.epoch << 32;
+#pragma unroll
+    for (int i = 0; i < SlotWords<T, Tr>::W; i++) store_agent(p.slots + i * nslots + s, tag | w[i]);
+}
+
+// false while any word of the slot still carries another tag
+template <typename T, typename Tr>
+__device__ __forceinline__ bool load_slot(const RedParams<T> &p, int64_t nslots, int64_t s, typename Tr::Acc &r)
+{
+    uint32_t w[3];
+    bool ok = true;
+#pragma unroll
+    for (int i = 0; i < SlotWords<T, Tr>::W; i++) {
+        const uint64_t v = load_agent(p.slots + i * nslots + s);
+        ok = ok && (uint32_t)(v >> 32) == p.epoch;
+        w[i] = (uint32_t)v;
+    }
+    T k;
+    __builtin_memcpy(&k, w, sizeof(T));
+    r = Tr::from_partial(k, Tr::kHasIdx ? (int32_t)w[SlotWords<T, Tr>::K] : 0);
+    return ok;
+}
+
 // Called by every thread of a workgroup after its partials are stored.  Returns true in the one
 // workgroup of the group that arrives last; it performs the fold.  No workgroup waits for
 // another.  Atomics of many workgroups on ONE address are served one after the other (measured:
@@ -353,84 +415,90 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(RedParams<T> p)
     const int lane_n = WAVE_ROW ? kWave : kBlock;
     const int lane = WAVE_ROW ? (threadIdx.x & (kWave - 1)) : threadIdx.x;
     int64_t o;
-    int split;
+    int my_split;
     if (WAVE_ROW) {
         o = (int64_t)blockIdx.x * kWaves + threadIdx.x / kWave;
-        split = 0;
+        my_split = 0;
     } else if (MODE == kBlockRow) {
         o = blockIdx.x;
-        split = 0;
+        my_split = 0;
     } else {            // grid = (splits, outputs): no division at the start of a workgroup
         o = blockIdx.y;
-        split = (int)blockIdx.x;
+        my_split = (int)blockIdx.x;
     }
     const bool active = o < p.nout;
-    A acc[U];
+
+    // what this lane accumulates of split `split` of output o, the U accumulators merged in a fixed tree
+    auto lane_partial = [&](int split) -> A {
+        A acc[U];
 #pragma unroll
-    for (int u = 0; u < U; u++) acc[u] = Tr::identity();
-    if (active) {
-        int64_t q = o, c = 0;
-        if (p.inner != 1) {
-            q = o / p.inner;
-            c = o - q * p.inner;
-        }
-        const int64_t base = q * p.outer_stride + c;
-        // The splits of an output interleave chunk by chunk (split s takes chunks s, s + splits,
-        // ...), so the workgroups of a launch sweep the source together as one moving window
-        // instead of each streaming its own far-apart segment in lockstep.
-        const int64_t R = p.R;
-        if (VEC > 1) {
-            const T *row = p.in + base;
-            const int64_t step = (int64_t)lane_n * VEC;
-            const int64_t chunk = U * step;
-            const int64_t stride = chunk * nsplit;
-            for (int64_t b = (int64_t)split * chunk; b < R; b += stride) {
-                int64_t r = b + (int64_t)lane * VEC;
-                if (b + chunk <= R) {      // U vectors in flight per lane
-                    Pack<T, VEC> x[U];
-#pragma unroll
-                    for (int u = 0; u < U; u++) x[u] = load_pack<T, VEC, NT>(row + r + u * step);
-#pragma unroll
-                    for (int u = 0; u < U; u++) {
-#pragma unroll
-                        for (int j = 0; j < VEC; j++) acc[u] = Tr::update(acc[u], x[u].v[j], r + u * step + j);
-                    }
-                } else {                   // the last, partial chunk of the row
-                    for (; r + VEC <= R; r += step) {
-                        Pack<T, VEC> x = load_pack<T, VEC, false>(row + r);
-#pragma unroll
-                        for (int j = 0; j < VEC; j++) acc[0] = Tr::update(acc[0], x.v[j], r + j);
-                    }
-                    if (r < R)             // ragged end (R % VEC != 0): one lane
-                        for (int j = 0; r + j < R; j++) acc[0] = Tr::update(acc[0], row[r + j], r + j);
-                }
+        for (int u = 0; u < U; u++) acc[u] = Tr::identity();
+        if (active) {
+            int64_t q = o, c = 0;
+            if (p.inner != 1) {
+                q = o / p.inner;
+                c = o - q * p.inner;
             }
-            if (split == 0 && lane == 0) acc[0] = Tr::first(acc[0], row[0]);
-        } else {
-            const int64_t chunk = (int64_t)U * lane_n;
-            const int64_t stride = chunk * nsplit;
-            for (int64_t b = (int64_t)split * chunk; b < R; b += stride) {
-                int64_t r = b + lane;
-                if (b + chunk <= R) {
+            const int64_t base = q * p.outer_stride + c;
+            // The splits of an output interleave chunk by chunk (split s takes chunks s, s + splits,
+            // ...), so the workgroups of a launch sweep the source together as one moving window
+            // instead of each streaming its own far-apart segment in lockstep.
+            const int64_t R = p.R;
+            if (VEC > 1) {
+                const T *row = p.in + base;
+                const int64_t step = (int64_t)lane_n * VEC;
+                const int64_t chunk = U * step;
+                const int64_t stride = chunk * nsplit;
+                for (int64_t b = (int64_t)split * chunk; b < R; b += stride) {
+                    int64_t r = b + (int64_t)lane * VEC;
+                    if (b + chunk <= R) {      // U vectors in flight per lane
+                        Pack<T, VEC> x[U];
 #pragma unroll
-                    for (int u = 0; u < U; u++) {
-                        const int64_t rr = r + (int64_t)u * lane_n;
-                        acc[u] = Tr::update(acc[u], p.in[base + rr * p.elem_stride], rr);
+                        for (int u = 0; u < U; u++) x[u] = load_pack<T, VEC, NT>(row + r + u * step);
+#pragma unroll
+                        for (int u = 0; u < U; u++) {
+#pragma unroll
+                            for (int j = 0; j < VEC; j++) acc[u] = Tr::update(acc[u], x[u].v[j], r + u * step + j);
+                        }
+                    } else {                   // the last, partial chunk of the row
+                        for (; r + VEC <= R; r += step) {
+                            Pack<T, VEC> x = load_pack<T, VEC, false>(row + r);
+#pragma unroll
+                            for (int j = 0; j < VEC; j++) acc[0] = Tr::update(acc[0], x.v[j], r + j);
+                        }
+                        if (r < R)             // ragged end (R % VEC != 0): one lane
+                            for (int j = 0; r + j < R; j++) acc[0] = Tr::update(acc[0], row[r + j], r + j);
                     }
-                } else {
-                    for (; r < R; r += lane_n) acc[0] = Tr::update(acc[0], p.in[base + r * p.elem_stride], r);
                 }
+                if (split == 0 && lane == 0) acc[0] = Tr::first(acc[0], row[0]);
+            } else {
+                const int64_t chunk = (int64_t)U * lane_n;
+                const int64_t stride = chunk * nsplit;
+                for (int64_t b = (int64_t)split * chunk; b < R; b += stride) {
+                    int64_t r = b + lane;
+                    if (b + chunk <= R) {
+#pragma unroll
+                        for (int u = 0; u < U; u++) {
+                            const int64_t rr = r + (int64_t)u * lane_n;
+                            acc[u] = Tr::update(acc[u], p.in[base + rr * p.elem_stride], rr);
+                        }
+                    } else {
+                        for (; r < R; r += lane_n) acc[0] = Tr::update(acc[0], p.in[base + r * p.elem_stride], r);
+                    }
+                }
+                if (split == 0 && lane == 0) acc[0] = Tr::first(acc[0], p.in[base]);
             }
-            if (split == 0 && lane == 0) acc[0] = Tr::first(acc[0], p.in[base]);
         }
-    }
-    // fixed tree over the U accumulators
+        // fixed tree over the U accumulators
 #pragma unroll
-    for (int w = 1; w < U; w *= 2) {
+        for (int w = 1; w < U; w *= 2) {
 #pragma unroll
-        for (int u = 0; u + w < U; u += 2 * w) acc[u] = Tr::merge(acc[u], acc[u + w]);
-    }
-    A a = acc[0];
+            for (int u = 0; u + w < U; u += 2 * w) acc[u] = Tr::merge(acc[u], acc[u + w]);
+        }
+        return acc[0];
+    };
+
+    A a = lane_partial(my_split);
     if (WAVE_ROW) {
         a = wave_allreduce<Tr>(a);
         if (active && lane == 0) emit_final<T, Tr>(p, o, a);
@@ -441,16 +509,59 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(RedParams<T> p)
         if (lane == 0) emit_final<T, Tr>(p, o, a);
         return;
     }
-    if (lane == 0) emit_partial<T, Tr>(p, o * p.splits + split, a);
-    if (!arrive_last(p.counters + o * p.cstride, split, p.splits, p.fan)) return;
-    // fold the splits of output o: lane l takes splits l, l + 256, ...; then the fixed block tree
+    const int splits = p.splits;
     A f = Tr::identity();
-    for (int s0 = lane; s0 < p.splits; s0 += 4 * kBlock) {
+    if (p.slots) {
+        // tagged words: store and leave; the workgroup with the highest index of the output folds
+        const int64_t nslots = p.nout * splits;
+        const int64_t s_base = o * splits;
+        if (lane == 0) emit_slot<T, Tr>(p, nslots, s_base + my_split, a);
+        if (my_split != splits - 1) return;
+        // lane l takes splits l, l + 256, ... in batches of kSlotBatch (few registers: every workgroup
+        // of the launch pays for what the folding one needs); merge in split order
+        for (int s0 = 0; s0 < splits; s0 += kSlotBatch * kBlock) {
+            A t[kSlotBatch];
+            int polls = 0;
+            for (;;) {
+                int ok = 1;
+#pragma unroll
+                for (int u = 0; u < kSlotBatch; u++) {
+                    const int sidx = s0 + lane + u * kBlock;
+                    t[u] = Tr::identity();
+                    if (sidx < splits && !load_slot<T, Tr>(p, nslots, s_base + sidx, t[u])) ok = 0;
+                }
+                if (__syncthreads_and(ok)) break;
+                if (++polls > p.spin_limit) {
+                    // compute what is still missing in this batch, as its owner would
+                    const int s_end = s0 + kSlotBatch * kBlock < splits ? s0 + kSlotBatch * kBlock : splits;
+                    for (int sp = s0; sp < s_end; sp++) {
+                        A probe;
+                        const int have = (lane == 0 && load_slot<T, Tr>(p, nslots, s_base + sp, probe)) ? 1 : 0;
+                        if (__syncthreads_or(have)) continue;
+                        const A r = block_allreduce<Tr>(lane_partial(sp));
+                        if (lane == 0) emit_slot<T, Tr>(p, nslots, s_base + sp, r);
+                    }
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the words are in place before the next poll
+                    __syncthreads();
+                    polls = 0;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kSlotBatch; u++) f = Tr::merge(f, t[u]);
+        }
+        f = block_allreduce<Tr>(f);
+        if (lane == 0) emit_final<T, Tr>(p, o, f);
+        return;
+    }
+    if (lane == 0) emit_partial<T, Tr>(p, o * splits + my_split, a);
+    if (!arrive_last(p.counters + o * p.cstride, my_split, splits, p.fan)) return;
+    // fold the splits of output o: lane l takes splits l, l + 256, ...; then the fixed block tree
+    for (int s0 = lane; s0 < splits; s0 += 4 * kBlock) {
         A t[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {   // issue the loads together, merge in split order
             const int sidx = s0 + u * kBlock;
-            t[u] = sidx < p.splits ? load_partial<T, Tr>(p, o * p.splits + sidx) : Tr::identity();
+            t[u] = sidx < splits ? load_partial<T, Tr>(p, o * splits + sidx) : Tr::identity();
         }
 #pragma unroll
         for (int u = 0; u < 4; u++) f = Tr::merge(f, t[u]);
@@ -505,61 +616,70 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, uin
     const int64_t group = q * col_tiles + ct;   // the workgroups that share these outputs
     const int64_t c = ((int64_t)ct * tx_n + tx) * VEC;
 
-    A acc[VEC];
-#pragma unroll
-    for (int j = 0; j < VEC; j++) acc[j] = Tr::identity();
-
     const int ncol = (c + VEC <= p.inner) ? VEC : (c < p.inner ? (int)(p.inner - c) : 0);
     const T *src = p.in + q * p.outer_stride + c;
-    // the splits interleave in chunks of U * ty_n source rows: all workgroups of a launch sweep
-    // the source top to bottom together
     constexpr int U = 4;
     const int64_t R = p.R;
-    const int64_t chunk = U * ty_n;
-    const int64_t row_step = (int64_t)ty_n * p.elem_stride;
-    if (ncol == VEC && VEC > 1) {
-        const T *ptr = src + ((int64_t)split * chunk + ty) * p.elem_stride;
-        const int64_t ptr_step = (int64_t)p.splits * chunk * p.elem_stride;
-        for (int64_t b = split * chunk; b < R; b += p.splits * chunk, ptr += ptr_step) {
-            const int64_t r = b + ty;
-            if (b + chunk <= R) {
-                Pack<T, VEC> x[U];
-#pragma unroll
-                for (int u = 0; u < U; u++) x[u] = load_pack<T, VEC, NT>(ptr + u * row_step);
-#pragma unroll
-                for (int u = 0; u < U; u++) {
-#pragma unroll
-                    for (int j = 0; j < VEC; j++) acc[j] = Tr::update(acc[j], x[u].v[j], r + u * ty_n);
-                }
-            } else {
-                const T *pt = ptr;
-                for (int64_t rr = r; rr < R; rr += ty_n, pt += row_step) {
-                    Pack<T, VEC> x = load_pack<T, VEC, false>(pt);
-#pragma unroll
-                    for (int j = 0; j < VEC; j++) acc[j] = Tr::update(acc[j], x.v[j], rr);
-                }
-            }
-        }
-    } else if (ncol > 0) {
-        for (int64_t b = split * chunk; b < R; b += p.splits * chunk)
-            for (int64_t r = b + ty; r < R && r < b + chunk; r += ty_n)
-                ZENU_FOR_COLS(j) acc[j] = Tr::update(acc[j], src[r * p.elem_stride + j], r);
-    }
-    if (split == 0 && ty == 0)
-        ZENU_FOR_COLS(j) acc[j] = Tr::first(acc[j], src[j]);
 
-    // combine the ty lanes in fixed order
-    if (ty_n > 1) {
+    // combine the ty lanes in fixed order: afterwards the row lane ty == 0 holds the result
+    auto combine_rows = [&](A (&acc)[VEC]) {
+        if (ty_n > 1) {
+            __syncthreads();
 #pragma unroll
-        for (int j = 0; j < VEC; j++) lds[j * kBlock + threadIdx.x] = acc[j];   // [vector element][thread]: consecutive lanes, consecutive banks
-        __syncthreads();
-        if (ty == 0) {   // row lane by row lane, the VEC columns side by side: ty_n - 1 dependent LDS round trips, not VEC times that
-            for (int w = 1; w < ty_n; w++) {
+            for (int j = 0; j < VEC; j++) lds[j * kBlock + threadIdx.x] = acc[j];   // [vector element][thread]: consecutive lanes, consecutive banks
+            __syncthreads();
+            if (ty == 0) {   // row lane by row lane, the VEC columns side by side: ty_n - 1 dependent LDS round trips, not VEC times that
+                for (int w = 1; w < ty_n; w++) {
 #pragma unroll
-                for (int j = 0; j < VEC; j++) acc[j] = Tr::merge(acc[j], lds[j * kBlock + w * tx_n + tx]);
+                    for (int j = 0; j < VEC; j++) acc[j] = Tr::merge(acc[j], lds[j * kBlock + w * tx_n + tx]);
+                }
             }
         }
-    }
+    };
+
+    // the partial result of split `split` for this workgroup's columns (valid where ty == 0)
+    auto partial_of = [&](int split, A (&acc)[VEC]) {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) acc[j] = Tr::identity();
+        // the splits interleave in chunks of U * ty_n source rows: all workgroups of a launch sweep
+        // the source top to bottom together
+        const int64_t chunk = U * ty_n;
+        const int64_t row_step = (int64_t)ty_n * p.elem_stride;
+        if (ncol == VEC && VEC > 1) {
+            const T *ptr = src + ((int64_t)split * chunk + ty) * p.elem_stride;
+            const int64_t ptr_step = (int64_t)p.splits * chunk * p.elem_stride;
+            for (int64_t b = split * chunk; b < R; b += p.splits * chunk, ptr += ptr_step) {
+                const int64_t r = b + ty;
+                if (b + chunk <= R) {
+                    Pack<T, VEC> x[U];
+#pragma unroll
+                    for (int u = 0; u < U; u++) x[u] = load_pack<T, VEC, NT>(ptr + u * row_step);
+#pragma unroll
+                    for (int u = 0; u < U; u++) {
+#pragma unroll
+                        for (int j = 0; j < VEC; j++) acc[j] = Tr::update(acc[j], x[u].v[j], r + u * ty_n);
+                    }
+                } else {
+                    const T *pt = ptr;
+                    for (int64_t rr = r; rr < R; rr += ty_n, pt += row_step) {
+                        Pack<T, VEC> x = load_pack<T, VEC, false>(pt);
+#pragma unroll
+                        for (int j = 0; j < VEC; j++) acc[j] = Tr::update(acc[j], x.v[j], rr);
+                    }
+                }
+            }
+        } else if (ncol > 0) {
+            for (int64_t b = split * chunk; b < R; b += p.splits * chunk)
+                for (int64_t r = b + ty; r < R && r < b + chunk; r += ty_n)
+                    ZENU_FOR_COLS(j) acc[j] = Tr::update(acc[j], src[r * p.elem_stride + j], r);
+        }
+        if (split == 0 && ty == 0)
+            ZENU_FOR_COLS(j) acc[j] = Tr::first(acc[j], src[j]);
+        combine_rows(acc);
+    };
+
+    A acc[VEC];
+    partial_of(split, acc);
     const int64_t o0 = q * p.inner + c;
     if (p.splits == 1) {
         if (ty == 0)
@@ -588,18 +708,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, uin
             for (int j = 0; j < VEC; j++) acc[j] = Tr::merge(acc[j], t[u][j]);
         }
     }
-    if (ty_n > 1) {
-        __syncthreads();
-#pragma unroll
-        for (int j = 0; j < VEC; j++) lds[j * kBlock + threadIdx.x] = acc[j];   // [vector element][thread]: consecutive lanes, consecutive banks
-        __syncthreads();
-        if (ty == 0) {   // row lane by row lane, the VEC columns side by side: ty_n - 1 dependent LDS round trips, not VEC times that
-            for (int w = 1; w < ty_n; w++) {
-#pragma unroll
-                for (int j = 0; j < VEC; j++) acc[j] = Tr::merge(acc[j], lds[j * kBlock + w * tx_n + tx]);
-            }
-        }
-    }
+    combine_rows(acc);
     if (ty == 0)
         ZENU_FOR_COLS(j) emit_final<T, Tr>(p, o0 + j, acc[j]);
     if (threadIdx.x == 0) store_agent(p.counters + group * p.cstride, 0);
@@ -719,6 +828,9 @@ int reduce_strided(const T *src, int64_t outer, int64_t R, int64_t inner, int64_
     p.counters = nullptr;
     p.fan = 1;
     p.cstride = 1;
+    p.slots = nullptr;
+    p.epoch = 0;
+    p.spin_limit = 0;
     p.gsrc = src;
     p.g_outer_stride = outer_stride;
     p.g_elem_stride = elem_stride;
@@ -760,6 +872,26 @@ int reduce_strided(const T *src, int64_t outer, int64_t R, int64_t inner, int64_
     }
     const size_t key_bytes = ((size_t)nout * splits * sizeof(T) + 255) / 256 * 256;
     const size_t idx_bytes = Tr::kHasIdx ? (size_t)nout * splits * sizeof(int32_t) : 0;
+    if (!fixed && !use_cols) {
+        // Tagged words from the stream's ring when the launch may use them (not while the stream
+        // records a graph, not beyond half the ring).  Rows only: with the column kernel's many
+        // groups the polls of one group queue behind the streaming of the others and the counters
+        // are faster (sum over axis 0 of [8192,4096] f32: 24.3 us against 25.1 us; of
+        // [131072,256]: 32 us against 49 us), while split rows gain 0.3 - 1.2 us.
+        uint32_t epoch = 0;
+        uint64_t *slots = reserve_slots(nout * splits * SlotWords<T, Tr>::W, s, &epoch);
+        if (slots) {
+            // The same request the counter path would make: it keeps a block of that size in the pool
+            // of this stream, so that a later capture of the same call (which takes the counter path)
+            // finds it there and does not have to go to the driver.
+            Workspace rehearse(key_bytes + idx_bytes, s);
+            if (rehearse.status) return rehearse.status;
+            p.slots = slots;
+            p.epoch = epoch;
+            p.spin_limit = reduce_spin_limit();
+            return launch_rows<T, Tr>(p, s);
+        }
+    }
     if (fixed) {
         // the caller may not allocate: counters and partials live in the static scratch, which
         // every such call on the device shares and which keeps the last call's contents

@@ -48,13 +48,18 @@ struct HipBackend : AllocBackend {
 };
 
 constexpr int64_t kNumCounters = 1 << 16;
+constexpr int64_t kNumSlotWords = 1 << 19;       // 4 MiB of tagged 64-bit partial-result words per stream
+constexpr size_t kRingBytes = kNumCounters * sizeof(int) + kNumSlotWords * sizeof(uint64_t);
 
 struct State {
     std::atomic<bool> ready{false};   // read without the init lock by every entry point
     bool use_pool = true;
-    // arrival counters of the reductions, zero at rest: one ring per stream, because only launches
-    // on the same stream are certain to run one after the other
-    struct Ring { int *base = nullptr; int64_t cursor = 0; };
+    // cross-workgroup memory of the split reductions, one ring per stream, because only launches on
+    // the same stream are certain to run one after the other: arrival counters (zero at rest), then
+    // tagged partial-result words.  A word is {tag, payload}; the tag is the ring's launch number
+    // (`epoch`, never zero, never repeated), so what an earlier launch left behind is never taken
+    // for a result of the current one and nothing has to be cleared.
+    struct Ring { int *base = nullptr; int64_t cursor = 0; int64_t slot_cursor = 0; uint32_t epoch = 0; };
     std::map<hipStream_t, Ring> rings;
     std::mutex counter_mu;
     DeviceInfo info;
@@ -64,6 +69,9 @@ struct State {
 
 State g_state;
 std::mutex g_init_mu;
+// polls of a folding workgroup before it computes missing partial results itself (about a
+// microsecond each); 0 makes every split reduction take that path at once (tests)
+std::atomic<int> g_reduce_spin_limit{1 << 20};
 
 // is `stream` recording a graph?  (the null stream never is)
 bool stream_is_capturing(hipStream_t stream)
@@ -84,8 +92,8 @@ int *make_ring(hipStream_t stream)
 {
     if (stream_is_capturing(stream)) return nullptr;
     int *base = nullptr;
-    hipError_t e = hipMalloc(reinterpret_cast<void **>(&base), kNumCounters * sizeof(int));
-    if (e == hipSuccess) e = hipMemset(base, 0, kNumCounters * sizeof(int));
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&base), kRingBytes);
+    if (e == hipSuccess) e = hipMemset(base, 0, kRingBytes);
     if (e == hipSuccess) e = hipDeviceSynchronize();
     if (e != hipSuccess) {
         set_last_hip_error(e);
@@ -154,6 +162,7 @@ __global__ __launch_bounds__(kFillBlock) void fill_zero_kernel(uint4 *dst16, siz
 
 const DeviceInfo &device_info() { return g_state.info; }
 bool library_ready() { return g_state.ready; }
+int reduce_spin_limit() { return g_reduce_spin_limit.load(std::memory_order_relaxed); }
 
 // Consecutive launches on a stream take consecutive ranges of that stream's ring; a range is reused
 // by a later launch of the same stream, which runs after the earlier one.  Every kernel leaves
@@ -174,6 +183,39 @@ int *reserve_counters(int64_t n, hipStream_t stream)
     }
     if (!make_ring(stream)) return nullptr;
     return reserve_counters(n, stream);
+}
+
+// `nwords` consecutive tagged words from the ring of `stream` and the tag (`*epoch`) that marks
+// this launch's results, or nullptr: the request is larger than half the ring, the stream has no
+// ring and cannot get one now, or the stream is recording a graph (a recorded launch would replay
+// its tag; such launches use the counters instead).
+uint64_t *reserve_slots(int64_t nwords, hipStream_t stream, uint32_t *epoch)
+{
+    if (nwords <= 0 || nwords > kNumSlotWords / 2 || !g_state.ready) return nullptr;
+    if (stream_is_capturing(stream)) return nullptr;
+    for (int attempt = 0; attempt < 2; attempt++) {
+        {
+            std::lock_guard<std::mutex> g(g_state.counter_mu);
+            auto it = g_state.rings.find(stream);
+            if (it != g_state.rings.end() && it->second.base) {
+                State::Ring &r = it->second;
+                if (r.epoch == 0xffffffffu) {
+                    // every tag has been used once: start over on a cleared ring (once in 2^32 launches)
+                    if (hipStreamSynchronize(stream) != hipSuccess) return nullptr;
+                    if (hipMemset(r.base + kNumCounters, 0, kNumSlotWords * sizeof(uint64_t)) != hipSuccess) return nullptr;
+                    if (hipDeviceSynchronize() != hipSuccess) return nullptr;
+                    r.epoch = 0;
+                }
+                if (r.slot_cursor + nwords > kNumSlotWords) r.slot_cursor = 0;
+                uint64_t *out = reinterpret_cast<uint64_t *>(r.base + kNumCounters) + r.slot_cursor;
+                r.slot_cursor += nwords;
+                *epoch = ++r.epoch;
+                return out;
+            }
+        }
+        if (!make_ring(stream)) return nullptr;
+    }
+    return nullptr;
 }
 
 int ensure_init()
@@ -305,6 +347,13 @@ int zenu_hip_free(void *ptr_dev, zenu_stream_t stream)
         return ZENU_OK;
     }
     return g_state.pool->free(ptr_dev, stream);
+}
+
+int zenu_hip_set_reduce_spin_limit(int polls)
+{
+    if (polls < 0) return ZENU_ERR_ARG;
+    g_reduce_spin_limit.store(polls, std::memory_order_relaxed);
+    return ZENU_OK;
 }
 
 int zenu_hip_release_captured(zenu_stream_t stream)
