@@ -628,6 +628,7 @@ def main():
     ap.add_argument("--workload", default="suite", choices=["suite", "c0", "c1", "c2", "c3", "c4", "fused", "next", "scaling"])
     ap.add_argument("--op-reps", type=int, default=50, help="launches per op in the per-op timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-c4", action="store_true", help="leave configs[4] out of the default line (profiling runs)")
     ap.add_argument("--profile-op", default=None, help="only launch this op (for rocprofv3 counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -735,7 +736,7 @@ def main():
 
     # ---- configs[4], the MLP training step: its own object on the default line ---------------------------
     c4 = None
-    if args.workload == "suite":
+    if args.workload == "suite" and not args.no_c4:
         t0 = time.time()
         c4 = c4_summary(z, args, sync)
         log(f"[c4] MLP step measured in {time.time() - t0:.1f} s: "
