@@ -78,8 +78,8 @@ template <typename T, int OP> struct ScalarF {
     __device__ __forceinline__ T operator()(T a, T) const { return bin_apply<T, OP>(a, s); }
 };
 
-__device__ __forceinline__ float dev_tanh(float x) { return zmath::tanhf_simd(x); }
-__device__ __forceinline__ double dev_tanh(double x) { return zmath::tanh_fdlibm(x); }
+__device__ __forceinline__ float dev_tanh(float x, const zmath::TanhRegs &rg) { return zmath::tanhf_simd(x, rg); }
+__device__ __forceinline__ double dev_tanh(double x, const zmath::TanhRegs &) { return zmath::tanh_fdlibm(x); }
 __device__ __forceinline__ float dev_sin(float x) { return zmath::sinf_glibc(x); }
 __device__ __forceinline__ double dev_sin(double x) { return sin(x); }
 __device__ __forceinline__ float dev_cos(float x) { return zmath::cosf_glibc(x); }
@@ -90,22 +90,24 @@ __device__ __forceinline__ float dev_acos(float x) { return zmath::acosf_fdlibm(
 __device__ __forceinline__ double dev_acos(double x) { return acos(x); }
 __device__ __forceinline__ float dev_atan(float x) { return zmath::atanf_fdlibm(x); }
 __device__ __forceinline__ double dev_atan(double x) { return atan(x); }
-__device__ __forceinline__ float dev_sigmoid(float x) { return zmath::sigmoidf_zenu(x); }
-__device__ __forceinline__ double dev_sigmoid(double x) { return zmath::sigmoid_zenu(x); }
+__device__ __forceinline__ float dev_sigmoid(float x, const zmath::TanhRegs &rg) { return zmath::sigmoidf_zenu(x, rg); }
+__device__ __forceinline__ double dev_sigmoid(double x, const zmath::TanhRegs &) { return zmath::sigmoid_zenu(x); }
 
 template <typename T, int FN> struct UnaryF {
     static constexpr int NIN = 1;
     zmath::ExpLog<T> m;     // exp / log state (f32: tables in LDS)
+    zmath::TanhRegs tr;     // f32 tanh / sigmoid: two constants held in vector registers
     __device__ __forceinline__ void init()
     {
         if constexpr (FN == ZENU_EXP || FN == ZENU_LOG || FN == ZENU_SINH || FN == ZENU_COSH)
             m.init(FN != ZENU_LOG, FN == ZENU_LOG);
+        if constexpr (FN == ZENU_TANH || FN == ZENU_SIGMOID) tr.pin();
     }
     __device__ __forceinline__ T operator()(T a, T) const
     {
         if constexpr (FN == ZENU_EXP) return m.exp(a);
         else if constexpr (FN == ZENU_LOG) return m.log(a);
-        else if constexpr (FN == ZENU_TANH) return dev_tanh(a);
+        else if constexpr (FN == ZENU_TANH) return dev_tanh(a, tr);
         else if constexpr (FN == ZENU_SQRT) return sqrt(a);
         else if constexpr (FN == ZENU_ABS) return fabs(a);
         else if constexpr (FN == ZENU_SIN) return dev_sin(a);
@@ -116,7 +118,7 @@ template <typename T, int FN> struct UnaryF {
         else if constexpr (FN == ZENU_ATAN) return dev_atan(a);
         else if constexpr (FN == ZENU_SINH) return m.sinh(a);
         else if constexpr (FN == ZENU_COSH) return m.cosh(a);
-        else return dev_sigmoid(a);
+        else return dev_sigmoid(a, tr);
     }
 };
 

@@ -193,42 +193,70 @@ ZM_HD float div_tanh(float a, float b)
 // The same tanh, restructured for 64-wide SIMD execution: one path through the argument
 // reduction, the rational core and ONE division pair for every lane, the per-k tails computed
 // side by side and selected, so that a wavefront whose lanes hold |x| on both sides of 1 and
-// different k does not execute the branches of tanhf_fdlibm one after another.  Every
-// arithmetic operation that reaches the result is the one tanhf_fdlibm performs, on the same
-// operands, so the bits are identical; this is checked over every f32 bit pattern against
-// tanhf_fdlibm and the host libm (tests/native/zmath_host_check.cpp).
+// different k does not execute the branches of tanhf_fdlibm one after another.  The results are
+// tanhf_fdlibm's and the host libm's on every f32 bit pattern (tests/native/zmath_host_check.cpp
+// on the host, tests/test_exhaustive_device.py on the device).
 //
 // The kernel is bound by its vector instructions (about 0.4 us per instruction and element on
-// 2^24 elements), so the count is what matters.  What was removed without changing a bit:
+// 2^24 elements), so the count is what matters.  Two kinds of savings.  Rewrites that perform
+// fdlibm's operations on fdlibm's operands:
 //   * hi = a - k*ln2_hi is one fused multiply-add: k*ln2_hi is exact (ln2_hi ends in 7 zero bits,
 //     |k| < 64), so fusing does not change the rounding;
 //   * the special cases |a| < 2^-25 (expm1 returns a) and |x| < 2^-55 (tanh returns x*(1+x)) need
 //     no select: the k = 0 formula returns a there (its correction term is below half a unit in
 //     the last place), and -a/(a+2) is then |x| exactly;
-//   * k == -1: 0.5*(xr - e1) - 0.5 = -0.5*(e1 - xr) - 0.5 shares e1 - xr with the other tails;
+//   * k == 0: the correction c is 0, so e1 equals xr*e - hxs and the tail xr - (xr*e - hxs) is
+//     -(e1 - xr): no arithmetic of its own;
+//   * k == -1: 0.5*(xr - e1) - 0.5 = -0.5*(e1 - xr) - 0.5 shares e1 - xr with the other tails, and
+//     is one fused multiply-add (the product is exact);
 //   * k <= -2 and 2 <= k < 23 are one formula, A - (e1 - xr) scaled by 2^k, with A = 1 (and a
-//     final - 1) or A = 1 - 2^-k;
+//     final - 1) or A = 1 - 2^-k; which of the two is decided by |x| >= 1 alone (then k >= 3,
+//     else k <= 0), and the bit pattern that builds 1 - 2^-k is 1 for the negative k;
 //   * |x| >= 9.02: 2/(expm1(2|x|) + 2) is below 2^-25 and vanishes against 1, so any large em1
 //     gives the result 1 (fdlibm takes its k > 56 tail and its |x| >= 22 exit for this);
 //     everything rare (k >= 23, i.e. |x| >= 7.8, and non-finite x) sits behind one test;
 //   * the sign goes back with one bit operation.
-ZM_HD float tanhf_simd(float x)
+// And departures from fdlibm's operation order whose only justification is the exhaustive check
+// (each was tried alone and together over all 2^32 arguments of tanh and of the sigmoid; fusing any
+// other multiply-add of the core changes between 15 and 17 526 results):
+//   * k is a/ln2 rounded to nearest-even in one fused step instead of trunc(a/ln2 +- 0.5) with the
+//     |a| <= 0.5 ln2 exception;
+//   * four of the five Horner steps of the polynomial are fused multiply-adds.
+// The core works on a2 = 2|x| (the sigmoid has it for free: tanh(x/2) needs a2 = |x|) and takes the
+// sign and the NaN payload from `x`.
+//
+// Two constants meet a second constant in a fused multiply-add, and one instruction holds only one
+// literal: the other has to sit in a vector register.  Left to the compiler it is written there
+// again for every element; a kernel pins the pair once per thread (TanhRegs::pin) and passes it in.
+struct TanhRegs {
+    float magic = 12582912.0f;               // 1.5 * 2^23: adding it rounds to an integer
+    float q4 = 4.0082177e-06f;               // 0x36867e54, the polynomial's fourth coefficient
+    ZM_HD void pin()
+    {
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("" : "+v"(magic), "+v"(q4));
+#endif
+    }
+};
+
+ZM_HD float tanhf_simd_core(float a2, float x, const TanhRegs &rg = TanhRegs())
 {
     const float one = 1.0f, two = 2.0f;
     const float ln2_hi = u2f(0x3f317180u), ln2_lo = u2f(0x3717f7d1u), invln2 = u2f(0x3fb8aa3bu);
     const float Q1 = u2f(0xbd088889u), Q2 = u2f(0x3ad00d01u), Q3 = u2f(0xb8a670cdu),
-                Q4 = u2f(0x36867e54u), Q5 = u2f(0xb457edbbu);
-    const uint32_t jx = f2u(x);
-    const uint32_t ix = jx & 0x7fffffffu;
-    const float ax = u2f(ix);
-    const bool big = ix >= 0x3f800000u;      // |x| >= 1: expm1(+2|x|), else expm1(-2|x|)
-    const float a2 = ax + ax;
+                Q5 = u2f(0xb457edbbu);
+    const bool big = a2 >= two;              // |x| >= 1: expm1(+2|x|), else expm1(-2|x|)
     const float a = big ? a2 : -a2;
 
-    // expm1(a), a in (-2, 0] or [2, 44): k = round(a / ln2) when |a| > 0.5 ln2, else 0
-    int32_t k = (int32_t)(invln2 * a + (big ? 0.5f : -0.5f));
-    k = (f2u(a2) > 0x3eb17218u) ? k : 0;
-    const float tk = (float)k;
+    // expm1(a), a in (-2, 0] or [2, 44).  fdlibm takes k = trunc(a/ln2 +- 0.5), and 0 when |a| <= 0.5 ln2;
+    // here k is a/ln2 rounded to the nearest integer by adding 1.5 * 2^23 in one fused step: the sum's
+    // low mantissa bits are k (as a two's complement number), and subtracting the constant again
+    // gives k as a float.  The two choices of k differ on a few ties, where either reduction gives
+    // the same final bits.
+    const float tkm = __builtin_fmaf(invln2, a, rg.magic);
+    const float tk = tkm - rg.magic;
+    const uint32_t kb = f2u(tkm);            // 0x4b400000 + k: only used where the upper bits fall out
+    const int32_t k = (int32_t)(kb - 0x4b400000u);
 #if defined(__HIP_DEVICE_COMPILE__)
     const float hi = __builtin_fmaf(-tk, ln2_hi, a);
 #else
@@ -240,36 +268,53 @@ ZM_HD float tanhf_simd(float x)
 
     const float hfx = 0.5f * xr;
     const float hxs = xr * hfx;
-    const float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    // four of the five steps of the polynomial are fused: their rounding differences stay below
+    // what reaches r1 on every argument (the last one, 1 + hxs * s, has to round twice)
+    float sp = __builtin_fmaf(hxs, Q5, rg.q4);
+    sp = __builtin_fmaf(hxs, sp, Q3);
+    sp = __builtin_fmaf(hxs, sp, Q2);
+    sp = __builtin_fmaf(hxs, sp, Q1);
+    const float r1 = one + hxs * sp;
     const float t = 3.0f - r1 * hfx;
     const float e = hxs * div_tanh(r1 - t, 6.0f - xr * t);
 
-    const float m0 = xr - (xr * e - hxs);                // k == 0
     float e1 = xr * (e - c) - c;
     e1 -= hxs;
     const float d = e1 - xr;
-    const float mneg1 = -0.5f * d - 0.5f;                // k == -1
-    const bool kpos = k >= 2;                            // 2 <= k < 23: (1 - 2^-k) - d, scaled; k <= -2: (1 - d) scaled, - 1
-    const float tt = u2f(0x3f800000u - (0x1000000u >> (k & 31)));
-    const float y = (kpos ? tt : one) - d;
-    const float ys = u2f(f2u(y) + ((uint32_t)k << 23));
-    float em1 = kpos ? ys : ys - one;
-    em1 = (k == -1) ? mneg1 : em1;
-    em1 = (k == 0) ? m0 : em1;
-    if (ix >= 0x40f00000u) {                             // |x| >= 7.5 (rare)
+    // k == 0: c is 0, so e1 is xr*e - hxs and fdlibm's xr - (xr*e - hxs) is -d
+#if defined(__HIP_DEVICE_COMPILE__)
+    const float mneg1 = __builtin_fmaf(-0.5f, d, -0.5f); // k == -1; -0.5*d is exact: fusing changes nothing
+#else
+    const float mneg1 = -0.5f * d - 0.5f;
+#endif
+    // |x| >= 1 has k >= 3: (1 - 2^-k) - d, scaled by 2^k.  |x| < 1 has k in {-3 .. 0}: (1 - d) scaled,
+    // minus 1 -- and the shift count (k & 31) >= 29 leaves nothing of 2^24, so tt is already 1 there
+    const float tt = u2f(0x3f800000u - (0x1000000u >> (kb & 31)));
+    const float y = tt - d;
+    const float ys = u2f(f2u(y) + (kb << 23));
+    float em1 = big ? ys : ys - one;
+    em1 = (kb == 0x4b3fffffu) ? mneg1 : em1;             // k == -1
+    em1 = (kb == 0x4b400000u) ? -d : em1;                // k == 0
+    if (!(a2 < 15.0f)) {                                 // |x| >= 7.5 (rare), or NaN
         if (k >= 23) {                                   // 2^-k no longer fits next to 1
-            const float t2 = u2f((uint32_t)(0x7f - k) << 23);
-            float y2 = xr - (e1 + t2);
+            const float t2 = __builtin_ldexpf(one, -k);  // (the scalings are spelled differently from the one
+            float y2 = xr - (e1 + t2);                   //  above so that it stays a single shift-and-add)
             y2 += one;
-            em1 = u2f(f2u(y2) + ((uint32_t)k << 23));
+            em1 = __builtin_ldexpf(y2, k);
         }
-        if (ix >= 0x411051ecu) em1 = u2f(0x4e800000u);   // |x| >= 9.02: the result is 1 for any large em1
-        if (ix > 0x7f800000u) em1 = x;                   // NaN stays NaN
+        if (a2 >= u2f(0x419051ecu)) em1 = u2f(0x4e800000u);   // |x| >= 9.02: the result is 1 for any large em1
+        if (a2 != a2) em1 = x;                           // NaN stays NaN
     }
     // |x| >= 1: 1 - 2/(t+2);  |x| < 1: -t/(t+2) = -(t/(t+2))
     const float q = div_tanh(big ? two : em1, em1 + two);
     const float z = big ? one - q : -q;
-    return u2f((f2u(z) & 0x7fffffffu) | (jx & 0x80000000u));
+    return u2f((f2u(z) & 0x7fffffffu) | (f2u(x) & 0x80000000u));
+}
+
+ZM_HD float tanhf_simd(float x, const TanhRegs &rg = TanhRegs())
+{
+    const float ax = u2f(f2u(x) & 0x7fffffffu);
+    return tanhf_simd_core(ax + ax, x, rg);
 }
 
 // ---- f32 exp and log: the table-driven routines glibc ships since 2.27 (from ARM's optimized routines) ----
@@ -1081,13 +1126,18 @@ ZM_HD double sinh_fdlibm(double x) { return sinh_fdlibm(x, exp_table()); }
 ZM_HD double cosh_fdlibm(double x) { return cosh_fdlibm(x, exp_table()); }
 
 // ZeNu's sigmoid composite in f32: each step rounded to f32, as the four autograd ops do.
-ZM_HD float sigmoidf_zenu(float x)
+ZM_HD float sigmoidf_zenu(float x, const TanhRegs &rg = TanhRegs())
 {
     const float half = 0.5f;
-    float xh = x * half;
-    float th = tanhf_simd(xh);
+    // tanh(x/2) needs 2|x/2| = |x|.  (Where x/2 underflows and rounds, tanh is below 2^-126 either
+    // way and vanishes against 0.5.)
+    float th = tanhf_simd_core(u2f(f2u(x) & 0x7fffffffu), x, rg);
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_fmaf(half, th, half);   // half*th is exact or vanishes against 0.5: same bits
+#else
     float ht = half * th;
     return half + ht;
+#endif
 }
 
 // tanh of an f32 evaluated in f64 and rounded once: NOT the host library's bits, but never more
