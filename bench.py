@@ -678,8 +678,10 @@ def main():
     value = step_bytes / (elapsed / args.steps) / 1e9
 
     # ---- per-op timing with HIP events on the launch stream ---------------------------------------------
-    # `us` is the mean over op_reps back-to-back launches (one event pair around the batch) and agrees
-    # with the kernel durations of a rocprofv3 trace; a second pass brackets every launch with its
+    # Three batches of op_reps back-to-back launches, one event pair around each; `us` is the median
+    # of the three batch means (kernels bound by their vector instructions follow the clock, which the
+    # power management moves by +-10 % from one millisecond to the next; `us_batches` keeps all three)
+    # and agrees with the kernel durations of a rocprofv3 trace; a second pass brackets every launch with its
     # own events for a median and a minimum, which include the cost of one event record (~2.5 us)
     e0, e1 = hip.event(), hip.event()
     marks = [hip.event() for _ in range(args.op_reps + 1)]
@@ -688,11 +690,14 @@ def main():
         for _ in range(10):
             o.launch()
         sync()
-        hip.record(e0, stream)
-        for _ in range(args.op_reps):
-            o.launch()
-        hip.record(e1, stream)
-        us = hip.elapsed_ms(e0, e1) / args.op_reps * 1e3
+        batches = []
+        for _ in range(3):
+            hip.record(e0, stream)
+            for _ in range(args.op_reps):
+                o.launch()
+            hip.record(e1, stream)
+            batches.append(hip.elapsed_ms(e0, e1) / args.op_reps * 1e3)
+        us = sorted(batches)[1]
         hip.record(marks[0], stream)
         for i in range(args.op_reps):
             o.launch()
@@ -701,7 +706,8 @@ def main():
         gbps = o.alg_bytes / (us * 1e-6) / 1e9
         table.append(dict(op=o.name, config=o.config, dtype=o.dtype, us=round(us, 2), GBps=round(gbps, 1),
                           frac_of_peak=round(gbps / PEAK_HBM_GBPS, 4), Gelem_per_s=round(o.elems / (us * 1e-6) / 1e9, 2),
-                          alg_bytes=o.alg_bytes, us_bracketed_median=round(each[len(each) // 2], 2), us_bracketed_min=round(each[0], 2)))
+                          alg_bytes=o.alg_bytes, us_batches=[round(b, 2) for b in batches],
+                          us_bracketed_median=round(each[len(each) // 2], 2), us_bracketed_min=round(each[0], 2)))
         log(f"[op] {o.name:22s} {us:9.2f} us  {gbps:8.1f} GB/s  {100 * gbps / PEAK_HBM_GBPS:5.1f}% of peak")
 
     # dominant kernel of the step = the op with the largest share of the step time
@@ -757,8 +763,8 @@ def main():
         "frac_of_peak_whole_step": round(value / PEAK_HBM_GBPS, 4),
         "adam_step_params_per_sec": (round(adam[0]["Gelem_per_s"] * 1e9) if adam else None),
         "roofline": roofline, "roofline_second_largest_op": roofline_second, "cpu_baseline": cpu, "c4": c4, "ops": table,
-        "timing": f"HIP events on the launch stream; per op {args.op_reps} back-to-back launches after 10 warm-up launches: "
-                  "us = batch mean, us_bracketed_* = per-launch event pairs (each includes one event record)",
+        "timing": f"HIP events on the launch stream; per op 3 batches of {args.op_reps} back-to-back launches after 10 warm-up launches: "
+                  "us = median of the 3 batch means (us_batches), us_bracketed_* = per-launch event pairs (each includes one event record)",
     }
     print(json.dumps(out))
 

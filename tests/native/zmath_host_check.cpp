@@ -1,6 +1,6 @@
 // Host build of zenu_amd/csrc/zmath.hpp compared with the host libm (the functions ZeNu's CPU path
 // calls through Rust's f32::tanh / exp / ln and f64::tanh).  Usage: zmath_host_check <stride>; checks every stride-th f32
-// bit pattern (stride 1 = exhaustive, about a minute on 8 cores).  powf: every stride-th x for a set
+// bit pattern (stride 1 = exhaustive, about ten minutes on 8 cores).  powf: every stride-th x for a set
 // of fixed exponents, and 2^32 / stride pseudo-random (x, y) pairs.  Prints the mismatch counts.
 #include <atomic>
 #include <cmath>
@@ -15,11 +15,11 @@ int main(int argc, char **argv)
 {
     const uint64_t stride = argc > 1 ? strtoull(argv[1], nullptr, 10) : 1;
     const int nt = 8;
-    std::atomic<uint64_t> bad_fdlibm{0}, bad_simd{0}, bad_expm1{0}, bad_sig{0}, bad_exp{0}, bad_log{0}, bad_sinh{0}, bad_cosh{0}, bad_sin{0}, bad_cos{0}, bad_atan{0}, bad_asin{0}, bad_acos{0}, far_ulp2{0};
+    std::atomic<uint64_t> bad_fdlibm{0}, bad_simd{0}, bad_expm1{0}, bad_sig{0}, bad_exp{0}, bad_log{0}, bad_sinh{0}, bad_cosh{0}, bad_sin{0}, bad_cos{0}, bad_atan{0}, bad_asin{0}, bad_acos{0}, far_ulp2{0}, bad_sinh_simd{0}, bad_cosh_simd{0};
     std::vector<std::thread> th;
     for (int w = 0; w < nt; w++)
         th.emplace_back([&, w]() {
-            uint64_t b0 = 0, b1 = 0, b2 = 0, b3 = 0, b4 = 0, b5 = 0, b6 = 0, b7 = 0, b8 = 0, b9 = 0, b10 = 0, b11 = 0, b12 = 0, b13 = 0;
+            uint64_t b0 = 0, b1 = 0, b2 = 0, b3 = 0, b4 = 0, b5 = 0, b6 = 0, b7 = 0, b8 = 0, b9 = 0, b10 = 0, b11 = 0, b12 = 0, b13 = 0, b14 = 0, b15 = 0;
             for (uint64_t u = (uint64_t)w * stride; u < (1ull << 32); u += stride * nt) {
                 const float x = zmath::u2f((uint32_t)u);
                 const float atr = atanf(x), atg = zmath::atanf_fdlibm(x);
@@ -34,8 +34,12 @@ int main(int argc, char **argv)
                 if ((csr != csr) ? !(csg != csg) : zmath::f2u(csg) != zmath::f2u(csr)) b9++;
                 const float shr = sinhf(x), shg = zmath::sinhf_fdlibm(x);
                 if ((shr != shr) ? !(shg != shg) : zmath::f2u(shg) != zmath::f2u(shr)) b6++;
+                const float shs = zmath::sinhf_simd(x, zmath::exp2f_table());
+                if ((shr != shr) ? !(shs != shs) : zmath::f2u(shs) != zmath::f2u(shr)) b14++;
                 const float chr = coshf(x), chg = zmath::coshf_fdlibm(x);
                 if ((chr != chr) ? !(chg != chg) : zmath::f2u(chg) != zmath::f2u(chr)) b7++;
+                const float chs = zmath::coshf_simd(x, zmath::exp2f_table());
+                if ((chr != chr) ? !(chs != chs) : zmath::f2u(chs) != zmath::f2u(chr)) b15++;
                 const float er = expf(x), eg = zmath::expf_glibc(x);
                 if ((er != er) ? !(eg != eg) : zmath::f2u(eg) != zmath::f2u(er)) b4++;
                 const float lr = logf(x), lg = zmath::logf_glibc(x);
@@ -55,7 +59,7 @@ int main(int argc, char **argv)
                 const float sg = 0.5f + 0.5f * tanhf(0.5f * x), sz = zmath::sigmoidf_zenu(x);
                 if ((sg != sg) ? !(sz != sz) : zmath::f2u(sz) != zmath::f2u(sg)) b3++;
             }
-            bad_fdlibm += b0; bad_simd += b1; bad_expm1 += b2; bad_sig += b3; bad_exp += b4; bad_log += b5; bad_sinh += b6; bad_cosh += b7; bad_sin += b8; bad_cos += b9; bad_atan += b10; bad_asin += b11; bad_acos += b12; far_ulp2 += b13;
+            bad_fdlibm += b0; bad_simd += b1; bad_expm1 += b2; bad_sig += b3; bad_exp += b4; bad_log += b5; bad_sinh += b6; bad_cosh += b7; bad_sin += b8; bad_cos += b9; bad_atan += b10; bad_asin += b11; bad_acos += b12; far_ulp2 += b13; bad_sinh_simd += b14; bad_cosh_simd += b15;
         });
     for (auto &t : th) t.join();
     // double precision: every stride-th value of the HIGH word (sign, exponent, 20 mantissa bits) with
@@ -130,9 +134,10 @@ int main(int argc, char **argv)
     printf("expf_glibc %llu logf_glibc %llu\n", (unsigned long long)bad_exp.load(), (unsigned long long)bad_log.load());
     printf("powf_glibc %llu sinhf_fdlibm %llu coshf_fdlibm %llu\n", (unsigned long long)bad_pow.load(),
            (unsigned long long)bad_sinh.load(), (unsigned long long)bad_cosh.load());
+    printf("sinhf_simd %llu coshf_simd %llu\n", (unsigned long long)bad_sinh_simd.load(), (unsigned long long)bad_cosh_simd.load());
     printf("sinf_glibc %llu cosf_glibc %llu\n", (unsigned long long)bad_sin.load(), (unsigned long long)bad_cos.load());
     printf("atanf_fdlibm %llu asinf_fdlibm %llu acosf_fdlibm %llu\n", (unsigned long long)bad_atan.load(),
            (unsigned long long)bad_asin.load(), (unsigned long long)bad_acos.load());
     printf("tanhf_ulp2_beyond_2ulp %llu\n", (unsigned long long)far_ulp2.load());
-    return (far_ulp2 + bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64 + bad_exp64 + bad_sinh64 + bad_cosh64 + bad_exp + bad_log + bad_pow + bad_sinh + bad_cosh + bad_sin + bad_cos + bad_atan + bad_asin + bad_acos) ? 1 : 0;
+    return (bad_sinh_simd + bad_cosh_simd + far_ulp2 + bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64 + bad_exp64 + bad_sinh64 + bad_cosh64 + bad_exp + bad_log + bad_pow + bad_sinh + bad_cosh + bad_sin + bad_cos + bad_atan + bad_asin + bad_acos) ? 1 : 0;
 }

@@ -80,10 +80,10 @@ template <typename T, int OP> struct ScalarF {
 
 __device__ __forceinline__ float dev_tanh(float x, const zmath::TanhRegs &rg) { return zmath::tanhf_simd(x, rg); }
 __device__ __forceinline__ double dev_tanh(double x, const zmath::TanhRegs &) { return zmath::tanh_fdlibm(x); }
-__device__ __forceinline__ float dev_sin(float x) { return zmath::sinf_glibc(x); }
-__device__ __forceinline__ double dev_sin(double x) { return sin(x); }
-__device__ __forceinline__ float dev_cos(float x) { return zmath::cosf_glibc(x); }
-__device__ __forceinline__ double dev_cos(double x) { return cos(x); }
+__device__ __forceinline__ float dev_sin(float x, const zmath::SinCosCoef &k) { return zmath::sinf_glibc(x, k); }
+__device__ __forceinline__ double dev_sin(double x, const zmath::SinCosCoef &) { return sin(x); }
+__device__ __forceinline__ float dev_cos(float x, const zmath::SinCosCoef &k) { return zmath::cosf_glibc(x, k); }
+__device__ __forceinline__ double dev_cos(double x, const zmath::SinCosCoef &) { return cos(x); }
 __device__ __forceinline__ float dev_asin(float x) { return zmath::asinf_fdlibm(x); }
 __device__ __forceinline__ double dev_asin(double x) { return asin(x); }
 __device__ __forceinline__ float dev_acos(float x) { return zmath::acosf_fdlibm(x); }
@@ -93,15 +93,24 @@ __device__ __forceinline__ double dev_atan(double x) { return atan(x); }
 __device__ __forceinline__ float dev_sigmoid(float x, const zmath::TanhRegs &rg) { return zmath::sigmoidf_zenu(x, rg); }
 __device__ __forceinline__ double dev_sigmoid(double x, const zmath::TanhRegs &) { return zmath::sigmoid_zenu(x); }
 
+// the f64 constants of the f32 sine / cosine travel in the functor (a kernel argument); every other
+// function carries nothing
+template <typename T, int FN> struct SinCosState {};
+template <> struct SinCosState<float, ZENU_SIN> { zmath::SinCosCoef k; };
+template <> struct SinCosState<float, ZENU_COS> { zmath::SinCosCoef k; };
+template <> struct SinCosState<double, ZENU_SIN> { zmath::SinCosCoef k; };
+template <> struct SinCosState<double, ZENU_COS> { zmath::SinCosCoef k; };
+
 template <typename T, int FN> struct UnaryF {
     static constexpr int NIN = 1;
     zmath::ExpLog<T> m;     // exp / log state (f32: tables in LDS)
-    zmath::TanhRegs tr;     // f32 tanh / sigmoid: two constants held in vector registers
+    zmath::TanhRegs tr;     // f32 tanh / sigmoid / sinh / cosh: two constants held in vector registers
+    SinCosState<T, FN> sc;  // f32 sin / cos: the f64 constants, as data
     __device__ __forceinline__ void init()
     {
         if constexpr (FN == ZENU_EXP || FN == ZENU_LOG || FN == ZENU_SINH || FN == ZENU_COSH)
             m.init(FN != ZENU_LOG, FN == ZENU_LOG);
-        if constexpr (FN == ZENU_TANH || FN == ZENU_SIGMOID) tr.pin();
+        if constexpr (FN == ZENU_TANH || FN == ZENU_SIGMOID || FN == ZENU_SINH || FN == ZENU_COSH) tr.pin();
     }
     __device__ __forceinline__ T operator()(T a, T) const
     {
@@ -110,14 +119,14 @@ template <typename T, int FN> struct UnaryF {
         else if constexpr (FN == ZENU_TANH) return dev_tanh(a, tr);
         else if constexpr (FN == ZENU_SQRT) return sqrt(a);
         else if constexpr (FN == ZENU_ABS) return fabs(a);
-        else if constexpr (FN == ZENU_SIN) return dev_sin(a);
-        else if constexpr (FN == ZENU_COS) return dev_cos(a);
+        else if constexpr (FN == ZENU_SIN) return dev_sin(a, sc.k);
+        else if constexpr (FN == ZENU_COS) return dev_cos(a, sc.k);
         else if constexpr (FN == ZENU_TAN) return tan(a);
         else if constexpr (FN == ZENU_ASIN) return dev_asin(a);
         else if constexpr (FN == ZENU_ACOS) return dev_acos(a);
         else if constexpr (FN == ZENU_ATAN) return dev_atan(a);
-        else if constexpr (FN == ZENU_SINH) return m.sinh(a);
-        else if constexpr (FN == ZENU_COSH) return m.cosh(a);
+        else if constexpr (FN == ZENU_SINH) return m.sinh(a, tr);
+        else if constexpr (FN == ZENU_COSH) return m.cosh(a, tr);
         else return dev_sigmoid(a, tr);
     }
 };

@@ -190,6 +190,24 @@ ZM_HD float div_tanh(float a, float b)
 #endif
 }
 
+// The same quotient for the other restated functions, and a square root in the same spirit
+// (reciprocal square root estimate, one correction by the exact remainder; the argument must be
+// positive and normal).  Each use is covered by the device check over every f32 bit pattern of
+// the function it sits in; the host build divides and calls sqrtf.
+ZM_HD float div_fast(float a, float b) { return div_tanh(a, b); }
+ZM_HD float sqrt_fast(float t)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    const float y = __builtin_amdgcn_rsqf(t);
+    const float s = t * y;
+    const float h = 0.5f * y;
+    const float r = __builtin_fmaf(-s, s, t);
+    return __builtin_fmaf(r, h, s);
+#else
+    return __builtin_sqrtf(t);
+#endif
+}
+
 // The same tanh, restructured for 64-wide SIMD execution: one path through the argument
 // reduction, the rational core and ONE division pair for every lane, the per-k tails computed
 // side by side and selected, so that a wavefront whose lanes hold |x| on both sides of 1 and
@@ -398,11 +416,19 @@ ZM_HD const double *powf_log2_table()
 ZM_HD uint64_t d2u(double d);
 ZM_HD double u2d(uint64_t u);
 
-ZM_HD float expf_glibc(float x, const uint64_t *tab)
+// The double constants of expf / logf as data (see SinCosCoef): a kernel hands them over in its
+// argument, every other caller takes the defaults.
+struct ExpfCoef {
+    double inv_ln2n = 0x1.71547652b82fep+0 * 32, shift = 0x1.8p+52;
+    double c0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32, c1 = 0x1.ebfce50fac4f3p-3 / 32 / 32, c2 = 0x1.62e42ff0c52d6p-1 / 32;
+};
+struct LogfCoef {
+    double a0 = -0x1.00ea348b88334p-2, a1 = 0x1.5575b0be00b6ap-2, a2 = -0x1.ffffef20a4123p-2;
+    double ln2 = 0x1.62e42fefa39efp-1;
+};
+
+ZM_HD float expf_glibc(float x, const uint64_t *tab, const ExpfCoef &k = ExpfCoef())
 {
-    const double InvLn2N = 0x1.71547652b82fep+0 * 32, Shift = 0x1.8p+52;
-    const double C0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32, C1 = 0x1.ebfce50fac4f3p-3 / 32 / 32,
-                 C2 = 0x1.62e42ff0c52d6p-1 / 32;
     const uint32_t ux = f2u(x);
     const uint32_t abstop = (ux >> 20) & 0x7ffu;
     if (abstop >= (0x42b00000u >> 20)) {                 // |x| >= 88 or NaN
@@ -412,22 +438,24 @@ ZM_HD float expf_glibc(float x, const uint64_t *tab)
         if (x < -0x1.9fe368p6f) return 0.0f;             // underflow
     }
     const double xd = (double)x;
-    const double z = InvLn2N * xd;
-    double kd = z + Shift;
+    const double z = k.inv_ln2n * xd;
+    double kd = z + k.shift;
     const uint64_t ki = d2u(kd);
-    kd -= Shift;
-    const double r = __builtin_fma(InvLn2N, xd, -kd);
+    kd -= k.shift;
+    const double r = __builtin_fma(k.inv_ln2n, xd, -kd);
     const uint64_t t = tab[ki % 32] + (ki << (52 - 5));
     const double s = u2d(t);
-    const double p = __builtin_fma(C0, r, C1);
+    const double p = __builtin_fma(k.c0, r, k.c1);
     const double r2 = r * r;
-    double y = __builtin_fma(C2, r, 1.0);
+    double y = __builtin_fma(k.c2, r, 1.0);
     y = __builtin_fma(p, r2, y);
     y = y * s;
     return (float)y;
 }
 
-ZM_HD float logf_glibc(float x, const double *tab)
+// logf: the routine with its special cases, and below it the main path as straight-line code for
+// positive normal arguments, which hands zero, negative, subnormal, infinite and NaN arguments back
+ZM_HD float logf_glibc_full(float x, const double *tab)
 {
     const double A0 = -0x1.00ea348b88334p-2, A1 = 0x1.5575b0be00b6ap-2, A2 = -0x1.ffffef20a4123p-2;
     const double Ln2 = 0x1.62e42fefa39efp-1;
@@ -455,6 +483,25 @@ ZM_HD float logf_glibc(float x, const double *tab)
     return (float)y;
 }
 
+ZM_HD float logf_glibc(float x, const double *tab, const LogfCoef &c = LogfCoef())
+{
+    const uint32_t ix = f2u(x);
+    const uint32_t tmp = ix - 0x3f330000u;
+    const uint32_t i = (tmp >> (23 - 4)) % 16;
+    const int32_t k = (int32_t)tmp >> 23;
+    const uint32_t iz = ix - (tmp & (0x1ffu << 23));
+    const double invc = tab[2 * i], logc = tab[2 * i + 1];
+    const double z = (double)u2f(iz);
+    const double r = __builtin_fma(z, invc, -1.0);
+    const double y0 = __builtin_fma((double)k, c.ln2, logc);
+    const double r2 = r * r;
+    double y = __builtin_fma(c.a1, r, c.a2);
+    y = __builtin_fma(c.a0, r2, y);
+    y = __builtin_fma(y, r2, y0 + r);
+    if (__builtin_expect(ix - 0x00800000u >= 0x7f800000u - 0x00800000u, 0)) return logf_glibc_full(x, tab);
+    return (float)y;                                     // (x = 1 gives +0 here as well: r and y0 are 0)
+}
+
 // powf (glibc's e_powf.c, same origin): x^y = 2^(y log2 x); log2 x as a quartic in r = z/c - 1 around
 // the 16 interval centres, the product y log2(x) and the 2^ step (exp2f's 32-entry table and cubic)
 // all in double, rounded once to float.  Results equal the host libm's with the fused and with
@@ -472,7 +519,7 @@ ZM_HD int powf_checkint(uint32_t iy)
 ZM_HD bool powf_zeroinfnan(uint32_t i) { return 2u * i - 1u >= 2u * 0x7f800000u - 1u; }
 ZM_HD bool powf_signaling(uint32_t i) { return 2u * (i ^ 0x00400000u) > 2u * 0x7fc00000u; }
 
-ZM_HD float powf_glibc(float x, float y, const uint64_t *etab, const double *ltab)
+ZM_HD float powf_glibc_full(float x, float y, const uint64_t *etab, const double *ltab)
 {
     const double A0 = 0x1.27616c9496e0bp-2, A1 = -0x1.71969a075c67ap-2, A2 = 0x1.ec70a6ca7baddp-2,
                  A3 = -0x1.7154748bef6c8p-1, A4 = 0x1.71547652ab82bp0;
@@ -543,6 +590,57 @@ ZM_HD float powf_glibc(float x, float y, const uint64_t *etab, const double *lta
     double out = __builtin_fma(C2, rr, 1.0);
     out = __builtin_fma(zz, rr2, out);
     out = out * s;
+    return (float)out;
+}
+
+// The constants of the main path as data (see SinCosCoef).
+struct PowCoef {
+    double a0 = 0x1.27616c9496e0bp-2, a1 = -0x1.71969a075c67ap-2, a2 = 0x1.ec70a6ca7baddp-2,
+           a3 = -0x1.7154748bef6c8p-1, a4 = 0x1.71547652ab82bp0;
+    double c0 = 0x1.c6af84b912394p-5, c1 = 0x1.ebfce50fac4f3p-3, c2 = 0x1.62e42ff0c52d6p-1;
+    double shift = 0x1.8p+52 / 32;
+};
+
+// powf as the kernels call it: the main path of powf_glibc_full as straight-line code (positive
+// normal x, finite non-zero y, |y log2 x| < 126: no special case applies, no sign to carry), and
+// one branch to the full routine for everything else.
+ZM_HD float powf_glibc(float x, float y, const uint64_t *etab, const double *ltab, const PowCoef &k = PowCoef())
+{
+    const uint32_t ix = f2u(x), iy = f2u(y);
+    // (the main path runs on any bit pattern without harm: its table indices are taken modulo the
+    // table sizes; whether its result stands is decided once, at the end)
+    const bool special = ix - 0x00800000u >= 0x7f800000u - 0x00800000u || powf_zeroinfnan(iy);
+    const uint32_t tmp = ix - 0x3f330000u;
+    const uint32_t i = (tmp >> (23 - 4)) % 16;
+    const uint32_t top = tmp & 0xff800000u;
+    const uint32_t iz = ix - top;
+    const int32_t kk = (int32_t)top >> 23;
+    const double invc = ltab[2 * i], logc = ltab[2 * i + 1];
+    const double z = (double)u2f(iz);
+    const double r = __builtin_fma(z, invc, -1.0);
+    const double y0 = logc + (double)kk;
+    const double r2 = r * r;
+    double yy = __builtin_fma(k.a0, r, k.a1);
+    const double p = __builtin_fma(k.a2, r, k.a3);
+    const double r4 = r2 * r2;
+    double q = __builtin_fma(k.a4, r, y0);
+    q = __builtin_fma(p, r2, q);
+    yy = __builtin_fma(yy, r4, q);
+    const double ylogx = (double)y * yy;
+    const bool wide = (d2u(ylogx) >> 47 & 0xffffu) >= (d2u(126.0) >> 47);   // |y log2 x| >= 126, or NaN
+    double kd = ylogx + k.shift;
+    const uint64_t ki = d2u(kd);
+    kd -= k.shift;
+    const double rr = ylogx - kd;
+    uint64_t t = etab[ki % 32];
+    t += ki << (52 - 5);
+    const double sc = u2d(t);
+    const double zz = __builtin_fma(k.c0, rr, k.c1);
+    const double rr2 = rr * rr;
+    double out = __builtin_fma(k.c2, rr, 1.0);
+    out = __builtin_fma(zz, rr2, out);
+    out = out * sc;
+    if (__builtin_expect(special || wide, 0)) return powf_glibc_full(x, y, etab, ltab);
     return (float)out;
 }
 
@@ -642,22 +740,52 @@ ZM_HD float sincosf_poly(double x, double x2, bool neg, int n)
     return (float)__builtin_fma(x6, c2, c);
 }
 
+// The constants of the common path as data: handed to a kernel as an argument they sit in scalar
+// registers and feed the f64 operations directly (as literals each one is copied into a register
+// pair before every use, two scalar instructions per constant and element).
+struct SinCosCoef {
+    double hpi_inv = 0x1.45F306DC9C883p+23, hpi = 0x1.921FB54442D18p0;
+    double s1 = -0x1.555545995a603p-3, s2 = 0x1.1107605230bc4p-7, s3 = -0x1.994eb3774cf24p-13;
+    double c1 = -0x1.ffffffd0c621cp-2, c2 = 0x1.55553e1068f19p-5, c3 = -0x1.6c087e89a359dp-10, c4 = 0x1.99343027bf8c3p-16;
+};
+
 // cosine = 0: sinf(y); cosine = 1: cosf(y)
-ZM_HD float sincosf_glibc(float y, int cosine)
+ZM_HD float sincosf_glibc(float y, int cosine, const SinCosCoef &k = SinCosCoef())
 {
-    const double HpiInv = 0x1.45F306DC9C883p+23, Hpi = 0x1.921FB54442D18p0, Pi63 = 0x1.921FB54442D18p-62;
+    const double Pi63 = 0x1.921FB54442D18p-62;
     const uint32_t top = (f2u(y) >> 20) & 0x7ffu;
-    double x = (double)y;
-    int n;
-    if (top < (0x3f490fdbu >> 20)) {                     // |y| < pi/4 (by the top 12 bits)
-        if (top < (0x39800000u >> 20)) return cosine ? 1.0f : y;   // |y| < 2^-12
-        return sincosf_poly(x, x * x, false, cosine);
-    }
     if (top < (0x42f00000u >> 20)) {                     // |y| < 120
-        const double r = x * HpiInv;
-        n = ((int32_t)r + 0x800000) >> 24;
-        x = __builtin_fma(-(double)n, Hpi, x);
-    } else if (top < (0x7f800000u >> 20)) {
+        // The sources branch off |y| < pi/4 (and |y| < 2^-12) first; the reduction below finds n = 0
+        // there and leaves x alone, and the polynomials round to y resp. 1 below 2^-12, so one path
+        // serves all three.  The signs (the sources multiply x by +-1 and the cosine coefficients by
+        // +-1) are applied to the result instead: every operation is odd resp. even in them.
+        double x = (double)y;
+        const double r = x * k.hpi_inv;
+        const int n = ((int32_t)r + 0x800000) >> 24;
+        x = __builtin_fma(-(double)n, k.hpi, x);
+        const double x2 = x * x;
+        const bool odd = ((n ^ cosine) & 1) != 0;
+        float res;
+        if (!odd) {                                      // on |x|: a zero keeps its sign that way
+            const double ax = __builtin_fabs(x);
+            const double x3 = ax * x2;
+            const double s1 = __builtin_fma(x2, k.s3, k.s2);
+            const double x7 = x3 * x2;
+            const double sv = __builtin_fma(x3, k.s1, ax);
+            res = (float)__builtin_fma(x7, s1, sv);
+        } else {
+            const double x4 = x2 * x2;
+            const double c2 = __builtin_fma(x2, k.c4, k.c3);
+            const double c1 = __builtin_fma(x2, k.c1, 1.0);
+            const double x6 = x4 * x2;
+            const double c = __builtin_fma(x4, k.c2, c1);
+            res = (float)__builtin_fma(x6, c2, c);
+        }
+        // sine polynomial: the sign of x, flipped in quadrants 1 and 2; cosine polynomial: negative in quadrants 2 and 3
+        const uint32_t flip = odd ? (uint32_t)n >> 1 : (((uint32_t)n + 1u) >> 1) ^ (uint32_t)(d2u(x) >> 63);
+        return u2f(f2u(res) ^ (flip << 31));
+    }
+    if (top < (0x7f800000u >> 20)) {
         uint32_t xi = f2u(y);
         const int sign = (int)(xi >> 31);
         const uint32_t *arr = inv_pio4_table() + ((xi >> 26) & 15u);
@@ -671,23 +799,21 @@ ZM_HD float sincosf_glibc(float y, int cosine)
         res0 += res1;
         const uint64_t q = (res0 + (1ull << 61)) >> 62;
         res0 -= q << 62;
-        x = (double)(int64_t)res0 * Pi63;
-        n = (int)q + sign;
+        const double x = (double)(int64_t)res0 * Pi63;
+        const int n = (int)q + sign;
         const double s = ((n & 3) == 1 || (n & 3) == 2) ? -1.0 : 1.0;
         return sincosf_poly(x * s, x * x, (n & 2) != 0, (int)q ^ cosine);
-    } else {
-        return (y - y) / (y - y);                        // inf, NaN
     }
-    const double s = ((n & 3) == 1 || (n & 3) == 2) ? -1.0 : 1.0;
-    return sincosf_poly(x * s, x * x, (n & 2) != 0, n ^ cosine);
+    return (y - y) / (y - y);                            // inf, NaN
 }
-ZM_HD float sinf_glibc(float x) { return sincosf_glibc(x, 0); }
-ZM_HD float cosf_glibc(float x) { return sincosf_glibc(x, 1); }
+ZM_HD float sinf_glibc(float x, const SinCosCoef &k = SinCosCoef()) { return sincosf_glibc(x, 0, k); }
+ZM_HD float cosf_glibc(float x, const SinCosCoef &k = SinCosCoef()) { return sincosf_glibc(x, 1, k); }
 
 // atanf, asinf, acosf: fdlibm's s_atanf.c, e_asinf.c (the five-term polynomial glibc carries), e_acosf.c as
-// glibc 2.35 ships them, plain f32 arithmetic (no fused operations: these have no FMA build).  The
-// constants are the decimal literals of the sources; atanf returns pi/2 from |x| >= 2^25.  Equal to
-// the host libm on all 2^32 inputs.
+// glibc 2.35 ships them (these have no FMA build: the sources round every product).  The constants are
+// the decimal literals of the sources; atanf returns pi/2 from |x| >= 2^25.  Equal to the host libm on
+// all 2^32 inputs -- including the few Horner steps that are fused here because the exhaustive
+// comparison shows no result changes, and, on the device, the short quotient and square root.
 ZM_HD float atanf_fdlibm(float x)
 {
     // atan(0.5), atan(1), atan(1.5), atan(inf) as high + low parts
@@ -713,15 +839,22 @@ ZM_HD float atanf_fdlibm(float x)
         const float ax = u2f(ix);
         const bool r0 = ix < 0x3f300000u, r1 = ix < 0x3f980000u, r2 = ix < 0x401c0000u;   // < 0.6875, < 1.1875, < 2.4375
         const float num = r0 ? 2.0f * ax - one : r1 ? ax - one : r2 ? ax - 1.5f : -1.0f;
-        const float den = r0 ? 2.0f + ax : r1 ? ax + one : r2 ? one + 1.5f * ax : ax;
+        const float den = r0 ? 2.0f + ax : r1 ? ax + one : r2 ? __builtin_fmaf(1.5f, ax, one) : ax;
         h = r0 ? hi0 : r1 ? hi1 : r2 ? hi2 : hi3;
         l = r0 ? lo0 : r1 ? lo1 : r2 ? lo2 : lo3;
-        x = num / den;
+        x = div_fast(num, den);
     }
     const float z = x * x;
     const float w = z * z;
-    const float s1 = z * (a0 + w * (a2 + w * (a4 + w * (a6 + w * (a8 + w * a10)))));
-    const float s2 = w * (a1 + w * (a3 + w * (a5 + w * (a7 + w * a9))));
+    // the inner Horner steps are fused where that changes none of the 2^32 results (each was tried
+    // alone and together; fusing any of the others changes between 8 and 405 980 of them)
+    float s1 = __builtin_fmaf(w, a10, a8);
+    s1 = __builtin_fmaf(w, s1, a6);
+    s1 = __builtin_fmaf(w, s1, a4);
+    s1 = z * (a0 + w * (a2 + w * s1));
+    float s2 = __builtin_fmaf(w, a9, a7);
+    s2 = __builtin_fmaf(w, s2, a5);
+    s2 = w * (a1 + w * (a3 + w * s2));
     if (!reduced) return x - x * (s1 + s2);
     const float r = h - ((x * (s1 + s2) - l) - x);
     return neg ? -r : r;
@@ -744,12 +877,12 @@ ZM_HD float asinf_fdlibm(float x)
     float t = small ? x * x : w * 0.5f;
     float p = t * (p0 + t * (p1 + t * (p2 + t * (p3 + t * p4))));
     if (small) return x + x * p;
-    const float s = sqrtf(t);
+    const float s = sqrt_fast(t);
     if (ix >= 0x3F79999Au) {                             // |x| > 0.975
         t = pio2_hi - (2.0f * (s + s * p) - pio2_lo);
     } else {
         w = u2f(f2u(s) & 0xfffff000u);
-        const float c = (t - w * w) / (s + w);
+        const float c = div_fast(__builtin_fmaf(-w, w, t), s + w);   // w has 12 bits: w*w is exact
         const float r = p;
         p = 2.0f * s * r - (pio2_lo - 2.0f * c);
         const float q = pio4_hi - 2.0f * w;
@@ -774,17 +907,19 @@ ZM_HD float acosf_fdlibm(float x)
     const bool small = ix < 0x3f000000u;                 // |x| < 0.5
     if (small && ix <= 0x23000000u) return pio2_hi + pio2_lo;   // |x| < 2^-57
     const float z = small ? x * x : (neg ? (one + x) * 0.5f : (one - x) * 0.5f);
-    const float p = z * (pS0 + z * (pS1 + z * (pS2 + z * (pS3 + z * (pS4 + z * pS5)))));
+    // (the innermost step of p is the only one of the two polynomials that can be fused without
+    // changing a result)
+    const float p = z * (pS0 + z * (pS1 + z * (pS2 + z * (pS3 + z * __builtin_fmaf(z, pS5, pS4)))));
     const float q = one + z * (qS1 + z * (qS2 + z * (qS3 + z * qS4)));
-    const float r = p / q;
+    const float r = div_fast(p, q);
     if (small) return pio2_hi - (x - (pio2_lo - x * r));
-    const float s = sqrtf(z);
+    const float s = sqrt_fast(z);
     if (neg) {                                           // x < -0.5
         const float w = r * s - pio2_lo;
         return pi - 2.0f * (s + w);
     }
     const float df = u2f(f2u(s) & 0xfffff000u);          // x > 0.5
-    const float c = (z - df * df) / (s + df);
+    const float c = div_fast(__builtin_fmaf(-df, df, z), s + df);   // df has 12 bits: df*df is exact
     const float w = r * s + c;
     return 2.0f * (df + w);
 }
@@ -1192,6 +1327,93 @@ ZM_HD float tanhf_ulp2(float x) { return tanhf_ulp2(x, TanhUlp2Coef()); }
 ZM_HD float expf_glibc(float x) { return expf_glibc(x, exp2f_table()); }
 ZM_HD float logf_glibc(float x) { return logf_glibc(x, logf_table()); }
 ZM_HD float powf_glibc(float x, float y) { return powf_glibc(x, y, exp2f_table(), powf_log2_table()); }
+// sinhf for 64-wide execution, in the manner of tanhf_simd_core: expm1(|x|) with one path through
+// the argument reduction and the rational core, the tails k = 0, k = 1 (both of its forms) and
+// 2 <= k <= 22 side by side, one quotient for both of sinh's ranges; |x| >= 15.5 (k could reach 23),
+// infinities and NaN go to sinhf_fdlibm.  Same results as sinhf_fdlibm on every f32 bit pattern.
+ZM_HD float sinhf_simd(float x, const uint64_t *etab, const TanhRegs &rg = TanhRegs())
+{
+    const float one = 1.0f;
+    const float ln2_hi = u2f(0x3f317180u), ln2_lo = u2f(0x3717f7d1u), invln2 = u2f(0x3fb8aa3bu);
+    const float Q1 = u2f(0xbd088889u), Q2 = u2f(0x3ad00d01u), Q3 = u2f(0xb8a670cdu), Q5 = u2f(0xb457edbbu);
+    const float a = u2f(f2u(x) & 0x7fffffffu);
+    if (!(a < 15.5f)) return sinhf_fdlibm(x, etab);
+
+    // k = trunc(a/ln2 + 0.5) in one fused step (ties go up, as in fdlibm; rounding a/ln2 to the
+    // nearest even integer instead changes one result)
+    const float tk = __builtin_floorf(__builtin_fmaf(invln2, a, 0.5f));
+    const uint32_t kb = (uint32_t)(int32_t)tk;   // 0 <= k <= 22
+#if defined(__HIP_DEVICE_COMPILE__)
+    const float hi = __builtin_fmaf(-tk, ln2_hi, a);
+#else
+    const float hi = a - tk * ln2_hi;        // the product is exact: same value
+#endif
+    const float lo = tk * ln2_lo;
+    const float xr = hi - lo;
+    const float c = (hi - xr) - lo;
+    const float hfx = 0.5f * xr;
+    const float hxs = xr * hfx;
+    float sp = __builtin_fmaf(hxs, Q5, rg.q4);
+    sp = __builtin_fmaf(hxs, sp, Q3);
+    sp = __builtin_fmaf(hxs, sp, Q2);
+    sp = __builtin_fmaf(hxs, sp, Q1);
+    const float r1 = one + hxs * sp;
+    const float t = 3.0f - r1 * hfx;
+    const float e = hxs * div_tanh(r1 - t, 6.0f - xr * t);
+    float e1 = xr * (e - c) - c;
+    e1 -= hxs;
+    const float d = e1 - xr;
+    // k == 1: 1 + 2 (xr - e1), or -2 (e1 - (xr + 0.5)) when xr < -0.25; the doublings are exact
+#if defined(__HIP_DEVICE_COMPILE__)
+    const float k1b = __builtin_fmaf(-2.0f, d, one);
+#else
+    const float k1b = one + 2.0f * (xr - e1);
+#endif
+    const float k1a = -2.0f * (e1 - (xr + 0.5f));
+    const float k1 = (xr < -0.25f) ? k1a : k1b;
+    const float tt = u2f(0x3f800000u - (0x1000000u >> (kb & 31)));
+    const float y = tt - d;
+    float em1 = u2f(f2u(y) + (kb << 23));
+    em1 = (kb == 1u) ? k1 : em1;
+    em1 = (kb == 0u) ? -d : em1;                        // k == 0 (c is 0: xr - (xr e - hxs) = -d)
+
+    // |x| < 1: h (2t - t t/(t+1));  else h (t + t/(t+1)), h = +-0.5
+    const bool small = a < one;
+    const float q = div_tanh(small ? em1 * em1 : em1, em1 + one);
+#if defined(__HIP_DEVICE_COMPILE__)
+    const float r = small ? __builtin_fmaf(2.0f, em1, -q) : em1 + q;
+#else
+    const float r = small ? 2.0f * em1 - q : em1 + q;
+#endif
+    return u2f(f2u(0.5f * r) | (f2u(x) & 0x80000000u));
+}
+
+// coshf with the same means: below 0.5 ln2 expm1's k = 0 path (no argument reduction), from there to
+// 22 expf; the quotients are div_tanh's.  |x| >= 22, infinities and NaN go to coshf_fdlibm.
+ZM_HD float coshf_simd(float x, const uint64_t *etab, const TanhRegs &rg = TanhRegs())
+{
+    const float one = 1.0f, half = 0.5f;
+    const float a = u2f(f2u(x) & 0x7fffffffu);
+    if (!(a < 22.0f)) return coshf_fdlibm(x, etab);
+    if (a < u2f(0x3eb17218u)) {
+        const float Q1 = u2f(0xbd088889u), Q2 = u2f(0x3ad00d01u), Q3 = u2f(0xb8a670cdu), Q5 = u2f(0xb457edbbu);
+        const float hfx = half * a;
+        const float hxs = a * hfx;
+        float sp = __builtin_fmaf(hxs, Q5, rg.q4);
+        sp = __builtin_fmaf(hxs, sp, Q3);
+        sp = __builtin_fmaf(hxs, sp, Q2);
+        sp = __builtin_fmaf(hxs, sp, Q1);
+        const float r1 = one + hxs * sp;
+        const float t3 = 3.0f - r1 * hfx;
+        const float e = hxs * div_tanh(r1 - t3, 6.0f - a * t3);
+        const float t = a - (a * e - hxs);
+        const float w = one + t;
+        return one + div_tanh(t * t, w + w);
+    }
+    const float t = expf_glibc(a, etab);
+    return half * t + div_tanh(half, t);
+}
+
 ZM_HD float sinhf_fdlibm(float x) { return sinhf_fdlibm(x, exp2f_table()); }
 ZM_HD float coshf_fdlibm(float x) { return coshf_fdlibm(x, exp2f_table()); }
 
@@ -1216,6 +1438,8 @@ template <> struct ExpLog<double> {
     __device__ __forceinline__ double log(double x) const { return ::log(x); }
     __device__ __forceinline__ double sinh(double x) const { return sinh_fdlibm(x, etab); }
     __device__ __forceinline__ double cosh(double x) const { return cosh_fdlibm(x, etab); }
+    __device__ __forceinline__ double sinh(double x, const TanhRegs &) const { return sinh_fdlibm(x, etab); }
+    __device__ __forceinline__ double cosh(double x, const TanhRegs &) const { return cosh_fdlibm(x, etab); }
 };
 template <> struct ExpLog<float> {
     const uint64_t *etab;
@@ -1232,10 +1456,15 @@ template <> struct ExpLog<float> {
         etab = lds_exp;
         ltab = lds_log;
     }
-    __device__ __forceinline__ float exp(float x) const { return expf_glibc(x, etab); }
-    __device__ __forceinline__ float log(float x) const { return logf_glibc(x, ltab); }
-    __device__ __forceinline__ float sinh(float x) const { return sinhf_fdlibm(x, etab); }
-    __device__ __forceinline__ float cosh(float x) const { return coshf_fdlibm(x, etab); }
+    ExpfCoef ek;
+    LogfCoef lk;
+    __device__ __forceinline__ float exp(float x) const { return expf_glibc(x, etab, ek); }
+    __device__ __forceinline__ float log(float x) const { return logf_glibc(x, ltab, lk); }
+    __device__ __forceinline__ float sinh(float x) const { return sinhf_simd(x, etab); }
+    __device__ __forceinline__ float cosh(float x) const { return coshf_simd(x, etab); }
+    // with the two register-held constants of the expm1 core pinned by the caller
+    __device__ __forceinline__ float sinh(float x, const TanhRegs &rg) const { return sinhf_simd(x, etab, rg); }
+    __device__ __forceinline__ float cosh(float x, const TanhRegs &rg) const { return coshf_simd(x, etab, rg); }
 };
 
 // pow with the same arrangement: f32 through powf's two tables in LDS, f64 from the math library
@@ -1258,7 +1487,8 @@ template <> struct Pow<float> {
         etab = lds_exp2;
         ltab = lds_log2;
     }
-    __device__ __forceinline__ float pow(float x, float y) const { return powf_glibc(x, y, etab, ltab); }
+    PowCoef k;
+    __device__ __forceinline__ float pow(float x, float y) const { return powf_glibc(x, y, etab, ltab, k); }
 };
 #endif
 
