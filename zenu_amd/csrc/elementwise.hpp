@@ -93,24 +93,35 @@ __device__ __forceinline__ double dev_atan(double x) { return atan(x); }
 __device__ __forceinline__ float dev_sigmoid(float x, const zmath::TanhRegs &rg) { return zmath::sigmoidf_zenu(x, rg); }
 __device__ __forceinline__ double dev_sigmoid(double x, const zmath::TanhRegs &) { return zmath::sigmoid_zenu(x); }
 
-// the f64 constants of the f32 sine / cosine travel in the functor (a kernel argument); every other
-// function carries nothing
-template <typename T, int FN> struct SinCosState {};
-template <> struct SinCosState<float, ZENU_SIN> { zmath::SinCosCoef k; };
-template <> struct SinCosState<float, ZENU_COS> { zmath::SinCosCoef k; };
-template <> struct SinCosState<double, ZENU_SIN> { zmath::SinCosCoef k; };
-template <> struct SinCosState<double, ZENU_COS> { zmath::SinCosCoef k; };
+// what single functions carry besides: the f64 constants of the f32 sine / cosine (in the functor, a
+// kernel argument), the range table of the f32 arc tangent (in LDS); every other function nothing
+template <typename T, int FN> struct UnaryExtra {
+    __device__ __forceinline__ void init() {}
+};
+template <typename T> struct UnaryExtra<T, ZENU_SIN> {
+    zmath::SinCosCoef k;
+    __device__ __forceinline__ void init() {}
+};
+template <typename T> struct UnaryExtra<T, ZENU_COS> {
+    zmath::SinCosCoef k;
+    __device__ __forceinline__ void init() {}
+};
+template <> struct UnaryExtra<float, ZENU_ATAN> {
+    zmath::AtanfLds t;
+    __device__ __forceinline__ void init() { t.init(); }
+};
 
 template <typename T, int FN> struct UnaryF {
     static constexpr int NIN = 1;
     zmath::ExpLog<T> m;     // exp / log state (f32: tables in LDS)
     zmath::TanhRegs tr;     // f32 tanh / sigmoid / sinh / cosh: two constants held in vector registers
-    SinCosState<T, FN> sc;  // f32 sin / cos: the f64 constants, as data
+    UnaryExtra<T, FN> sc;   // f32 sin / cos: the f64 constants, as data; f32 atan: its table
     __device__ __forceinline__ void init()
     {
         if constexpr (FN == ZENU_EXP || FN == ZENU_LOG || FN == ZENU_SINH || FN == ZENU_COSH)
             m.init(FN != ZENU_LOG, FN == ZENU_LOG);
         if constexpr (FN == ZENU_TANH || FN == ZENU_SIGMOID || FN == ZENU_SINH || FN == ZENU_COSH) tr.pin();
+        sc.init();
     }
     __device__ __forceinline__ T operator()(T a, T) const
     {
@@ -124,7 +135,10 @@ template <typename T, int FN> struct UnaryF {
         else if constexpr (FN == ZENU_TAN) return tan(a);
         else if constexpr (FN == ZENU_ASIN) return dev_asin(a);
         else if constexpr (FN == ZENU_ACOS) return dev_acos(a);
-        else if constexpr (FN == ZENU_ATAN) return dev_atan(a);
+        else if constexpr (FN == ZENU_ATAN) {
+            if constexpr (sizeof(T) == 4) return zmath::atanf_fdlibm(a, sc.t.tab);
+            else return dev_atan(a);
+        }
         else if constexpr (FN == ZENU_SINH) return m.sinh(a, tr);
         else if constexpr (FN == ZENU_COSH) return m.cosh(a, tr);
         else return dev_sigmoid(a, tr);

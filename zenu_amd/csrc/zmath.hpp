@@ -814,37 +814,55 @@ ZM_HD float cosf_glibc(float x, const SinCosCoef &k = SinCosCoef()) { return sin
 // the decimal literals of the sources; atanf returns pi/2 from |x| >= 2^25.  Equal to the host libm on
 // all 2^32 inputs -- including the few Horner steps that are fused here because the exhaustive
 // comparison shows no result changes, and, on the device, the short quotient and square root.
-ZM_HD float atanf_fdlibm(float x)
+// Per argument range: numerator = n1 |x| + n0 and denominator = d1 |x| + d0 of the reduction, and
+// atan of the range's centre as high + low part.  Ranges: |x| < 0.4375 (no reduction: |x| / 1),
+// < 0.6875 ((2|x| - 1) / (2 + |x|)), < 1.1875 ((|x| - 1) / (|x| + 1)), < 2.4375 ((|x| - 1.5) / (1 + 1.5 |x|)),
+// above (-1 / |x|).  Each n1 |x| + n0 as one fused multiply-add rounds like the sources' expression
+// (the products are exact, except 1.5 |x|, where the exhaustive comparison shows no change).
+#define ZM_ATANF_TAB                                                                                        \
+    { 1.0f, 0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 0.0f, 0.0f,                                                       \
+      2.0f, -1.0f, 1.0f, 2.0f, 4.6364760399e-01f, 5.0121582440e-09f, 0.0f, 0.0f,                            \
+      1.0f, -1.0f, 1.0f, 1.0f, 7.8539812565e-01f, 3.7748947079e-08f, 0.0f, 0.0f,                            \
+      1.0f, -1.5f, 1.5f, 1.0f, 9.8279368877e-01f, 3.4473217170e-08f, 0.0f, 0.0f,                            \
+      0.0f, -1.0f, 1.0f, 0.0f, 1.5707962513e+00f, 7.5497894159e-08f, 0.0f, 0.0f }
+static const float kAtanfTabHost[40] = ZM_ATANF_TAB;
+#if defined(__HIPCC__)
+static __device__ const float kAtanfTabDev[40] = ZM_ATANF_TAB;
+#endif
+ZM_HD const float *atanf_table()
 {
-    // atan(0.5), atan(1), atan(1.5), atan(inf) as high + low parts
-    const float hi0 = 4.6364760399e-01f, hi1 = 7.8539812565e-01f, hi2 = 9.8279368877e-01f, hi3 = 1.5707962513e+00f;
-    const float lo0 = 5.0121582440e-09f, lo1 = 3.7748947079e-08f, lo2 = 3.4473217170e-08f, lo3 = 7.5497894159e-08f;
+#if defined(__HIP_DEVICE_COMPILE__)
+    return kAtanfTabDev;
+#else
+    return kAtanfTabHost;
+#endif
+}
+
+ZM_HD float atanf_fdlibm(float x, const float *tab)
+{
+    const float hi3 = 1.5707962513e+00f, lo3 = 7.5497894159e-08f;
     const float a0 = 3.3333334327e-01f, a1 = -2.0000000298e-01f, a2 = 1.4285714924e-01f, a3 = -1.1111110449e-01f,
                 a4 = 9.0908870101e-02f, a5 = -7.6918758452e-02f, a6 = 6.6610731184e-02f, a7 = -5.8335702866e-02f,
                 a8 = 4.9768779427e-02f, a9 = -3.6531571299e-02f, a10 = 1.6285819933e-02f;
-    const float one = 1.0f;
     const uint32_t hx = f2u(x);
     const uint32_t ix = hx & 0x7fffffffu;
-    const bool neg = (hx >> 31) != 0;
-    if (ix >= 0x4c000000u) {                             // |x| >= 2^25
+    if (__builtin_expect(ix >= 0x4c000000u, 0)) {        // |x| >= 2^25
         if (ix > 0x7f800000u) return x + x;              // NaN
-        return neg ? -hi3 - lo3 : hi3 + lo3;
+        return (hx >> 31) ? -hi3 - lo3 : hi3 + lo3;
     }
-    // The four argument reductions are one division each in the sources; here the numerator and
-    // denominator are selected first, so a wavefront with arguments in several ranges divides once.
-    const bool reduced = ix >= 0x3ee00000u;              // |x| >= 0.4375
-    if (!reduced && ix < 0x31000000u) return x;          // |x| < 2^-29
-    float h = 0.0f, l = 0.0f;
-    if (reduced) {
-        const float ax = u2f(ix);
-        const bool r0 = ix < 0x3f300000u, r1 = ix < 0x3f980000u, r2 = ix < 0x401c0000u;   // < 0.6875, < 1.1875, < 2.4375
-        const float num = r0 ? 2.0f * ax - one : r1 ? ax - one : r2 ? ax - 1.5f : -1.0f;
-        const float den = r0 ? 2.0f + ax : r1 ? ax + one : r2 ? __builtin_fmaf(1.5f, ax, one) : ax;
-        h = r0 ? hi0 : r1 ? hi1 : r2 ? hi2 : hi3;
-        l = r0 ? lo0 : r1 ? lo1 : r2 ? lo2 : lo3;
-        x = div_fast(num, den);
-    }
-    const float z = x * x;
+    // One path for all five ranges (a wavefront holds arguments of several): the range picks a table
+    // row, the reduced argument is one quotient, the sign goes back at the end (every step is odd
+    // in x).  Without a reduction the sources return x - x (s1 + s2), which is h - ((x (s1 + s2) - l) - x)
+    // with h = l = 0; below 2^-29 they return x, and so does this (s1 + s2 vanishes against 1).
+    const uint32_t id = (uint32_t)(ix >= 0x3ee00000u) + (uint32_t)(ix >= 0x3f300000u) + (uint32_t)(ix >= 0x3f980000u) +
+                        (uint32_t)(ix >= 0x401c0000u);
+    const float *e = tab + 8 * id;
+    const float ax = u2f(ix);
+    const float num = __builtin_fmaf(e[0], ax, e[1]);
+    const float den = __builtin_fmaf(e[2], ax, e[3]);
+    const float h = e[4], l = e[5];
+    const float xr = div_fast(num, den);
+    const float z = xr * xr;
     const float w = z * z;
     // the inner Horner steps are fused where that changes none of the 2^32 results (each was tried
     // alone and together; fusing any of the others changes between 8 and 405 980 of them)
@@ -855,10 +873,10 @@ ZM_HD float atanf_fdlibm(float x)
     float s2 = __builtin_fmaf(w, a9, a7);
     s2 = __builtin_fmaf(w, s2, a5);
     s2 = w * (a1 + w * (a3 + w * s2));
-    if (!reduced) return x - x * (s1 + s2);
-    const float r = h - ((x * (s1 + s2) - l) - x);
-    return neg ? -r : r;
+    const float r = h - ((xr * (s1 + s2) - l) - xr);
+    return u2f(f2u(r) | (hx & 0x80000000u));
 }
+ZM_HD float atanf_fdlibm(float x) { return atanf_fdlibm(x, atanf_table()); }
 
 ZM_HD float asinf_fdlibm(float x)
 {
@@ -1465,6 +1483,18 @@ template <> struct ExpLog<float> {
     // with the two register-held constants of the expm1 core pinned by the caller
     __device__ __forceinline__ float sinh(float x, const TanhRegs &rg) const { return sinhf_simd(x, etab, rg); }
     __device__ __forceinline__ float cosh(float x, const TanhRegs &rg) const { return coshf_simd(x, etab, rg); }
+};
+
+// atanf's range table in LDS, same arrangement (init() by every thread of the workgroup, once)
+struct AtanfLds {
+    const float *tab;
+    __device__ __forceinline__ void init()
+    {
+        __shared__ float lds_atan[40];
+        if (threadIdx.x < 40) lds_atan[threadIdx.x] = kAtanfTabDev[threadIdx.x];
+        __syncthreads();
+        tab = lds_atan;
+    }
 };
 
 // pow with the same arrangement: f32 through powf's two tables in LDS, f64 from the math library
