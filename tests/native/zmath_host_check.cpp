@@ -74,20 +74,29 @@ int main(int argc, char **argv)
                 const uint32_t lows[3] = {(uint32_t)rng, 0u, 0xffffffffu};
                 for (uint32_t lo : lows) {
                     const double x = zmath::u2d((u << 32) | lo);
-                    const double ref = tanh(x), got = zmath::tanh_fdlibm(x);
+                    const double ref = tanh(x), got = zmath::tanh_fdlibm(x), got2 = zmath::tanh_simd(x);
                     if ((ref != ref) ? !(got != got) : zmath::d2u(got) != zmath::d2u(ref)) b0++;
+                    if ((ref != ref) ? !(got2 != got2) : zmath::d2u(got2) != zmath::d2u(ref)) b0++;   // the form the kernels use
                     if (fabs(x) < 700.0 && zmath::d2u(zmath::expm1_fdlibm(x)) != zmath::d2u(expm1(x))) b1++;
                     const double sg = 0.5 + 0.5 * tanh(0.5 * x), sz = zmath::sigmoid_zenu(x);
                     if ((sg != sg) ? !(sz != sz) : zmath::d2u(sz) != zmath::d2u(sg)) b2++;
                     const double er = exp(x), eg = zmath::exp_glibc(x);
                     if ((er != er) ? !(eg != eg) : zmath::d2u(eg) != zmath::d2u(er)) b3++;
-                    const double shr = sinh(x), shg = zmath::sinh_fdlibm(x);
+                    const double shr = sinh(x), shg = zmath::sinh_fdlibm(x), shs = zmath::sinh_simd(x, zmath::exp_table());
                     if ((shr != shr) ? !(shg != shg) : zmath::d2u(shg) != zmath::d2u(shr)) b4++;
+                    if ((shr != shr) ? !(shs != shs) : zmath::d2u(shs) != zmath::d2u(shr)) b4++;   // the form the kernels use
                     const double chr = cosh(x), chg = zmath::cosh_fdlibm(x);
                     if ((chr != chr) ? !(chg != chg) : zmath::d2u(chg) != zmath::d2u(chr)) b5++;
                 }
                 // arguments where exp is finite and not 1: uniform in +-745 and in +-4
                 const double m = (double)(int64_t)rng / 9.2233720368547758e18;
+                // tanh and the sigmoid where they are neither x nor +-1: uniform in +-1, +-4 and +-20
+                for (double x : {m, m * 4.0, m * 20.0}) {
+                    if (zmath::d2u(zmath::sinh_simd(x, zmath::exp_table())) != zmath::d2u(sinh(x))) b4++;
+                    const double ref = tanh(x);
+                    if (zmath::d2u(zmath::tanh_fdlibm(x)) != zmath::d2u(ref) || zmath::d2u(zmath::tanh_simd(x)) != zmath::d2u(ref)) b0++;
+                    if (zmath::d2u(zmath::sigmoid_zenu(x)) != zmath::d2u(0.5 + 0.5 * tanh(0.5 * x))) b2++;
+                }
                 for (double x : {m * 745.0, m * 4.0}) {
                     const double er = exp(x), eg = zmath::exp_glibc(x);
                     if (zmath::d2u(eg) != zmath::d2u(er)) b3++;

@@ -35,7 +35,9 @@ def test_zmath_matches_host_libm(tmp_path):
     each; stride 1, all 2^32, was run during development with the same result); powf on every 31st
     base for 19 fixed exponents and on two pseudo-random (base, exponent) pairs per base; f64 tanh,
     expm1, exp, sinh, cosh and the sigmoid composite on every 31st high word with three low words
-    each plus uniform samples in +-745 and +-4 (about 700 M points).  tanhf_ulp2, the variant that
+    each plus uniform samples in +-745 and +-4 (about 700 M points); f64 tanh in both of its forms
+    (fdlibm's branches and the single path the kernels use) and the sigmoid also on 400 M uniform
+    samples in +-1, +-4 and +-20.  tanhf_ulp2, the variant that
     is not meant to give libm's bits, must stay within 2 units in the last place of tanhf on the
     same f32 points (stride 1: the largest distance is 2)."""
     exe = build("zmath_host_check.cpp", str(tmp_path / "zmath_check"), ("-ffp-contract=off", "-fno-fast-math"))

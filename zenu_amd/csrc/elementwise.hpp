@@ -79,7 +79,7 @@ template <typename T, int OP> struct ScalarF {
 };
 
 __device__ __forceinline__ float dev_tanh(float x, const zmath::TanhRegs &rg) { return zmath::tanhf_simd(x, rg); }
-__device__ __forceinline__ double dev_tanh(double x, const zmath::TanhRegs &) { return zmath::tanh_fdlibm(x); }
+__device__ __forceinline__ double dev_tanh(double x, const zmath::TanhRegs &) { return zmath::tanh_simd(x); }
 __device__ __forceinline__ float dev_sin(float x, const zmath::SinCosCoef &k) { return zmath::sinf_glibc(x, k); }
 __device__ __forceinline__ double dev_sin(double x, const zmath::SinCosCoef &) { return sin(x); }
 __device__ __forceinline__ float dev_cos(float x, const zmath::SinCosCoef &k) { return zmath::cosf_glibc(x, k); }

@@ -1216,13 +1216,79 @@ ZM_HD double tanh_fdlibm(double x)
     return neg ? -z : z;
 }
 
-// ZeNu's sigmoid composite in f64
+// The same tanh for 64-wide execution, as tanhf_simd_core does it in f32, but with only those
+// rewrites that perform fdlibm's operations on fdlibm's operands (no f64 function can be compared on
+// all of its arguments, so nothing here rests on an exhaustive check):
+//   * one path through the argument reduction, the rational core and one division pair; k is fdlibm's
+//     (0 up to 0.5 ln2 by the high word, trunc(a/ln2 +- 0.5) above; between 0.5 ln2 and 1.5 ln2 the
+//     sources take k = +-1 with hi = a -+ ln2_hi, lo = +-ln2_lo, which is what the general formula gives:
+//     the bounds on the high word keep a/ln2 +- 0.5 inside (1, 2));
+//   * hi = a - k ln2_hi fused: ln2_hi ends in 21 zero bits, the product is exact;
+//   * |a| < 2^-54 (expm1 returns a) and |x| < 2^-55 (tanh returns x (1 + x) = x) go through the k = 0
+//     formula, whose correction term is below half a unit in the last place there;
+//   * the tails share d = e1 - xr: k = 0 is -d (c is 0 there), k = -1 is -0.5 d - 0.5 in one fused step
+//     (exact product), k <= -2 and 3 <= k < 20 are (A - d) 2^k with A = 1 (and a final - 1) or
+//     A = 1 - 2^-k, whose bit pattern comes out as 1 for the negative k; |x| >= 1 decides which;
+//   * |x| >= 6.5 (k could reach 20), infinities and NaN go to tanh_fdlibm.
+// The core works on a2 = 2|x|; the sigmoid passes |x| (see sigmoidf_zenu).
+ZM_HD double tanh_simd_core(double a2, double x)
+{
+    const double one = 1.0, two = 2.0;
+    const double ln2_hi = u2d(0x3fe62e42fee00000ull), ln2_lo = u2d(0x3dea39ef35793c76ull), invln2 = u2d(0x3ff71547652b82feull);
+    const double Q1 = u2d(0xBFA11111111110F4ull), Q2 = u2d(0x3F5A01A019FE5585ull), Q3 = u2d(0xBF14CE199EAADBB7ull),
+                 Q4 = u2d(0x3ED0CFCA86E65239ull), Q5 = u2d(0xBE8AFDB76E09C32Dull);
+    const bool big = a2 >= two;              // |x| >= 1: expm1(+2|x|), else expm1(-2|x|)
+    const double a = big ? a2 : -a2;
+    int32_t k = (int32_t)(invln2 * a + (big ? 0.5 : -0.5));
+    k = (hi_word(a2) > 0x3fd62e42u) ? k : 0;
+    const double tk = (double)k;
+    const double hi = __builtin_fma(-tk, ln2_hi, a);
+    const double lo = tk * ln2_lo;
+    const double xr = hi - lo;
+    const double c = (hi - xr) - lo;
+    const double hfx = 0.5 * xr;
+    const double hxs = xr * hfx;
+    const double R1 = one + hxs * Q1;
+    const double h2 = hxs * hxs;
+    const double R2 = Q2 + hxs * Q3;
+    const double h4 = h2 * h2;
+    const double R3 = Q4 + hxs * Q5;
+    const double r1 = R1 + h2 * R2 + h4 * R3;
+    const double t = 3.0 - r1 * hfx;
+    const double e = hxs * ((r1 - t) / (6.0 - xr * t));
+    double e1 = xr * (e - c) - c;
+    e1 -= hxs;
+    const double d = e1 - xr;
+    const double mneg1 = __builtin_fma(-0.5, d, -0.5);
+    const double tt = from_hi_word(0x3ff00000u - (0x200000u >> (k & 31)));
+    const double y = tt - d;
+    const double ys = add_to_hi_word(y, (uint32_t)k << 20);
+    double em1 = big ? ys : ys - one;
+    em1 = (k == -1) ? mneg1 : em1;
+    em1 = (k == 0) ? -d : em1;
+    const double q = (big ? two : em1) / (em1 + two);
+    const double z = big ? one - q : -q;
+    return u2d((d2u(z) & 0x7fffffffffffffffull) | (d2u(x) & 0x8000000000000000ull));
+}
+
+ZM_HD double tanh_simd(double x)
+{
+    const double ax = u2d(d2u(x) & 0x7fffffffffffffffull);
+    if (__builtin_expect(!(ax < 6.5), 0)) return tanh_fdlibm(x);
+    return tanh_simd_core(ax + ax, x);
+}
+
+// ZeNu's sigmoid composite in f64: tanh(x/2) needs 2|x/2| = |x| (where x/2 underflows and rounds,
+// tanh is below 2^-1022 either way and vanishes against 0.5); 0.5 tanh is exact or vanishes, so
+// the last two steps are one fused multiply-add
 ZM_HD double sigmoid_zenu(double x)
 {
-    double xh = x * 0.5;
-    double th = tanh_fdlibm(xh);
-    double ht = 0.5 * th;
-    return 0.5 + ht;
+    const double ax = u2d(d2u(x) & 0x7fffffffffffffffull);
+    if (__builtin_expect(!(ax < 13.0), 0)) {
+        const double th = tanh_fdlibm(x * 0.5);
+        return 0.5 + 0.5 * th;
+    }
+    return __builtin_fma(0.5, tanh_simd_core(ax, x), 0.5);
 }
 
 // sinh / cosh in f64 (fdlibm e_sinh.c / e_cosh.c as glibc 2.35 ships them) over the expm1 and exp above
@@ -1248,6 +1314,54 @@ ZM_HD double sinh_fdlibm(double x, const uint64_t *etab)
         return t * w;
     }
     return x * shuge;                                    // overflow
+}
+
+// sinh in f64 for 64-wide execution, with the means of tanh_simd_core (only rewrites that keep
+// fdlibm's operations and operands): expm1(|x|) on one path with the tails k = 0, k = 1 in both of
+// its forms and 2 <= k < 20 side by side, one division for both of sinh's ranges.  |x| >= 13
+// (k could reach 20), infinities and NaN go to sinh_fdlibm; |x| < 2^-28 returns x as in the sources.
+ZM_HD double sinh_simd(double x, const uint64_t *etab)
+{
+    const double one = 1.0;
+    const double ln2_hi = u2d(0x3fe62e42fee00000ull), ln2_lo = u2d(0x3dea39ef35793c76ull), invln2 = u2d(0x3ff71547652b82feull);
+    const double Q1 = u2d(0xBFA11111111110F4ull), Q2 = u2d(0x3F5A01A019FE5585ull), Q3 = u2d(0xBF14CE199EAADBB7ull),
+                 Q4 = u2d(0x3ED0CFCA86E65239ull), Q5 = u2d(0xBE8AFDB76E09C32Dull);
+    const double a = u2d(d2u(x) & 0x7fffffffffffffffull);
+    if (__builtin_expect(!(a < 13.0), 0)) return sinh_fdlibm(x, etab);
+    const uint32_t ix = hi_word(a);
+    int32_t k = (int32_t)(invln2 * a + 0.5);
+    k = (ix > 0x3fd62e42u) ? k : 0;
+    const double tk = (double)k;
+    const double hi = __builtin_fma(-tk, ln2_hi, a);     // the product is exact
+    const double lo = tk * ln2_lo;
+    const double xr = hi - lo;
+    const double c = (hi - xr) - lo;
+    const double hfx = 0.5 * xr;
+    const double hxs = xr * hfx;
+    const double R1 = one + hxs * Q1;
+    const double h2 = hxs * hxs;
+    const double R2 = Q2 + hxs * Q3;
+    const double h4 = h2 * h2;
+    const double R3 = Q4 + hxs * Q5;
+    const double r1 = R1 + h2 * R2 + h4 * R3;
+    const double t = 3.0 - r1 * hfx;
+    const double e = hxs * ((r1 - t) / (6.0 - xr * t));
+    double e1 = xr * (e - c) - c;
+    e1 -= hxs;
+    const double d = e1 - xr;
+    const double k1b = __builtin_fma(-2.0, d, one);      // 1 + 2 (xr - e1): the doubling is exact
+    const double k1a = -2.0 * (e1 - (xr + 0.5));
+    const double k1 = (xr < -0.25) ? k1a : k1b;
+    const double tt = from_hi_word(0x3ff00000u - (0x200000u >> (k & 31)));
+    const double y = tt - d;
+    double em1 = add_to_hi_word(y, (uint32_t)k << 20);
+    em1 = (k == 1) ? k1 : em1;
+    em1 = (k == 0) ? -d : em1;                           // c is 0: xr - (xr e - hxs) = -d
+    const bool small = a < one;
+    const double q = (small ? em1 * em1 : em1) / (em1 + one);
+    const double r = small ? __builtin_fma(2.0, em1, -q) : em1 + q;   // 2 em1 is exact
+    const double res = u2d(d2u(0.5 * r) | (d2u(x) & 0x8000000000000000ull));
+    return (ix < 0x3e300000u) ? x : res;
 }
 
 ZM_HD double cosh_fdlibm(double x, const uint64_t *etab)
@@ -1454,9 +1568,9 @@ template <> struct ExpLog<double> {
     }
     __device__ __forceinline__ double exp(double x) const { return exp_glibc(x, etab); }
     __device__ __forceinline__ double log(double x) const { return ::log(x); }
-    __device__ __forceinline__ double sinh(double x) const { return sinh_fdlibm(x, etab); }
+    __device__ __forceinline__ double sinh(double x) const { return sinh_simd(x, etab); }
     __device__ __forceinline__ double cosh(double x) const { return cosh_fdlibm(x, etab); }
-    __device__ __forceinline__ double sinh(double x, const TanhRegs &) const { return sinh_fdlibm(x, etab); }
+    __device__ __forceinline__ double sinh(double x, const TanhRegs &) const { return sinh_simd(x, etab); }
     __device__ __forceinline__ double cosh(double x, const TanhRegs &) const { return cosh_fdlibm(x, etab); }
 };
 template <> struct ExpLog<float> {
