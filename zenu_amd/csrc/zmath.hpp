@@ -32,8 +32,12 @@
 
 #if defined(__HIPCC__)
 #define ZM_HD __host__ __device__ __forceinline__
+// a rarely taken path kept out of line: one copy per kernel instead of one per element of the
+// unrolled loop (the branchy fdlibm forms are thousands of instructions when inlined eight times)
+#define ZM_RARE __host__ __device__ __attribute__((noinline)) static
 #else
 #define ZM_HD static inline
+#define ZM_RARE static
 #endif
 
 namespace zmath {
@@ -483,6 +487,8 @@ ZM_HD float logf_glibc_full(float x, const double *tab)
     return (float)y;
 }
 
+ZM_RARE float logf_rare(float x, const double *tab) { return logf_glibc_full(x, tab); }
+
 ZM_HD float logf_glibc(float x, const double *tab, const LogfCoef &c = LogfCoef())
 {
     const uint32_t ix = f2u(x);
@@ -498,7 +504,7 @@ ZM_HD float logf_glibc(float x, const double *tab, const LogfCoef &c = LogfCoef(
     double y = __builtin_fma(c.a1, r, c.a2);
     y = __builtin_fma(c.a0, r2, y);
     y = __builtin_fma(y, r2, y0 + r);
-    if (__builtin_expect(ix - 0x00800000u >= 0x7f800000u - 0x00800000u, 0)) return logf_glibc_full(x, tab);
+    if (__builtin_expect(ix - 0x00800000u >= 0x7f800000u - 0x00800000u, 0)) return logf_rare(x, tab);
     return (float)y;                                     // (x = 1 gives +0 here as well: r and y0 are 0)
 }
 
@@ -604,6 +610,8 @@ struct PowCoef {
 // powf as the kernels call it: the main path of powf_glibc_full as straight-line code (positive
 // normal x, finite non-zero y, |y log2 x| < 126: no special case applies, no sign to carry), and
 // one branch to the full routine for everything else.
+ZM_RARE float powf_rare(float x, float y, const uint64_t *etab, const double *ltab) { return powf_glibc_full(x, y, etab, ltab); }
+
 ZM_HD float powf_glibc(float x, float y, const uint64_t *etab, const double *ltab, const PowCoef &k = PowCoef())
 {
     const uint32_t ix = f2u(x), iy = f2u(y);
@@ -640,7 +648,7 @@ ZM_HD float powf_glibc(float x, float y, const uint64_t *etab, const double *lta
     double out = __builtin_fma(k.c2, rr, 1.0);
     out = __builtin_fma(zz, rr2, out);
     out = out * sc;
-    if (__builtin_expect(special || wide, 0)) return powf_glibc_full(x, y, etab, ltab);
+    if (__builtin_expect(special || wide, 0)) return powf_rare(x, y, etab, ltab);
     return (float)out;
 }
 
@@ -1271,10 +1279,12 @@ ZM_HD double tanh_simd_core(double a2, double x)
     return u2d((d2u(z) & 0x7fffffffffffffffull) | (d2u(x) & 0x8000000000000000ull));
 }
 
+ZM_RARE double tanh_rare(double x) { return tanh_fdlibm(x); }
+
 ZM_HD double tanh_simd(double x)
 {
     const double ax = u2d(d2u(x) & 0x7fffffffffffffffull);
-    if (__builtin_expect(!(ax < 6.5), 0)) return tanh_fdlibm(x);
+    if (__builtin_expect(!(ax < 6.5), 0)) return tanh_rare(x);
     return tanh_simd_core(ax + ax, x);
 }
 
@@ -1285,7 +1295,7 @@ ZM_HD double sigmoid_zenu(double x)
 {
     const double ax = u2d(d2u(x) & 0x7fffffffffffffffull);
     if (__builtin_expect(!(ax < 13.0), 0)) {
-        const double th = tanh_fdlibm(x * 0.5);
+        const double th = tanh_rare(x * 0.5);
         return 0.5 + 0.5 * th;
     }
     return __builtin_fma(0.5, tanh_simd_core(ax, x), 0.5);
@@ -1320,6 +1330,8 @@ ZM_HD double sinh_fdlibm(double x, const uint64_t *etab)
 // fdlibm's operations and operands): expm1(|x|) on one path with the tails k = 0, k = 1 in both of
 // its forms and 2 <= k < 20 side by side, one division for both of sinh's ranges.  |x| >= 13
 // (k could reach 20), infinities and NaN go to sinh_fdlibm; |x| < 2^-28 returns x as in the sources.
+ZM_RARE double sinh_rare(double x, const uint64_t *etab) { return sinh_fdlibm(x, etab); }
+
 ZM_HD double sinh_simd(double x, const uint64_t *etab)
 {
     const double one = 1.0;
@@ -1327,7 +1339,7 @@ ZM_HD double sinh_simd(double x, const uint64_t *etab)
     const double Q1 = u2d(0xBFA11111111110F4ull), Q2 = u2d(0x3F5A01A019FE5585ull), Q3 = u2d(0xBF14CE199EAADBB7ull),
                  Q4 = u2d(0x3ED0CFCA86E65239ull), Q5 = u2d(0xBE8AFDB76E09C32Dull);
     const double a = u2d(d2u(x) & 0x7fffffffffffffffull);
-    if (__builtin_expect(!(a < 13.0), 0)) return sinh_fdlibm(x, etab);
+    if (__builtin_expect(!(a < 13.0), 0)) return sinh_rare(x, etab);
     const uint32_t ix = hi_word(a);
     int32_t k = (int32_t)(invln2 * a + 0.5);
     k = (ix > 0x3fd62e42u) ? k : 0;
@@ -1463,13 +1475,16 @@ ZM_HD float powf_glibc(float x, float y) { return powf_glibc(x, y, exp2f_table()
 // the argument reduction and the rational core, the tails k = 0, k = 1 (both of its forms) and
 // 2 <= k <= 22 side by side, one quotient for both of sinh's ranges; |x| >= 15.5 (k could reach 23),
 // infinities and NaN go to sinhf_fdlibm.  Same results as sinhf_fdlibm on every f32 bit pattern.
+ZM_RARE float sinhf_rare(float x, const uint64_t *etab) { return sinhf_fdlibm(x, etab); }
+ZM_RARE float coshf_rare(float x, const uint64_t *etab) { return coshf_fdlibm(x, etab); }
+
 ZM_HD float sinhf_simd(float x, const uint64_t *etab, const TanhRegs &rg = TanhRegs())
 {
     const float one = 1.0f;
     const float ln2_hi = u2f(0x3f317180u), ln2_lo = u2f(0x3717f7d1u), invln2 = u2f(0x3fb8aa3bu);
     const float Q1 = u2f(0xbd088889u), Q2 = u2f(0x3ad00d01u), Q3 = u2f(0xb8a670cdu), Q5 = u2f(0xb457edbbu);
     const float a = u2f(f2u(x) & 0x7fffffffu);
-    if (!(a < 15.5f)) return sinhf_fdlibm(x, etab);
+    if (__builtin_expect(!(a < 15.5f), 0)) return sinhf_rare(x, etab);
 
     // k = trunc(a/ln2 + 0.5) in one fused step (ties go up, as in fdlibm; rounding a/ln2 to the
     // nearest even integer instead changes one result)
@@ -1526,7 +1541,7 @@ ZM_HD float coshf_simd(float x, const uint64_t *etab, const TanhRegs &rg = TanhR
 {
     const float one = 1.0f, half = 0.5f;
     const float a = u2f(f2u(x) & 0x7fffffffu);
-    if (!(a < 22.0f)) return coshf_fdlibm(x, etab);
+    if (__builtin_expect(!(a < 22.0f), 0)) return coshf_rare(x, etab);
     if (a < u2f(0x3eb17218u)) {
         const float Q1 = u2f(0xbd088889u), Q2 = u2f(0x3ad00d01u), Q3 = u2f(0xb8a670cdu), Q5 = u2f(0xb457edbbu);
         const float hfx = half * a;
