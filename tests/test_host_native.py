@@ -39,7 +39,8 @@ def test_zmath_matches_host_libm(tmp_path):
     (fdlibm's branches and the single path the kernels use) and the sigmoid also on 400 M uniform
     samples in +-1, +-4 and +-20.  tanhf_ulp2, the variant that
     is not meant to give libm's bits, must stay within 2 units in the last place of tanhf on the
-    same f32 points (stride 1: the largest distance is 2)."""
+    same f32 points (stride 1: the largest distance is 2), and tanf_ulp1, the f32 tangent the kernels
+    use, within 1 of tanf (stride 1: 97.5 % equal, 2.5 % one apart)."""
     exe = build("zmath_host_check.cpp", str(tmp_path / "zmath_check"), ("-ffp-contract=off", "-fno-fast-math"))
     out = subprocess.run([exe, "31"], capture_output=True, text=True)
     assert out.returncode == 0, out.stdout
@@ -49,4 +50,4 @@ def test_zmath_matches_host_libm(tmp_path):
                                   "expf_glibc", "0", "logf_glibc", "0", "powf_glibc", "0",
                                   "sinhf_fdlibm", "0", "coshf_fdlibm", "0", "sinhf_simd", "0", "coshf_simd", "0", "sinf_glibc", "0", "cosf_glibc", "0",
                                   "atanf_fdlibm", "0", "asinf_fdlibm", "0", "acosf_fdlibm", "0",
-                                  "tanhf_ulp2_beyond_2ulp", "0"]
+                                  "tanhf_ulp2_beyond_2ulp", "0", "tanf_ulp1_beyond_1ulp", "0"]

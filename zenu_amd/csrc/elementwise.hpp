@@ -106,6 +106,10 @@ template <typename T> struct UnaryExtra<T, ZENU_COS> {
     zmath::SinCosCoef k;
     __device__ __forceinline__ void init() {}
 };
+template <> struct UnaryExtra<float, ZENU_TAN> {
+    zmath::SinCosCoef k;
+    __device__ __forceinline__ void init() {}
+};
 template <> struct UnaryExtra<float, ZENU_ATAN> {
     zmath::AtanfLds t;
     __device__ __forceinline__ void init() { t.init(); }
@@ -132,7 +136,10 @@ template <typename T, int FN> struct UnaryF {
         else if constexpr (FN == ZENU_ABS) return fabs(a);
         else if constexpr (FN == ZENU_SIN) return dev_sin(a, sc.k);
         else if constexpr (FN == ZENU_COS) return dev_cos(a, sc.k);
-        else if constexpr (FN == ZENU_TAN) return tan(a);
+        else if constexpr (FN == ZENU_TAN) {
+            if constexpr (sizeof(T) == 4) return zmath::tanf_ulp1(a, sc.k);
+            else return tan(a);
+        }
         else if constexpr (FN == ZENU_ASIN) return dev_asin(a);
         else if constexpr (FN == ZENU_ACOS) return dev_acos(a);
         else if constexpr (FN == ZENU_ATAN) {
