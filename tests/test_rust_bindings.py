@@ -2,7 +2,7 @@
 place of the bindgen output of zenu-cuda-kernel-sys/build.rs:35-53) is generated from
 include/zenu_hip.h.  Regenerate it and compare, and check it independently against the header's
 symbol list and the ctypes signature table, so neither the .rs file nor the excerpt shown in
-INTEGRATION.md can drift from the header.  The file itself was never compiled (no Rust here)."""
+the binder's guide at the repository root can drift from the header.  The file itself was never compiled (no Rust here)."""
 import ctypes as C
 import importlib.util
 import os
@@ -84,10 +84,10 @@ def test_struct_layout_matches_the_ctypes_mirror():
 
 
 def test_integration_excerpt_is_taken_from_the_generated_file():
-    """every `pub fn` line shown in INTEGRATION.md must be a line of the generated file"""
+    """every `pub fn` line the binder's guide shows must be a line of the generated file"""
     doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     gen = open(os.path.join(ROOT, "bindings", "zenu_hip_sys.rs")).read()
     shown = re.findall(r"^\s*(pub fn \w+\(.*\).*;)\s*$", doc, re.M)
-    assert shown, "INTEGRATION.md shows no binding lines"
+    assert shown, "the guide shows no binding lines"
     for line in shown:
         assert line in gen, line
