@@ -143,6 +143,43 @@ def test_softmax_strided_views(hip):
     assert np.all(big.to_numpy()[:, 1::2] == 0)
 
 
+def test_softmax_rows_divide_like_the_chain(hip):
+    """The workgroup-per-row kernel adds the row in a tree, so its sum S may differ from the chain's
+    index-order sum by a few units in the last place -- but every element of a row must be the
+    correctly rounded exp(x - max) / S for ONE such S, as the chain's element-wise division would
+    give.  Rows: random
+    logits of several spreads, spreads that put elements below 2^-80 and at zero, -inf entries, equal
+    entries (S a power of two), lengths on both sides of the row-in-registers limit."""
+    import zenu_oracle as zo
+    r = np.random.default_rng(11)
+    for R in (4096, 1000, 5000):
+        rows = [r.standard_normal(R) * s for s in (0.1, 1.0, 3.0, 10.0, 30.0)]
+        rows.append(np.linspace(-120.0, 0.0, R))                       # tiny, subnormal and zero quotients
+        rows.append(np.where(r.random(R) < 0.3, -np.inf, r.standard_normal(R)))
+        rows.append(np.full(R, 0.25))
+        rows += [r.standard_normal(R) * 2.0 for _ in range(24)]
+        x = np.ascontiguousarray(np.array(rows, dtype=np.float32))
+        out = hip.Matrix.zeros(x.shape)
+        out.softmax_assign(hip.Matrix.from_numpy(x), 1)
+        got = out.to_numpy()
+        m = x.max(axis=1, keepdims=True)
+        a = np.empty_like(x)
+        zo.unary(zo.EXP, a, np.ascontiguousarray(x - m))               # the chain's exp, bit-exact on the device
+        for i in range(x.shape[0]):
+            s0 = np.float32(a[i].astype(np.float64).sum())             # the exact sum, rounded: any summation order lands near it
+            cand = s0
+            for _ in range(64):
+                cand = np.nextafter(cand, np.float32(0))
+            matched = False
+            for _ in range(129):
+                with np.errstate(all="ignore"):
+                    if bits_equal(got[i], (a[i] / cand).astype(np.float32)):
+                        matched = True
+                        break
+                cand = np.nextafter(cand, np.float32(np.inf))
+            assert matched, f"R={R} row {i}: no single divisor near {s0!r} reproduces the row"
+
+
 def test_softmax_special_rows(hip):
     """NaN in position 0 / elsewhere and an all -inf row poison the row exactly as in the chain; a row
     with +inf gives NaN at the inf (inf - inf) and 0 elsewhere... all NaN after the division"""
