@@ -94,10 +94,12 @@ __global__ __launch_bounds__(kBlock) void softmax_lines_kernel(const T *x, T *y,
 
 template <typename T, int VEC, bool CE, bool REG, bool NT, int kBlock = 256, int kRegPacks = 4>
 __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, int64_t R, const T *target,
-                                                               T *rowloss)
+                                                               T *rowloss, zmath::ExpLog<T> ml)
 {
+    // (ml arrives as an argument so that the f64 constants of exp / log sit in scalar registers; written
+    // as literals each is copied into a register pair per use, and this kernel is bound by its scalar
+    // instructions: the branch-free exp for the same reason)
     __shared__ T lds[4];
-    zmath::ExpLog<T> ml;
     if (!REG) ml.init(true, CE);
     const int64_t row = blockIdx.x;
     const T *xr = x + row * R;
@@ -127,7 +129,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
             if (first + k * step < R) {
 #pragma unroll
                 for (int j = 0; j < VEC; j++) {
-                    v[k].v[j] = ml.exp(v[k].v[j] - m);
+                    v[k].v[j] = ml.exp_flat(v[k].v[j] - m);
                     sum = sum + v[k].v[j];
                 }
             }
@@ -162,7 +164,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
             Pack<T, VEC> v = load_pack<T, VEC, false>(xr + r);
 #pragma unroll
             for (int j = 0; j < VEC; j++) {
-                v.v[j] = ml.exp(v.v[j] - m);
+                v.v[j] = ml.exp_flat(v.v[j] - m);
                 sum = sum + v.v[j];
             }
             store_pack<T, VEC, false>(yr + r, v);
@@ -430,11 +432,11 @@ int softmax_forward_launch(const T *x, T *y, Geometry g, const T *target, T *row
         const unsigned grid = (unsigned)lines;
         const bool nt = vec && reg && lines * g.R * (int64_t)sizeof(T) * 2 >= kStreamBytes;
         // (one wavefront or 128 threads per row with more vectors per lane measured 4-9 % slower)
-        if (nt)               softmax_rows_kernel<T, VEC, CE, true, true><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
-        else if (vec && reg)  softmax_rows_kernel<T, VEC, CE, true, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
-        else if (vec)         softmax_rows_kernel<T, VEC, CE, false, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
-        else if (reg)         softmax_rows_kernel<T, 1, CE, true, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
-        else                  softmax_rows_kernel<T, 1, CE, false, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss);
+        if (nt)               softmax_rows_kernel<T, VEC, CE, true, true><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss, zmath::ExpLog<T>());
+        else if (vec && reg)  softmax_rows_kernel<T, VEC, CE, true, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss, zmath::ExpLog<T>());
+        else if (vec)         softmax_rows_kernel<T, VEC, CE, false, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss, zmath::ExpLog<T>());
+        else if (reg)         softmax_rows_kernel<T, 1, CE, true, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss, zmath::ExpLog<T>());
+        else                  softmax_rows_kernel<T, 1, CE, false, false><<<grid, kBlock, 0, s>>>(x, y, g.R, target, rowloss, zmath::ExpLog<T>());
     }
     ZENU_LAUNCH_CHECK();
     return ZENU_OK;

@@ -457,6 +457,31 @@ ZM_HD float expf_glibc(float x, const uint64_t *tab, const ExpfCoef &k = ExpfCoe
     return (float)y;
 }
 
+// The same expf without a branch, for kernels whose scalar unit is the busy one (a branch per element
+// is half a dozen scalar instructions): the main path runs on any bit pattern (the table index is
+// taken modulo the table size; a NaN stays a NaN), overflow and underflow are two selects.  Same
+// results as expf_glibc except for the payload of a NaN.
+ZM_HD float expf_glibc_flat(float x, const uint64_t *tab, const ExpfCoef &k = ExpfCoef())
+{
+    const double xd = (double)x;
+    const double z = k.inv_ln2n * xd;
+    double kd = z + k.shift;
+    const uint64_t ki = d2u(kd);
+    kd -= k.shift;
+    const double r = __builtin_fma(k.inv_ln2n, xd, -kd);
+    const uint64_t t = tab[ki % 32] + (ki << (52 - 5));
+    const double s = u2d(t);
+    const double p = __builtin_fma(k.c0, r, k.c1);
+    const double r2 = r * r;
+    double y = __builtin_fma(k.c2, r, 1.0);
+    y = __builtin_fma(p, r2, y);
+    y = y * s;
+    float res = (float)y;
+    res = (x > 0x1.62e42ep6f) ? u2f(0x7f800000u) : res;  // overflow, +inf
+    res = (x < -0x1.9fe368p6f) ? 0.0f : res;             // underflow, -inf
+    return res;
+}
+
 // logf: the routine with its special cases, and below it the main path as straight-line code for
 // positive normal arguments, which hands zero, negative, subnormal, infinite and NaN arguments back
 ZM_HD float logf_glibc_full(float x, const double *tab)
@@ -1639,6 +1664,7 @@ template <> struct ExpLog<double> {
         etab = lds_exp64;
     }
     __device__ __forceinline__ double exp(double x) const { return exp_glibc(x, etab); }
+    __device__ __forceinline__ double exp_flat(double x) const { return exp_glibc(x, etab); }
     __device__ __forceinline__ double log(double x) const { return ::log(x); }
     __device__ __forceinline__ double sinh(double x) const { return sinh_simd(x, etab); }
     __device__ __forceinline__ double cosh(double x) const { return cosh_fdlibm(x, etab); }
@@ -1663,6 +1689,7 @@ template <> struct ExpLog<float> {
     ExpfCoef ek;
     LogfCoef lk;
     __device__ __forceinline__ float exp(float x) const { return expf_glibc(x, etab, ek); }
+    __device__ __forceinline__ float exp_flat(float x) const { return expf_glibc_flat(x, etab, ek); }
     __device__ __forceinline__ float log(float x) const { return logf_glibc(x, ltab, lk); }
     __device__ __forceinline__ float sinh(float x) const { return sinhf_simd(x, etab); }
     __device__ __forceinline__ float cosh(float x) const { return coshf_simd(x, etab); }
