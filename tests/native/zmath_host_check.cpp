@@ -91,14 +91,16 @@ int main(int argc, char **argv)
                     const double shr = sinh(x), shg = zmath::sinh_fdlibm(x), shs = zmath::sinh_simd(x, zmath::exp_table());
                     if ((shr != shr) ? !(shg != shg) : zmath::d2u(shg) != zmath::d2u(shr)) b4++;
                     if ((shr != shr) ? !(shs != shs) : zmath::d2u(shs) != zmath::d2u(shr)) b4++;   // the form the kernels use
-                    const double chr = cosh(x), chg = zmath::cosh_fdlibm(x);
+                    const double chr = cosh(x), chg = zmath::cosh_fdlibm(x), chs = zmath::cosh_simd(x, zmath::exp_table());
                     if ((chr != chr) ? !(chg != chg) : zmath::d2u(chg) != zmath::d2u(chr)) b5++;
+                    if ((chr != chr) ? !(chs != chs) : zmath::d2u(chs) != zmath::d2u(chr)) b5++;   // the form the kernels use
                 }
                 // arguments where exp is finite and not 1: uniform in +-745 and in +-4
                 const double m = (double)(int64_t)rng / 9.2233720368547758e18;
                 // tanh and the sigmoid where they are neither x nor +-1: uniform in +-1, +-4 and +-20
                 for (double x : {m, m * 4.0, m * 20.0}) {
                     if (zmath::d2u(zmath::sinh_simd(x, zmath::exp_table())) != zmath::d2u(sinh(x))) b4++;
+                    if (zmath::d2u(zmath::cosh_simd(x, zmath::exp_table())) != zmath::d2u(cosh(x))) b5++;
                     const double ref = tanh(x);
                     if (zmath::d2u(zmath::tanh_fdlibm(x)) != zmath::d2u(ref) || zmath::d2u(zmath::tanh_simd(x)) != zmath::d2u(ref)) b0++;
                     if (zmath::d2u(zmath::sigmoid_zenu(x)) != zmath::d2u(0.5 + 0.5 * tanh(0.5 * x))) b2++;

@@ -1483,6 +1483,36 @@ ZM_HD double cosh_fdlibm(double x, const uint64_t *etab)
     if (ix >= 0x7ff00000u) return x * x;                 // inf, NaN
     return huge * huge;                                  // overflow
 }
+// cosh in f64 as the kernels call it: below 0.5 ln2 expm1's k = 0 path written out (the general
+// expm1 brings all of its branches along; below 2^-54, where it returns its argument, and below 2^-55,
+// where cosh returns 1, the k = 0 formula gives the same), exp above, |x| >= 22 out of line.
+ZM_RARE double cosh_rare(double x, const uint64_t *etab) { return cosh_fdlibm(x, etab); }
+ZM_HD double cosh_simd(double x, const uint64_t *etab)
+{
+    const double one = 1.0, half = 0.5;
+    const double a = u2d(d2u(x) & 0x7fffffffffffffffull);
+    if (__builtin_expect(!(a < 22.0), 0)) return cosh_rare(x, etab);
+    if (hi_word(a) < 0x3fd62e43u) {                      // |x| < 0.5 ln2
+        const double Q1 = u2d(0xBFA11111111110F4ull), Q2 = u2d(0x3F5A01A019FE5585ull), Q3 = u2d(0xBF14CE199EAADBB7ull),
+                     Q4 = u2d(0x3ED0CFCA86E65239ull), Q5 = u2d(0xBE8AFDB76E09C32Dull);
+        const double hfx = half * a;
+        const double hxs = a * hfx;
+        const double R1 = one + hxs * Q1;
+        const double h2 = hxs * hxs;
+        const double R2 = Q2 + hxs * Q3;
+        const double h4 = h2 * h2;
+        const double R3 = Q4 + hxs * Q5;
+        const double r1 = R1 + h2 * R2 + h4 * R3;
+        const double t3 = 3.0 - r1 * hfx;
+        const double e = hxs * ((r1 - t3) / (6.0 - a * t3));
+        const double t = a - (a * e - hxs);
+        const double w = one + t;
+        return one + (t * t) / (w + w);
+    }
+    const double t = exp_glibc(a, etab);
+    return half * t + half / t;
+}
+
 ZM_HD double sinh_fdlibm(double x) { return sinh_fdlibm(x, exp_table()); }
 ZM_HD double cosh_fdlibm(double x) { return cosh_fdlibm(x, exp_table()); }
 
@@ -1667,9 +1697,9 @@ template <> struct ExpLog<double> {
     __device__ __forceinline__ double exp_flat(double x) const { return exp_glibc(x, etab); }
     __device__ __forceinline__ double log(double x) const { return ::log(x); }
     __device__ __forceinline__ double sinh(double x) const { return sinh_simd(x, etab); }
-    __device__ __forceinline__ double cosh(double x) const { return cosh_fdlibm(x, etab); }
+    __device__ __forceinline__ double cosh(double x) const { return cosh_simd(x, etab); }
     __device__ __forceinline__ double sinh(double x, const TanhRegs &) const { return sinh_simd(x, etab); }
-    __device__ __forceinline__ double cosh(double x, const TanhRegs &) const { return cosh_fdlibm(x, etab); }
+    __device__ __forceinline__ double cosh(double x, const TanhRegs &) const { return cosh_simd(x, etab); }
 };
 template <> struct ExpLog<float> {
     const uint64_t *etab;
