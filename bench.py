@@ -323,6 +323,17 @@ def build_ops(z, workload, stream):
                       mk(lambda A, P, U, R, O, V, S: (lambda d=V.desc(), s_=A.desc(): check(l.zenu_hip_sum_to(_lib.F32, ref(d), ref(s_), stream), "sum_to"))),
                       lambda: zo.sum_to(a, col_h)))
         ops[-1].keep = sets
+        # the f64 side of the unary family ([4096,4096] f64: 128 MiB in, 128 MiB out)
+        a64 = a.astype(np.float64)
+        out64_h = np.empty_like(a64)
+        sets64 = [(M.from_numpy(a64), M.alloc((n, n), dtype=np.float64)) for _ in range(nsets(4 * nb))]
+        for name, fn in (("exp f64", _lib.EXP), ("tanh f64", _lib.TANH), ("sigmoid f64", _lib.SIGMOID), ("sinh f64", _lib.SINH),
+                         ("cosh f64", _lib.COSH)):
+            ls = [(lambda d=O.desc(), s_=A.desc(), fn=fn: check(l.zenu_hip_unary(fn, _lib.F64, ref(d), ref(s_), stream), "unary f64"))
+                  for A, O in sets64]
+            cpu = (lambda: zo.sigmoid(out64_h, a64)) if fn == _lib.SIGMOID else (lambda fn=fn: zo.unary(fn, out64_h, a64))
+            ops.append(Op(name, "next", "f64", 4 * nb, n * n, ls, cpu))
+        ops[-1].keep = (sets, sets64)
 
     # ---- the same kernels on larger tensors: how much of the distance to the roofline is the fixed
     # cost of a launch at the BASELINE sizes (not a BASELINE config) --------------------------------------
@@ -752,13 +763,13 @@ def main():
         "metric": "achieved HBM GB/s (% of MI355X peak) per op; Adam step params/sec",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32" if args.workload != "suite" and args.workload != "c2" else "f32+f64", "data": "synthetic",
+        "dtype": "f32" if args.workload not in ("suite", "c2", "next") else "f32+f64", "data": "synthetic",
         "config": {"workload": {"suite": "configs[0..3]: every op once per step", "c0": "configs[0]", "c1": "configs[1]",
                                 "c2": "configs[2]", "c3": "configs[3]",
                                 "fused": "fused entry points on [8192,4096] f32 (not a BASELINE config)",
                                 "scaling": "copy, add, sums and tanh on 64 MiB, 256 MiB and 1 GiB f32 tensors (not a BASELINE config)",
-                                "next": "strided copy, broadcast, the remaining unary functions, powf, asum and sum_to on [4096,4096] f32 "
-                                        "(not a BASELINE config)"}[args.workload],
+                                "next": "strided copy, broadcast, the remaining unary functions, powf, asum and sum_to on [4096,4096] f32, "
+                                        "and exp / tanh / sigmoid / sinh / cosh on [4096,4096] f64 (not a BASELINE config)"}[args.workload],
                    "ops_per_step": len(table), "algorithmic_bytes_per_step": step_bytes},
         "frac_of_peak_whole_step": round(value / PEAK_HBM_GBPS, 4),
         "adam_step_params_per_sec": (round(adam[0]["Gelem_per_s"] * 1e9) if adam else None),

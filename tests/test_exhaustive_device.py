@@ -23,7 +23,8 @@ THREADS = 16
 # (Matrix method, oracle function id or None for the sigmoid composite, largest allowed distance in ulp)
 FUNCTIONS = [("tanh", zo.TANH, 0), ("sigmoid", None, 0), ("exp", zo.EXP, 0), ("log", zo.LOG, 0),
              ("sinh", zo.SINH, 0), ("cosh", zo.COSH, 0), ("sin", zo.SIN, 0), ("cos", zo.COS, 0),
-             ("asin", zo.ASIN, 0), ("acos", zo.ACOS, 0), ("atan", zo.ATAN, 0), ("tanh_ulp2", zo.TANH, 2)]
+             ("asin", zo.ASIN, 0), ("acos", zo.ACOS, 0), ("atan", zo.ATAN, 0), ("tanh_ulp2", zo.TANH, 2),
+             ("tan", zo.TAN, 1)]
 
 
 def oracle_chunk(fn, x, exponent=None):
