@@ -53,6 +53,12 @@ inline zenu_stream_t &current_stream()
     return s;
 }
 inline void synchronize() { check(zenu_hip_stream_synchronize(current_stream()), "stream_synchronize"); }
+// The first failure behind the reference-named void entry points of this thread since the last call
+// (ZENU_OK if none); reading clears it.
+inline int last_status() { return zenu_hip_last_status(); }
+// After the graphs captured on `stream` are destroyed: hand the blocks their captured calls took from
+// the pool back to it.
+inline void release_captured(zenu_stream_t stream) { check(zenu_hip_release_captured(stream), "release_captured"); }
 
 template <typename T> struct DType;
 template <> struct DType<float> { static constexpr int value = ZENU_F32; };
@@ -436,6 +442,13 @@ public:
         zenu_tensor_t o = out.desc(), s = desc();
         check(zenu_hip_sum_axis(dt(), &o, &s, axis, st()), "sum");
         return keep_dim ? out.add_axis(axis) : out;
+    }
+    // the same sum into an existing `out` through the entry point that allocates nothing (for callers that
+    // cannot allocate: its scratch is a fixed device array, see zenu_hip.h for the limits)
+    void sum_noalloc(int axis, const Matrix &out) const
+    {
+        zenu_tensor_t o = out.desc(), s = desc();
+        check(zenu_hip_sum_axis_noalloc(dt(), &o, &s, axis, st()), "sum_noalloc");
     }
     Matrix sum_all() const
     {

@@ -197,6 +197,11 @@ static void sum_4d()          // sum.rs:109-245
     a.sum_to(tot);
     REQUIRE(eq(tot, {7140.f}));
     REQUIRE(eq(a.sum_all(), {7140.f}));
+    // the entry point that allocates nothing gives the same sums into an existing matrix
+    M s0b = M::zeros({3, 4, 5});
+    a.sum_noalloc(0, s0b);
+    REQUIRE(eq(s0b, exp));
+    REQUIRE(zenu_hip::last_status() == ZENU_OK);
 }
 
 static void max_cases()       // max.rs:157-245
