@@ -472,6 +472,12 @@ def c4_summary(z, args, sync):
     return {
         "workload": C4_WORKLOAD, "dtype": "f32", "unit": "ms per training step",
         "eager_compiled_host_ms_per_step": ms_of("ops"),
+        # the part of it the host needs just to issue the launches (it runs ahead of the GPU): when this is
+        # close to the step time the step is bound by the host's per-launch cost, not by the kernels
+        "eager_compiled_host_issue_ms_per_step": (comp.get("ops") or {}).get("host_issue_ms_per_step") if isinstance(comp, dict) else None,
+        "fused_compiled_host_issue_ms_per_step": (comp.get("fused") or {}).get("host_issue_ms_per_step") if isinstance(comp, dict) else None,
+        # one-element adds issued back to back through the C ABI: the cost of a launch as such
+        "smallest_launch_us": (comp.get("floor") or {}).get("launch_us") if isinstance(comp, dict) else None,
         "fused_compiled_host_ms_per_step": ms_of("fused"),
         "fused_transposed_views_compiled_host_ms_per_step": ms_of("lean"),
         "eager_python_mirror_ms_per_step": round(r["ms"], 4),
@@ -507,7 +513,7 @@ def compiled_host_c4(x, t, params, args):
     res = {}
     for line in out.stdout.splitlines():
         w = line.split()
-        if len(w) == 3 and w[1] in ("ms_per_step", "final_loss"):
+        if len(w) == 3 and w[1] in ("ms_per_step", "host_issue_ms_per_step", "final_loss", "launch_us"):
             res.setdefault(w[0], {})[w[1]] = float(w[2])
     return res
 

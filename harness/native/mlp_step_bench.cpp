@@ -257,6 +257,19 @@ int main(int argc, char **argv)
             std::printf("rocblas init failed\n");
             return 1;
         }
+        {   // what one launch costs when the kernel does next to nothing: one-element adds issued back to
+            // back through the C ABI (the rate at which the HIP runtime and the dispatcher hand out kernels)
+            zenu_hip::Matrix<float> a = zenu_hip::Matrix<float>::zeros({1}), b = zenu_hip::Matrix<float>::zeros({1}),
+                                    c = zenu_hip::Matrix<float>::zeros({1});
+            zenu_tensor_t ta = a.desc(), tb = b.desc(), tc = c.desc();
+            const int n = 20000;
+            for (int i = 0; i < 2000; i++) zenu_hip_binary(ZENU_ADD, ZENU_F32, &tc, &ta, &tb, stream);
+            synchronize();
+            const auto t0 = std::chrono::steady_clock::now();
+            for (int i = 0; i < n; i++) zenu_hip_binary(ZENU_ADD, ZENU_F32, &tc, &ta, &tb, stream);
+            synchronize();
+            std::printf("floor launch_us %.3f\n", std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count() / n);
+        }
         for (int fused = 0; fused < 3; fused++) {
             const char *name = fused == 2 ? "lean" : fused ? "fused" : "ops";
             Step st;
@@ -269,9 +282,12 @@ int main(int argc, char **argv)
             synchronize();
             const auto t0 = std::chrono::steady_clock::now();
             for (int i = 0; i < steps; i++) st.run(fused);
+            // time the host needed to issue the steps (it runs ahead of the GPU until the queue is full)
+            const double issue_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / steps;
             synchronize();
             const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / steps;
             std::printf("%s ms_per_step %.4f\n", name, ms);
+            std::printf("%s host_issue_ms_per_step %.4f\n", name, issue_ms);
             std::printf("%s final_loss %.9g\n", name, (double)st.loss.to_vec()[0]);
             std::fflush(stdout);
         }
