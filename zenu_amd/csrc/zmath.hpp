@@ -1533,8 +1533,9 @@ ZM_HD float sigmoidf_zenu(float x, const TanhRegs &rg = TanhRegs())
 
 // tanh of an f32 evaluated in f64 and rounded once: NOT the host library's bits, but never more
 // than 2 units in the last place away from them (the largest distance over all 2^32 arguments
-// is 2: 97.23 % equal, 2.76 % one apart, 0.017 % two apart) at a third of the instructions of
-// tanhf_simd.  tanh|x| = em1 / (em1 + 2) with em1 = exp(2|x|) - 1 = 2^k (1 + r p(r)) - 1, where
+// is 2: 97.23 % equal, 2.76 % one apart, 0.017 % two apart) in about 37 vector instructions.
+// (tanhf_simd has since come down to 57 and is the faster of the two: its f32 instructions cost one
+// issue slot each, the f64 division and conversions here more.)  tanh|x| = em1 / (em1 + 2) with em1 = exp(2|x|) - 1 = 2^k (1 + r p(r)) - 1, where
 // 2|x| = k ln2 + r, |r| <= ln2 / 2, and p is a degree-8 fit of (exp(r) - 1) / r (relative error
 // of exp below 2^-44).  With k = 0 the term 2^k - 1 vanishes and em1 = r p(r) keeps its relative
 // accuracy down to the smallest subnormal.  Only IEEE operations, so host and device agree bit
