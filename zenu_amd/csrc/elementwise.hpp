@@ -93,8 +93,8 @@ __device__ __forceinline__ double dev_atan(double x) { return atan(x); }
 __device__ __forceinline__ float dev_sigmoid(float x, const zmath::TanhRegs &rg) { return zmath::sigmoidf_zenu(x, rg); }
 __device__ __forceinline__ double dev_sigmoid(double x, const zmath::TanhRegs &) { return zmath::sigmoid_zenu(x); }
 
-// what single functions carry besides: the f64 constants of the f32 sine / cosine (in the functor, a
-// kernel argument), the range table of the f32 arc tangent (in LDS); every other function nothing
+// what single functions carry besides: the f64 constants of the f32 sine / cosine / tangent (in the
+// functor, a kernel argument), the range table of the f32 arc tangent (in LDS); every other function nothing
 template <typename T, int FN> struct UnaryExtra {
     __device__ __forceinline__ void init() {}
 };
@@ -119,7 +119,7 @@ template <typename T, int FN> struct UnaryF {
     static constexpr int NIN = 1;
     zmath::ExpLog<T> m;     // exp / log state (f32: tables in LDS)
     zmath::TanhRegs tr;     // f32 tanh / sigmoid / sinh / cosh: two constants held in vector registers
-    UnaryExtra<T, FN> sc;   // f32 sin / cos: the f64 constants, as data; f32 atan: its table
+    UnaryExtra<T, FN> sc;   // f32 sin / cos / tan: the f64 constants, as data; f32 atan: its table
     __device__ __forceinline__ void init()
     {
         if constexpr (FN == ZENU_EXP || FN == ZENU_LOG || FN == ZENU_SINH || FN == ZENU_COSH)
