@@ -522,6 +522,7 @@ struct TileParams {
     int vec_ok;                 // alignment allows 128-bit accesses on full tiles
     int grid3d;                 // the grid is (tiles_c, tiles_r, nbatch); else linear, tiles_c fastest
     int64_t tiles_r, tiles_c;
+    uint32_t tiles_r_magic;     // min(floor(2^32 / tiles_r), 2^32 - 1): x mod tiles_r from one high multiply and a fix-up
 };
 
 template <typename T, bool NT, typename F>
@@ -552,31 +553,50 @@ __global__ __launch_bounds__((TileThreads<T, F>::value)) void ew_tile_kernel(T *
     // The grid is (column tiles, row tiles, batch) when that fits the grid limits, so that no
     // workgroup starts with a chain of integer divisions (in 64 bits they were most of this kernel's
     // instructions); otherwise a linear grid below 2^31, decomposed in 32 bits.
+    // Every wave of the workgroup runs this scalar prologue, and nothing is in flight before it ends:
+    // the fields it needs are read from the argument block together (one wait, not one per branch),
+    // and the diagonal's remainder comes from a multiplier that the host prepared, not from a division.
+    int grid3d = p.grid3d, vec_ok = p.vec_ok, nouter = p.outer.nouter;
+    uint32_t ntr = (uint32_t)p.tiles_r, magic = p.tiles_r_magic;
+    int64_t R = p.R, C = p.C;
+    int64_t ldr0 = p.ldr[0], ldr1 = p.ldr[1], ldr2 = p.ldr[2], ldc1 = p.ldc[1], ldc2 = p.ldc[2];
+    int trans_a = p.trans_a, trans_b = p.trans_b;
+    asm volatile("" : "+s"(grid3d), "+s"(vec_ok), "+s"(nouter), "+s"(ntr), "+s"(magic), "+s"(R), "+s"(C),
+                      "+s"(ldr0), "+s"(ldr1), "+s"(ldr2), "+s"(ldc1), "+s"(ldc2), "+s"(trans_a), "+s"(trans_b),
+                      "+s"(out), "+s"(a), "+s"(b));
     uint32_t tc32, tr32, batch32;
-    if (p.grid3d) {
+    if (grid3d) {
         tc32 = blockIdx.x;
         tr32 = blockIdx.y;
         batch32 = blockIdx.z;
     } else {
-        const uint32_t ntc = (uint32_t)p.tiles_c, ntr = (uint32_t)p.tiles_r;
+        const uint32_t ntc = (uint32_t)p.tiles_c;
         const uint32_t q = blockIdx.x / ntc;
         tc32 = blockIdx.x - q * ntc;
         batch32 = q / ntr;
         tr32 = q - batch32 * ntr;
     }
-    tr32 = (tr32 + tc32) % (uint32_t)p.tiles_r;
+    {
+        // (tr + tc) mod tiles_r: the multiplier is floor(2^32 / tiles_r) (2^32 - 1 for one tile row),
+        // which is less than 1 below 2^32 / tiles_r, so for every 32-bit argument the quotient is
+        // exact or one too small (the sum is below 2^32: both grids are)
+        const uint32_t x = tr32 + tc32;
+        const uint32_t q = __umulhi(x, magic);
+        const uint32_t r = x - q * ntr;
+        tr32 = r >= ntr ? r - ntr : r;
+    }
     const int64_t tc = tc32, tr = tr32;
-    int64_t oo, oa, ob;
-    decompose32(p.outer, batch32, oo, oa, ob);
+    int64_t oo = 0, oa = 0, ob = 0;
+    if (nouter > 0) decompose32(p.outer, batch32, oo, oa, ob);
     const int64_t r0 = tr * kTile, c0 = tc * kTile;
-    const int64_t nr = (p.R - r0 < kTile) ? p.R - r0 : kTile;
-    const int64_t nc = (p.C - c0 < kTile) ? p.C - c0 : kTile;
-    const bool full = (nr == kTile) && (nc == kTile) && p.vec_ok;
+    const int64_t nr = (R - r0 < kTile) ? R - r0 : kTile;
+    const int64_t nc = (C - c0 < kTile) ? C - c0 : kTile;
+    const bool full = (nr == kTile) & (nc == kTile) & (vec_ok != 0);
     const int tid = threadIdx.x;
 
-    T *obase = out + oo + r0 * p.ldr[0] + c0;
-    const T *abase = a + oa + r0 * p.ldr[1] + c0 * p.ldc[1];
-    const T *bbase = (F::NIN == 2) ? b + ob + r0 * p.ldr[2] + c0 * p.ldc[2] : abase;
+    T *obase = out + oo + r0 * ldr0 + c0;
+    const T *abase = a + oa + r0 * ldr1 + c0 * ldc1;
+    const T *bbase = (F::NIN == 2) ? b + ob + r0 * ldr2 + c0 * ldc2 : abase;
 
     if (full) {
         // All global loads of the tile are issued first -- the transposed inputs along R (their
@@ -588,20 +608,20 @@ __global__ __launch_bounds__((TileThreads<T, F>::value)) void ew_tile_kernel(T *
         const int seg_v = (tid % VPS) * VEC;            // vector position inside the segment
         auto other_of = [&](int k) { return ((k * kBlock + tid) / VPS) % kTile; };                  // position along the other dim
         auto vec_of = [&](int k) { return seg_v + (((k * kBlock + tid) / VPS) / kTile) * VPS * VEC; };  // element position along the vector dim
-        const bool ta = p.trans_a != 0;
-        const bool tb = (F::NIN == 2) && p.trans_b != 0;
+        const bool ta = trans_a != 0;
+        const bool tb = (F::NIN == 2) && trans_b != 0;
         Pack<T, VEC> xa[K], xb[K];
 #pragma unroll
         for (int k = 0; k < K; k++) {
             const int o = other_of(k);
             const int lane_v = vec_of(k);
-            if (ta) xa[k] = load_pack<T, VEC, NT>(abase + lane_v + (int64_t)o * p.ldc[1]);
-            else if (p.ldc[1] == 0) xa[k] = splat<T, VEC>(abase[(int64_t)o * p.ldr[1]]);
-            else xa[k] = load_pack<T, VEC, NT>(abase + (int64_t)o * p.ldr[1] + lane_v);
+            if (ta) xa[k] = load_pack<T, VEC, NT>(abase + lane_v + (int64_t)o * ldc1);
+            else if (ldc1 == 0) xa[k] = splat<T, VEC>(abase[(int64_t)o * ldr1]);
+            else xa[k] = load_pack<T, VEC, NT>(abase + (int64_t)o * ldr1 + lane_v);
             if constexpr (F::NIN == 2) {
-                if (tb) xb[k] = load_pack<T, VEC, NT>(bbase + lane_v + (int64_t)o * p.ldc[2]);
-                else if (p.ldc[2] == 0) xb[k] = splat<T, VEC>(bbase[(int64_t)o * p.ldr[2]]);
-                else xb[k] = load_pack<T, VEC, NT>(bbase + (int64_t)o * p.ldr[2] + lane_v);
+                if (tb) xb[k] = load_pack<T, VEC, NT>(bbase + lane_v + (int64_t)o * ldc2);
+                else if (ldc2 == 0) xb[k] = splat<T, VEC>(bbase[(int64_t)o * ldr2]);
+                else xb[k] = load_pack<T, VEC, NT>(bbase + (int64_t)o * ldr2 + lane_v);
             }
         }
         if (ta || tb) {
@@ -637,17 +657,17 @@ __global__ __launch_bounds__((TileThreads<T, F>::value)) void ew_tile_kernel(T *
             } else {
                 y = x;
             }
-            store_pack<T, VEC, NT>(obase + (int64_t)r * p.ldr[0] + lane_v, apply_pack<T, VEC, F>(f, x, y));
+            store_pack<T, VEC, NT>(obase + (int64_t)r * ldr0 + lane_v, apply_pack<T, VEC, F>(f, x, y));
         }
     } else {
         // edge tiles and unaligned operands: element-wise with bounds checks
-        if (p.trans_a || (F::NIN == 2 && p.trans_b)) {
+        if (trans_a || (F::NIN == 2 && trans_b)) {
             for (int e = tid; e < kTile * kTile; e += kBlock) {
                 const int r = e % kTile, c = e / kTile;
                 if (r < nr && c < nc) {
-                    if (p.trans_a) lds_a[r * kPitch + c] = abase[r + (int64_t)c * p.ldc[1]];
+                    if (trans_a) lds_a[r * kPitch + c] = abase[r + (int64_t)c * ldc1];
                     if constexpr (F::NIN == 2) {
-                        if (p.trans_b) lds_b[r * kPitch + c] = bbase[r + (int64_t)c * p.ldc[2]];
+                        if (trans_b) lds_b[r * kPitch + c] = bbase[r + (int64_t)c * ldc2];
                     }
                 }
             }
@@ -656,12 +676,12 @@ __global__ __launch_bounds__((TileThreads<T, F>::value)) void ew_tile_kernel(T *
         for (int e = tid; e < kTile * kTile; e += kBlock) {
             const int c = e % kTile, r = e / kTile;
             if (r < nr && c < nc) {
-                T x = p.trans_a ? lds_a[r * kPitch + c] : abase[(int64_t)r * p.ldr[1] + (int64_t)c * p.ldc[1]];
+                T x = trans_a ? lds_a[r * kPitch + c] : abase[(int64_t)r * ldr1 + (int64_t)c * ldc1];
                 T y = x;
                 if constexpr (F::NIN == 2)
-                    y = p.trans_b ? lds_b[r * kPitch + c]
-                                  : bbase[(int64_t)r * p.ldr[2] + (int64_t)c * p.ldc[2]];
-                obase[(int64_t)r * p.ldr[0] + c] = f(x, y);
+                    y = trans_b ? lds_b[r * kPitch + c]
+                                  : bbase[(int64_t)r * ldr2 + (int64_t)c * ldc2];
+                obase[(int64_t)r * ldr0 + c] = f(x, y);
             }
         }
     }
@@ -950,6 +970,10 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
             constexpr int kTile = TileOf<T>::N;
             tp.tiles_r = (tp.R + kTile - 1) / kTile;
             tp.tiles_c = (tp.C + kTile - 1) / kTile;
+            {
+                const uint64_t m = (1ull << 32) / (uint64_t)tp.tiles_r;
+                tp.tiles_r_magic = m > 0xffffffffull ? 0xffffffffu : (uint32_t)m;
+            }
             int64_t grid = tp.nbatch * tp.tiles_r * tp.tiles_c;
             if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
             tp.grid3d = (tp.tiles_r <= 65535 && tp.nbatch <= 65535) ? 1 : 0;
