@@ -826,6 +826,33 @@ def test_copy_transpose_large(hip):
     assert_bits(dst.to_numpy(), np.ascontiguousarray(a.T), "copy into transposed")
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("pitch_out,pitch_in", [(1024, 1024), (1024, 1100), (1100, 1024), (1100, 1100),
+                                                (1028, 2048), (2048, 1028)])
+def test_transposed_views_every_tile_walk(hip, dt, pitch_out, pitch_in):
+    # The tile kernel walks its tiles row by row, column by column or along diagonals, picked by
+    # how close the operands' pitches are to a multiple of 4 KiB: all three orders, with ragged
+    # edge tiles (neither extent is a multiple of the tile) and with whole tiles, copy and a + b^T.
+    r = rng(31)
+    for rows, cols in ((300, 210), (256, 192)):
+        b = r.standard_normal((cols, pitch_in)).astype(dt)
+        a = r.standard_normal((rows, pitch_out)).astype(dt)
+        B, A = hip.Matrix.from_numpy(b), hip.Matrix.from_numpy(a)
+        bt = b[:, :rows].T                                  # [rows, cols], unit stride along rows
+        Bt = B.slice(slice(None), slice(0, rows)).transpose()
+        av = a[:, :cols]
+        Av = A.slice(slice(None), slice(0, cols))
+        out = hip.Matrix.zeros((rows, pitch_out), dt)
+        Ov = out.slice(slice(None), slice(0, cols))
+        Ov.copy_from(Bt)
+        assert_bits(out.to_numpy()[:, :cols], bt, f"copy b^T {rows}x{cols} pitches {pitch_out}/{pitch_in}")
+        assert not out.to_numpy()[:, cols:].any(), "wrote outside the view"
+        Ov.add_array(Av, Bt)
+        exp = np.empty((rows, cols), dtype=dt)
+        zo.binary_array(zo.ADD, exp, av, bt)
+        assert_bits(out.to_numpy()[:, :cols], exp, f"a + b^T {rows}x{cols} pitches {pitch_out}/{pitch_in}")
+
+
 # ---- config[2]: [8192,4096] reductions, normal(0,1), seed 2, ~1% duplicate maxima ---------------------------
 
 def make_c2(dt):

@@ -512,6 +512,8 @@ template <typename T, typename F> struct TileThreads {
     static constexpr int value = F::NIN == 1 ? TileOf<T>::N * TileOf<T>::N / VecOf<T>::N : 256;
 };
 
+enum { kWalkRows = 0, kWalkCols = 1, kWalkDiagonal = 2 };
+
 struct TileParams {
     OuterDesc outer;      // batch dims (everything except the two tile dims)
     int64_t nbatch;
@@ -521,6 +523,7 @@ struct TileParams {
     int trans_a, trans_b;       // input goes through LDS
     int vec_ok;                 // alignment allows 128-bit accesses on full tiles
     int grid3d;                 // the grid is (tiles_c, tiles_r, nbatch); else linear, tiles_c fastest
+    int walk;                   // order of the tiles: kWalkRows, kWalkCols (3-d grids only) or kWalkDiagonal
     int64_t tiles_r, tiles_c;
     uint32_t tiles_r_magic;     // min(floor(2^32 / tiles_r), 2^32 - 1): x mod tiles_r from one high multiply and a fix-up
 };
@@ -545,29 +548,34 @@ __global__ __launch_bounds__((TileThreads<T, F>::value)) void ew_tile_kernel(T *
     __shared__ T lds_b[(F::NIN == 2) ? kTile * kPitch : 1];
     f.init();
 
-    // Tiles are walked along diagonals: consecutive workgroups (which run together) differ in BOTH
-    // tile coordinates.  Walking a tile row, they would read (or, walking a tile column, write) row
-    // pieces whose addresses differ by multiples of the matrix pitch; with a power-of-two pitch those
-    // fall on the same few memory channels (transposed copy of [4096,4096]: 26.8 us row by row,
-    // 29.1 us column by column, 25.2 us diagonally with the same 64x64 tiles).
+    // The order in which the tiles are walked decides which addresses the workgroups that run
+    // together touch.  Row by row (consecutive workgroups along the output's rows) they read pieces
+    // of a transposed input that lie a tile's height times ITS pitch apart; column by column they
+    // write pieces (and read those of the other inputs) that far apart by the output's pitch; along
+    // diagonals consecutive workgroups differ in both tile coordinates.  A distance that is a
+    // multiple of 4 KiB lands on few memory channels, so the host picks the walk by the pitches
+    // (transposed copy of 4096 x 4096 f32, pitch of the output / of the input in elements, us row by
+    // row / column by column / diagonally: 4096 / 4096: 26.3 / 27.6 / 24.0; 4096 / 4352: 24.1 / 28.5 /
+    // 26.7; 4352 / 4096: 26.4 / 24.9 / 28.3; 4352 / 4352: 24.1 / 25.3 / 31.2; 5120 / 5120: 26.6 / 29.4 / 25.8).
     // The grid is (column tiles, row tiles, batch) when that fits the grid limits, so that no
     // workgroup starts with a chain of integer divisions (in 64 bits they were most of this kernel's
     // instructions); otherwise a linear grid below 2^31, decomposed in 32 bits.
     // Every wave of the workgroup runs this scalar prologue, and nothing is in flight before it ends:
     // the fields it needs are read from the argument block together (one wait, not one per branch),
     // and the diagonal's remainder comes from a multiplier that the host prepared, not from a division.
-    int grid3d = p.grid3d, vec_ok = p.vec_ok, nouter = p.outer.nouter;
+    int grid3d = p.grid3d, vec_ok = p.vec_ok, nouter = p.outer.nouter, walk = p.walk;
     uint32_t ntr = (uint32_t)p.tiles_r, magic = p.tiles_r_magic;
     int64_t R = p.R, C = p.C;
     int64_t ldr0 = p.ldr[0], ldr1 = p.ldr[1], ldr2 = p.ldr[2], ldc1 = p.ldc[1], ldc2 = p.ldc[2];
     int trans_a = p.trans_a, trans_b = p.trans_b;
-    asm volatile("" : "+s"(grid3d), "+s"(vec_ok), "+s"(nouter), "+s"(ntr), "+s"(magic), "+s"(R), "+s"(C),
+    asm volatile("" : "+s"(grid3d), "+s"(vec_ok), "+s"(nouter), "+s"(walk), "+s"(ntr), "+s"(magic), "+s"(R), "+s"(C),
                       "+s"(ldr0), "+s"(ldr1), "+s"(ldr2), "+s"(ldc1), "+s"(ldc2), "+s"(trans_a), "+s"(trans_b),
                       "+s"(out), "+s"(a), "+s"(b));
     uint32_t tc32, tr32, batch32;
     if (grid3d) {
-        tc32 = blockIdx.x;
-        tr32 = blockIdx.y;
+        const bool by_cols = walk == kWalkCols;       // then the grid is (row tiles, column tiles, batch)
+        tc32 = by_cols ? blockIdx.y : blockIdx.x;
+        tr32 = by_cols ? blockIdx.x : blockIdx.y;
         batch32 = blockIdx.z;
     } else {
         const uint32_t ntc = (uint32_t)p.tiles_c;
@@ -576,7 +584,7 @@ __global__ __launch_bounds__((TileThreads<T, F>::value)) void ew_tile_kernel(T *
         batch32 = q / ntr;
         tr32 = q - batch32 * ntr;
     }
-    {
+    if (walk == kWalkDiagonal) {
         // (tr + tc) mod tiles_r: the multiplier is floor(2^32 / tiles_r) (2^32 - 1 for one tile row),
         // which is less than 1 below 2^32 / tiles_r, so for every 32-bit argument the quotient is
         // exact or one too small (the sum is below 2^32: both grids are)
@@ -977,7 +985,23 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
             int64_t grid = tp.nbatch * tp.tiles_r * tp.tiles_c;
             if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
             tp.grid3d = (tp.tiles_r <= 65535 && tp.nbatch <= 65535) ? 1 : 0;
-            const dim3 g = tp.grid3d ? dim3((unsigned)tp.tiles_c, (unsigned)tp.tiles_r, (unsigned)tp.nbatch) : dim3((unsigned)grid);
+            // Row by row unless a transposed input's pitch is within one row piece of a multiple of
+            // 4 KiB; then column by column if no other operand's pitch is, else along diagonals.
+            auto near_4k = [](int64_t elems) {
+                const int64_t r = ((elems < 0 ? -elems : elems) * (int64_t)sizeof(T)) % 4096;
+                return (r < 4096 - r ? r : 4096 - r) < kTile * (int64_t)sizeof(T);
+            };
+            bool trans_near = false, direct_near = near_4k(tp.ldr[0]);
+            for (int o = 1; o <= nin; o++) {
+                if (trans[o]) trans_near = trans_near || near_4k(tp.ldc[o]);
+                else if (tp.ldc[o] == 1) direct_near = direct_near || near_4k(tp.ldr[o]);
+            }
+            tp.walk = !trans_near ? kWalkRows
+                      : (!direct_near && tp.grid3d && tp.tiles_c <= 65535) ? kWalkCols : kWalkDiagonal;
+            const bool by_cols = tp.walk == kWalkCols;
+            const dim3 g = !tp.grid3d ? dim3((unsigned)grid)
+                           : by_cols ? dim3((unsigned)tp.tiles_r, (unsigned)tp.tiles_c, (unsigned)tp.nbatch)
+                                     : dim3((unsigned)tp.tiles_c, (unsigned)tp.tiles_r, (unsigned)tp.nbatch);
             if (nt) ew_tile_kernel<T, true, F><<<g, TileThreads<T, F>::value, 0, stream>>>(out, a, b, tp, f);
             else    ew_tile_kernel<T, false, F><<<g, TileThreads<T, F>::value, 0, stream>>>(out, a, b, tp, f);
             ZENU_LAUNCH_CHECK();
