@@ -428,6 +428,7 @@ struct RowsParams {
     int inner_b;       // inner stride of input b: 1 or 0
     int tx_shift;      // threads along the row = 1 << tx_shift (<= 256)
     int64_t col_tiles; // column tiles per row
+    int grid2d;        // the grid is (column tiles, row blocks); else linear, column tiles fastest
 };
 
 // NTA / NTB: input a / b is streamed once (not broadcast along an outer dim); the output is
@@ -438,18 +439,38 @@ __global__ __launch_bounds__(kBlock) void ew_rows_kernel(T *out, const T *a, con
                                                          RowsParams p, F f)
 {
     f.init();
-    const int tx_n = 1 << p.tx_shift;
-    const int ty_n = kBlock >> p.tx_shift;
+    // The workgroups are short-lived, so the scalar work before the first load counts: every field
+    // of the argument block that the common case needs is read here, together (one wait instead of
+    // one per branch), and a 2-d grid spares the division of the workgroup index.
+    int tx_shift = p.tx_shift, inner_a = p.inner_a, inner_b = p.inner_b, nouter = p.outer.nouter, grid2d = p.grid2d;
+    int64_t nrows = p.nrows, ncols = p.ncols;
+    int64_t so0 = p.outer.stride[0][0], sa0 = p.outer.stride[1][0], sb0 = p.outer.stride[2][0];
+    asm volatile("" : "+s"(tx_shift), "+s"(inner_a), "+s"(inner_b), "+s"(nouter), "+s"(grid2d), "+s"(nrows),
+                      "+s"(ncols), "+s"(so0), "+s"(sa0), "+s"(sb0), "+s"(out), "+s"(a), "+s"(b));
+    const int tx_n = 1 << tx_shift;
+    const int ty_n = kBlock >> tx_shift;
     const int tx = threadIdx.x & (tx_n - 1);
-    const int ty = threadIdx.x >> p.tx_shift;
-    // grid and col_tiles fit 32 bits (checked at launch)
-    const uint32_t row_blk32 = blockIdx.x / (uint32_t)p.col_tiles;
-    const int64_t row_blk = row_blk32;
-    const int64_t col_tile = blockIdx.x - row_blk32 * (uint32_t)p.col_tiles;
-    const int64_t row = row_blk * ty_n + ty;
-    if (row >= p.nrows) return;
+    const int ty = threadIdx.x >> tx_shift;
+    uint32_t row_blk32, col_tile32;
+    if (grid2d) {
+        col_tile32 = blockIdx.x;
+        row_blk32 = blockIdx.y;
+    } else {
+        // grid and col_tiles fit 32 bits (checked at launch)
+        row_blk32 = blockIdx.x / (uint32_t)p.col_tiles;
+        col_tile32 = blockIdx.x - row_blk32 * (uint32_t)p.col_tiles;
+    }
+    const int64_t col_tile = col_tile32;
+    const int64_t row = (int64_t)row_blk32 * ty_n + ty;
+    if (row >= nrows) return;
     int64_t oo, oa, ob;
-    decompose(p.outer, row, oo, oa, ob);
+    if (nouter == 1) {            // one outer dim: the row index is its coordinate
+        oo = row * so0;
+        oa = row * sa0;
+        ob = row * sb0;
+    } else {
+        decompose(p.outer, row, oo, oa, ob);
+    }
     T *orow = out + oo;
     const T *arow = a + oa;
     const T *brow = (F::NIN == 2) ? b + ob : arow;
@@ -457,16 +478,16 @@ __global__ __launch_bounds__(kBlock) void ew_rows_kernel(T *out, const T *a, con
     const int64_t cols_per_tile = (int64_t)tx_n * VEC * kUnroll;
     const int64_t c0 = col_tile * cols_per_tile;
     Pack<T, VEC> sa, sb;
-    if (p.inner_a == 0) sa = splat<T, VEC>(arow[0]);
-    if (F::NIN == 2 && p.inner_b == 0) sb = splat<T, VEC>(brow[0]);
+    if (inner_a == 0) sa = splat<T, VEC>(arow[0]);
+    if (F::NIN == 2 && inner_b == 0) sb = splat<T, VEC>(brow[0]);
 
-    if (c0 + cols_per_tile <= p.ncols) {
+    if (c0 + cols_per_tile <= ncols) {
         Pack<T, VEC> va[kUnroll], vb[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             int64_t c = c0 + ((int64_t)u * tx_n + tx) * VEC;
-            va[u] = p.inner_a ? load_pack<T, VEC, NTA>(arow + c) : sa;
-            if constexpr (F::NIN == 2) vb[u] = p.inner_b ? load_pack<T, VEC, NTB>(brow + c) : sb;
+            va[u] = inner_a ? load_pack<T, VEC, NTA>(arow + c) : sa;
+            if constexpr (F::NIN == 2) vb[u] = inner_b ? load_pack<T, VEC, NTB>(brow + c) : sb;
             else vb[u] = va[u];
         }
 #pragma unroll
@@ -477,17 +498,17 @@ __global__ __launch_bounds__(kBlock) void ew_rows_kernel(T *out, const T *a, con
     } else {
         for (int u = 0; u < kUnroll; u++) {
             int64_t c = c0 + ((int64_t)u * tx_n + tx) * VEC;
-            if (c + VEC <= p.ncols) {
-                Pack<T, VEC> x = p.inner_a ? load_pack<T, VEC, false>(arow + c) : sa;
+            if (c + VEC <= ncols) {
+                Pack<T, VEC> x = inner_a ? load_pack<T, VEC, false>(arow + c) : sa;
                 Pack<T, VEC> y = x;
-                if constexpr (F::NIN == 2) y = p.inner_b ? load_pack<T, VEC, false>(brow + c) : sb;
+                if constexpr (F::NIN == 2) y = inner_b ? load_pack<T, VEC, false>(brow + c) : sb;
                 store_pack<T, VEC, false>(orow + c, apply_pack<T, VEC, F>(f, x, y));
             } else {
                 for (int j = 0; j < VEC; j++) {
-                    if (c + j < p.ncols) {
-                        T x = p.inner_a ? arow[c + j] : sa.v[0];
+                    if (c + j < ncols) {
+                        T x = inner_a ? arow[c + j] : sa.v[0];
                         T y = x;
-                        if constexpr (F::NIN == 2) y = p.inner_b ? brow[c + j] : sb.v[0];
+                        if constexpr (F::NIN == 2) y = inner_b ? brow[c + j] : sb.v[0];
                         orow[c + j] = f(x, y);
                     }
                 }
@@ -708,6 +729,7 @@ struct StridedRowsParams {
     int64_t inner[kMaxOperands];   // stride along the innermost dim per operand (any value)
     int tx_shift;
     int64_t col_tiles;
+    int grid2d;        // the grid is (column tiles, row blocks); else linear, column tiles fastest
 };
 
 template <typename T, typename F, int kUnroll, bool NT>
@@ -715,26 +737,45 @@ __global__ __launch_bounds__(kBlock) void ew_strided_rows_kernel(T *out, const T
                                                                  StridedRowsParams p, F f)
 {
     f.init();
-    const int tx_n = 1 << p.tx_shift;
-    const int ty_n = kBlock >> p.tx_shift;
+    // as in the rows kernel: the argument block is read once, at the top, and a 2-d grid spares the division
+    int tx_shift = p.tx_shift, nouter = p.outer.nouter, grid2d = p.grid2d;
+    int64_t nrows = p.nrows, ncols = p.ncols;
+    int64_t so0 = p.outer.stride[0][0], sa0 = p.outer.stride[1][0], sb0 = p.outer.stride[2][0];
+    int64_t so = p.inner[0], sa = p.inner[1], sb = p.inner[2];
+    asm volatile("" : "+s"(tx_shift), "+s"(nouter), "+s"(grid2d), "+s"(nrows), "+s"(ncols), "+s"(so0), "+s"(sa0),
+                      "+s"(sb0), "+s"(so), "+s"(sa), "+s"(sb), "+s"(out), "+s"(a), "+s"(b));
+    const int tx_n = 1 << tx_shift;
+    const int ty_n = kBlock >> tx_shift;
     const int tx = threadIdx.x & (tx_n - 1);
-    const int ty = threadIdx.x >> p.tx_shift;
-    const uint32_t row_blk32 = blockIdx.x / (uint32_t)p.col_tiles;   // grid and col_tiles fit 32 bits (checked at launch)
-    const int64_t col_tile = blockIdx.x - row_blk32 * (uint32_t)p.col_tiles;
+    const int ty = threadIdx.x >> tx_shift;
+    uint32_t row_blk32, col_tile32;
+    if (grid2d) {
+        col_tile32 = blockIdx.x;
+        row_blk32 = blockIdx.y;
+    } else {
+        row_blk32 = blockIdx.x / (uint32_t)p.col_tiles;   // grid and col_tiles fit 32 bits (checked at launch)
+        col_tile32 = blockIdx.x - row_blk32 * (uint32_t)p.col_tiles;
+    }
+    const int64_t col_tile = col_tile32;
     const int64_t row = (int64_t)row_blk32 * ty_n + ty;
-    if (row >= p.nrows) return;
+    if (row >= nrows) return;
     int64_t oo, oa, ob;
-    decompose(p.outer, row, oo, oa, ob);
+    if (nouter == 1) {
+        oo = row * so0;
+        oa = row * sa0;
+        ob = row * sb0;
+    } else {
+        decompose(p.outer, row, oo, oa, ob);
+    }
     T *orow = out + oo;
     const T *arow = a + oa;
     const T *brow = (F::NIN == 2) ? b + ob : arow;
-    const int64_t so = p.inner[0], sa = p.inner[1], sb = p.inner[2];
     const int64_t c0 = col_tile * ((int64_t)tx_n * kUnroll) + tx;
     T x[kUnroll], y[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {          // all loads of the thread first
         const int64_t c = c0 + (int64_t)u * tx_n;
-        if (c < p.ncols) {
+        if (c < ncols) {
             x[u] = load_pack<T, 1, NT>(arow + c * sa).v[0];
             y[u] = (F::NIN == 2) ? load_pack<T, 1, NT>(brow + c * sb).v[0] : x[u];
         }
@@ -742,7 +783,7 @@ __global__ __launch_bounds__(kBlock) void ew_strided_rows_kernel(T *out, const T
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
         const int64_t c = c0 + (int64_t)u * tx_n;
-        if (c < p.ncols) {
+        if (c < ncols) {
             Pack<T, 1> r;
             r.v[0] = f(x[u], y[u]);
             store_pack<T, 1, NT>(orow + c * so, r);
@@ -911,13 +952,15 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
             int64_t cols_per_tile = ((int64_t)1 << shift) * v * U;
             rp.col_tiles = (rp.ncols + cols_per_tile - 1) / cols_per_tile;
             int64_t rows_per_blk = B >> shift;
-            int64_t grid = ((rp.nrows + rows_per_blk - 1) / rows_per_blk) * rp.col_tiles;
-            if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-            if (!vec)            ew_rows_kernel<T, 1, false, false, F, B, U><<<(unsigned)grid, B, 0, stream>>>(out, a, b, rp, f);
-            else if (nta && ntb) ew_rows_kernel<T, VEC, true, true, F, B, U><<<(unsigned)grid, B, 0, stream>>>(out, a, b, rp, f);
-            else if (nta)        ew_rows_kernel<T, VEC, true, false, F, B, U><<<(unsigned)grid, B, 0, stream>>>(out, a, b, rp, f);
-            else if (ntb)        ew_rows_kernel<T, VEC, false, true, F, B, U><<<(unsigned)grid, B, 0, stream>>>(out, a, b, rp, f);
-            else                 ew_rows_kernel<T, VEC, false, false, F, B, U><<<(unsigned)grid, B, 0, stream>>>(out, a, b, rp, f);
+            const int64_t row_blks = (rp.nrows + rows_per_blk - 1) / rows_per_blk;
+            if (row_blks * rp.col_tiles > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
+            rp.grid2d = row_blks <= 65535 ? 1 : 0;
+            const dim3 grid = rp.grid2d ? dim3((unsigned)rp.col_tiles, (unsigned)row_blks) : dim3((unsigned)(row_blks * rp.col_tiles));
+            if (!vec)            ew_rows_kernel<T, 1, false, false, F, B, U><<<grid, B, 0, stream>>>(out, a, b, rp, f);
+            else if (nta && ntb) ew_rows_kernel<T, VEC, true, true, F, B, U><<<grid, B, 0, stream>>>(out, a, b, rp, f);
+            else if (nta)        ew_rows_kernel<T, VEC, true, false, F, B, U><<<grid, B, 0, stream>>>(out, a, b, rp, f);
+            else if (ntb)        ew_rows_kernel<T, VEC, false, true, F, B, U><<<grid, B, 0, stream>>>(out, a, b, rp, f);
+            else                 ew_rows_kernel<T, VEC, false, false, F, B, U><<<grid, B, 0, stream>>>(out, a, b, rp, f);
             return ZENU_OK;
         };
         int rc = small ? launch(std::integral_constant<int, ZENU_EW1_BLOCK>(), std::integral_constant<int, ZENU_EW1_UNROLL>())
@@ -1027,15 +1070,17 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
     const int64_t cols_per_tile = ((int64_t)1 << shift) * kStridedUnroll;
     sp.col_tiles = (sp.ncols + cols_per_tile - 1) / cols_per_tile;
     const int64_t rows_per_blk = kBlock >> shift;
-    const int64_t grid = ((sp.nrows + rows_per_blk - 1) / rows_per_blk) * sp.col_tiles;
-    if (grid > 0x7fffffffLL || sp.col_tiles > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
+    const int64_t row_blks = (sp.nrows + rows_per_blk - 1) / rows_per_blk;
+    if (row_blks * sp.col_tiles > 0x7fffffffLL || sp.col_tiles > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
+    sp.grid2d = row_blks <= 65535 ? 1 : 0;
+    const dim3 grid = sp.grid2d ? dim3((unsigned)sp.col_tiles, (unsigned)row_blks) : dim3((unsigned)(row_blks * sp.col_tiles));
     // streaming hint only when every cache line an access touches is used up by the same wavefront
     // (small inner strides); with large strides the neighbours of an element belong to other rows
     bool snt = nt;
     for (int o = 0; o <= nin; o++)
         if (sp.inner[o] > 4) snt = false;
-    if (snt) ew_strided_rows_kernel<T, F, kStridedUnroll, true><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, sp, f);
-    else     ew_strided_rows_kernel<T, F, kStridedUnroll, false><<<(unsigned)grid, kBlock, 0, stream>>>(out, a, b, sp, f);
+    if (snt) ew_strided_rows_kernel<T, F, kStridedUnroll, true><<<grid, kBlock, 0, stream>>>(out, a, b, sp, f);
+    else     ew_strided_rows_kernel<T, F, kStridedUnroll, false><<<grid, kBlock, 0, stream>>>(out, a, b, sp, f);
     ZENU_LAUNCH_CHECK();
     return ZENU_OK;
 }
