@@ -445,8 +445,8 @@ __global__ __launch_bounds__(kBlock) void ew_rows_kernel(T *out, const T *a, con
     int tx_shift = p.tx_shift, inner_a = p.inner_a, inner_b = p.inner_b, nouter = p.outer.nouter, grid2d = p.grid2d;
     int64_t nrows = p.nrows, ncols = p.ncols;
     int64_t so0 = p.outer.stride[0][0], sa0 = p.outer.stride[1][0], sb0 = p.outer.stride[2][0];
-    asm volatile("" : "+s"(tx_shift), "+s"(inner_a), "+s"(inner_b), "+s"(nouter), "+s"(grid2d), "+s"(nrows),
-                      "+s"(ncols), "+s"(so0), "+s"(sa0), "+s"(sb0), "+s"(out), "+s"(a), "+s"(b));
+    asm volatile("" : : "s"(tx_shift), "s"(inner_a), "s"(inner_b), "s"(nouter), "s"(grid2d), "s"(nrows),
+                      "s"(ncols), "s"(so0), "s"(sa0), "s"(sb0), "s"(out), "s"(a), "s"(b));
     const int tx_n = 1 << tx_shift;
     const int ty_n = kBlock >> tx_shift;
     const int tx = threadIdx.x & (tx_n - 1);
@@ -527,10 +527,11 @@ __global__ __launch_bounds__(kBlock) void ew_rows_kernel(T *out, const T *a, con
 // four vectors each; 32x32 tiles with 256 threads copy as fast (24.1 us) but leave operands that
 // are not transposed with 128-byte row pieces.
 template <typename T> struct TileOf { static constexpr int N = sizeof(T) == 4 ? 64 : 32; };
-// With two inputs (three streams, a + b^T) four vectors per thread and operand at 256 threads keep
-// more bytes in flight per compute unit and win: 39.5 us against 41.1 us.
+// With two inputs (three streams, a + b^T) two vectors per thread and operand at 512 threads are the
+// fastest (stand-alone probe: 36.2 us with four at 256 threads, 35.5 us with two at 512, 35.7 us with
+// one at 1024).
 template <typename T, typename F> struct TileThreads {
-    static constexpr int value = F::NIN == 1 ? TileOf<T>::N * TileOf<T>::N / VecOf<T>::N : 256;
+    static constexpr int value = F::NIN == 1 ? TileOf<T>::N * TileOf<T>::N / VecOf<T>::N : 512;
 };
 
 enum { kWalkRows = 0, kWalkCols = 1, kWalkDiagonal = 2 };
@@ -565,8 +566,11 @@ __global__ __launch_bounds__((TileThreads<T, F>::value)) void ew_tile_kernel(T *
     constexpr int VPS = 8;                  // vectors per segment
     constexpr int SEG = kTile / (VPS * VEC);// segments per tile row (2)
     static_assert(SEG >= 1 && (kTile * SEG * VPS) % kBlock == 0, "tile geometry");
-    __shared__ T lds_a[kTile * kPitch];
-    __shared__ T lds_b[(F::NIN == 2) ? kTile * kPitch : 1];
+    // One staging tile per TRANSPOSED input, sized at launch: with a static tile per input, `a + b^T`
+    // held 33 KB of LDS per workgroup for the one tile it uses, and four workgroups fit a CU instead
+    // of eight (38.9 us against 36.2 us on [4096,4096] f32).
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    T *const lds_a = reinterpret_cast<T *>(lds_raw);
     f.init();
 
     // The order in which the tiles are walked decides which addresses the workgroups that run
@@ -589,9 +593,10 @@ __global__ __launch_bounds__((TileThreads<T, F>::value)) void ew_tile_kernel(T *
     int64_t R = p.R, C = p.C;
     int64_t ldr0 = p.ldr[0], ldr1 = p.ldr[1], ldr2 = p.ldr[2], ldc1 = p.ldc[1], ldc2 = p.ldc[2];
     int trans_a = p.trans_a, trans_b = p.trans_b;
-    asm volatile("" : "+s"(grid3d), "+s"(vec_ok), "+s"(nouter), "+s"(walk), "+s"(ntr), "+s"(magic), "+s"(R), "+s"(C),
-                      "+s"(ldr0), "+s"(ldr1), "+s"(ldr2), "+s"(ldc1), "+s"(ldc2), "+s"(trans_a), "+s"(trans_b),
-                      "+s"(out), "+s"(a), "+s"(b));
+    asm volatile("" : : "s"(grid3d), "s"(vec_ok), "s"(nouter), "s"(walk), "s"(ntr), "s"(magic), "s"(R), "s"(C),
+                      "s"(ldr0), "s"(ldr1), "s"(ldr2), "s"(ldc1), "s"(ldc2), "s"(trans_a), "s"(trans_b),
+                      "s"(out), "s"(a), "s"(b));
+    T *const lds_b = lds_a + ((F::NIN == 2 && trans_a) ? kTile * kPitch : 0);
     uint32_t tc32, tr32, batch32;
     if (grid3d) {
         const bool by_cols = walk == kWalkCols;       // then the grid is (row tiles, column tiles, batch)
@@ -639,54 +644,68 @@ __global__ __launch_bounds__((TileThreads<T, F>::value)) void ew_tile_kernel(T *
         auto vec_of = [&](int k) { return seg_v + (((k * kBlock + tid) / VPS) / kTile) * VPS * VEC; };  // element position along the vector dim
         const bool ta = trans_a != 0;
         const bool tb = (F::NIN == 2) && trans_b != 0;
+        // A transposed input is read along R with its pitch ldc between the vectors, any other along C
+        // with its pitch ldr: the same expression with the pitch selected, so the loads of one thread
+        // follow each other without a branch between them.  (With a branch per load the compiler put a
+        // wait for all earlier loads in front of each one: `a + b^T` 38.9 us instead of 36 us.)
+        const int64_t pitch_a = ta ? ldc1 : ldr1;
+        const int64_t pitch_b = tb ? ldc2 : ldr2;
         Pack<T, VEC> xa[K], xb[K];
 #pragma unroll
         for (int k = 0; k < K; k++) {
             const int o = other_of(k);
             const int lane_v = vec_of(k);
-            if (ta) xa[k] = load_pack<T, VEC, NT>(abase + lane_v + (int64_t)o * ldc1);
-            else if (ldc1 == 0) xa[k] = splat<T, VEC>(abase[(int64_t)o * ldr1]);
-            else xa[k] = load_pack<T, VEC, NT>(abase + (int64_t)o * ldr1 + lane_v);
-            if constexpr (F::NIN == 2) {
-                if (tb) xb[k] = load_pack<T, VEC, NT>(bbase + lane_v + (int64_t)o * ldc2);
-                else if (ldc2 == 0) xb[k] = splat<T, VEC>(bbase[(int64_t)o * ldr2]);
-                else xb[k] = load_pack<T, VEC, NT>(bbase + (int64_t)o * ldr2 + lane_v);
-            }
+            xa[k] = load_pack<T, VEC, NT>(abase + lane_v + (int64_t)o * pitch_a);
+            if constexpr (F::NIN == 2) xb[k] = load_pack<T, VEC, NT>(bbase + lane_v + (int64_t)o * pitch_b);
         }
-        if (ta || tb) {
+        if (ta) {
 #pragma unroll
             for (int k = 0; k < K; k++) {
                 const int c = other_of(k);               // the loaded vector holds rows lane_v.. of column c
                 const int lane_v = vec_of(k);
 #pragma unroll
-                for (int j = 0; j < VEC; j++) {
-                    if (ta) lds_a[(lane_v + j) * kPitch + c] = xa[k].v[j];
-                    if constexpr (F::NIN == 2) {
-                        if (tb) lds_b[(lane_v + j) * kPitch + c] = xb[k].v[j];
-                    }
+                for (int j = 0; j < VEC; j++) lds_a[(lane_v + j) * kPitch + c] = xa[k].v[j];
+            }
+        }
+        if constexpr (F::NIN == 2) {
+            if (tb) {
+#pragma unroll
+                for (int k = 0; k < K; k++) {
+                    const int c = other_of(k);
+                    const int lane_v = vec_of(k);
+#pragma unroll
+                    for (int j = 0; j < VEC; j++) lds_b[(lane_v + j) * kPitch + c] = xb[k].v[j];
                 }
             }
-            __syncthreads();
+        }
+        __syncthreads();                                 // at least one input is transposed
+        if (ta) {
+#pragma unroll
+            for (int k = 0; k < K; k++) {
+                const int r = other_of(k);
+                const int lane_v = vec_of(k);
+#pragma unroll
+                for (int j = 0; j < VEC; j++) xa[k].v[j] = lds_a[r * kPitch + lane_v + j];
+            }
+        }
+        if constexpr (F::NIN == 2) {
+            if (tb) {
+#pragma unroll
+                for (int k = 0; k < K; k++) {
+                    const int r = other_of(k);
+                    const int lane_v = vec_of(k);
+#pragma unroll
+                    for (int j = 0; j < VEC; j++) xb[k].v[j] = lds_b[r * kPitch + lane_v + j];
+                }
+            }
         }
 #pragma unroll
         for (int k = 0; k < K; k++) {
             const int r = other_of(k);
             const int lane_v = vec_of(k);
-            Pack<T, VEC> x = xa[k], y;
-            if (ta) {
-#pragma unroll
-                for (int j = 0; j < VEC; j++) x.v[j] = lds_a[r * kPitch + lane_v + j];
-            }
-            if constexpr (F::NIN == 2) {
-                y = xb[k];
-                if (tb) {
-#pragma unroll
-                    for (int j = 0; j < VEC; j++) y.v[j] = lds_b[r * kPitch + lane_v + j];
-                }
-            } else {
-                y = x;
-            }
-            store_pack<T, VEC, NT>(obase + (int64_t)r * ldr0 + lane_v, apply_pack<T, VEC, F>(f, x, y));
+            Pack<T, VEC> y = xa[k];
+            if constexpr (F::NIN == 2) y = xb[k];
+            store_pack<T, VEC, NT>(obase + (int64_t)r * ldr0 + lane_v, apply_pack<T, VEC, F>(f, xa[k], y));
         }
     } else {
         // edge tiles and unaligned operands: element-wise with bounds checks
@@ -742,8 +761,8 @@ __global__ __launch_bounds__(kBlock) void ew_strided_rows_kernel(T *out, const T
     int64_t nrows = p.nrows, ncols = p.ncols;
     int64_t so0 = p.outer.stride[0][0], sa0 = p.outer.stride[1][0], sb0 = p.outer.stride[2][0];
     int64_t so = p.inner[0], sa = p.inner[1], sb = p.inner[2];
-    asm volatile("" : "+s"(tx_shift), "+s"(nouter), "+s"(grid2d), "+s"(nrows), "+s"(ncols), "+s"(so0), "+s"(sa0),
-                      "+s"(sb0), "+s"(so), "+s"(sa), "+s"(sb), "+s"(out), "+s"(a), "+s"(b));
+    asm volatile("" : : "s"(tx_shift), "s"(nouter), "s"(grid2d), "s"(nrows), "s"(ncols), "s"(so0), "s"(sa0),
+                      "s"(sb0), "s"(so), "s"(sa), "s"(sb), "s"(out), "s"(a), "s"(b));
     const int tx_n = 1 << tx_shift;
     const int ty_n = kBlock >> tx_shift;
     const int tx = threadIdx.x & (tx_n - 1);
@@ -774,11 +793,13 @@ __global__ __launch_bounds__(kBlock) void ew_strided_rows_kernel(T *out, const T
     T x[kUnroll], y[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {          // all loads of the thread first
+        // A column past the end reads the last one again (and stores nothing): with the loads under
+        // the bounds check the compiler waits for the first before it issues the others.
         const int64_t c = c0 + (int64_t)u * tx_n;
-        if (c < ncols) {
-            x[u] = load_pack<T, 1, NT>(arow + c * sa).v[0];
-            y[u] = (F::NIN == 2) ? load_pack<T, 1, NT>(brow + c * sb).v[0] : x[u];
-        }
+        const int64_t cl = c < ncols ? c : ncols - 1;
+        x[u] = load_pack<T, 1, NT>(arow + cl * sa).v[0];
+        if constexpr (F::NIN == 2) y[u] = load_pack<T, 1, NT>(brow + cl * sb).v[0];
+        else y[u] = x[u];
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
@@ -1017,6 +1038,10 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
                     if (s % VEC) vec = false;
                 }
             }
+            // the vector path reads whole vectors along C from the inputs that are not transposed: one
+            // that is broadcast along C (a column beside a transposed operand) takes the element path
+            for (int o = 1; o <= nin; o++)
+                if (!trans[o] && tp.ldc[o] == 0) vec = false;
             tp.vec_ok = vec ? 1 : 0;
             constexpr int kTile = TileOf<T>::N;
             tp.tiles_r = (tp.R + kTile - 1) / kTile;
@@ -1045,8 +1070,9 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
             const dim3 g = !tp.grid3d ? dim3((unsigned)grid)
                            : by_cols ? dim3((unsigned)tp.tiles_r, (unsigned)tp.tiles_c, (unsigned)tp.nbatch)
                                      : dim3((unsigned)tp.tiles_c, (unsigned)tp.tiles_r, (unsigned)tp.nbatch);
-            if (nt) ew_tile_kernel<T, true, F><<<g, TileThreads<T, F>::value, 0, stream>>>(out, a, b, tp, f);
-            else    ew_tile_kernel<T, false, F><<<g, TileThreads<T, F>::value, 0, stream>>>(out, a, b, tp, f);
+            const size_t lds = (size_t)(tp.trans_a + tp.trans_b) * kTile * (kTile + 1) * sizeof(T);
+            if (nt) ew_tile_kernel<T, true, F><<<g, TileThreads<T, F>::value, lds, stream>>>(out, a, b, tp, f);
+            else    ew_tile_kernel<T, false, F><<<g, TileThreads<T, F>::value, lds, stream>>>(out, a, b, tp, f);
             ZENU_LAUNCH_CHECK();
             return ZENU_OK;
         }

@@ -266,13 +266,22 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_rows_kernel(const T *y, co
     constexpr int64_t step = (int64_t)kBlock * VEC;
     T sum = (T)0;
     if (REG) {   // the row of y and of t = y * gy stays in registers: two reads, one write
-        Pack<T, VEC> yv[kRegPacks], t[kRegPacks];
+        Pack<T, VEC> yv[kRegPacks], gv[kRegPacks], t[kRegPacks];
+        // all loads of the thread first (a pack past the end of the row reads the row's first one and
+        // is not used): with the loads inside the bounds check the compiler waits for each pair
+        // before it issues the next, because the running sum orders the blocks
+#pragma unroll
+        for (int k = 0; k < kRegPacks; k++) {
+            const int64_t r = first + k * step;
+            const int64_t rl = r < R ? r : 0;
+            yv[k] = load_pack<T, VEC, NT && !CE>(yr + rl);
+            gv[k] = load_pack<T, VEC, NT>(sr + rl);
+        }
 #pragma unroll
         for (int k = 0; k < kRegPacks; k++) {
             const int64_t r = first + k * step;
             if (r < R) {
-                yv[k] = load_pack<T, VEC, NT && !CE>(yr + r);
-                const Pack<T, VEC> g = load_pack<T, VEC, NT>(sr + r);
+                const Pack<T, VEC> g = gv[k];
 #pragma unroll
                 for (int j = 0; j < VEC; j++) {
                     const T gyv = CE ? (g.v[j] * g_total) / yv[k].v[j] : g.v[j];
