@@ -827,6 +827,29 @@ def test_copy_transpose_large(hip):
 
 
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_transposed_operand_beside_a_broadcast_one(hip, dt):
+    # whole tiles (both extents are multiples of the tile): a transposed input together with a
+    # column [R,1] (broadcast along the rows' direction of the output: the element path), with a
+    # row [1,C] and with a second transposed input (the vector path)
+    r = rng(32)
+    rows, cols = 256, 192
+    a = r.standard_normal((cols, rows)).astype(dt)
+    b = r.standard_normal((cols, rows)).astype(dt)
+    col = r.standard_normal((rows, 1)).astype(dt)
+    row = r.standard_normal((1, cols)).astype(dt)
+    A, B = hip.Matrix.from_numpy(a), hip.Matrix.from_numpy(b)
+    COL, ROW = hip.Matrix.from_numpy(col), hip.Matrix.from_numpy(row)
+    out = hip.Matrix.zeros((rows, cols), dt)
+    exp = np.empty((rows, cols), dtype=dt)
+    for name, X, Y, x, y in (("a^T + col", A.transpose(), COL, a.T, col), ("col - a^T", COL, A.transpose(), col, a.T),
+                             ("a^T + row", A.transpose(), ROW, a.T, row), ("a^T * b^T", A.transpose(), B.transpose(), a.T, b.T)):
+        op = zo.SUB if "-" in name else zo.MUL if "*" in name else zo.ADD
+        zo.binary_array(op, exp, x, y)
+        (out.sub_array if op == zo.SUB else out.mul_array if op == zo.MUL else out.add_array)(X, Y)
+        assert_bits(out.to_numpy(), exp, name)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
 @pytest.mark.parametrize("pitch_out,pitch_in", [(1024, 1024), (1024, 1100), (1100, 1024), (1100, 1100),
                                                 (1028, 2048), (2048, 1028)])
 def test_transposed_views_every_tile_walk(hip, dt, pitch_out, pitch_in):
