@@ -15,6 +15,7 @@
 //
 // Geometry: operands are row-major [outer, R, inner] with the softmax axis R in the middle;
 // views that are not in default stride are staged through a contiguous temporary.
+#include <type_traits>
 #include <math.h>
 
 #include "common.hpp"
@@ -124,6 +125,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
         m = block_red<T, true, kBlock>(m, lds);
         if (x0 != x0) m = x0;   // a NaN in position 0 is never replaced
         T sum = (T)0;
+        T least = INFINITY;     // the smallest of this thread's terms
 #pragma unroll
         for (int k = 0; k < kRegPacks; k++) {
             if (first + k * step < R) {
@@ -131,25 +133,51 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
                 for (int j = 0; j < VEC; j++) {
                     v[k].v[j] = ml.exp_flat(v[k].v[j] - m);
                     sum = sum + v[k].v[j];
+                    least = v[k].v[j] < least ? v[k].v[j] : least;
                 }
             }
         }
         sum = block_red<T, false, kBlock>(sum, lds);
-#pragma unroll
-        for (int k = 0; k < kRegPacks; k++) {
-            const int64_t r = first + k * step;
-            if (r < R) {
-                Pack<T, VEC> t;
-                if (CE) t = load_pack<T, VEC, NT>(tr + r);
-#pragma unroll
-                for (int j = 0; j < VEC; j++) {
-                    const T s = v[k].v[j] / sum;
-                    v[k].v[j] = s;
-                    if (CE) acc = acc + t.v[j] * ml.log(s);
-                }
-                store_pack<T, VEC, NT && !CE>(yr + r, v[k]);   // the CE output is read again by the backward pass
-            }
+        // Every quotient of the row has the same divisor.  With r = RN(1 / sum): q0 = RN(a r), the
+        // exact remainder a - sum q0 (one fma) and q = fma(remainder, r, q0) is the correctly rounded
+        // a / sum (Markstein) unless the divisor's mantissa is all ones, as long as nothing underflows:
+        // three instructions per element instead of the division's eleven.  The thread takes that road
+        // when its terms are at least 2^-64 and the sum lies in [1, 2^23) (quotient and remainder stay
+        // normal); otherwise it divides.  On 9.6e9 random pairs from those ranges (terms down to 2^-80)
+        // the host finds no quotient that differs from the division's.
+        bool shared_divisor = false;
+        if constexpr (sizeof(T) == 4) {
+            uint32_t sb;
+            __builtin_memcpy(&sb, &sum, 4);
+            shared_divisor = least >= (T)0x1p-64f && sum >= (T)1 && sum < (T)0x1p23f && (sb & 0x7fffffu) != 0x7fffffu;
         }
+        auto finish = [&](auto by_reciprocal) {
+            const T rcp = decltype(by_reciprocal)::value ? (T)1 / sum : (T)0;
+#pragma unroll
+            for (int k = 0; k < kRegPacks; k++) {
+                const int64_t r = first + k * step;
+                if (r < R) {
+                    Pack<T, VEC> t;
+                    if (CE) t = load_pack<T, VEC, NT>(tr + r);
+#pragma unroll
+                    for (int j = 0; j < VEC; j++) {
+                        T s;
+                        if constexpr (decltype(by_reciprocal)::value && sizeof(T) == 4) {
+                            const float a = v[k].v[j];
+                            const float q0 = a * rcp;
+                            s = __builtin_fmaf(__builtin_fmaf(-sum, q0, a), rcp, q0);
+                        } else {
+                            s = v[k].v[j] / sum;
+                        }
+                        v[k].v[j] = s;
+                        if (CE) acc = acc + t.v[j] * ml.log(s);
+                    }
+                    store_pack<T, VEC, NT && !CE>(yr + r, v[k]);   // the CE output is read again by the backward pass
+                }
+            }
+        };
+        if (shared_divisor) finish(std::true_type());
+        else finish(std::false_type());
     } else {     // long rows: three passes; the second and third find the row in cache
         T m = -INFINITY;
         for (int64_t r = first; r < R; r += step) {
