@@ -874,6 +874,15 @@ def test_transposed_views_every_tile_walk(hip, dt, pitch_out, pitch_in):
         exp = np.empty((rows, cols), dtype=dt)
         zo.binary_array(zo.ADD, exp, av, bt)
         assert_bits(out.to_numpy()[:, :cols], exp, f"a + b^T {rows}x{cols} pitches {pitch_out}/{pitch_in}")
+    # the same walks with a batch dim in front (a 3-d grid): out[n] = b[n]^T
+    rows, cols = 130, 70
+    b3 = r.standard_normal((3, cols, pitch_in)).astype(dt)
+    B3 = hip.Matrix.from_numpy(b3).slice(slice(None), slice(None), slice(0, rows)).transpose_by_index((0, 2, 1))
+    out3 = hip.Matrix.zeros((3, rows, pitch_out), dt)
+    out3.slice(slice(None), slice(None), slice(0, cols)).copy_from(B3)
+    got3 = out3.to_numpy()
+    assert_bits(got3[:, :, :cols], np.ascontiguousarray(b3[:, :, :rows].transpose(0, 2, 1)), f"batched copy b^T pitches {pitch_out}/{pitch_in}")
+    assert not got3[:, :, cols:].any(), "wrote outside the batched view"
 
 
 # ---- config[2]: [8192,4096] reductions, normal(0,1), seed 2, ~1% duplicate maxima ---------------------------
