@@ -336,7 +336,7 @@ int zenu_hip_adam_step_multi(int dtype, int n_tensors, void *const *p_dev, const
 /* They let the unchanged zenu-cuda/src/kernel/mod.rs wrappers link.            */
 /* ------------------------------------------------------------------------- */
 
-/* The reference's functions return void (kernel/*.h) and so do these; what the descriptor entry
+/* The reference's functions return void (the headers under kernel/) and so do these; what the descriptor entry
  * point behind one of them returned is kept per thread instead.  zenu_hip_last_status() returns
  * the first status other than ZENU_OK that any of them produced on this thread since the last
  * call, and clears it: a wrapper can poll it after a batch of calls (no counterpart in the
