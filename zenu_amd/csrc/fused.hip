@@ -121,6 +121,16 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
 #pragma unroll
             for (int j = 0; j < VEC; j++) m = combine<T, true>(m, v[k].v[j]);
         }
+        // the targets of the cross-entropy terms travel with the row: loaded where they are used, each
+        // pack cost the end of the kernel a round trip of its own
+        Pack<T, VEC> tg[kRegPacks];
+        if (CE) {
+#pragma unroll
+            for (int k = 0; k < kRegPacks; k++) {
+                const int64_t r = first + k * step;
+                tg[k] = load_pack<T, VEC, NT>(tr + (r < R ? r : 0));
+            }
+        }
         ml.init(true, CE);      // after the row's loads are issued: the table fetch overlaps them
         m = block_red<T, true, kBlock>(m, lds);
         if (x0 != x0) m = x0;   // a NaN in position 0 is never replaced
@@ -157,8 +167,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
             for (int k = 0; k < kRegPacks; k++) {
                 const int64_t r = first + k * step;
                 if (r < R) {
-                    Pack<T, VEC> t;
-                    if (CE) t = load_pack<T, VEC, NT>(tr + r);
+                    const Pack<T, VEC> t = tg[k];
 #pragma unroll
                     for (int j = 0; j < VEC; j++) {
                         T s;
