@@ -826,6 +826,22 @@ def test_copy_transpose_large(hip):
     assert_bits(dst.to_numpy(), np.ascontiguousarray(a.T), "copy into transposed")
 
 
+@pytest.mark.parametrize("shape", [(70, 1024), (1024, 70), (64, 4096), (33, 2048)])
+def test_transposed_copy_wide_and_tall(hip, shape):
+    # many more tile columns than tile rows and the reverse, with pitches that are multiples of
+    # 4 KiB: the diagonal walk wraps around the tile rows several times
+    r = rng(33)
+    a = r.standard_normal(shape).astype(np.float32)
+    A = hip.Matrix.from_numpy(a)
+    assert_bits(A.transpose().to_default_stride().to_numpy(), np.ascontiguousarray(a.T), f"transpose copy {shape}")
+    b = r.standard_normal(shape[::-1]).astype(np.float32)
+    out = hip.Matrix.zeros(shape[::-1])
+    out.add_array(hip.Matrix.from_numpy(b), A.transpose())
+    exp = np.empty(shape[::-1], dtype=np.float32)
+    zo.binary_array(zo.ADD, exp, b, a.T)
+    assert_bits(out.to_numpy(), exp, f"b + a^T {shape}")
+
+
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
 def test_transposed_operand_beside_a_broadcast_one(hip, dt):
     # whole tiles (both extents are multiples of the tile): a transposed input together with a
