@@ -568,7 +568,7 @@ __global__ __launch_bounds__((TileThreads<T, F>::value)) void ew_tile_kernel(T *
     static_assert(SEG >= 1 && (kTile * SEG * VPS) % kBlock == 0, "tile geometry");
     // One staging tile per TRANSPOSED input, sized at launch: with a static tile per input, `a + b^T`
     // held 33 KB of LDS per workgroup for the one tile it uses, and four workgroups fit a CU instead
-    // of eight (38.9 us against 36.2 us on [4096,4096] f32).
+    // of eight (on a [4096,4096] f32 view of pitch 4160: 37.6 us against 36.0 us).
     extern __shared__ __align__(16) unsigned char lds_raw[];
     T *const lds_a = reinterpret_cast<T *>(lds_raw);
     f.init();
