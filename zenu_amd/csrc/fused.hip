@@ -55,6 +55,8 @@ template <typename T, bool MAX, int BLOCK = kBlock> __device__ __forceinline__ T
 // ---- forward ---------------------------------------------------------------------------------------------
 // CE: additionally rowloss[line] = sum_r target * log(softmax)   (inner == 1 only)
 
+constexpr int kLineRegs = 16;   // lines up to this length are kept in registers by the lines kernel
+
 template <typename T, bool CE>
 __global__ __launch_bounds__(kBlock) void softmax_lines_kernel(const T *x, T *y, int64_t lines, int64_t R,
                                                                 int64_t inner, const T *target, T *rowloss)
@@ -71,6 +73,41 @@ __global__ __launch_bounds__(kBlock) void softmax_lines_kernel(const T *x, T *y,
     const int64_t base = q * R * inner + c;
     const T *xl = x + base;
     T *yl = y + base;
+    if (R <= kLineRegs) {
+        // a short line (the classes of a classifier head) stays in registers: its loads, and those of
+        // the targets, are issued together instead of one per loop iteration, and nothing is read
+        // back.  The operations and their order are those of the loops below.
+        T v[kLineRegs], tg[kLineRegs];
+#pragma unroll
+        for (int r = 0; r < kLineRegs; r++) {
+            const int64_t rl = r < R ? r : 0;
+            v[r] = xl[rl * inner];
+            if (CE) tg[r] = target[base + rl * inner];
+        }
+        T m = v[0];
+#pragma unroll
+        for (int r = 1; r < kLineRegs; r++)
+            if (r < R && v[r] > m) m = v[r];
+        T sum = (T)0;
+#pragma unroll
+        for (int r = 0; r < kLineRegs; r++) {
+            if (r < R) {
+                v[r] = ml.exp(v[r] - m);
+                sum = sum + v[r];
+            }
+        }
+        T acc = (T)0;
+#pragma unroll
+        for (int r = 0; r < kLineRegs; r++) {
+            if (r < R) {
+                const T s = v[r] / sum;
+                yl[r * inner] = s;
+                if (CE) acc = acc + tg[r] * ml.log(s);
+            }
+        }
+        if (CE) rowloss[line] = acc;
+        return;
+    }
     // max_axis: strict '>' from element 0 (max.rs:19-34)
     T m = xl[0];
     for (int64_t r = 1; r < R; r++) {
@@ -275,6 +312,27 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_lines_kernel(const T *y, c
         c = line - q * inner;
     }
     const int64_t base = q * R * inner + c;
+    if (R <= kLineRegs) {     // a short line in registers, as in the forward kernel: same operations, same order
+        T yv[kLineRegs], pv[kLineRegs], t[kLineRegs];
+#pragma unroll
+        for (int r = 0; r < kLineRegs; r++) {
+            const int64_t off = base + (r < R ? r : 0) * inner;
+            yv[r] = y[off];
+            pv[r] = gy_or_target[off];
+        }
+        T sum = (T)0;
+#pragma unroll
+        for (int r = 0; r < kLineRegs; r++) {
+            if (r < R) {
+                t[r] = yv[r] * (CE ? (pv[r] * src.g_total) / yv[r] : pv[r]);
+                sum = sum + t[r];
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < kLineRegs; r++)
+            if (r < R) gx[base + r * inner] = t[r] - yv[r] * sum;
+        return;
+    }
     T sum = (T)0;
     for (int64_t r = 0; r < R; r++) {
         const int64_t off = base + r * inner;
