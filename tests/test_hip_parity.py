@@ -842,6 +842,19 @@ def test_transposed_copy_wide_and_tall(hip, shape):
     assert_bits(out.to_numpy(), exp, f"b + a^T {shape}")
 
 
+def test_transposed_copy_of_many_small_matrices(hip):
+    # more batches than a grid's y / z extent holds: the tile kernel's linear grid, decomposed in the kernel
+    r = rng(34)
+    a = r.standard_normal((70000, 5, 3)).astype(np.float32)
+    A = hip.Matrix.from_numpy(a)
+    got = A.transpose_by_index((0, 2, 1)).to_default_stride().to_numpy()
+    assert_bits(got, np.ascontiguousarray(a.transpose(0, 2, 1)), "70000 transposed 5x3 matrices")
+    b = r.standard_normal((70000, 3, 5)).astype(np.float32)
+    out = hip.Matrix.zeros((70000, 3, 5))
+    out.add_array(hip.Matrix.from_numpy(b), A.transpose_by_index((0, 2, 1)))
+    assert_bits(out.to_numpy(), b + a.transpose(0, 2, 1), "b + a^T, 70000 batches")
+
+
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
 def test_transposed_operand_beside_a_broadcast_one(hip, dt):
     # whole tiles (both extents are multiples of the tile): a transposed input together with a
