@@ -855,6 +855,28 @@ def test_transposed_copy_of_many_small_matrices(hip):
     assert_bits(out.to_numpy(), b + a.transpose(0, 2, 1), "b + a^T, 70000 batches")
 
 
+def test_sliced_views_with_more_row_blocks_than_a_grid_dim(hip):
+    # the rows kernel and the strided-rows kernel take a 2-d grid (column tiles, row blocks) up to
+    # 65535 row blocks and a linear one beyond: both sides of that limit
+    r = rng(35)
+    for nrows in (600000, 4000):
+        w = r.standard_normal((nrows, 256)).astype(np.float32)          # 4 rows per workgroup: 75000 row blocks
+        W = hip.Matrix.from_numpy(w)
+        rows = W.slice(slice(None, None, 2), slice(None))             # every other row: rows kernel
+        assert_bits(rows.to_default_stride().to_numpy(), np.ascontiguousarray(w[::2]), f"row-sliced copy, {nrows} rows")
+        del W, rows, w
+        a = r.standard_normal((nrows, 64)).astype(np.float32)           # 8 rows per workgroup: 75000 row blocks
+        A = hip.Matrix.from_numpy(a)
+        cols = A.slice(slice(None), slice(None, None, 2))             # every other column: strided rows
+        assert_bits(cols.to_default_stride().to_numpy(), np.ascontiguousarray(a[:, ::2]), f"column-sliced copy, {nrows} rows")
+        out = hip.Matrix.zeros((nrows, 64))
+        out.slice(slice(None), slice(None, None, 2)).copy_from(cols)    # strided destination
+        exp = np.zeros_like(a)
+        exp[:, ::2] = a[:, ::2]
+        assert_bits(out.to_numpy(), exp, f"strided destination, {nrows} rows")
+        del A, cols, out
+
+
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
 def test_transposed_operand_beside_a_broadcast_one(hip, dt):
     # whole tiles (both extents are multiples of the tile): a transposed input together with a
