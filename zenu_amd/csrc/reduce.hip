@@ -714,6 +714,118 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, uin
     if (threadIdx.x == 0) store_agent(p.counters + group * p.cstride, 0);
 }
 
+// ---- kernel B, regular geometry ----------------------------------------------------------------------------
+// Kernel B for the shape it mostly runs on -- vector columns, every column tile full (inner a
+// multiple of 32 vectors), the reduced axis split over workgroups, a 3-d grid, a flat arrival
+// counter -- with everything that cannot happen there taken out of the instruction stream: no
+// per-column predicates, one 128-bit LDS exchange per thread instead of one per column, partials
+// stored and loaded as whole vectors' worth of device-scope words without a branch each.  The
+// accumulation order, the order of the LDS combine and the order of the fold are kernel B's, so
+// both give the same bits.
+template <typename T, typename Tr, int VEC, bool NT>
+__global__ __launch_bounds__(kBlock) void reduce_cols_regular_kernel(RedParams<T> p)
+{
+    typedef typename Tr::Acc A;
+    struct Cols {
+        A a[VEC];
+    };
+    __shared__ Cols lds[kBlock];
+    constexpr int TX = 32, TY = kBlock / TX, U = 4;
+    const int tx = threadIdx.x & (TX - 1), ty = threadIdx.x / TX;
+    const int split = (int)blockIdx.y, splits = p.splits;
+    const int64_t q = blockIdx.z;
+    const int64_t c = ((int64_t)blockIdx.x * TX + tx) * VEC;
+    const T *src = p.in + q * p.outer_stride + c;
+    const int64_t R = p.R, es = p.elem_stride;
+
+    // afterwards the row lane ty == 0 holds the result of the TY lanes, merged in lane order
+    auto combine_rows = [&](Cols &acc) {
+        __syncthreads();
+        lds[threadIdx.x] = acc;
+        __syncthreads();
+        if (ty == 0) {
+#pragma unroll
+            for (int w = 1; w < TY; w++) {
+                const Cols o = lds[w * TX + tx];
+#pragma unroll
+                for (int j = 0; j < VEC; j++) acc.a[j] = Tr::merge(acc.a[j], o.a[j]);
+            }
+        }
+    };
+
+    Cols acc;
+#pragma unroll
+    for (int j = 0; j < VEC; j++) acc.a[j] = Tr::identity();
+    constexpr int chunk = U * TY;
+    for (int64_t b = (int64_t)split * chunk; b < R; b += (int64_t)splits * chunk) {
+        const int64_t r = b + ty;
+        if (b + chunk <= R) {
+            Pack<T, VEC> x[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) x[u] = load_pack<T, VEC, NT>(src + (r + u * TY) * es);
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+#pragma unroll
+                for (int j = 0; j < VEC; j++) acc.a[j] = Tr::update(acc.a[j], x[u].v[j], r + u * TY);
+            }
+        } else {
+            for (int64_t rr = r; rr < R; rr += TY) {
+                const Pack<T, VEC> x = load_pack<T, VEC, false>(src + rr * es);
+#pragma unroll
+                for (int j = 0; j < VEC; j++) acc.a[j] = Tr::update(acc.a[j], x.v[j], rr);
+            }
+        }
+    }
+    if (split == 0 && ty == 0) {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) acc.a[j] = Tr::first(acc.a[j], src[j]);
+    }
+    combine_rows(acc);
+
+    const int64_t o0 = q * p.inner + c;
+    if (ty == 0) {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) emit_partial<T, Tr>(p, (int64_t)split * p.nout + o0 + j, acc.a[j]);
+    }
+    const int64_t group = q * gridDim.x + blockIdx.x;
+    if (!arrive_last(p.counters + group, split, splits, splits)) return;
+    // fold this column tile: row lane ty takes splits ty, ty + TY, ... two at a time, then the LDS order
+#pragma unroll
+    for (int j = 0; j < VEC; j++) acc.a[j] = Tr::identity();
+    for (int s0 = ty; s0 < splits; s0 += 2 * TY) {
+        A t[2][VEC];
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int sidx = s0 + u * TY;
+            if (sidx < splits) {
+#pragma unroll
+                for (int j = 0; j < VEC; j++) t[u][j] = load_partial<T, Tr>(p, (int64_t)sidx * p.nout + o0 + j);
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; j++) t[u][j] = Tr::identity();
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+#pragma unroll
+            for (int j = 0; j < VEC; j++) acc.a[j] = Tr::merge(acc.a[j], t[u][j]);
+        }
+    }
+    combine_rows(acc);
+    if (ty == 0) {
+        if constexpr (!Tr::kHasIdx) {
+            Pack<T, VEC> r;
+#pragma unroll
+            for (int j = 0; j < VEC; j++) r.v[j] = Tr::key(acc.a[j]);
+            store_pack<T, VEC, false>(p.out_val + o0, r);
+        } else {
+#pragma unroll
+            for (int j = 0; j < VEC; j++) emit_final<T, Tr>(p, o0 + j, acc.a[j]);
+        }
+    }
+    if (threadIdx.x == 0) store_agent(p.counters + group, 0);
+}
+
 // ---- host side ---------------------------------------------------------------------------------------------
 
 // the source is read once; when it is larger than the caches the loads carry the streaming hint
@@ -786,6 +898,15 @@ int launch_cols(const RedParams<T> &p, hipStream_t s)
     const int g3 = (p.splits <= 65535 && outer <= 65535) ? 1 : 0;
     const dim3 g = g3 ? dim3((unsigned)col_tiles, (unsigned)p.splits, (unsigned)outer) : dim3((unsigned)grid);
     const uint32_t ctl = (uint32_t)col_tiles;
+    // the regular geometry: full vector tiles of 32 x 8 threads, a split axis with a flat counter
+    const bool regular = vec && g3 && shift == 5 && p.inner % per_tile == 0 && p.splits > 1 && p.fan >= p.splits &&
+                         p.cstride == 1 && (Tr::kHasIdx || aligned16(p.out_val));
+    if (regular) {
+        if (nt) reduce_cols_regular_kernel<T, Tr, VEC, true><<<g, kBlock, 0, s>>>(p);
+        else    reduce_cols_regular_kernel<T, Tr, VEC, false><<<g, kBlock, 0, s>>>(p);
+        ZENU_LAUNCH_CHECK();
+        return ZENU_OK;
+    }
     if (nt)       reduce_cols_kernel<T, Tr, VEC, true><<<g, kBlock, 0, s>>>(p, ctl, shift, g3);
     else if (vec) reduce_cols_kernel<T, Tr, VEC, false><<<g, kBlock, 0, s>>>(p, ctl, shift, g3);
     else          reduce_cols_kernel<T, Tr, 1, false><<<g, kBlock, 0, s>>>(p, ctl, shift, g3);
