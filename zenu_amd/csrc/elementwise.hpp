@@ -290,7 +290,10 @@ __global__ __launch_bounds__(ContigShape<F>::kBlock) void ew_contig_kernel(T *ou
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             int64_t i = base + ((int64_t)u * kBlock + tid) * VEC;
-            store_pack<T, VEC, NT>(out + i, apply_pack<T, VEC, F>(f, va[u], vb[u]));
+            const Pack<T, VEC> r = apply_pack<T, VEC, F>(f, va[u], vb[u]);
+            // one streamed input, one streamed output: the written-through streaming store (vecmem.hpp)
+            if constexpr (NT && ContigShape<F>::kSmall && VEC > 1) store_pack_wt<T, VEC>(out + i, r);
+            else store_pack<T, VEC, NT>(out + i, r);
         }
     } else {
         f.init();
