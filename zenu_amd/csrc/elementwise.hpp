@@ -352,8 +352,9 @@ __global__ __launch_bounds__(kBlock) void ew_periodic_kernel(T *out, const T *x,
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             const uint32_t i0 = base + (uint32_t)(u * kBlock + threadIdx.x) * VEC;
-            store_pack<T, VEC, NT>(out + i0, Y_FIRST ? apply_pack<T, VEC, F>(f, yv[u], xv[u])
-                                                     : apply_pack<T, VEC, F>(f, xv[u], yv[u]));
+            const Pack<T, VEC> r = Y_FIRST ? apply_pack<T, VEC, F>(f, yv[u], xv[u]) : apply_pack<T, VEC, F>(f, xv[u], yv[u]);
+            if constexpr (NT && VEC > 1) store_pack_wt<T, VEC>(out + i0, r);   // at most one streamed input beside the output
+            else store_pack<T, VEC, NT>(out + i0, r);
         }
     } else {
         for (int u = 0; u < kUnroll; u++) {
@@ -496,7 +497,9 @@ __global__ __launch_bounds__(kBlock) void ew_rows_kernel(T *out, const T *a, con
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
             int64_t c = c0 + ((int64_t)u * tx_n + tx) * VEC;
-            store_pack<T, VEC, (NTA || NTB)>(orow + c, apply_pack<T, VEC, F>(f, va[u], vb[u]));
+            const Pack<T, VEC> r = apply_pack<T, VEC, F>(f, va[u], vb[u]);
+            if constexpr ((NTA != NTB || (F::NIN == 1 && NTA)) && VEC > 1) store_pack_wt<T, VEC>(orow + c, r);   // one streamed input
+            else store_pack<T, VEC, (NTA || NTB)>(orow + c, r);
         }
     } else {
         for (int u = 0; u < kUnroll; u++) {

@@ -218,7 +218,9 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const T *x, T *y, 
                         v[k].v[j] = s;
                         if (CE) acc = acc + t.v[j] * ml.log(s);
                     }
-                    store_pack<T, VEC, NT && !CE>(yr + r, v[k]);   // the CE output is read again by the backward pass
+                    // the CE output is read again by the backward pass; plain softmax is one stream in, one out
+                    if constexpr (NT && !CE && VEC > 1) store_pack_wt<T, VEC>(yr + r, v[k]);
+                    else store_pack<T, VEC, false>(yr + r, v[k]);
                 }
             }
         };
@@ -464,8 +466,13 @@ __global__ __launch_bounds__(kTileLanes) void bias_relu_tile_kernel(const T *z, 
         a.v[j] = v.v[j] + b.v[j];
         h.v[j] = a.v[j] > (T)0 ? a.v[j] : alpha * a.v[j];
     }
-    if (pre) store_pack<T, VEC, NT>(pre + off, a);
-    store_pack<T, VEC, NT>(act + off, h);
+    if constexpr (NT && VEC > 1) {
+        if (pre) store_pack_wt<T, VEC>(pre + off, a);
+        store_pack_wt<T, VEC>(act + off, h);
+    } else {
+        if (pre) store_pack<T, VEC, NT>(pre + off, a);
+        store_pack<T, VEC, NT>(act + off, h);
+    }
 }
 
 // ---- host side ------------------------------------------------------------------------------------------------
