@@ -15,8 +15,11 @@
  *   - every function returns ZENU_OK (0) or an error code; nothing aborts.  Where the
  *     reference panics (shape / rank / axis mismatch) the code is ZENU_ERR_SHAPE,
  *     ZENU_ERR_RANK or ZENU_ERR_AXIS and nothing is launched.
- *   - exactly aliased input/output (the *_assign forms) is supported; partially
- *     overlapping operands are not.
+ *   - an input may be the output's own view (the *_assign forms: same pointer, same strides);
+ *     an input that shares memory with an output in any other way (shifted, transposed or
+ *     broadcast views of it; a reduction's result inside its source; optimizer arrays that
+ *     overlap) is refused with ZENU_ERR_ARG and nothing is launched.  ZeNu's `&mut` outputs
+ *     cannot alias their `&` inputs, so no call the reference can make is affected.
  */
 #ifndef ZENU_HIP_H
 #define ZENU_HIP_H
@@ -83,6 +86,14 @@ int zenu_hip_init(int device);
 int zenu_hip_shutdown(void);
 const char *zenu_hip_status_string(int status);
 /* hipError_t of the last failed runtime call on this thread, and its text. */
+/* The host math library whose results the device's exp, log, tanh, sigmoid, powf, sinh, cosh, sin,
+ * cos, asin, acos and atan reproduce bit for bit (the routines are restated from it and compared
+ * with it on every f32 argument).  ZeNu's CPU device calls whatever libm the host has: on a host
+ * whose libm rounds some of these functions differently (glibc 2.41 and later return correctly
+ * rounded results from several f32 functions), CPU and device results differ by the difference between
+ * the two libms -- at most 1 ulp for the functions themselves, more for the sigmoid, whose last
+ * addition cancels.  No counterpart in the reference. */
+const char *zenu_hip_validated_libm(void);
 int zenu_hip_last_hip_error(void);
 const char *zenu_hip_last_hip_error_string(void);
 
@@ -99,7 +110,10 @@ int zenu_hip_device_synchronize(void);
  * of zenu_hip_free is the last stream that used the block.
  * On out-of-memory the cache is trimmed and the request retried once
  * (the flow zenu-matrix/src/memory_pool/mod.rs:9-20 documents).  Thread-safe.
- * Honours ZENU_USE_MEMPOOL=0 (zenu-matrix/src/lib.rs:36): every call goes to hipMalloc/hipFree. */
+ * Honours ZENU_USE_MEMPOOL=0 (zenu-matrix/src/lib.rs:36): every call goes to hipMalloc/hipFree;
+ * in that mode both functions, and with them every entry point that needs scratch memory, return
+ * ZENU_ERR_UNSUPPORTED while `stream` records a graph (hipFree synchronises, and memory freed
+ * during a capture would still be written by every replay): nothing is recorded. */
 int zenu_hip_malloc(void **ptr_dev, size_t bytes, zenu_stream_t stream);
 int zenu_hip_free(void *ptr_dev, zenu_stream_t stream);
 /* Stream capture (HIP graphs).  Kernels recorded into a graph keep the addresses they were
@@ -247,11 +261,19 @@ int zenu_hip_sum_axis(int dtype, const zenu_tensor_t *out, const zenu_tensor_t *
 int zenu_hip_sum_axis_noalloc(int dtype, const zenu_tensor_t *out, const zenu_tensor_t *src, int axis,
                               zenu_stream_t stream);
 /* Split reductions hand their partial results from many workgroups to one.  That workgroup polls
- * for them; after `polls` fruitless polls (about a microsecond each; default 2^20) it computes the
+ * for them; after `polls` fruitless polls (about a microsecond each; default 2^13, about the time
+ * one workgroup needs to recompute every split of a 128 MiB reduction) it computes the
  * missing ones itself, so no launch ever depends on the order in which workgroups are dispatched.
- * 0 makes every split reduction take that path at once: a switch for tests, results are the same
- * bits either way.  No counterpart in the reference. */
+ * 0 makes the folding workgroup of every split reduction compute every partial itself without
+ * polling at all: a switch for tests, results are the same bits either way.  No counterpart in
+ * the reference. */
 int zenu_hip_set_reduce_spin_limit(int polls);
+/* *count = how many times, since zenu_hip_init, a folding workgroup gave up polling and computed
+ * missing partials itself (once per batch of up to 512 partials).  Such launches are correct but
+ * can be a poll limit slower than normal; a non-zero count on a GPU that is not shared says that
+ * workgroups are being dispatched far out of order.  Blocking (a device-to-host copy).  No
+ * counterpart in the reference. */
+int zenu_hip_reduce_fallback_count(uint64_t *count);
 /* *out_dev = sum of every element (sum_to(x, []), sum.rs:35-94). */
 int zenu_hip_sum_all(int dtype, void *out_dev, const zenu_tensor_t *src, zenu_stream_t stream);
 /* target = sum_to(src) for any legal target shape (sum.rs:35-94). */

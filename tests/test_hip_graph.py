@@ -146,3 +146,61 @@ def test_library_calls_in_a_captured_graph(hip):
         import gc
         gc.collect()
         _lib.check(l.zenu_hip_stream_destroy(stream), "stream_destroy")
+
+
+_POOL_OFF_CAPTURE = r"""
+import ctypes as C, sys
+import numpy as np
+sys.path.insert(0, sys.argv[1])
+import zenu_amd
+from zenu_amd import _lib
+rt = C.CDLL("libamdhip64.so")
+vp = C.c_void_p
+rt.hipStreamBeginCapture.argtypes = [vp, C.c_int]
+rt.hipStreamEndCapture.argtypes = [vp, C.POINTER(vp)]
+rt.hipGraphDestroy.argtypes = [vp]
+l = zenu_amd.lib()
+_lib.check(l.zenu_hip_init(0), "init")
+stream = vp()
+_lib.check(l.zenu_hip_stream_create(C.byref(stream)), "stream_create")
+M = zenu_amd.Matrix
+a = M.from_numpy(np.ones((4096, 256), dtype=np.float32))
+out = M.alloc((256,))
+p = vp()
+_lib.check(l.zenu_hip_malloc(C.byref(p), 1 << 20, stream), "eager malloc with the pool off")
+_lib.check(l.zenu_hip_sum_axis(_lib.F32, C.byref(out.desc()), C.byref(a.desc()), 0, stream), "eager split reduction")
+assert rt.hipStreamBeginCapture(stream, 2) == 0
+q = vp()
+rc_malloc = l.zenu_hip_malloc(C.byref(q), 1 << 20, stream)
+rc_free = l.zenu_hip_free(p, stream)
+rc_reduce = l.zenu_hip_sum_axis(_lib.F32, C.byref(out.desc()), C.byref(a.desc()), 0, stream)   # needs partials
+graph = vp()
+rc_end = rt.hipStreamEndCapture(stream, C.byref(graph))
+print("RC", rc_malloc, rc_free, rc_reduce, rc_end, bool(q.value))
+if graph.value:
+    rt.hipGraphDestroy(graph)
+_lib.check(l.zenu_hip_free(p, stream), "free after the capture")
+_lib.check(l.zenu_hip_sum_axis(_lib.F32, C.byref(out.desc()), C.byref(a.desc()), 0, stream), "reduction after the capture")
+_lib.check(l.zenu_hip_stream_synchronize(stream), "sync")
+assert np.array_equal(out.to_numpy(), np.full(256, 4096.0, dtype=np.float32))
+print("DONE")
+"""
+
+
+def test_pool_off_refuses_scratch_while_capturing():
+    """ZENU_USE_MEMPOOL=0: a capturing stream gets ZENU_ERR_UNSUPPORTED from the allocator and from a
+    reduction that needs partials, before anything is recorded; the capture ends cleanly (no replay
+    is needed to see that) and the same calls work again afterwards."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, ZENU_USE_MEMPOOL="0")
+    r = subprocess.run([sys.executable, "-c", _POOL_OFF_CAPTURE, root], env=env, capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stdout + r.stderr
+    line = [ln for ln in r.stdout.splitlines() if ln.startswith("RC")][0].split()
+    from zenu_amd import _lib
+    unsupported = str(_lib.ERR_UNSUPPORTED)
+    assert line[1:4] == [unsupported] * 3, line
+    assert line[4] == "0" and line[5] == "False", line
+    assert "DONE" in r.stdout

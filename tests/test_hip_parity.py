@@ -247,6 +247,23 @@ def _oracle_threads(fn, x, threads=16):
     return out
 
 
+def _libm_note(hip):
+    """what to say when a bit-exact transcendental check fails: the device restates one particular libm"""
+    import platform
+    return "host libc %s; the device functions restate %s" % (" ".join(platform.libc_ver()),
+                                                              hip.lib().zenu_hip_validated_libm().decode())
+
+
+def test_validated_libm_is_named(hip):
+    note = _libm_note(hip)
+    assert "glibc 2.35" in note
+    import platform
+    if platform.libc_ver() == ("glibc", "2.35"):
+        return
+    # another host libm: the 0-ulp tests below compare against it and may legitimately differ
+    print("note:", note)
+
+
 def test_tanh_sigmoid_dense_sweep(hip):
     """every 16th f32 bit pattern (268 M arguments per function, all exponents, both signs, NaN and
     infinities included): tanh, sigmoid, exp, log, sinh, cosh, sin, cos, atan, asin, acos are the host
@@ -254,19 +271,19 @@ def test_tanh_sigmoid_dense_sweep(hip):
     bits = np.arange(0, 1 << 32, 16, dtype=np.uint64).astype(np.uint32)
     x = bits.view(np.float32)
     X = hip.Matrix.from_numpy(x)
-    assert max_ulp(X.tanh().to_numpy(), _oracle_threads(zo.TANH, x)) == 0
-    assert max_ulp(X.sigmoid().to_numpy(), _oracle_threads(None, x)) == 0
+    assert max_ulp(X.tanh().to_numpy(), _oracle_threads(zo.TANH, x)) == 0, _libm_note(hip)
+    assert max_ulp(X.sigmoid().to_numpy(), _oracle_threads(None, x)) == 0, _libm_note(hip)
     fin = np.isfinite(x)
     exp = _oracle_threads(zo.EXP, x)
     got = X.exp().to_numpy()
-    assert max_ulp(got[fin], exp[fin]) == 0
+    assert max_ulp(got[fin], exp[fin]) == 0, _libm_note(hip)
     nan = np.isnan(x)
     assert np.all(np.isnan(got[nan])) and got[np.isposinf(x)][0] == np.inf and got[np.isneginf(x)][0] == 0
     exp = _oracle_threads(zo.LOG, x)
     got = X.log().to_numpy()
     ok = ~np.isnan(exp)                                    # log of negatives and NaN is NaN on both sides
     assert np.array_equal(np.isnan(got), np.isnan(exp))
-    assert max_ulp(got[ok], exp[ok]) == 0                  # includes zeros (-inf), subnormals and +inf
+    assert max_ulp(got[ok], exp[ok]) == 0, _libm_note(hip)   # includes zeros (-inf), subnormals and +inf
     # cosh is what tanh's backward evaluates; sin / cos include the large-argument reduction
     for name, fn in (("sinh", zo.SINH), ("cosh", zo.COSH), ("sin", zo.SIN), ("cos", zo.COS), ("atan", zo.ATAN),
                      ("asin", zo.ASIN), ("acos", zo.ACOS)):
@@ -274,7 +291,7 @@ def test_tanh_sigmoid_dense_sweep(hip):
         got = getattr(X, name)().to_numpy()
         ok = ~np.isnan(exp)
         assert np.array_equal(np.isnan(got), np.isnan(exp)), name
-        assert max_ulp(got[ok], exp[ok]) == 0, name
+        assert max_ulp(got[ok], exp[ok]) == 0, (name, _libm_note(hip))
 
 
 def test_tanh_ulp2_variant(hip):
@@ -1615,15 +1632,83 @@ def test_split_reduction_handoff_repeatable(hip):
     _lib.check(l.zenu_hip_stream_destroy(s2), "destroy")
 
 
+def test_partially_overlapping_operands_are_refused(hip):
+    """An input may be the output's own view (the *_assign forms); any other sharing of memory between
+    an output and an input -- shifted, transposed or broadcast views of the output's memory, a
+    reduction's result inside its source, optimizer arrays that overlap -- is refused with
+    ZENU_ERR_ARG before anything is launched.  (ZeNu's `&mut` outputs cannot alias `&` inputs, so no
+    call the reference can make is refused.)"""
+    import ctypes as C
+    from zenu_amd import _lib
+    l = hip.lib()
+    M = hip.Matrix
+    r = rng(17)
+    x = r.standard_normal((64, 64)).astype(np.float32)
+    A = M.from_numpy(x)
+    B = M.from_numpy(x)
+
+    def refused(fn):
+        with pytest.raises(_lib.ZenuHipError) as e:
+            fn()
+        assert e.value.status == _lib.ERR_ARG
+        assert np.array_equal(A.to_numpy(), x), "a refused call wrote something"
+
+    # the output's own view: in place
+    A.add_assign(A)
+    assert np.array_equal(A.to_numpy(), x + x)
+    A.copy_from(B)
+    A.slice(slice(0, 32)).add_array(A.slice(slice(0, 32)), B.slice(slice(0, 32)))   # lhs is the output's view
+    A.copy_from(B)
+    # shifted rows, transposed, broadcast row of the output
+    refused(lambda: A.slice(slice(0, 63)).add_array(A.slice(slice(1, 64)), B.slice(slice(0, 63))))
+    refused(lambda: A.slice(slice(0, 63)).add_assign(A.slice(slice(1, 64))))
+    refused(lambda: A.add_array(B, A.transpose()))
+    refused(lambda: A.add_assign(A.slice(slice(0, 1))))
+    refused(lambda: A.copy_from(A.transpose()))
+    refused(lambda: A.slice(slice(0, 64), slice(0, 32)).exp_array(A.slice(slice(0, 64), slice(16, 48))))
+    # neighbours that only touch are fine
+    A.slice(slice(0, 32)).add_assign(A.slice(slice(32, 64)))
+    exp = x.copy()
+    exp[:32] += exp[32:]
+    assert np.array_equal(A.to_numpy(), exp)
+    A.copy_from(B)
+    # a reduction that writes into its source
+    row0 = A.index_axis(0, 0)
+    rc = l.zenu_hip_sum_axis(_lib.F32, C.byref(row0.desc()), C.byref(A.desc()), 0, hip.get_stream())
+    assert rc == _lib.ERR_ARG
+    rc = l.zenu_hip_sum_all(_lib.F32, A.as_ptr(), C.byref(A.desc()), hip.get_stream())
+    assert rc == _lib.ERR_ARG
+    assert np.array_equal(A.to_numpy(), x)
+    # optimizer arrays
+    n = 1000
+    P, G, Mm = (M.from_numpy(r.standard_normal(n + 8).astype(np.float32)) for _ in range(3))
+    pv, gv, mv = P.as_ptr(), G.as_ptr(), Mm.as_ptr()
+    rc = l.zenu_hip_adam_step(_lib.F32, pv, gv, mv, mv + 16, n, 1e-3, 0.9, 0.999, 1e-8, 1.0, hip.get_stream())
+    assert rc == _lib.ERR_ARG
+    rc = l.zenu_hip_sgd_step(_lib.F32, pv, pv + 4 * (n - 1), n, 1e-3, hip.get_stream())
+    assert rc == _lib.ERR_ARG
+    rc = l.zenu_hip_sgd_step(_lib.F32, pv, pv + 4 * n, 8, 1e-3, hip.get_stream())     # adjacent, disjoint
+    assert rc == _lib.OK
+
+
 def test_split_reductions_when_the_folding_workgroup_computes_everything_itself(hip):
     """The workgroup that folds a split reduction polls for the other workgroups' partial results and,
     after a bounded number of polls, computes the missing ones itself.  With the bound at 0 it takes
     that path at once, for partials that have not landed yet; the results must be the bits of the
     ordinary path (same partials, same merge order), in f32 and f64, for sums, asum, max and arg-max
     over rows, columns and the whole tensor.  Forced from the host; every kernel still exits normally."""
+    import ctypes as C
     from zenu_amd import _lib
     l = hip.lib()
     r = rng(91)
+
+    def fallbacks():
+        n = C.c_uint64()
+        _lib.check(l.zenu_hip_reduce_fallback_count(C.byref(n)), "fallback count")
+        return n.value
+
+    # every reduction this process has run so far found its partials by polling
+    assert fallbacks() == 0, "a split reduction gave up polling and recomputed partials in an ordinary run"
 
     def run_all(X, x):
         out = [X.sum_all().to_numpy().copy(), X.sum(0).to_numpy().copy(), X.max_axis(0).to_numpy().copy(),
@@ -1638,6 +1723,8 @@ def test_split_reductions_when_the_folding_workgroup_computes_everything_itself(
         x[5, 7] = x[2000, 7] = x.max() + 1          # a tie across splits: the first index must win
         X = hip.Matrix.from_numpy(x)
         ref = run_all(X, x)
+        before = fallbacks()
+        assert before == (0 if dt == np.float32 else hip._forced_fallbacks)
         _lib.check(l.zenu_hip_set_reduce_spin_limit(0), "spin limit")
         try:
             for rep in range(3):
@@ -1645,7 +1732,11 @@ def test_split_reductions_when_the_folding_workgroup_computes_everything_itself(
                 for i, (a, b) in enumerate(zip(got, ref)):
                     assert bits_equal(np.asarray(a), np.asarray(b)), (np.dtype(dt).name, rep, i)
         finally:
-            _lib.check(l.zenu_hip_set_reduce_spin_limit(1 << 20), "spin limit")
+            _lib.check(l.zenu_hip_set_reduce_spin_limit(1 << 13), "spin limit")
+        hip._forced_fallbacks = fallbacks()          # the forced path is counted ...
+        assert hip._forced_fallbacks > before
+        run_all(X, x)
+        assert fallbacks() == hip._forced_fallbacks  # ... and the ordinary one is not
         assert ref[3][7] == 5 and tuple(ref[5]) == (5, 7)
         assert_sum_close(ref[1], zo.sum_axis(x, 0), x, 0, "sum axis 0")
         del X

@@ -98,3 +98,13 @@ def test_sum_axis_noalloc_views_and_limits(hip):
     assert np.all(o.to_numpy() == 3.0)
     assert b"static scratch" in l.zenu_hip_status_string(_lib.ERR_SCRATCH_LIMIT)
     del big, bview, src2
+
+
+def test_zz_no_ordinary_reduction_fell_back(hip):
+    """Runs last: apart from the launches that tests/test_hip_parity.py forced onto that path (spin limit
+    0), no split reduction of this process gave up polling for its partial results."""
+    import ctypes as C
+    from zenu_amd import _lib
+    n = C.c_uint64()
+    _lib.check(hip.lib().zenu_hip_reduce_fallback_count(C.byref(n)), "fallback count")
+    assert n.value == getattr(hip, "_forced_fallbacks", 0)

@@ -89,6 +89,7 @@ SIGNATURES = {
     "zenu_hip_sum_axis": [_i, _TP, _TP, _i, _vp],
     "zenu_hip_sum_axis_noalloc": [_i, _TP, _TP, _i, _vp],
     "zenu_hip_set_reduce_spin_limit": [_i],
+    "zenu_hip_reduce_fallback_count": [C.POINTER(C.c_uint64)],
     "zenu_hip_sum_all": [_i, _vp, _TP, _vp],
     "zenu_hip_sum_to": [_i, _TP, _TP, _vp],
     "zenu_hip_max_axis": [_i, _TP, _TP, _i, _vp],
@@ -142,6 +143,8 @@ def lib():
         fn.restype = C.c_int
     l.zenu_hip_status_string.argtypes = [C.c_int]
     l.zenu_hip_status_string.restype = C.c_char_p
+    l.zenu_hip_validated_libm.argtypes = []
+    l.zenu_hip_validated_libm.restype = C.c_char_p
     l.zenu_hip_last_hip_error_string.argtypes = []
     l.zenu_hip_last_hip_error_string.restype = C.c_char_p
     _lib = l

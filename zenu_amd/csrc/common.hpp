@@ -82,6 +82,11 @@ struct EwProblem {
 void ew_set_operand(EwProblem &p, int slot, const zenu_tensor_t &t, int out_ndim,
                     const int64_t *out_shape);
 void ew_collapse(EwProblem &p);
+// ZENU_ERR_ARG when an input shares memory with the output other than as the output's own view
+int ew_check_alias(const EwProblem &p, size_t esz);
+int check_output_alias(const zenu_tensor_t &out, const zenu_tensor_t &in, size_t esz);
+bool ranges_overlap(const void *a, size_t a_bytes, const void *b, size_t b_bytes);
+bool view_overlaps(const zenu_tensor_t &t, size_t esz, const void *ptr, size_t bytes);
 
 // ---- device properties cached at init ---------------------------------------------------------
 struct DeviceInfo {

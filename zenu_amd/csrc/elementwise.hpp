@@ -825,6 +825,7 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
     constexpr int VEC = VecOf<T>::N;
     ew_collapse(p);
     if (p.numel == 0) return ZENU_OK;
+    if (int rc = ew_check_alias(p, sizeof(T))) return rc;
     T *out = static_cast<T *>(p.ptr[0]);
     const T *a = static_cast<const T *>(p.ptr[1]);
     const T *b = (F::NIN == 2) ? static_cast<const T *>(p.ptr[2]) : a;

@@ -256,12 +256,20 @@ AdamConsts<T> make_consts(double lr, double beta1, double beta2, double eps, dou
     return k;
 }
 
+// the parameter, gradient and moment arrays of one tensor are four different arrays
+inline bool adam_arrays_overlap(const void *p, const void *g, const void *m, const void *v, size_t bytes)
+{
+    return ranges_overlap(p, bytes, g, bytes) || ranges_overlap(p, bytes, m, bytes) || ranges_overlap(p, bytes, v, bytes) ||
+           ranges_overlap(g, bytes, m, bytes) || ranges_overlap(g, bytes, v, bytes) || ranges_overlap(m, bytes, v, bytes);
+}
+
 template <typename T>
 int adam_t(void *p, const void *g, void *m, void *v, int64_t n, const AdamConsts<T> &k, int decay,
            hipStream_t s)
 {
     constexpr int VEC = VecOf<T>::N;
     if (n == 0) return ZENU_OK;
+    if (adam_arrays_overlap(p, g, m, v, (size_t)n * sizeof(T))) return ZENU_ERR_ARG;
     const bool vec = aligned16(p) && aligned16(g) && aligned16(m) && aligned16(v);
     const bool nt = n * (int64_t)sizeof(T) * 7 >= kStreamBytes;  // 7 passes exceed the caches: stream
     if (vec) {
@@ -293,6 +301,8 @@ int adam_multi_t(int nt, void *const *p, const void *const *g, void *const *m, v
     constexpr int64_t kTile = (int64_t)kBlock * VEC * kUnroll;
     for (int i = 0; i < nt; i++)
         if (sizes[i] < 0 || (sizes[i] > 0 && (!p[i] || !g[i] || !m[i] || !v[i]))) return ZENU_ERR_ARG;
+    for (int i = 0; i < nt; i++)
+        if (adam_arrays_overlap(p[i], g[i], m[i], v[i], (size_t)sizes[i] * sizeof(T))) return ZENU_ERR_ARG;
     int i = 0;
     while (i < nt) {
         MultiArgs a;
@@ -333,6 +343,8 @@ int sgd_multi_t(int nt, void *const *p, const void *const *g, const int64_t *siz
     constexpr int64_t kTile = (int64_t)kBlock * VEC * kSgdUnroll;
     for (int i = 0; i < nt; i++)
         if (sizes[i] < 0 || (sizes[i] > 0 && (!p[i] || !g[i]))) return ZENU_ERR_ARG;
+    for (int i = 0; i < nt; i++)
+        if (ranges_overlap(p[i], (size_t)sizes[i] * sizeof(T), g[i], (size_t)sizes[i] * sizeof(T))) return ZENU_ERR_ARG;
     int i = 0;
     while (i < nt) {
         MultiArgs a;
@@ -392,6 +404,8 @@ int zenu_hip_sgd_step(int dtype, void *p_dev, const void *g_dev, int64_t n, doub
     int rc = ensure_init();
     if (rc) return rc;
     if (n == 0) return ZENU_OK;
+    if (ranges_overlap(p_dev, (size_t)n * (dtype == ZENU_F64 ? 8 : 4), g_dev, (size_t)n * (dtype == ZENU_F64 ? 8 : 4)))
+        return ZENU_ERR_ARG;
     hipStream_t s = as_stream(stream);
     const bool vec = aligned16(p_dev) && aligned16(g_dev);
     if (dtype == ZENU_F32) {

@@ -60,6 +60,11 @@ constexpr size_t kScratchBytes = kScratchCounterBytes + kScratchPartialBytes + k
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 unsigned char *g_scratch_ptr = nullptr;   // device address of `scratch` (one device per process)
 
+// How often a folding workgroup gave up polling and computed missing partials itself (see "hand-off
+// through tagged words").  Such a launch is correct but slow, and nothing else would show it.
+static __device__ unsigned int fold_fallbacks;
+unsigned int *g_fold_fallbacks_ptr = nullptr;   // device address of `fold_fallbacks`
+
 // where a reduction finds its cross-workgroup memory when it may not allocate
 struct FixedScratch {
     int *counters;
@@ -238,6 +243,7 @@ template <typename T> struct RedParams {
     uint64_t *slots;
     uint32_t epoch;          // this launch's tag, never zero
     int spin_limit;          // polls before the folding workgroup computes what is missing itself
+    unsigned int *fallbacks; // bumped once per batch of partials that the folding workgroup had to compute
     // value gather for max: value = gsrc[q * g_outer_stride + c + idx * g_elem_stride]
     const T *gsrc;
     int64_t g_outer_stride, g_elem_stride;
@@ -522,6 +528,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(RedParams<T> p)
         for (int s0 = 0; s0 < splits; s0 += kSlotBatch * kBlock) {
             A t[kSlotBatch];
             int polls = 0;
+            bool force = p.spin_limit == 0;   // the host asks for the fallback itself: every partial of the batch
             for (;;) {
                 int ok = 1;
 #pragma unroll
@@ -530,13 +537,15 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(RedParams<T> p)
                     t[u] = Tr::identity();
                     if (sidx < splits && !load_slot<T, Tr>(p, nslots, s_base + sidx, t[u])) ok = 0;
                 }
-                if (__syncthreads_and(ok)) break;
-                if (++polls > p.spin_limit) {
+                if (__syncthreads_and(ok) && !force) break;
+                if (force || ++polls > p.spin_limit) {
                     // compute what is still missing in this batch, as its owner would
+                    if (lane == 0 && p.fallbacks)
+                        __hip_atomic_fetch_add(p.fallbacks, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     const int s_end = s0 + kSlotBatch * kBlock < splits ? s0 + kSlotBatch * kBlock : splits;
                     for (int sp = s0; sp < s_end; sp++) {
                         A probe;
-                        const int have = (lane == 0 && load_slot<T, Tr>(p, nslots, s_base + sp, probe)) ? 1 : 0;
+                        const int have = (!force && lane == 0 && load_slot<T, Tr>(p, nslots, s_base + sp, probe)) ? 1 : 0;
                         if (__syncthreads_or(have)) continue;
                         const A r = block_allreduce<Tr>(lane_partial(sp));
                         if (lane == 0) emit_slot<T, Tr>(p, nslots, s_base + sp, r);
@@ -544,6 +553,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(RedParams<T> p)
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the words are in place before the next poll
                     __syncthreads();
                     polls = 0;
+                    force = false;
                 }
             }
 #pragma unroll
@@ -952,6 +962,7 @@ int reduce_strided(const T *src, int64_t outer, int64_t R, int64_t inner, int64_
     p.slots = nullptr;
     p.epoch = 0;
     p.spin_limit = 0;
+    p.fallbacks = g_fold_fallbacks_ptr;
     p.gsrc = src;
     p.g_outer_stride = outer_stride;
     p.g_elem_stride = elem_stride;
@@ -1194,6 +1205,14 @@ int reduce_axis(int kind, int dtype, const zenu_tensor_t *out, int64_t *out_idx,
     if (rc) return rc;
     if (axis < 0 || axis >= src->ndim) return ZENU_ERR_AXIS;
     if (out && !reduced_shape_ok(*out, *src, axis)) return ZENU_ERR_SHAPE;
+    {   // results that share memory with the source would be read back as input by other workgroups
+        const size_t esz = dtype == ZENU_F64 ? 8 : 4;
+        int64_t nout = 1;
+        for (int i = 0; i < src->ndim; i++)
+            if (i != axis) nout *= src->shape[i];
+        if (out && src->shape[axis] > 1 && check_output_alias(*out, *src, esz)) return ZENU_ERR_ARG;
+        if (out_idx && view_overlaps(*src, esz, out_idx, (size_t)nout * sizeof(int64_t))) return ZENU_ERR_ARG;
+    }
     if (dtype == ZENU_F32) return reduce_axis_t<float>(kind, dtype, out, out_idx, *src, axis, s, fixed);
     if (dtype == ZENU_F64) return reduce_axis_t<double>(kind, dtype, out, out_idx, *src, axis, s, fixed);
     return ZENU_ERR_ARG;
@@ -1208,6 +1227,9 @@ int reduce_all(int kind, int dtype, void *out_val, int64_t *out_idx, const zenu_
     const int64_t n = num_elm(*src);
     const size_t esz = dtype == ZENU_F32 ? 4 : 8;
     if (dtype != ZENU_F32 && dtype != ZENU_F64) return ZENU_ERR_ARG;
+    if (n > 1 && ((out_val && view_overlaps(*src, esz, out_val, esz)) ||
+                  (out_idx && view_overlaps(*src, esz, out_idx, sizeof(int64_t)))))
+        return ZENU_ERR_ARG;   // the result would overwrite an element other workgroups still read
     if (n <= 0) {   // nothing to add: 0; nothing to take a maximum of: an error
         if (kind == kMax) return ZENU_ERR_SHAPE;
         return zenu_hip_memset_zero(out_val, esz, reinterpret_cast<zenu_stream_t>(s));
@@ -1247,6 +1269,11 @@ int init_static_scratch()
     ZENU_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
     if (!p) return ZENU_ERR_HIP;
     g_scratch_ptr = static_cast<unsigned char *>(p);
+    void *f = nullptr;
+    ZENU_HIP_TRY(hipGetSymbolAddress(&f, HIP_SYMBOL(fold_fallbacks)));
+    if (!f) return ZENU_ERR_HIP;
+    ZENU_HIP_TRY(hipMemset(f, 0, sizeof(unsigned int)));
+    g_fold_fallbacks_ptr = static_cast<unsigned int *>(f);
     return ZENU_OK;
 }
 
@@ -1270,6 +1297,16 @@ int zenu_hip_sum_axis_noalloc(int dtype, const zenu_tensor_t *out, const zenu_te
     fx.stage = g_scratch_ptr + kScratchCounterBytes + kScratchPartialBytes;
     fx.stage_bytes = kScratchStageBytes;
     return reduce_axis(kSum, dtype, out, nullptr, src, axis, as_stream(stream), &fx);
+}
+
+int zenu_hip_reduce_fallback_count(uint64_t *count)
+{
+    if (!count) return ZENU_ERR_ARG;
+    if (!library_ready() || !g_fold_fallbacks_ptr) return ZENU_ERR_NOT_INIT;
+    unsigned int v = 0;
+    ZENU_HIP_TRY(hipMemcpy(&v, g_fold_fallbacks_ptr, sizeof v, hipMemcpyDeviceToHost));   // waits for the device
+    *count = v;
+    return ZENU_OK;
 }
 
 int zenu_hip_sum_axis(int dtype, const zenu_tensor_t *out, const zenu_tensor_t *src, int axis,

@@ -71,7 +71,10 @@ State g_state;
 std::mutex g_init_mu;
 // polls of a folding workgroup before it computes missing partial results itself (about a
 // microsecond each); 0 makes every split reduction take that path at once (tests)
-std::atomic<int> g_reduce_spin_limit{1 << 20};
+// polls (about a microsecond each) before a folding workgroup computes missing partials itself:
+// about as long as recomputing every split of a 128 MiB reduction takes one workgroup (6 ms at
+// 22 GB/s); waiting longer than that for workgroups that have not been dispatched buys nothing
+std::atomic<int> g_reduce_spin_limit{1 << 13};
 
 // is `stream` recording a graph?  (the null stream never is)
 bool stream_is_capturing(hipStream_t stream)
@@ -281,6 +284,11 @@ const char *zenu_hip_status_string(int status)
     }
 }
 
+const char *zenu_hip_validated_libm(void)
+{
+    return "glibc 2.35 libm, x86-64 (the variants selected on CPUs with FMA)";
+}
+
 int zenu_hip_last_hip_error(void) { return (int)tl_last_hip_error; }
 const char *zenu_hip_last_hip_error_string(void) { return hipGetErrorString(tl_last_hip_error); }
 
@@ -330,6 +338,10 @@ int zenu_hip_malloc(void **ptr_dev, size_t bytes, zenu_stream_t stream)
     int rc = ensure_init();
     if (rc) return rc;
     if (!g_state.use_pool) {
+        // Without the pool every request goes to the driver and every release is a hipFree, which
+        // synchronises: inside a capture that invalidates the recording or, in relaxed mode, frees
+        // memory whose address the recorded kernels keep.  Refused before anything is recorded.
+        if (stream_is_capturing(as_stream(stream))) return ZENU_ERR_UNSUPPORTED;
         *ptr_dev = nullptr;
         if (g_state.backend.raw_alloc(ptr_dev, bytes ? bytes : 1) != 0) return ZENU_ERR_OOM;
         return ZENU_OK;
@@ -343,6 +355,7 @@ int zenu_hip_free(void *ptr_dev, zenu_stream_t stream)
     int rc = ensure_init();
     if (rc) return rc;
     if (!g_state.use_pool) {
+        if (stream_is_capturing(as_stream(stream))) return ZENU_ERR_UNSUPPORTED;   // see zenu_hip_malloc
         ZENU_HIP_TRY(hipFree(ptr_dev));
         return ZENU_OK;
     }

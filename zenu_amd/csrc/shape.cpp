@@ -5,6 +5,7 @@
 // legality rules are checked once, the operands are folded into one iteration space, and a
 // single launch covers it.
 #include <algorithm>
+#include <cstdint>
 #include <utility>
 
 #include "common.hpp"
@@ -138,6 +139,70 @@ static int broadcast_walk(const int64_t *to, int nt, const int64_t *src, int ns)
 int check_broadcast(const zenu_tensor_t &to, const zenu_tensor_t &source)
 {
     return broadcast_walk(to.shape, to.ndim, source.shape, source.ndim);
+}
+
+// ---- operand aliasing -------------------------------------------------------------------------------
+// ZeNu's ops take `&mut` outputs and `&` inputs, so an output never shares memory with an input
+// except as the very same view (the *_assign forms).  Through a C ABI anything can be passed:
+// operands that overlap only partly (shifted, transposed or broadcast views of the output's
+// memory) would be read by some threads after others have overwritten them.  They are refused.
+
+// [lo, hi) in bytes of everything a view can touch (strides are non-negative)
+static void byte_range(const void *ptr, int ndim, const int64_t *shape, const int64_t *stride, size_t esz,
+                       uintptr_t &lo, uintptr_t &hi)
+{
+    int64_t last = 0;
+    bool empty = false;
+    for (int d = 0; d < ndim; d++) {
+        if (shape[d] == 0) empty = true;
+        else last += (shape[d] - 1) * stride[d];
+    }
+    lo = reinterpret_cast<uintptr_t>(ptr);
+    hi = empty ? lo : lo + (uintptr_t)(last + 1) * esz;
+}
+
+bool ranges_overlap(const void *a, size_t a_bytes, const void *b, size_t b_bytes)
+{
+    const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+    return a_bytes && b_bytes && a0 < b0 + b_bytes && b0 < a0 + a_bytes;
+}
+
+bool view_overlaps(const zenu_tensor_t &t, size_t esz, const void *ptr, size_t bytes)
+{
+    uintptr_t lo, hi;
+    byte_range(t.ptr, t.ndim, t.shape, t.stride, esz, lo, hi);
+    return ranges_overlap(reinterpret_cast<const void *>(lo), (size_t)(hi - lo), ptr, bytes);
+}
+
+int check_output_alias(const zenu_tensor_t &out, const zenu_tensor_t &in, size_t esz)
+{
+    uintptr_t o0, o1, i0, i1;
+    byte_range(out.ptr, out.ndim, out.shape, out.stride, esz, o0, o1);
+    byte_range(in.ptr, in.ndim, in.shape, in.stride, esz, i0, i1);
+    if (o0 >= i1 || i0 >= o1 || o0 == o1 || i0 == i1) return ZENU_OK;
+    if (out.ptr != in.ptr || out.ndim != in.ndim) return ZENU_ERR_ARG;
+    for (int d = 0; d < out.ndim; d++) {
+        if (out.shape[d] != in.shape[d]) return ZENU_ERR_ARG;
+        if (out.shape[d] > 1 && out.stride[d] != in.stride[d]) return ZENU_ERR_ARG;
+    }
+    return ZENU_OK;
+}
+
+int ew_check_alias(const EwProblem &p, size_t esz)
+{
+    uintptr_t o0, o1;
+    byte_range(p.ptr[0], p.ndim, p.shape, p.stride[0], esz, o0, o1);
+    if (o0 == o1) return ZENU_OK;
+    for (int o = 1; o < p.nops; o++) {
+        uintptr_t i0, i1;
+        byte_range(p.ptr[o], p.ndim, p.shape, p.stride[o], esz, i0, i1);
+        if (o0 >= i1 || i0 >= o1) continue;
+        // overlapping: only the output's own view is allowed (same start, same stride on every dim)
+        if (p.ptr[o] != p.ptr[0]) return ZENU_ERR_ARG;
+        for (int d = 0; d < p.ndim; d++)
+            if (p.shape[d] > 1 && p.stride[o][d] != p.stride[0][d]) return ZENU_ERR_ARG;
+    }
+    return ZENU_OK;
 }
 
 void ew_set_operand(EwProblem &p, int slot, const zenu_tensor_t &t, int out_ndim,
