@@ -100,6 +100,82 @@ def test_sum_axis_noalloc_views_and_limits(hip):
     del big, bview, src2
 
 
+def test_noalloc_large_split_then_small_split_reuses_the_same_scratch(hip):
+    """A large split reduction fills the static partials; the small one after it uses the first bytes of
+    the same area with fewer splits and different data: nothing of the large call's partials may
+    reach the small call's result (and the other way round on the third call)."""
+    r = np.random.default_rng(9)
+    big = (r.standard_normal((8192, 1024)) * 1000).astype(np.float32)      # 16 splits x 1024 outputs
+    small = r.standard_normal((520, 256)).astype(np.float32)                # fewer splits, fewer outputs
+    B, S = hip.Matrix.from_numpy(big), hip.Matrix.from_numpy(small)
+    for X, x in ((B, big), (S, small), (B, big), (S, small)):
+        got, ref = _both(hip, X, 0, (x.shape[1],), np.float32)
+        assert bits_equal(got, ref), x.shape
+        assert_sum_close(got, zo.sum_axis(x, 0), x, 0, f"{x.shape} axis 0")
+
+
+def test_noalloc_call_recorded_into_a_graph(hip):
+    """The call is meant for code under HIP-graph capture: record it (a split column reduction and a split
+    row reduction, with their counter fills) into a graph, replay the graph on new inputs with eager
+    reductions on the same stream in between, and compare every replay bit for bit with
+    zenu_hip_sum_axis on the same inputs.  The pool's counters do not move during the capture."""
+    from zenu_amd import _lib
+    from test_hip_graph import _hip_runtime
+    rt = _hip_runtime()
+    l = hip.lib()
+    M = hip.Matrix
+    stream = C.c_void_p()
+    _lib.check(l.zenu_hip_stream_create(C.byref(stream)), "stream_create")
+    old = hip.get_stream()
+    hip.set_stream(stream)
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    try:
+        r = np.random.default_rng(10)
+        inputs = [r.standard_normal((4096, 512)).astype(np.float32) * s for s in (1.0, 3.0, 0.25)]
+        X = M.from_numpy(inputs[0])
+        Xr = X.reshape((4, 4096 * 128))
+        cols, rows = M.alloc((512,)), M.alloc((4,))
+        ecols, erows = M.alloc((512,)), M.alloc((4,))
+
+        def sequence(fn, oc, orow):
+            _lib.check(fn(_lib.F32, C.byref(oc.desc()), C.byref(X.desc()), 0, stream), "cols")
+            _lib.check(fn(_lib.F32, C.byref(orow.desc()), C.byref(Xr.desc()), 1, stream), "rows")
+
+        sequence(l.zenu_hip_sum_axis_noalloc, cols, rows)                 # eager once
+        hip.synchronize()
+        before = _stats(hip)
+        assert rt.hipStreamBeginCapture(stream, 2) == 0
+        try:
+            sequence(l.zenu_hip_sum_axis_noalloc, cols, rows)
+        finally:
+            rc = rt.hipStreamEndCapture(stream, C.byref(graph))
+        assert rc == 0
+        after = _stats(hip)
+        assert after.n_alloc_calls == before.n_alloc_calls and after.n_driver_allocs == before.n_driver_allocs
+        assert rt.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+        for i, inp in enumerate(inputs + inputs[:1]):
+            _lib.check(l.zenu_hip_memcpy_h2d(X.as_ptr(), inp.ctypes.data, inp.nbytes, stream), "h2d")
+            _lib.check(l.zenu_hip_memset_zero(cols.as_ptr(), 512 * 4, stream), "zero")
+            _lib.check(l.zenu_hip_memset_zero(rows.as_ptr(), 4 * 4, stream), "zero")
+            assert rt.hipGraphLaunch(gexec, stream) == 0
+            hip.synchronize()
+            got = cols.to_numpy().copy(), rows.to_numpy().copy()
+            sequence(l.zenu_hip_sum_axis, ecols, erows)                   # eager work between the replays
+            hip.synchronize()
+            assert bits_equal(got[0], ecols.to_numpy()) and bits_equal(got[1], erows.to_numpy()), i
+            assert_sum_close(got[0], zo.sum_axis(inp, 0), inp, 0, "replayed column sums")
+    finally:
+        hip.synchronize()
+        if gexec:
+            rt.hipGraphExecDestroy(gexec)
+        if graph:
+            rt.hipGraphDestroy(graph)
+        hip.set_stream(old)
+        X = Xr = cols = rows = ecols = erows = None      # freed before their stream goes
+        import gc
+        gc.collect()
+        _lib.check(l.zenu_hip_stream_destroy(stream), "stream_destroy")
+
 def test_zz_no_ordinary_reduction_fell_back(hip):
     """Runs last: apart from the launches that tests/test_hip_parity.py forced onto that path (spin limit
     0), no split reduction of this process gave up polling for its partial results."""

@@ -42,6 +42,7 @@ int *reserve_counters(int64_t n, hipStream_t stream);
 // `nwords` tagged 64-bit words from the ring of `stream` and this launch's tag, or nullptr
 uint64_t *reserve_slots(int64_t nwords, hipStream_t stream, uint32_t *epoch);
 int reduce_spin_limit();
+bool rehearsal_needed(size_t bytes, hipStream_t stream);
 bool library_ready();
 
 namespace {
@@ -1013,11 +1014,13 @@ int reduce_strided(const T *src, int64_t outer, int64_t R, int64_t inner, int64_
         uint32_t epoch = 0;
         uint64_t *slots = reserve_slots(nout * splits * SlotWords<T, Tr>::W, s, &epoch);
         if (slots) {
-            // The same request the counter path would make: it keeps a block of that size in the pool
-            // of this stream, so that a later capture of the same call (which takes the counter path)
-            // finds it there and does not have to go to the driver.
-            Workspace rehearse(key_bytes + idx_bytes, s);
-            if (rehearse.status) return rehearse.status;
+            // The request the counter path would make, once per stream and size: it leaves a block of
+            // that size in the pool of this stream, so that a later capture of the same call (which
+            // takes the counter path) finds it there and does not have to go to the driver.
+            if (rehearsal_needed(key_bytes + idx_bytes, s)) {
+                Workspace rehearse(key_bytes + idx_bytes, s);
+                if (rehearse.status) return rehearse.status;
+            }
             p.slots = slots;
             p.epoch = epoch;
             p.spin_limit = reduce_spin_limit();

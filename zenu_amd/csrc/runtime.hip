@@ -59,7 +59,7 @@ struct State {
     // tagged partial-result words.  A word is {tag, payload}; the tag is the ring's launch number
     // (`epoch`, never zero, never repeated), so what an earlier launch left behind is never taken
     // for a result of the current one and nothing has to be cleared.
-    struct Ring { int *base = nullptr; int64_t cursor = 0; int64_t slot_cursor = 0; uint32_t epoch = 0; };
+    struct Ring { int *base = nullptr; int64_t cursor = 0; int64_t slot_cursor = 0; uint32_t epoch = 0; size_t rehearsed = 0; };
     std::map<hipStream_t, Ring> rings;
     std::mutex counter_mu;
     DeviceInfo info;
@@ -69,8 +69,6 @@ struct State {
 
 State g_state;
 std::mutex g_init_mu;
-// polls of a folding workgroup before it computes missing partial results itself (about a
-// microsecond each); 0 makes every split reduction take that path at once (tests)
 // polls (about a microsecond each) before a folding workgroup computes missing partials itself:
 // about as long as recomputing every split of a 128 MiB reduction takes one workgroup (6 ms at
 // 22 GB/s); waiting longer than that for workgroups that have not been dispatched buys nothing
@@ -219,6 +217,22 @@ uint64_t *reserve_slots(int64_t nwords, hipStream_t stream, uint32_t *epoch)
         if (!make_ring(stream)) return nullptr;
     }
     return nullptr;
+}
+
+// A split reduction that uses tagged words needs no workspace, but the same call recorded into a
+// graph would (it takes the counter path): the eager call then requests and releases a block of
+// that size once, so the pool of its stream holds one when a capture comes.  True when `bytes` is
+// larger than anything rehearsed on `stream` so far; never with the pool switched off (the block
+// would go straight back to the driver).
+bool rehearsal_needed(size_t bytes, hipStream_t stream)
+{
+    if (!g_state.use_pool || bytes == 0) return false;
+    std::lock_guard<std::mutex> g(g_state.counter_mu);
+    auto it = g_state.rings.find(stream);
+    if (it == g_state.rings.end()) return false;
+    if (bytes <= it->second.rehearsed) return false;
+    it->second.rehearsed = bytes;
+    return true;
 }
 
 int ensure_init()
@@ -382,6 +396,10 @@ int zenu_hip_mempool_trim(void)
 {
     int rc = ensure_init();
     if (rc) return rc;
+    {   // the blocks that rehearsals left are gone with the rest
+        std::lock_guard<std::mutex> g(g_state.counter_mu);
+        for (auto &kv : g_state.rings) kv.second.rehearsed = 0;
+    }
     return g_state.pool->trim();
 }
 
