@@ -521,8 +521,8 @@ def compiled_host_c4(x, t, params, args):
 def capture_and_replay_c4(z, st, args, sync):
     """Capture one whole step (62 launches, 37 with the fused entry points, all on the library's stream, all allocations
     served by the caching pool) into a HIP graph and time its replays: the step without the
-    host's per-launch cost.  Every replay is checked against an eager step from the same state.
-    The Adam step number is a kernel argument and so is frozen in the graph."""
+    host's per-launch cost.  The recorded Adam update is the scheduled one, so consecutive replays are
+    consecutive training steps; the first three are checked bit for bit against three eager steps."""
     import numpy as np
     rt = C.CDLL("libamdhip64.so")
     stream = z.get_stream()
@@ -547,12 +547,15 @@ def capture_and_replay_c4(z, st, args, sync):
             st.opt.step = s[3]
 
         s0 = snapshot()
-        eager_loss, _ = st.step()
-        eager = (float(eager_loss.to_numpy()), {k: v.to_numpy() for k, v in st.p.items()})
-        for _ in range(2):      # rehearse with the live set the capture will see: every request a pool hit
-            rehearsal = st.step()
+        eager = []
+        for _ in range(3):      # three consecutive eager steps: the reference results, and the rehearsal that
+            eager_loss, rehearsal = st.step()   # leaves every block the capture will ask the pool for
+            eager.append((float(eager_loss.to_numpy()), {k: v.to_numpy() for k, v in st.p.items()}))
             del rehearsal
         restore(s0)
+        # Adam's step advances on every update (adam.rs:21-25): the recorded update takes 1 - beta^t from a
+        # table in device memory whose cursor it advances, so replay i is step i
+        st.opt.use_schedule(args.steps + 16)
         sync()
         if rt.hipStreamBeginCapture(stream, 2) != 0:   # hipStreamCaptureModeRelaxed
             return {"error": "hipStreamBeginCapture failed"}
@@ -567,14 +570,12 @@ def capture_and_replay_c4(z, st, args, sync):
         if rt.hipGraphInstantiate(C.byref(ge), g, None, None, 0) != 0:
             return {"error": "hipGraphInstantiate failed"}
         checks = 0
-        for _ in range(3):                              # replays, each checked against the eager result
-            restore(s0)
-            st.opt.step = s0[3] + 1
+        for i in range(3):                              # consecutive replays = consecutive steps, each checked
             assert rt.hipGraphLaunch(ge, stream) == 0
             sync()
-            ok = float(loss.to_numpy()) == eager[0] and all(np.array_equal(st.p[k].to_numpy(), eager[1][k]) for k in st.p)
+            ok = float(loss.to_numpy()) == eager[i][0] and all(np.array_equal(st.p[k].to_numpy(), eager[i][1][k]) for k in st.p)
             if not ok:
-                return {"error": "graph replay differs from the eager step"}
+                return {"error": f"graph replay {i} differs from eager step {i}"}
             checks += 1
         sync()
         t0 = time.perf_counter()
@@ -582,7 +583,11 @@ def capture_and_replay_c4(z, st, args, sync):
             rt.hipGraphLaunch(ge, stream)
         sync()
         ms = (time.perf_counter() - t0) / args.steps * 1e3
-        return {"ms_per_step": round(ms, 4), "steps_per_s": round(1e3 / ms, 1), "replays_checked_bit_exact": checks}
+        nxt, left, refused = st.opt.schedule_state()
+        st.opt.drop_schedule()
+        return {"ms_per_step": round(ms, 4), "steps_per_s": round(1e3 / ms, 1), "consecutive_steps_checked_bit_exact": checks,
+                "adam_step": "advances on the device with every replay (scheduled update)", "steps_taken": nxt - 1,
+                "updates_refused": refused}
     except Exception as e:  # the eager figures above stand on their own
         return {"error": repr(e)}
 

@@ -351,6 +351,30 @@ int zenu_hip_adam_step_multi(int dtype, int n_tensors, void *const *p_dev, const
                              void *const *m_dev, void *const *v_dev, const int64_t *sizes, double lr,
                              double beta1, double beta2, double eps, double weight_decay,
                              const int32_t *apply_decay, double step, zenu_stream_t stream);
+/* The same update for callers that record it into a HIP graph.  `Adam::update` advances its step
+ * on every call (adam.rs:21-25) and forms 1-beta^step on the host; a recorded launch would replay
+ * one step's scalars for ever.  A schedule holds those scalars for steps first_step ..
+ * first_step + n_steps - 1 in device memory -- computed on the host in dtype with libm's powf /
+ * pow, exactly as the eager call computes them -- and a cursor, also in device memory, that every
+ * scheduled update advances (a one-thread launch after the update's own).  A recorded scheduled
+ * update is therefore the NEXT step on every replay, bit for bit what consecutive eager calls
+ * give.  An update asked for after the last step of the table changes nothing and is counted
+ * (`refused` of the query): create a new schedule from `next_step` before that happens.
+ * create / destroy / query block and may not be called while `stream` records a graph; the
+ * scheduled update never blocks and allocates nothing.  One device array per schedule
+ * (16 bytes + 2 elements per step).  No counterpart in the reference. */
+int zenu_hip_adam_schedule_create(void **schedule, int dtype, double beta1, double beta2,
+                                  int64_t first_step, int n_steps, zenu_stream_t stream);
+int zenu_hip_adam_schedule_destroy(void *schedule, zenu_stream_t stream);
+/* any of the three outputs may be NULL */
+int zenu_hip_adam_schedule_query(void *schedule, int64_t *next_step, int64_t *steps_left,
+                                 int64_t *refused, zenu_stream_t stream);
+/* zenu_hip_adam_step_multi with beta1, beta2 and the step taken from `schedule` */
+int zenu_hip_adam_step_multi_scheduled(int dtype, int n_tensors, void *const *p_dev,
+                                       const void *const *g_dev, void *const *m_dev,
+                                       void *const *v_dev, const int64_t *sizes, double lr, double eps,
+                                       double weight_decay, const int32_t *apply_decay, void *schedule,
+                                       zenu_stream_t stream);
 
 /* ------------------------------------------------------------------------- */
 /* Entry points with the reference's own names and argument order              */

@@ -148,6 +148,112 @@ def test_library_calls_in_a_captured_graph(hip):
         _lib.check(l.zenu_hip_stream_destroy(stream), "stream_destroy")
 
 
+def test_scheduled_adam_steps_through_graph_replays(hip):
+    """`Adam::update` advances its step on every call (adam.rs:21-25).  A recorded update whose step is a
+    kernel argument replays ONE step for ever; the scheduled update reads 1 - beta^t from a table in
+    device memory and advances a device cursor, so replay i of one recorded update is step i.  Five
+    consecutive eager AdamW steps with changing gradients, then the same five as replays of one graph:
+    parameters and both moments equal bit for bit after every step; past the end of the table an
+    update changes nothing and is counted."""
+    from zenu_amd import _lib
+    rt = _hip_runtime()
+    l = hip.lib()
+    M = hip.Matrix
+    stream = C.c_void_p()
+    _lib.check(l.zenu_hip_stream_create(C.byref(stream)), "stream_create")
+    old = hip.get_stream()
+    hip.set_stream(stream)
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    opt = None
+    try:
+        r = np.random.default_rng(77)
+        shapes = {"w1": (300, 257), "b1": (257,), "w2": (1 << 18,)}
+        p0 = {k: (r.standard_normal(s) * 0.02).astype(np.float32) for k, s in shapes.items()}
+        grads = [{k: (r.standard_normal(s) * (10.0 ** -i)).astype(np.float32) for k, s in shapes.items()} for i in range(9)]
+        P = {k: M.from_numpy(v) for k, v in p0.items()}
+        G = {k: M.alloc(s) for k, s in shapes.items()}
+        params = {k: (P[k], G[k]) for k in shapes}
+
+        def set_grads(i):
+            for k in shapes:
+                _lib.check(l.zenu_hip_memcpy_h2d(G[k].as_ptr(), grads[i][k].ctypes.data, grads[i][k].nbytes, stream), "h2d")
+
+        def snapshot(o):
+            hip.synchronize()
+            return [t.to_numpy().copy() for k in shapes for t in (P[k], o.m[k], o.v[k])]
+
+        eager = []
+        ref = hip.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, params, ["w1", "w2"])
+        for i in range(5):
+            set_grads(i)
+            ref.update(params)
+            eager.append(snapshot(ref))
+
+        for k in shapes:                                  # start again
+            _lib.check(l.zenu_hip_memcpy_h2d(P[k].as_ptr(), p0[k].ctypes.data, p0[k].nbytes, stream), "h2d")
+        opt = hip.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, params, ["w1", "w2"])
+        opt.use_schedule(8)
+        assert opt.schedule_state() == (1, 8, 0)
+        hip.synchronize()
+        assert rt.hipStreamBeginCapture(stream, 2) == 0
+        try:
+            opt.update(params)                            # recorded, not executed
+        finally:
+            rc = rt.hipStreamEndCapture(stream, C.byref(graph))
+        assert rc == 0
+        assert rt.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+        assert opt.schedule_state() == (1, 8, 0)          # recording advanced nothing
+        for i in range(5):
+            set_grads(i)
+            assert rt.hipGraphLaunch(gexec, stream) == 0
+            got = snapshot(opt)
+            for a, b in zip(got, eager[i]):
+                assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), ("replay", i)
+            (P["w1"] + P["w1"]).sum(0)                    # eager work between the replays
+        assert opt.schedule_state() == (6, 3, 0)
+        # an eager (not recorded) scheduled call is the next step as well
+        set_grads(5)
+        opt.update(params)                                # step 6 through the schedule
+        after6 = snapshot(opt)
+        names = list(shapes)
+        for j, k in enumerate(names):                     # the same step with the step number as a kernel argument
+            _lib.check(l.zenu_hip_memcpy_h2d(P[k].as_ptr(), eager[4][3 * j].ctypes.data, p0[k].nbytes, stream), "h2d")
+        ref2 = hip.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, params, ["w1", "w2"])
+        for j, k in enumerate(names):
+            _lib.check(l.zenu_hip_memcpy_h2d(ref2.m[k].as_ptr(), eager[4][3 * j + 1].ctypes.data, p0[k].nbytes, stream), "h2d")
+            _lib.check(l.zenu_hip_memcpy_h2d(ref2.v[k].as_ptr(), eager[4][3 * j + 2].ctypes.data, p0[k].nbytes, stream), "h2d")
+        ref2.step = 5
+        ref2.update(params)
+        for a, b in zip(after6, snapshot(ref2)):
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), "eager scheduled step 6"
+        for j, k in enumerate(names):                     # opt's parameters again
+            _lib.check(l.zenu_hip_memcpy_h2d(P[k].as_ptr(), after6[3 * j].ctypes.data, p0[k].nbytes, stream), "h2d")
+        # steps 7 and 8 exist; a ninth changes nothing and is counted
+        for i in (6, 7):
+            set_grads(i)
+            assert rt.hipGraphLaunch(gexec, stream) == 0
+        assert opt.schedule_state() == (9, 0, 0)
+        before = snapshot(opt)
+        set_grads(8)
+        assert rt.hipGraphLaunch(gexec, stream) == 0
+        for a, b in zip(snapshot(opt), before):
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+        assert opt.schedule_state() == (9, 0, 1)
+    finally:
+        hip.synchronize()
+        if gexec:
+            rt.hipGraphExecDestroy(gexec)
+        if graph:
+            rt.hipGraphDestroy(graph)
+        if opt is not None:
+            opt.drop_schedule()
+        hip.set_stream(old)
+        P = G = params = ref = ref2 = opt = None   # freed before their stream goes
+        import gc
+        gc.collect()
+        _lib.check(l.zenu_hip_stream_destroy(stream), "stream_destroy")
+
+
 _POOL_OFF_CAPTURE = r"""
 import ctypes as C, sys
 import numpy as np

@@ -102,6 +102,11 @@ SIGNATURES = {
     "zenu_hip_adamw_step": [_i, _vp, _vp, _vp, _vp, _i64, _d, _d, _d, _d, _d, _i, _d, _vp],
     "zenu_hip_adam_step_multi": [_i, _i, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
                                  C.POINTER(_i64), _d, _d, _d, _d, _d, C.POINTER(C.c_int32), _d, _vp],
+    "zenu_hip_adam_schedule_create": [C.POINTER(_vp), _i, _d, _d, _i64, _i, _vp],
+    "zenu_hip_adam_schedule_destroy": [_vp, _vp],
+    "zenu_hip_adam_schedule_query": [_vp, C.POINTER(_i64), C.POINTER(_i64), C.POINTER(_i64), _vp],
+    "zenu_hip_adam_step_multi_scheduled": [_i, _i, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
+                                           C.POINTER(_i64), _d, _d, _d, C.POINTER(C.c_int32), _vp, _vp],
 }
 
 _BIN = ("add", "sub", "mul", "div")

@@ -16,6 +16,8 @@
 // 1-b, b^t and 1-b^t are formed on the host in T, as adam.rs:22-25,45-51 does.
 #include <math.h>
 
+#include <vector>
+
 #include "common.hpp"
 #include "vecmem.hpp"
 
@@ -140,9 +142,40 @@ struct MultiArgs {
     int32_t count;
 };
 
-template <typename T, int VEC>
-__global__ __launch_bounds__(kBlock) void adam_multi_kernel(MultiArgs a, AdamConsts<T> k)
+// The step-dependent scalars of a scheduled update: 1 - beta1^t and 1 - beta2^t for consecutive
+// steps t, formed on the host in T exactly as an eager call forms them, and a cursor on the device
+// that says which pair the next update uses.  A launch recorded into a graph carries the schedule's
+// address, not a step number, so every replay is the next step.
+struct ScheduleHeader {
+    uint32_t cursor;      // index of the pair the next update uses
+    uint32_t n;           // pairs in the table
+    uint32_t exhausted;   // updates that were asked for after the last pair (they change nothing)
+    uint32_t pad;
+};
+
+template <typename T>
+__device__ __forceinline__ bool schedule_consts(const ScheduleHeader *h, AdamConsts<T> &k)
 {
+    if (!h) return true;
+    const uint32_t i = h->cursor;
+    if (i >= h->n) return false;
+    const T *table = reinterpret_cast<const T *>(h + 1);
+    k.c1 = table[2 * i];
+    k.c2 = table[2 * i + 1];
+    return true;
+}
+
+// after every launch of one scheduled update: move on to the next step
+__global__ void schedule_advance_kernel(ScheduleHeader *h)
+{
+    if (h->cursor < h->n) h->cursor = h->cursor + 1;
+    else h->exhausted = h->exhausted + 1;
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void adam_multi_kernel(MultiArgs a, AdamConsts<T> k, const ScheduleHeader *sched)
+{
+    if (!schedule_consts<T>(sched, k)) return;
     int t = 0;
     while (t + 1 < a.count && (int)blockIdx.x >= a.first_block[t + 1]) t++;
     const MultiEntry &e = a.e[t];
@@ -295,7 +328,8 @@ int adam_t(void *p, const void *g, void *m, void *v, int64_t n, const AdamConsts
 
 template <typename T>
 int adam_multi_t(int nt, void *const *p, const void *const *g, void *const *m, void *const *v,
-                 const int64_t *sizes, const AdamConsts<T> &k, const int32_t *decay, hipStream_t s)
+                 const int64_t *sizes, const AdamConsts<T> &k, const int32_t *decay, hipStream_t s,
+                 ScheduleHeader *sched = nullptr)
 {
     constexpr int VEC = VecOf<T>::N;
     constexpr int64_t kTile = (int64_t)kBlock * VEC * kUnroll;
@@ -330,7 +364,11 @@ int adam_multi_t(int nt, void *const *p, const void *const *g, void *const *m, v
         }
         if (a.count == 0) break;
         a.first_block[a.count] = (int32_t)blocks;
-        adam_multi_kernel<T, VEC><<<(unsigned)blocks, kBlock, 0, s>>>(a, k);
+        adam_multi_kernel<T, VEC><<<(unsigned)blocks, kBlock, 0, s>>>(a, k, sched);
+        ZENU_LAUNCH_CHECK();
+    }
+    if (sched) {
+        schedule_advance_kernel<<<1, 1, 0, s>>>(sched);
         ZENU_LAUNCH_CHECK();
     }
     return ZENU_OK;
@@ -473,6 +511,111 @@ int zenu_hip_adam_step_multi(int dtype, int n_tensors, void *const *p_dev, const
                                     make_consts<double>(lr, beta1, beta2, eps, weight_decay, step),
                                     apply_decay, as_stream(stream));
     return ZENU_ERR_ARG;
+}
+
+// host side of a schedule (the handle the C ABI passes around)
+struct AdamScheduleHost {
+    ScheduleHeader *dev;
+    int dtype;
+    double beta1, beta2;
+    int64_t first_step;
+    int n_steps;
+};
+
+int zenu_hip_adam_schedule_create(void **schedule, int dtype, double beta1, double beta2, int64_t first_step,
+                                  int n_steps, zenu_stream_t stream)
+{
+    if (!schedule || first_step < 1 || n_steps < 1 || n_steps > (1 << 24)) return ZENU_ERR_ARG;
+    if (dtype != ZENU_F32 && dtype != ZENU_F64) return ZENU_ERR_ARG;
+    int rc = ensure_init();
+    if (rc) return rc;
+    hipStream_t s = as_stream(stream);
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (s && hipStreamIsCapturing(s, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone) return ZENU_ERR_UNSUPPORTED;
+    const size_t esz = dtype == ZENU_F32 ? 4 : 8;
+    const size_t bytes = sizeof(ScheduleHeader) + (size_t)n_steps * 2 * esz;
+    std::vector<unsigned char> host(bytes);
+    ScheduleHeader *h = reinterpret_cast<ScheduleHeader *>(host.data());
+    h->cursor = 0;
+    h->n = (uint32_t)n_steps;
+    h->exhausted = 0;
+    h->pad = 0;
+    for (int i = 0; i < n_steps; i++) {
+        const double step = (double)(first_step + i);
+        if (dtype == ZENU_F32) {
+            const AdamConsts<float> k = make_consts<float>(0, beta1, beta2, 0, 0, step);
+            float *t = reinterpret_cast<float *>(h + 1);
+            t[2 * i] = k.c1;
+            t[2 * i + 1] = k.c2;
+        } else {
+            const AdamConsts<double> k = make_consts<double>(0, beta1, beta2, 0, 0, step);
+            double *t = reinterpret_cast<double *>(h + 1);
+            t[2 * i] = k.c1;
+            t[2 * i + 1] = k.c2;
+        }
+    }
+    void *dev = nullptr;
+    rc = zenu_hip_raw_malloc(&dev, bytes);
+    if (rc) return rc;
+    rc = zenu_hip_memcpy_h2d(dev, host.data(), bytes, stream);   // blocking: `host` may go
+    if (rc) {
+        (void)zenu_hip_raw_free(dev);
+        return rc;
+    }
+    AdamScheduleHost *hs = new AdamScheduleHost;
+    hs->dev = static_cast<ScheduleHeader *>(dev);
+    hs->dtype = dtype;
+    hs->beta1 = beta1;
+    hs->beta2 = beta2;
+    hs->first_step = first_step;
+    hs->n_steps = n_steps;
+    *schedule = hs;
+    return ZENU_OK;
+}
+
+int zenu_hip_adam_schedule_destroy(void *schedule, zenu_stream_t stream)
+{
+    if (!schedule) return ZENU_OK;
+    AdamScheduleHost *hs = static_cast<AdamScheduleHost *>(schedule);
+    ZENU_HIP_TRY(hipStreamSynchronize(as_stream(stream)));   // the updates that read it are done
+    int rc = zenu_hip_raw_free(hs->dev);
+    delete hs;
+    return rc;
+}
+
+int zenu_hip_adam_schedule_query(void *schedule, int64_t *next_step, int64_t *steps_left, int64_t *refused,
+                                 zenu_stream_t stream)
+{
+    if (!schedule) return ZENU_ERR_ARG;
+    AdamScheduleHost *hs = static_cast<AdamScheduleHost *>(schedule);
+    ScheduleHeader h;
+    int rc = zenu_hip_memcpy_d2h(&h, hs->dev, sizeof h, stream);   // blocking
+    if (rc) return rc;
+    if (next_step) *next_step = hs->first_step + h.cursor;
+    if (steps_left) *steps_left = (int64_t)h.n - h.cursor;
+    if (refused) *refused = h.exhausted;
+    return ZENU_OK;
+}
+
+int zenu_hip_adam_step_multi_scheduled(int dtype, int n_tensors, void *const *p_dev, const void *const *g_dev,
+                                       void *const *m_dev, void *const *v_dev, const int64_t *sizes, double lr,
+                                       double eps, double weight_decay, const int32_t *apply_decay,
+                                       void *schedule, zenu_stream_t stream)
+{
+    if (n_tensors < 0 || !schedule) return ZENU_ERR_ARG;
+    AdamScheduleHost *hs = static_cast<AdamScheduleHost *>(schedule);
+    if (hs->dtype != dtype) return ZENU_ERR_ARG;
+    if (n_tensors > 0 && (!p_dev || !g_dev || !m_dev || !v_dev || !sizes)) return ZENU_ERR_ARG;
+    int rc = ensure_init();
+    if (rc) return rc;
+    // the step-dependent scalars come from the table; everything else as in the eager call
+    if (dtype == ZENU_F32)
+        return adam_multi_t<float>(n_tensors, p_dev, g_dev, m_dev, v_dev, sizes,
+                                   make_consts<float>(lr, hs->beta1, hs->beta2, eps, weight_decay, 1.0),
+                                   apply_decay, as_stream(stream), hs->dev);
+    return adam_multi_t<double>(n_tensors, p_dev, g_dev, m_dev, v_dev, sizes,
+                                make_consts<double>(lr, hs->beta1, hs->beta2, eps, weight_decay, 1.0),
+                                apply_decay, as_stream(stream), hs->dev);
 }
 
 }  // extern "C"

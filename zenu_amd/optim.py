@@ -57,6 +57,36 @@ class _AdamBase:
         # zeros_like per parameter (adam.rs:62-88)
         self.m = {k: Matrix.zeros(p.shape, p.dtype) for k, (p, _) in parameters.items()}
         self.v = {k: Matrix.zeros(p.shape, p.dtype) for k, (p, _) in parameters.items()}
+        self._schedule = None
+
+    def use_schedule(self, n_steps, dtype=np.float32):
+        """Take the step-dependent scalars of the next `n_steps` updates from a table in device memory
+        whose cursor every update advances, so that an `update` recorded into a HIP graph is the next
+        step on every replay (no counterpart in the reference, which never records graphs)."""
+        self.drop_schedule()
+        h = C.c_void_p()
+        check(_lib.lib().zenu_hip_adam_schedule_create(C.byref(h), _dt(dtype), float(self.beta1), float(self.beta2),
+                                                       self.step + 1, int(n_steps), get_stream()), "adam_schedule_create")
+        self._schedule = h
+        self._schedule_dtype = np.dtype(dtype)
+
+    def drop_schedule(self):
+        if self._schedule is not None:
+            check(_lib.lib().zenu_hip_adam_schedule_destroy(self._schedule, get_stream()), "adam_schedule_destroy")
+            self._schedule = None
+
+    def schedule_state(self):
+        """(next step, steps left in the table, updates refused because the table had run out)"""
+        a, b, c = C.c_int64(), C.c_int64(), C.c_int64()
+        check(_lib.lib().zenu_hip_adam_schedule_query(self._schedule, C.byref(a), C.byref(b), C.byref(c), get_stream()),
+              "adam_schedule_query")
+        return a.value, b.value, c.value
+
+    def __del__(self):
+        try:
+            self.drop_schedule()
+        except Exception:
+            pass
 
     def _update(self, parameters, weight_decay, weight_keys, multi):
         self.step += 1
@@ -76,11 +106,20 @@ class _AdamBase:
                 M[i] = _flat(self.m[k])[0]
                 V[i] = _flat(self.v[k])[0]
                 decay[i] = 1 if (weight_keys is not None and k in weight_keys) else 0
+            if self._schedule is not None:
+                if np.dtype(dtype) != self._schedule_dtype:
+                    raise ValueError("the schedule was made for another dtype")
+                check(_lib.lib().zenu_hip_adam_step_multi_scheduled(
+                    _dt(dtype), n, P, G, M, V, sizes, float(self.learning_rate), float(self.epsilon),
+                    float(weight_decay), decay, self._schedule, get_stream()), "adam_step_multi_scheduled")
+                return
             check(_lib.lib().zenu_hip_adam_step_multi(
                 _dt(dtype), n, P, G, M, V, sizes, float(self.learning_rate), float(self.beta1),
                 float(self.beta2), float(self.epsilon), float(weight_decay), decay, float(self.step),
                 get_stream()), "adam_step_multi")
             return
+        if self._schedule is not None:
+            raise ValueError("a scheduled update takes the multi-tensor path: one dtype, multi_tensor=True")
         for k, d, g in items:
             p, n = _flat(d)
             decay = 1 if (weight_keys is not None and k in weight_keys) else 0
