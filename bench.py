@@ -63,6 +63,46 @@ class Hip:
         return ms.value
 
 
+class ClockProbe:
+    """The shader clock right after a batch of launches (harness/native/clock_probe.hip: a chain of
+    dependent multiply-adds run by one wavefront between the shader-clock counter and the 100 MHz
+    constant-rate counter).  None-valued when the helper library is not built."""
+
+    def __init__(self, z, slots=4):
+        self.lib = None
+        path = os.path.join(ROOT, "harness", "native", "bin", "libclock_probe.so")
+        if not os.path.exists(path):
+            return
+        try:
+            lib = C.CDLL(path)
+            lib.clock_probe_launch.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
+            self.wall_khz = lib.clock_probe_wall_rate_khz()
+            self.buf = C.c_void_p()
+            if z.lib().zenu_hip_raw_malloc(C.byref(self.buf), 32 * slots) != 0 or self.wall_khz <= 0:
+                return
+            self.z, self.lib = z, lib
+        except OSError:
+            self.lib = None
+
+    def sample(self, slot, stream):
+        """queue one sample (about 15 us of one wavefront) on `stream`"""
+        if self.lib is not None:
+            self.lib.clock_probe_launch(C.c_void_p(self.buf.value + 32 * slot), 300, stream)
+
+    def read_mhz(self, n, stream):
+        """shader clock in MHz for slots 0..n-1 (after their stream work has finished), or None"""
+        if self.lib is None:
+            return None
+        host = (C.c_uint64 * (4 * n))()
+        if self.z.lib().zenu_hip_memcpy_d2h(host, self.buf, 32 * n, stream) != 0:
+            return None
+        out = []
+        for i in range(n):
+            c, w = host[4 * i], host[4 * i + 1]
+            out.append(round(c / w * self.wall_khz / 1e3, 0) if w else None)
+        return out
+
+
 class Op:
     """one op of the step: a list of pre-bound launch closures, one per rotating buffer set"""
 
@@ -642,6 +682,68 @@ def roofline_of(row, op):
                 avg_launch_us=row["us"])
 
 
+def time_ops(ops, args, hip, stream, sync, probe, bracketed=True):
+    """Per-op timing with HIP events on the launch stream.
+    Three batches of op_reps back-to-back launches, one event pair around each; `us` is the median
+    of the three batch means (kernels bound by their vector instructions follow the clock, which the
+    power management moves by +-10 % from one millisecond to the next; `us_batches` keeps all three,
+    `shader_mhz_batches` the clock sampled right after each batch) and agrees with the kernel durations
+    of a rocprofv3 trace; a second pass brackets every launch with its own events for a median and a
+    minimum, which include the cost of one event record (~2.5 us)."""
+    e0, e1 = hip.event(), hip.event()
+    marks = [hip.event() for _ in range(args.op_reps + 1)] if bracketed else []
+    table = []
+    for o in ops:
+        for _ in range(10):
+            o.launch()
+        sync()
+        batches = []
+        for b in range(3):
+            hip.record(e0, stream)
+            for _ in range(args.op_reps):
+                o.launch()
+            hip.record(e1, stream)
+            probe.sample(b, stream)
+            batches.append(hip.elapsed_ms(e0, e1) / args.op_reps * 1e3)
+        mhz = probe.read_mhz(3, stream)
+        us = sorted(batches)[1]
+        gbps = o.alg_bytes / (us * 1e-6) / 1e9
+        row = dict(op=o.name, config=o.config, dtype=o.dtype, us=round(us, 2), GBps=round(gbps, 1),
+                   frac_of_peak=round(gbps / PEAK_HBM_GBPS, 4), Gelem_per_s=round(o.elems / (us * 1e-6) / 1e9, 2),
+                   alg_bytes=o.alg_bytes, us_batches=[round(b, 2) for b in batches], shader_mhz_batches=mhz)
+        if bracketed:
+            hip.record(marks[0], stream)
+            for i in range(args.op_reps):
+                o.launch()
+                hip.record(marks[i + 1], stream)
+            each = sorted(hip.elapsed_ms(marks[i], marks[i + 1]) * 1e3 for i in range(args.op_reps))
+            row.update(us_bracketed_median=round(each[len(each) // 2], 2), us_bracketed_min=round(each[0], 2))
+        table.append(row)
+        log(f"[op] {o.name:22s} {us:9.2f} us  {gbps:8.1f} GB/s  {100 * gbps / PEAK_HBM_GBPS:5.1f}% of peak  clock {mhz}")
+    return table
+
+
+def extra_rows(z, workload, args, hip, stream, sync, probe):
+    """the rows that come after the BASELINE configs, compact, for the default line: op -> [us, % of peak,
+    shader MHz of the median batch]; never `value`, never `roofline`, no CPU leg"""
+    try:
+        t0 = time.time()
+        ops = build_ops(z, workload, stream)
+        sync()
+        rows = time_ops(ops, args, hip, stream, sync, probe, bracketed=False)
+        out = {}
+        for r in rows:
+            mid = sorted(range(3), key=lambda i: r["us_batches"][i])[1]
+            mhz = r["shader_mhz_batches"][mid] if r["shader_mhz_batches"] else None
+            out[r["op"]] = [r["us"], round(100 * r["frac_of_peak"], 1), mhz]
+        del ops
+        log(f"[{workload}] {len(out)} ops measured in {time.time() - t0:.1f} s")
+        return {"columns": ["us per launch (median of 3 batches)", "% of the 8 TB/s HBM peak by algorithmic bytes",
+                            "shader clock in MHz right after that batch"], "ops": out}
+    except Exception as e:      # the configs[0..3] figures stand on their own
+        return {"error": repr(e)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -670,6 +772,7 @@ def main():
 
     if args.workload == "c4":
         return run_c4(z, args, sync)
+    probe = ClockProbe(z)
 
     t0 = time.time()
     ops = build_ops(z, args.workload, stream)
@@ -699,38 +802,7 @@ def main():
     ms_per_step = elapsed / args.steps * 1e3
     value = step_bytes / (elapsed / args.steps) / 1e9
 
-    # ---- per-op timing with HIP events on the launch stream ---------------------------------------------
-    # Three batches of op_reps back-to-back launches, one event pair around each; `us` is the median
-    # of the three batch means (kernels bound by their vector instructions follow the clock, which the
-    # power management moves by +-10 % from one millisecond to the next; `us_batches` keeps all three)
-    # and agrees with the kernel durations of a rocprofv3 trace; a second pass brackets every launch with its
-    # own events for a median and a minimum, which include the cost of one event record (~2.5 us)
-    e0, e1 = hip.event(), hip.event()
-    marks = [hip.event() for _ in range(args.op_reps + 1)]
-    table = []
-    for o in ops:
-        for _ in range(10):
-            o.launch()
-        sync()
-        batches = []
-        for _ in range(3):
-            hip.record(e0, stream)
-            for _ in range(args.op_reps):
-                o.launch()
-            hip.record(e1, stream)
-            batches.append(hip.elapsed_ms(e0, e1) / args.op_reps * 1e3)
-        us = sorted(batches)[1]
-        hip.record(marks[0], stream)
-        for i in range(args.op_reps):
-            o.launch()
-            hip.record(marks[i + 1], stream)
-        each = sorted(hip.elapsed_ms(marks[i], marks[i + 1]) * 1e3 for i in range(args.op_reps))
-        gbps = o.alg_bytes / (us * 1e-6) / 1e9
-        table.append(dict(op=o.name, config=o.config, dtype=o.dtype, us=round(us, 2), GBps=round(gbps, 1),
-                          frac_of_peak=round(gbps / PEAK_HBM_GBPS, 4), Gelem_per_s=round(o.elems / (us * 1e-6) / 1e9, 2),
-                          alg_bytes=o.alg_bytes, us_batches=[round(b, 2) for b in batches],
-                          us_bracketed_median=round(each[len(each) // 2], 2), us_bracketed_min=round(each[0], 2)))
-        log(f"[op] {o.name:22s} {us:9.2f} us  {gbps:8.1f} GB/s  {100 * gbps / PEAK_HBM_GBPS:5.1f}% of peak")
+    table = time_ops(ops, args, hip, stream, sync, probe)
 
     # dominant kernel of the step = the op with the largest share of the step time
     by_time = sorted(table, key=lambda t: -t["us"])
@@ -770,6 +842,13 @@ def main():
         log(f"[c4] MLP step measured in {time.time() - t0:.1f} s: "
             f"{c4.get('eager_compiled_host_ms_per_step')} ms eager, {c4.get('fused_compiled_host_ms_per_step')} ms fused")
 
+    # ---- the rows after the BASELINE configs: compact objects on the default line ---------------------------
+    nxt = fused = None
+    if args.workload == "suite" and not args.no_c4:
+        del ops
+        nxt = extra_rows(z, "next", args, hip, stream, sync, probe)
+        fused = extra_rows(z, "fused", args, hip, stream, sync, probe)
+
     out = {
         "metric": "achieved HBM GB/s (% of MI355X peak) per op; Adam step params/sec",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -784,9 +863,10 @@ def main():
                    "ops_per_step": len(table), "algorithmic_bytes_per_step": step_bytes},
         "frac_of_peak_whole_step": round(value / PEAK_HBM_GBPS, 4),
         "adam_step_params_per_sec": (round(adam[0]["Gelem_per_s"] * 1e9) if adam else None),
-        "roofline": roofline, "roofline_second_largest_op": roofline_second, "cpu_baseline": cpu, "c4": c4, "ops": table,
+        "roofline": roofline, "roofline_second_largest_op": roofline_second, "cpu_baseline": cpu, "c4": c4, "next": nxt, "fused": fused, "ops": table,
         "timing": f"HIP events on the launch stream; per op 3 batches of {args.op_reps} back-to-back launches after 10 warm-up launches: "
-                  "us = median of the 3 batch means (us_batches), us_bracketed_* = per-launch event pairs (each includes one event record)",
+                  "us = median of the 3 batch means (us_batches), us_bracketed_* = per-launch event pairs (each includes one event record); "
+                  "shader_mhz_batches = the shader clock sampled by a one-wavefront kernel right after each batch",
     }
     print(json.dumps(out))
 
