@@ -16,7 +16,8 @@ Op sequence followed (reference file:line):
   Adam::update                                                          zenu-optimizer/src/adam.rs:19-59
 
 With fused=True the same step uses the fused entry points (bias add + ReLU, softmax cross-entropy
-forward and backward, ReLU backward): 37 launches instead of 62 on the HIP device.  On the CPU
+forward and backward, ReLU backward, the two backward calls also producing the bias gradients): 30
+launches instead of 62 on the HIP device.  On the CPU
 device those names are the op-by-op chains, so both settings compute the same thing there.
 
 GEMM stays on the library path (`dev.gemm`): numpy/OpenBLAS for the CPU leg, rocBLAS for the HIP
@@ -88,12 +89,14 @@ class MlpStep:
         Wt2, a2, h2 = self._linear_relu_fwd(2, h1)
         Wt3, logits = self._linear_fwd(3, h2)
         loss, s = dev.F.cross_entropy(logits, self.t); tick("reduction")
-        g = dev.F.cross_entropy_backward(s, self.t, self.one); tick("reduction")
+        # each bias gradient comes out of the launch that produces the gradient it sums (no zero fill:
+        # it is overwritten)
+        gb = M.alloc([LAYERS[2][1]], dt)
+        g = dev.F.cross_entropy_backward_bias_grad(s, self.t, gb, self.one); tick("reduction")
         grads = {}
         acts = [(self.x, Wt1, a1), (h1, Wt2, a2), (h2, Wt3, None)]
         for i in (3, 2, 1):
             inp, Wt, _ = acts[i - 1]
-            gb = M.zeros([LAYERS[i - 1][1]], dt); dev.sum_to(g, gb); tick("reduction")
             grads[f"linear{i}.bias"] = gb
             inpT = inp.transpose().to_default_stride(); tick("copy")
             gWt = dev.gemm(inpT, g); tick("gemm")
@@ -101,7 +104,8 @@ class MlpStep:
             if i > 1:
                 WtT = Wt.transpose().to_default_stride(); tick("copy")
                 g_h = dev.gemm(g, WtT); tick("gemm")
-                g = g_h.alloc_like(); g.relu_backward(g_h, acts[i - 2][2], 0.0); tick("elementwise")
+                g = g_h.alloc_like(); gb = M.alloc([LAYERS[i - 2][1]], dt)
+                g.relu_backward_bias_grad(gb, g_h, acts[i - 2][2], 0.0); tick("elementwise")
         self.opt.update({k: (self.p[k], grads[k]) for k in self.p}); tick("update")
         return loss, grads
 

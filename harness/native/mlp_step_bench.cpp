@@ -88,11 +88,18 @@ struct Step {
         opt = new Adam<float>(1e-3f, 0.9f, 0.999f, 1e-8f, p);
     }
 
-    void backward_linears(M g, const M acts_in[3], const M Wt[3], const M pre[3], bool fused)
+    // `gb_in`: the bias gradient of the last layer when the caller's fused call has already produced it
+    void backward_linears(M g, const M acts_in[3], const M Wt[3], const M pre[3], bool fused, M gb_in = M())
     {
+        M gb_next = gb_in;
         for (int i = 2; i >= 0; i--) {
-            M gb = M::zeros({kLayers[i][1]});
-            g.sum_to(gb);                                               // bias gradient
+            M gb;
+            if (fused) {
+                gb = gb_next;                                           // came with the gradient, same launch
+            } else {
+                gb = M::zeros({kLayers[i][1]});
+                g.sum_to(gb);                                           // bias gradient
+            }
             M inT = acts_in[i].transpose().to_default_stride();
             M gWt = gemm(inT, g);                                       // dW^T = X^T dY
             p[wk[i]] = ParamGrad<float>(p[wk[i]].data, gWt.transpose().to_default_stride());
@@ -102,7 +109,8 @@ struct Step {
                 M gh = gemm(g, WtT);                                    // dX = dY W
                 if (fused) {
                     M gn = gh.alloc_like();
-                    gn.relu_backward(gh, pre[i - 1], 0.f);
+                    gb_next = M::alloc({kLayers[i - 1][1]});
+                    gn.relu_backward_bias_grad(gb_next, gh, pre[i - 1], 0.f);
                     g = gn;
                 } else {
                     M mask = pre[i - 1].alloc_like();
@@ -134,11 +142,10 @@ struct Step {
         }
         auto lp = cross_entropy(logits, t);
         loss = lp.first;
-        M g = cross_entropy_backward(lp.second, t, &one);
+        M gb = M::alloc({kLayers[2][1]});
+        M g = cross_entropy_backward_bias_grad(lp.second, t, gb, &one);
         for (int i = 2; i >= 0; i--) {
             const int in = kLayers[i][0], out = kLayers[i][1];
-            M gb = M::alloc({out});
-            g.sum_to(gb);
             M gW = gemm_rm(true, false, out, in, kBatch, g, out, act_in[i], in);        // dY^T X, already [out, in]
             M w = p[wk[i]].data;
             p[wk[i]] = ParamGrad<float>(w, gW);
@@ -146,7 +153,8 @@ struct Step {
             if (i > 0) {
                 M gh = gemm_rm(false, false, kBatch, in, out, g, out, w, in);           // dY W
                 M gn = gh.alloc_like();
-                gn.relu_backward(gh, pre[i - 1], 0.f);
+                gb = M::alloc({in});
+                gn.relu_backward_bias_grad(gb, gh, pre[i - 1], 0.f);
                 g = gn;
             }
         }
@@ -178,11 +186,12 @@ struct Step {
                 h = a;
             }
         }
-        M g;
+        M g, gb_last;
         if (fused) {
             auto lp = cross_entropy(logits, t);
             loss = lp.first;
-            g = cross_entropy_backward(lp.second, t, &one);
+            gb_last = M::alloc({kLayers[2][1]});
+            g = cross_entropy_backward_bias_grad(lp.second, t, gb_last, &one);
         } else {
             M diff = logits - logits.max_axis(1, true);                 // softmax_assign
             M e = diff.exp();
@@ -200,7 +209,7 @@ struct Step {
             M gx = s * g_s;
             g = gx - s * gx.sum(1, true);
         }
-        backward_linears(g, act_in, Wt, pre, fused);
+        backward_linears(g, act_in, Wt, pre, fused, gb_last);
     }
 };
 

@@ -321,6 +321,27 @@ int zenu_hip_softmax_cross_entropy_backward(int dtype, const zenu_tensor_t *gpre
 int zenu_hip_bias_add_relu(int dtype, const zenu_tensor_t *pre, const zenu_tensor_t *act,
                            const zenu_tensor_t *z, const zenu_tensor_t *bias, double alpha,
                            zenu_stream_t stream);
+/* The backward pass of a Linear layer needs the gradient of its output and that gradient's column
+ * sums (the bias gradient: zenu-layer/src/layers/linear.rs:27-31 through the `sum_to` of
+ * zenu-autograd/src/lib.rs:466-486).  Both in one pass over the incoming gradient:
+ *   gx = gy * relu'(x)   (zenu_hip_relu_backward),   gbias[j] = sum over every leading index of gx[.., j]
+ * gx, gy, x have the same shape [.., N]; gbias holds N elements ([N], [1, N], ..).  One launch (the
+ * column-reduction kernel with the ReLU gradient applied to its loads) when the tensors are whole,
+ * 16-byte aligned and N is a multiple of the vector width and at least 16; otherwise the two calls it
+ * stands for.  gx is bit-identical to zenu_hip_relu_backward's and, for a 2-d gradient, gbias to
+ * zenu_hip_sum_to(gbias, gx).
+ * No counterpart in the reference (two autograd nodes there). */
+int zenu_hip_relu_backward_bias_grad(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *gbias,
+                                     const zenu_tensor_t *gy, const zenu_tensor_t *x, double alpha,
+                                     zenu_stream_t stream);
+/* zenu_hip_softmax_cross_entropy_backward that also writes the column sums of gpred to gbias (the bias
+ * gradient of the layer that produced the logits).  One launch for a classifier head (at most 256
+ * rows, at most 16 classes; each column folded over the rows in a fixed order), otherwise the two
+ * calls it stands for.  No counterpart in the reference. */
+int zenu_hip_softmax_cross_entropy_backward_bias_grad(int dtype, const zenu_tensor_t *gpred,
+                                                      const zenu_tensor_t *gbias, const zenu_tensor_t *prob,
+                                                      const zenu_tensor_t *ans, const zenu_tensor_t *gloss,
+                                                      zenu_stream_t stream);
 
 /* ------------------------------------------------------------------------- */
 /* Fused optimizer updates (one launch, 4 loads + 3 stores per element)        */

@@ -390,6 +390,12 @@ public:
         zenu_tensor_t t = desc(), g = gy.desc(), xx = x.desc();
         check(zenu_hip_relu_backward(dt(), &t, &g, &xx, (double)alpha, st()), "relu_backward");
     }
+    // *this = gy * relu'(x) and gbias = its column sums (the bias gradient of the layer before), one pass
+    void relu_backward_bias_grad(const Matrix &gbias, const Matrix &gy, const Matrix &x, T alpha) const
+    {
+        zenu_tensor_t t = desc(), b = gbias.desc(), g = gy.desc(), xx = x.desc();
+        check(zenu_hip_relu_backward_bias_grad(dt(), &t, &b, &g, &xx, (double)alpha, st()), "relu_backward_bias_grad");
+    }
     void tanh_backward(const Matrix &gy, const Matrix &x) const      // functions/tanh.rs:30-37
     {
         zenu_tensor_t t = desc(), g = gy.desc(), xx = x.desc();
@@ -562,6 +568,21 @@ Matrix<T> cross_entropy_backward(const Matrix<T> &prob, const Matrix<T> &ans, co
     if (gloss) gl = gloss->desc();
     check(zenu_hip_softmax_cross_entropy_backward(DType<T>::value, &gd, &p, &a, gloss ? &gl : nullptr, current_stream()),
           "cross_entropy_backward");
+    return g;
+}
+
+// cross_entropy_backward that also writes the column sums of the gradient (the bias gradient of the
+// layer that produced the logits) to gbias
+template <typename T>
+Matrix<T> cross_entropy_backward_bias_grad(const Matrix<T> &prob, const Matrix<T> &ans, const Matrix<T> &gbias,
+                                           const Matrix<T> *gloss = nullptr)
+{
+    Matrix<T> g = prob.alloc_like();
+    zenu_tensor_t gd = g.desc(), b = gbias.desc(), p = prob.desc(), a = ans.desc(), gl;
+    if (gloss) gl = gloss->desc();
+    check(zenu_hip_softmax_cross_entropy_backward_bias_grad(DType<T>::value, &gd, &b, &p, &a, gloss ? &gl : nullptr,
+                                                            current_stream()),
+          "cross_entropy_backward_bias_grad");
     return g;
 }
 

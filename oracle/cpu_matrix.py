@@ -146,6 +146,12 @@ class CpuMatrix:
         mask.relu_backward_mask(x, alpha)
         self.mul_array(gy, mask)
 
+    def relu_backward_bias_grad(self, gbias, gy, x, alpha):
+        """the two nodes the fused call stands for: relu backward, then the bias gradient's sum_to
+        (zenu-autograd/src/lib.rs:466-486)"""
+        self.relu_backward(gy, x, alpha)
+        sum_to(self, gbias)
+
     # clip.rs:289-318
     def clip(self, lo, hi):
         out = self.alloc_like()
@@ -293,6 +299,13 @@ def cross_entropy(pred, ans):
     sum_to(y_log_pred, total)
     neg_n = CpuMatrix.from_vec([-float(pred.shape[0])], (), pred.dtype)
     return total / neg_n, prob
+
+
+def cross_entropy_backward_bias_grad(prob, ans, gbias, gloss=None):
+    """cross_entropy_backward, then the bias gradient's sum_to"""
+    g = cross_entropy_backward(prob, ans, gloss)
+    sum_to(g, gbias)
+    return g
 
 
 def cross_entropy_backward(prob, ans, gloss=None):

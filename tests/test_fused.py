@@ -399,3 +399,127 @@ def test_tanh_and_sigmoid_backward(hip):
     assert bits_equal(ho.to_numpy(), co.a)
     with pytest.raises(hip.ZenuHipError):
         ho.tanh_backward(hg, hip.Matrix.zeros((64, 96)))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("shape", [(256, 512), (256, 10), (1000, 130), (3, 40, 64), (8192, 4096), (64, 18), (5000, 16)])
+@pytest.mark.parametrize("alpha", [0.0, 0.2])
+def test_relu_backward_bias_grad(hip, dtype, shape, alpha):
+    """gx and the bias gradient in one pass: gx is the bits of relu_backward (and of the oracle's mask
+    chain), the bias gradient the bits of sum_to over that gx when the gradient is 2-d (same kernel,
+    same geometry) and within the bar of every sum against the oracle and the exact f64 sums; shapes
+    on both sides of the one-launch conditions (column count below 16 or no multiple of the vector
+    width, more than two dims)."""
+    print(f"[case] relu_backward_bias_grad {shape} {np.dtype(dtype).name} alpha {alpha}", flush=True)
+    r = np.random.default_rng(shape[0] + 7 * shape[-1])
+    x = r.standard_normal(shape).astype(dtype)
+    x.reshape(-1)[::13] = 0.0
+    x.reshape(-1)[3::31] = -0.0
+    gy = r.standard_normal(shape).astype(dtype)
+    n = shape[-1]
+    M = hip.Matrix
+    X, GY = M.from_numpy(x), M.from_numpy(gy)
+    gx, gb = M.alloc(shape, dtype), M.from_numpy(np.full(n, 77.0, dtype=dtype))
+    gx.relu_backward_bias_grad(gb, GY, X, alpha)
+    gx2 = M.alloc(shape, dtype)
+    gx2.relu_backward(GY, X, alpha)
+    assert bits_equal(gx.to_numpy(), gx2.to_numpy())
+    gref, gbref = CpuMatrix.zeros(shape, dtype), CpuMatrix.zeros((n,), dtype)
+    gref.relu_backward_bias_grad(gbref, CpuMatrix.from_numpy(gy), CpuMatrix.from_numpy(x), alpha)
+    assert bits_equal(gx.to_numpy(), gref.a)
+    if len(shape) == 2:
+        gb2 = M.alloc((n,), dtype)
+        hip.sum_to(gx2, gb2)
+        assert bits_equal(gb.to_numpy(), gb2.to_numpy())
+    g64 = gref.a.astype(np.float64).reshape(-1, n)
+    exact = g64.sum(0)
+    scale = np.maximum(np.abs(exact), np.abs(g64).sum(0) / np.sqrt(g64.shape[0]))
+    tol = 1e-5 if dtype == np.float32 else 1e-12
+    assert np.all(np.abs(gb.to_numpy() - exact) <= tol * scale)
+    assert np.all(np.abs(gb.to_numpy() - gbref.a) <= 2 * tol * scale)
+    # twice in a row: the same bits (fixed merge order), and in place (gx == gy)
+    gb3 = M.alloc((n,), dtype)
+    GY.relu_backward_bias_grad(gb3, GY, X, alpha)
+    assert bits_equal(GY.to_numpy(), gx.to_numpy()) and bits_equal(gb3.to_numpy(), gb.to_numpy())
+
+
+def test_relu_backward_bias_grad_views_and_errors(hip):
+    """strided operands take the two-call road with the same results; shape errors and a bias gradient
+    inside the gradient are refused"""
+    from zenu_amd import _lib
+    r = np.random.default_rng(3)
+    M = hip.Matrix
+    x = r.standard_normal((300, 96)).astype(np.float32)
+    gy = r.standard_normal((300, 96)).astype(np.float32)
+    X, GY = M.from_numpy(x), M.from_numpy(gy)
+    xv, gv = X.slice(slice(0, 300, 2), slice(None)), GY.slice(slice(0, 300, 2), slice(None))   # every other row
+    gx, gb = M.alloc((150, 96)), M.alloc((96,))
+    gx.relu_backward_bias_grad(gb, gv, xv, 0.1)
+    ref = gy[::2] * np.where(x[::2] > 0, np.float32(1), np.float32(0.1) * np.float32(-1))
+    assert bits_equal(gx.to_numpy(), ref.astype(np.float32))
+    assert np.allclose(gb.to_numpy(), ref.astype(np.float64).sum(0), rtol=1e-5, atol=1e-5)
+    gb1 = M.alloc((1, 96))                                  # [1, N] is the same bias gradient
+    gx.relu_backward_bias_grad(gb1, gv, xv, 0.1)
+    assert bits_equal(gb1.to_numpy().reshape(-1), gb.to_numpy())
+    with pytest.raises(_lib.ZenuHipError) as e:
+        gx.relu_backward_bias_grad(M.alloc((95,)), gv, xv, 0.1)
+    assert e.value.status == _lib.ERR_SHAPE
+    with pytest.raises(_lib.ZenuHipError) as e:
+        gx.relu_backward_bias_grad(gb, GY, xv, 0.1)
+    assert e.value.status == _lib.ERR_SHAPE
+    with pytest.raises(_lib.ZenuHipError) as e:
+        gx.relu_backward_bias_grad(gx.index_axis(0, 0), gv, xv, 0.1)
+    assert e.value.status == _lib.ERR_ARG
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("n,c", [(256, 10), (1, 4), (200, 16), (257, 10), (64, 17), (1000, 64)])
+def test_cross_entropy_backward_bias_grad(hip, dtype, n, c):
+    """gradient and its column sums from one call: the gradient is the bits of cross_entropy_backward,
+    the column sums are within the bar of every sum of the oracle's sum_to and of the exact sums, and
+    the same bits on every run; sizes on both sides of the one-launch conditions (<= 256 rows, <= 16 classes)"""
+    print(f"[case] cross_entropy_backward_bias_grad {n}x{c} {np.dtype(dtype).name}", flush=True)
+    r = np.random.default_rng(n * 17 + c)
+    pred = r.standard_normal((n, c)).astype(dtype)
+    ans = np.zeros((n, c), dtype=dtype)
+    ans[np.arange(n), r.integers(0, c, n)] = 1
+    M = hip.Matrix
+    _, prob = hip.cross_entropy(M.from_numpy(pred), M.from_numpy(ans))
+    p = prob.to_numpy()
+    gl = np.array(1.75, dtype=dtype)
+    for gloss in (None, gl):
+        G = M.from_numpy(gloss) if gloss is not None else None
+        gb = M.from_numpy(np.full(c, -3.0, dtype=dtype))
+        g = hip.cross_entropy_backward_bias_grad(prob, M.from_numpy(ans), gb, G)
+        g0 = hip.cross_entropy_backward(prob, M.from_numpy(ans), G)
+        assert bits_equal(g.to_numpy(), g0.to_numpy())
+        gbref = CpuMatrix.zeros((c,), dtype)
+        gref = cpu_matrix.cross_entropy_backward_bias_grad(CpuMatrix.from_numpy(p), CpuMatrix.from_numpy(ans), gbref,
+                                                           CpuMatrix.from_numpy(gloss) if gloss is not None else None)
+        assert bits_equal(g.to_numpy(), gref.a)
+        g64 = gref.a.astype(np.float64)
+        exact = g64.sum(0)
+        scale = np.maximum(np.abs(exact), np.abs(g64).sum(0) / np.sqrt(n))
+        tol = 1e-5 if dtype == np.float32 else 1e-12
+        assert np.all(np.abs(gb.to_numpy() - exact) <= tol * scale)
+        assert np.all(np.abs(gb.to_numpy() - gbref.a) <= 2 * tol * scale)
+        gb2 = M.alloc((c,), dtype)
+        hip.cross_entropy_backward_bias_grad(prob, M.from_numpy(ans), gb2, G)
+        assert bits_equal(gb2.to_numpy(), gb.to_numpy())
+
+
+def test_cross_entropy_single_launch_equals_two_launches(hip):
+    """up to 256 rows the cross-entropy forward folds its row terms in the workgroup that computed them;
+    257 rows take the two-launch road: on the first 256 rows of the same data both give the same
+    probabilities, and each loss is its own rows' exact value"""
+    r = np.random.default_rng(8)
+    pred = r.standard_normal((257, 10)).astype(np.float32)
+    ans = np.zeros((257, 10), dtype=np.float32)
+    ans[np.arange(257), r.integers(0, 10, 257)] = 1
+    M = hip.Matrix
+    la, pa = hip.cross_entropy(M.from_numpy(pred[:256]), M.from_numpy(ans[:256]))
+    lb, pb = hip.cross_entropy(M.from_numpy(pred), M.from_numpy(ans))
+    assert bits_equal(pa.to_numpy(), pb.to_numpy()[:256])
+    for loss, rows in ((la, 256), (lb, 257)):
+        lref, _ = cpu_matrix.cross_entropy(CpuMatrix.from_numpy(pred[:rows]), CpuMatrix.from_numpy(ans[:rows]))
+        assert abs(float(loss.to_numpy()) - float(lref.a)) <= 4e-5 * abs(float(lref.a))

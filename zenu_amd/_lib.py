@@ -86,6 +86,8 @@ SIGNATURES = {
     "zenu_hip_softmax_cross_entropy": [_i, _TP, _TP, _TP, _TP, _vp],
     "zenu_hip_softmax_cross_entropy_backward": [_i, _TP, _TP, _TP, _TP, _vp],
     "zenu_hip_bias_add_relu": [_i, _TP, _TP, _TP, _TP, _d, _vp],
+    "zenu_hip_relu_backward_bias_grad": [_i, _TP, _TP, _TP, _TP, _d, _vp],
+    "zenu_hip_softmax_cross_entropy_backward_bias_grad": [_i, _TP, _TP, _TP, _TP, _TP, _vp],
     "zenu_hip_sum_axis": [_i, _TP, _TP, _i, _vp],
     "zenu_hip_sum_axis_noalloc": [_i, _TP, _TP, _i, _vp],
     "zenu_hip_set_reduce_spin_limit": [_i],

@@ -58,13 +58,37 @@ template <typename T, bool MAX, int BLOCK = kBlock> __device__ __forceinline__ T
 constexpr int kLineRegs = 16;   // lines up to this length are kept in registers by the lines kernel
 
 template <typename T, bool CE>
+__device__ __forceinline__ T softmax_line(const zmath::ExpLog<T> &ml, const T *x, T *y, int64_t line, int64_t R,
+                                          int64_t inner, const T *target, T *rowloss);
+
+// With `loss` set (cross-entropy, every line in this one workgroup) the kernel also folds the row
+// terms and divides by -N, in the order of ce_finalize_kernel: the whole loss in one launch.
+template <typename T, bool CE>
 __global__ __launch_bounds__(kBlock) void softmax_lines_kernel(const T *x, T *y, int64_t lines, int64_t R,
-                                                                int64_t inner, const T *target, T *rowloss)
+                                                                int64_t inner, const T *target, T *rowloss,
+                                                                T *loss, T neg_n)
 {
     zmath::ExpLog<T> ml;
     ml.init(true, CE);
     const int64_t line = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (line >= lines) return;
+    T row_term = (T)0;
+    if (line < lines) row_term = softmax_line<T, CE>(ml, x, y, line, R, inner, target, rowloss);
+    if constexpr (CE) {
+        if (loss) {     // uniform: every thread of the workgroup gets here
+            __shared__ T lds[kWaves];
+            T acc = (T)0;
+            if (line < lines) acc = acc + row_term;
+            acc = block_red<T, false>(acc, lds);
+            if (threadIdx.x == 0) *loss = acc / neg_n;
+        }
+    }
+}
+
+// one softmax line by one thread; returns the line's cross-entropy term (also stored to rowloss when set)
+template <typename T, bool CE>
+__device__ __forceinline__ T softmax_line(const zmath::ExpLog<T> &ml, const T *x, T *y, int64_t line, int64_t R,
+                                          int64_t inner, const T *target, T *rowloss)
+{
     int64_t q = line, c = 0;
     if (inner != 1) {
         q = line / inner;
@@ -105,8 +129,8 @@ __global__ __launch_bounds__(kBlock) void softmax_lines_kernel(const T *x, T *y,
                 if (CE) acc = acc + tg[r] * ml.log(s);
             }
         }
-        if (CE) rowloss[line] = acc;
-        return;
+        if (CE && rowloss) rowloss[line] = acc;
+        return acc;
     }
     // max_axis: strict '>' from element 0 (max.rs:19-34)
     T m = xl[0];
@@ -127,7 +151,8 @@ __global__ __launch_bounds__(kBlock) void softmax_lines_kernel(const T *x, T *y,
         yl[r * inner] = s;
         if (CE) acc = acc + target[base + r * inner] * ml.log(s);
     }
-    if (CE) rowloss[line] = acc;
+    if (CE && rowloss) rowloss[line] = acc;
+    return acc;
 }
 
 template <typename T, int VEC, bool CE, bool REG, bool NT, int kBlock = 256, int kRegPacks = 4>
@@ -298,12 +323,49 @@ template <typename T, bool CE> struct GySource {
     }
 };
 
+// With `colsum` set (every line in this one workgroup, lines of at most kLineRegs elements, inner == 1)
+// the kernel also writes the column sums of gx -- the bias gradient of the Linear layer that
+// produced the logits (zenu-layer/src/layers/linear.rs:27-31 through the `sum_to` of
+// zenu-autograd/src/lib.rs:466-486) -- each folded over the lines in the fixed order of block_red.
 template <typename T, bool CE>
 __global__ __launch_bounds__(kBlock) void softmax_bwd_lines_kernel(const T *y, const T *gy_or_target, T *gx,
                                                                     int64_t lines, int64_t R, int64_t inner,
-                                                                    const T *gout, T neg_n)
+                                                                    const T *gout, T neg_n, T *colsum)
 {
     const int64_t line = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (colsum) {    // uniform; the host sends this only with R <= kLineRegs, inner == 1, one workgroup
+        __shared__ T lds[kWaves];
+        const bool active = line < lines;
+        const T g_total = CE ? (gout ? *gout : (T)1) / neg_n : (T)0;
+        const int64_t base = (active ? line : 0) * R;
+        T yv[kLineRegs], pv[kLineRegs], t[kLineRegs];
+#pragma unroll
+        for (int r = 0; r < kLineRegs; r++) {
+            const int64_t off = base + (r < R ? r : 0);
+            yv[r] = y[off];
+            pv[r] = gy_or_target[off];
+        }
+        T sum = (T)0;
+#pragma unroll
+        for (int r = 0; r < kLineRegs; r++) {
+            if (r < R) {
+                t[r] = yv[r] * (CE ? (pv[r] * g_total) / yv[r] : pv[r]);
+                sum = sum + t[r];
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < kLineRegs; r++) {
+            if (r < R) {
+                const T g = t[r] - yv[r] * sum;
+                if (active) gx[base + r] = g;
+                T c = (T)0;
+                if (active) c = c + g;
+                c = block_red<T, false>(c, lds);
+                if (threadIdx.x == 0) colsum[r] = c;
+            }
+        }
+        return;
+    }
     if (line >= lines) return;
     GySource<T, CE> src;
     src.p = gy_or_target;
@@ -527,15 +589,24 @@ Geometry geometry(const zenu_tensor_t &t, int axis)
 
 inline bool grid_ok(int64_t blocks) { return blocks > 0 && blocks <= 0x7fffffffLL; }
 
+// true when the cross-entropy forward of this geometry is one workgroup of the lines kernel, which
+// then also produces the loss (no row terms in memory, no second launch)
+inline bool ce_single_workgroup(const Geometry &g)
+{
+    return g.inner == 1 && g.R <= kLineMaxR && g.outer <= kBlock;
+}
+
 template <typename T, bool CE>
-int softmax_forward_launch(const T *x, T *y, Geometry g, const T *target, T *rowloss, hipStream_t s)
+int softmax_forward_launch(const T *x, T *y, Geometry g, const T *target, T *rowloss, hipStream_t s,
+                           T *loss = nullptr, T neg_n = (T)0)
 {
     constexpr int VEC = VecOf<T>::N;
     const int64_t lines = g.outer * g.inner;
     if (g.inner != 1 || g.R <= kLineMaxR) {
         const int64_t blocks = (lines + kBlock - 1) / kBlock;
         if (!grid_ok(blocks)) return ZENU_ERR_UNSUPPORTED;
-        softmax_lines_kernel<T, CE><<<(unsigned)blocks, kBlock, 0, s>>>(x, y, lines, g.R, g.inner, target, rowloss);
+        T *fold = (CE && blocks == 1) ? loss : nullptr;
+        softmax_lines_kernel<T, CE><<<(unsigned)blocks, kBlock, 0, s>>>(x, y, lines, g.R, g.inner, target, rowloss, fold, neg_n);
     } else {
         if (!grid_ok(lines)) return ZENU_ERR_UNSUPPORTED;
         const bool vec = g.R % VEC == 0 && aligned16(x) && aligned16(y) && (!CE || aligned16(target));
@@ -555,14 +626,15 @@ int softmax_forward_launch(const T *x, T *y, Geometry g, const T *target, T *row
 
 template <typename T, bool CE>
 int softmax_backward_launch(const T *y, const T *gy_or_target, T *gx, Geometry g, const T *gout, T neg_n,
-                            hipStream_t s)
+                            hipStream_t s, T *colsum = nullptr)
 {
     const int64_t lines = g.outer * g.inner;
+    if (colsum && !(g.inner == 1 && g.R <= kLineRegs && lines <= kBlock)) return ZENU_ERR_UNSUPPORTED;
     if (g.inner != 1 || g.R <= kLineMaxR) {
         const int64_t blocks = (lines + kBlock - 1) / kBlock;
         if (!grid_ok(blocks)) return ZENU_ERR_UNSUPPORTED;
         softmax_bwd_lines_kernel<T, CE><<<(unsigned)blocks, kBlock, 0, s>>>(y, gy_or_target, gx, lines, g.R, g.inner,
-                                                                             gout, neg_n);
+                                                                             gout, neg_n, colsum);
     } else {
         if (!grid_ok(lines)) return ZENU_ERR_UNSUPPORTED;
         constexpr int VEC = VecOf<T>::N;
@@ -619,13 +691,18 @@ int cross_entropy_t(int dtype, const zenu_tensor_t &loss, const zenu_tensor_t &p
     if (tin.status) return tin.status;
     ContigOut<T> out(prob, dtype, s);
     if (out.status) return out.status;
+    // n = T::from_usize(rows); Variable::from(-n)  (cross_entropy.rs:20-21)
+    const T neg_n = -(T)n;
+    if (ce_single_workgroup(geometry(pred, 1))) {   // a classifier head's batch: probabilities and loss in one launch
+        int rc1 = softmax_forward_launch<T, true>(in.ptr, out.ptr, geometry(pred, 1), tin.ptr, nullptr, s,
+                                                  static_cast<T *>(loss.ptr), neg_n);
+        return rc1 ? rc1 : out.finish();
+    }
     Workspace rows((size_t)n * sizeof(T), s);
     if (rows.status) return rows.status;
     T *rowloss = static_cast<T *>(rows.ptr);
     int rc = softmax_forward_launch<T, true>(in.ptr, out.ptr, geometry(pred, 1), tin.ptr, rowloss, s);
     if (rc) return rc;
-    // n = T::from_usize(rows); Variable::from(-n)  (cross_entropy.rs:20-21)
-    const T neg_n = -(T)n;
     if (n <= 65536) {
         ce_finalize_kernel<T><<<1, kBlock, 0, s>>>(rowloss, n, static_cast<T *>(loss.ptr), neg_n);
         ZENU_LAUNCH_CHECK();
@@ -644,9 +721,10 @@ int cross_entropy_t(int dtype, const zenu_tensor_t &loss, const zenu_tensor_t &p
 
 template <typename T>
 int cross_entropy_backward_t(int dtype, const zenu_tensor_t &gpred, const zenu_tensor_t &prob,
-                             const zenu_tensor_t &ans, const zenu_tensor_t *gloss, hipStream_t s)
+                             const zenu_tensor_t &ans, const zenu_tensor_t *gloss, hipStream_t s,
+                             const zenu_tensor_t *gbias = nullptr)
 {
-    if (num_elm(prob) == 0) return ZENU_OK;
+    if (num_elm(prob) == 0) return gbias ? ZENU_ERR_SHAPE : ZENU_OK;
     ContigIn<T> yin(prob, dtype, s);
     if (yin.status) return yin.status;
     ContigIn<T> tin(ans, dtype, s);
@@ -655,7 +733,8 @@ int cross_entropy_backward_t(int dtype, const zenu_tensor_t &gpred, const zenu_t
     if (out.status) return out.status;
     const T neg_n = -(T)prob.shape[0];
     const T *gout = gloss ? static_cast<const T *>(gloss->ptr) : nullptr;
-    int rc = softmax_backward_launch<T, true>(yin.ptr, tin.ptr, out.ptr, geometry(prob, 1), gout, neg_n, s);
+    T *colsum = gbias ? static_cast<T *>(gbias->ptr) : nullptr;
+    int rc = softmax_backward_launch<T, true>(yin.ptr, tin.ptr, out.ptr, geometry(prob, 1), gout, neg_n, s, colsum);
     return rc ? rc : out.finish();
 }
 
@@ -771,6 +850,37 @@ int zenu_hip_softmax_cross_entropy_backward(int dtype, const zenu_tensor_t *gpre
     if (dtype == ZENU_F32) return cross_entropy_backward_t<float>(dtype, *gpred, *prob, *ans, gloss, as_stream(stream));
     if (dtype == ZENU_F64) return cross_entropy_backward_t<double>(dtype, *gpred, *prob, *ans, gloss, as_stream(stream));
     return ZENU_ERR_ARG;
+}
+
+int zenu_hip_softmax_cross_entropy_backward_bias_grad(int dtype, const zenu_tensor_t *gpred, const zenu_tensor_t *gbias,
+                                                      const zenu_tensor_t *prob, const zenu_tensor_t *ans,
+                                                      const zenu_tensor_t *gloss, zenu_stream_t stream)
+{
+    const zenu_tensor_t *ts[] = {gpred, gbias, prob, ans};
+    int rc = check_all(ts, 4);
+    if (rc) return rc;
+    if (gloss && (validate_tensor(gloss) || gloss->ndim != 0)) return ZENU_ERR_SHAPE;
+    if (prob->ndim != 2) return ZENU_ERR_SHAPE;
+    if (!same_shape(*gpred, *prob) || !same_shape(*ans, *prob)) return ZENU_ERR_SHAPE;
+    if (gbias->ndim < 1 || gbias->shape[gbias->ndim - 1] != prob->shape[1] || num_elm(*gbias) != prob->shape[1])
+        return ZENU_ERR_SHAPE;
+    if (dtype != ZENU_F32 && dtype != ZENU_F64) return ZENU_ERR_ARG;
+    const size_t esz = dtype == ZENU_F32 ? 4 : 8;
+    const size_t gb_bytes = (size_t)num_elm(*gbias) * esz;
+    if (view_overlaps(*gpred, esz, gbias->ptr, gb_bytes) || view_overlaps(*prob, esz, gbias->ptr, gb_bytes) ||
+        view_overlaps(*ans, esz, gbias->ptr, gb_bytes))
+        return ZENU_ERR_ARG;
+    // a classifier head's batch (every line in one workgroup, at most 16 classes): gradient and its column
+    // sums in one launch; anything else is the two calls it stands for
+    if (prob->shape[0] <= kBlock && prob->shape[1] <= kLineRegs && is_default_stride_strict(*gbias)) {
+        rc = dtype == ZENU_F32
+                 ? cross_entropy_backward_t<float>(dtype, *gpred, *prob, *ans, gloss, as_stream(stream), gbias)
+                 : cross_entropy_backward_t<double>(dtype, *gpred, *prob, *ans, gloss, as_stream(stream), gbias);
+        if (rc != ZENU_ERR_UNSUPPORTED) return rc;
+    }
+    rc = zenu_hip_softmax_cross_entropy_backward(dtype, gpred, prob, ans, gloss, stream);
+    if (rc) return rc;
+    return zenu_hip_sum_to(dtype, gbias, gpred, stream);
 }
 
 int zenu_hip_bias_add_relu(int dtype, const zenu_tensor_t *pre, const zenu_tensor_t *act, const zenu_tensor_t *z,

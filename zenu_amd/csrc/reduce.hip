@@ -32,6 +32,8 @@
 // (NaN payload, sign of zero) are the source's.
 #include <math.h>
 
+#include <type_traits>
+
 #include "common.hpp"
 #include "vecmem.hpp"
 
@@ -245,6 +247,14 @@ template <typename T> struct RedParams {
     uint32_t epoch;          // this launch's tag, never zero
     int spin_limit;          // polls before the folding workgroup computes what is missing itself
     unsigned int *fallbacks; // bumped once per batch of partials that the folding workgroup had to compute
+    // optional transform of the source on its way in (column kernels, vector path, sums only):
+    // the reduced value is in[i] * (pre_x[i] > 0 ? 1 : pre_alpha * -1), the gradient of ReLU
+    // (zenu-autograd/src/activation/relu.rs:35-44), which is also stored to pre_out[i]; the three
+    // arrays share the source's layout.  Every source element is loaded by exactly one thread of
+    // the launch, so every element of pre_out is written once.
+    const T *pre_x;
+    T *pre_out;
+    T pre_alpha;
     // value gather for max: value = gsrc[q * g_outer_stride + c + idx * g_elem_stride]
     const T *gsrc;
     int64_t g_outer_stride, g_elem_stride;
@@ -314,6 +324,21 @@ __device__ __forceinline__ typename Tr::Acc load_partial(const RedParams<T> &p, 
     int32_t i = 0;
     if (Tr::kHasIdx) i = load_agent(p.part_idx + slot);
     return Tr::from_partial(k, i);
+}
+
+// a vector of the source; with PRE the ReLU-gradient transform described at RedParams::pre_x
+template <typename T, int VEC, bool NT, bool PRE>
+__device__ __forceinline__ Pack<T, VEC> load_src(const RedParams<T> &p, const T *ptr)
+{
+    Pack<T, VEC> g = load_pack<T, VEC, NT>(ptr);
+    if constexpr (PRE) {
+        const int64_t off = ptr - p.in;
+        const Pack<T, VEC> x = load_pack<T, VEC, NT>(p.pre_x + off);
+#pragma unroll
+        for (int j = 0; j < VEC; j++) g.v[j] = g.v[j] * ((x.v[j] > (T)0) ? (T)1 : p.pre_alpha * (T)-1);
+        store_pack<T, VEC, NT>(p.pre_out + off, g);
+    }
+    return g;
 }
 
 // ---- hand-off through tagged words ---------------------------------------------------------------------
@@ -597,7 +622,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(RedParams<T> p)
 // which sits in host memory: 2-10 us before the first load (measured on the arg-max kernel).
 #define ZENU_FOR_COLS(j) _Pragma("unroll") for (int j = 0; j < VEC; j++) if (j < ncol)
 
-template <typename T, typename Tr, int VEC, bool NT>
+template <typename T, typename Tr, int VEC, bool NT, bool PRE = false>
 __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, uint32_t col_tiles, int tx_shift, int grid3d)
 {
     typedef typename Tr::Acc A;
@@ -664,7 +689,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, uin
                 if (b + chunk <= R) {
                     Pack<T, VEC> x[U];
 #pragma unroll
-                    for (int u = 0; u < U; u++) x[u] = load_pack<T, VEC, NT>(ptr + u * row_step);
+                    for (int u = 0; u < U; u++) x[u] = load_src<T, VEC, NT, PRE>(p, ptr + u * row_step);
 #pragma unroll
                     for (int u = 0; u < U; u++) {
 #pragma unroll
@@ -673,7 +698,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, uin
                 } else {
                     const T *pt = ptr;
                     for (int64_t rr = r; rr < R; rr += ty_n, pt += row_step) {
-                        Pack<T, VEC> x = load_pack<T, VEC, false>(pt);
+                        Pack<T, VEC> x = load_src<T, VEC, false, PRE>(p, pt);
 #pragma unroll
                         for (int j = 0; j < VEC; j++) acc[j] = Tr::update(acc[j], x.v[j], rr);
                     }
@@ -733,7 +758,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, uin
 // stored and loaded as whole vectors' worth of device-scope words without a branch each.  The
 // accumulation order, the order of the LDS combine and the order of the fold are kernel B's, so
 // both give the same bits.
-template <typename T, typename Tr, int VEC, bool NT>
+template <typename T, typename Tr, int VEC, bool NT, bool PRE = false>
 __global__ __launch_bounds__(kBlock) void reduce_cols_regular_kernel(RedParams<T> p)
 {
     typedef typename Tr::Acc A;
@@ -773,7 +798,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_regular_kernel(RedParams<T
         if (b + chunk <= R) {
             Pack<T, VEC> x[U];
 #pragma unroll
-            for (int u = 0; u < U; u++) x[u] = load_pack<T, VEC, NT>(src + (r + u * TY) * es);
+            for (int u = 0; u < U; u++) x[u] = load_src<T, VEC, NT, PRE>(p, src + (r + u * TY) * es);
 #pragma unroll
             for (int u = 0; u < U; u++) {
 #pragma unroll
@@ -781,7 +806,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_regular_kernel(RedParams<T
             }
         } else {
             for (int64_t rr = r; rr < R; rr += TY) {
-                const Pack<T, VEC> x = load_pack<T, VEC, false>(src + rr * es);
+                const Pack<T, VEC> x = load_src<T, VEC, false, PRE>(p, src + rr * es);
 #pragma unroll
                 for (int j = 0; j < VEC; j++) acc.a[j] = Tr::update(acc.a[j], x.v[j], rr);
             }
@@ -912,6 +937,20 @@ int launch_cols(const RedParams<T> &p, hipStream_t s)
     // the regular geometry: full vector tiles of 32 x 8 threads, a split axis with a flat counter
     const bool regular = vec && g3 && shift == 5 && p.inner % per_tile == 0 && p.splits > 1 && p.fan >= p.splits &&
                          p.cstride == 1 && (Tr::kHasIdx || aligned16(p.out_val));
+    if constexpr (!Tr::kHasIdx && std::is_same<Tr, SumTr<T>>::value) {
+        if (p.pre_x) {   // the transform rides on the vector paths only (the caller has checked the layout)
+            if (!vec) return ZENU_ERR_UNSUPPORTED;
+            if (regular) {
+                if (nt) reduce_cols_regular_kernel<T, Tr, VEC, true, true><<<g, kBlock, 0, s>>>(p);
+                else    reduce_cols_regular_kernel<T, Tr, VEC, false, true><<<g, kBlock, 0, s>>>(p);
+            } else {
+                if (nt) reduce_cols_kernel<T, Tr, VEC, true, true><<<g, kBlock, 0, s>>>(p, ctl, shift, g3);
+                else    reduce_cols_kernel<T, Tr, VEC, false, true><<<g, kBlock, 0, s>>>(p, ctl, shift, g3);
+            }
+            ZENU_LAUNCH_CHECK();
+            return ZENU_OK;
+        }
+    }
     if (regular) {
         if (nt) reduce_cols_regular_kernel<T, Tr, VEC, true><<<g, kBlock, 0, s>>>(p);
         else    reduce_cols_regular_kernel<T, Tr, VEC, false><<<g, kBlock, 0, s>>>(p);
@@ -930,7 +969,8 @@ int launch_cols(const RedParams<T> &p, hipStream_t s)
 template <typename T, typename Tr>
 int reduce_strided(const T *src, int64_t outer, int64_t R, int64_t inner, int64_t outer_stride,
                    int64_t elem_stride, T *out_val, int64_t *out_idx, hipStream_t s,
-                   const FixedScratch *fixed = nullptr)
+                   const FixedScratch *fixed = nullptr, const T *pre_x = nullptr, T *pre_out = nullptr,
+                   T pre_alpha = (T)0)
 {
     constexpr int VEC = VecOf<T>::N;
     const int64_t nout = outer * inner;
@@ -964,11 +1004,15 @@ int reduce_strided(const T *src, int64_t outer, int64_t R, int64_t inner, int64_
     p.epoch = 0;
     p.spin_limit = 0;
     p.fallbacks = g_fold_fallbacks_ptr;
+    p.pre_x = pre_x;
+    p.pre_out = pre_out;
+    p.pre_alpha = pre_alpha;
     p.gsrc = src;
     p.g_outer_stride = outer_stride;
     p.g_elem_stride = elem_stride;
 
     const bool use_cols = inner >= 16;
+    if (pre_x && (!use_cols || !cols_vec_ok(p))) return ZENU_ERR_UNSUPPORTED;   // the caller falls back to two launches
     int64_t splits = 1, groups = nout;
     if (use_cols) {
         const int v = cols_vec_ok(p) ? VEC : 1;
@@ -1260,6 +1304,17 @@ int reduce_all(int kind, int dtype, void *out_val, int64_t *out_idx, const zenu_
     return reduce_contiguous<double, ArgmaxTr<double>>(d, 1, n, 1, ov, out_idx, s);
 }
 
+template <typename T>
+int relu_backward_bias_grad_t(const zenu_tensor_t &gx, const zenu_tensor_t &gbias, const zenu_tensor_t &gy,
+                                     const zenu_tensor_t &x, double alpha, hipStream_t s)
+{
+    const int64_t n = gbias.shape[gbias.ndim - 1];
+    const int64_t rows = num_elm(gy) / n;
+    return reduce_strided<T, SumTr<T>>(static_cast<const T *>(gy.ptr), 1, rows, n, rows * n, n,
+                                       static_cast<T *>(gbias.ptr), nullptr, s, nullptr,
+                                       static_cast<const T *>(x.ptr), static_cast<T *>(gx.ptr), (T)alpha);
+}
+
 }  // namespace
 
 // Called once by the library's init, with its device current: the device address of the static
@@ -1384,6 +1439,42 @@ int zenu_hip_max_idx(int dtype, int64_t *out_flat_idx_dev, void *out_val_dev, co
 {
     if (!out_flat_idx_dev && !out_val_dev) return ZENU_ERR_ARG;
     return reduce_all(kMax, dtype, out_val_dev, out_flat_idx_dev, src, as_stream(stream));
+}
+
+int zenu_hip_relu_backward_bias_grad(int dtype, const zenu_tensor_t *gx, const zenu_tensor_t *gbias,
+                                     const zenu_tensor_t *gy, const zenu_tensor_t *x, double alpha,
+                                     zenu_stream_t stream)
+{
+    int rc = validate_tensor(gx);
+    if (!rc) rc = validate_tensor(gbias);
+    if (!rc) rc = validate_tensor(gy);
+    if (!rc) rc = validate_tensor(x);
+    if (!rc) rc = ensure_init();
+    if (rc) return rc;
+    if (dtype != ZENU_F32 && dtype != ZENU_F64) return ZENU_ERR_ARG;
+    if (!same_shape(*gx, *gy) || !same_shape(*gx, *x)) return ZENU_ERR_SHAPE;
+    const size_t esz = dtype == ZENU_F32 ? 4 : 8;
+    if (view_overlaps(*gx, esz, gbias->ptr, (size_t)num_elm(*gbias) * esz) ||
+        view_overlaps(*gy, esz, gbias->ptr, (size_t)num_elm(*gbias) * esz) ||
+        view_overlaps(*x, esz, gbias->ptr, (size_t)num_elm(*gbias) * esz) || check_output_alias(*gx, *x, esz))
+        return ZENU_ERR_ARG;
+    // one launch when the gradient is a whole [.., N] tensor and the bias gradient its [N] (or [1, .., N])
+    // column sums; anything else is the two calls it stands for
+    bool fused = gx->ndim >= 2 && gbias->ndim >= 1 && num_elm(*gy) > 0 && is_default_stride_strict(*gx) &&
+                 is_default_stride_strict(*gy) && is_default_stride_strict(*x) && is_default_stride_strict(*gbias) &&
+                 aligned16(gx->ptr) && aligned16(x->ptr) && aligned16(gy->ptr);
+    if (fused) {
+        const int64_t n = gx->shape[gx->ndim - 1];
+        fused = gbias->shape[gbias->ndim - 1] == n && num_elm(*gbias) == n;
+    }
+    if (fused) {
+        rc = dtype == ZENU_F32 ? relu_backward_bias_grad_t<float>(*gx, *gbias, *gy, *x, alpha, as_stream(stream))
+                               : relu_backward_bias_grad_t<double>(*gx, *gbias, *gy, *x, alpha, as_stream(stream));
+        if (rc != ZENU_ERR_UNSUPPORTED) return rc;
+    }
+    rc = zenu_hip_relu_backward(dtype, gx, gy, x, alpha, stream);
+    if (rc) return rc;
+    return zenu_hip_sum_to(dtype, gbias, gx, stream);
 }
 
 int zenu_hip_sum_to(int dtype, const zenu_tensor_t *target, const zenu_tensor_t *src, zenu_stream_t stream)

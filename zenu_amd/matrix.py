@@ -345,6 +345,13 @@ class Matrix:
         check(_lib.lib().zenu_hip_relu_backward(_dt(self.dtype), C.byref(self.desc()), C.byref(gy.desc()),
                                                 C.byref(x.desc()), float(alpha), _stream), "relu_backward")
 
+    def relu_backward_bias_grad(self, gbias, gy, x, alpha):
+        """self = gy * relu'(x) and gbias = the column sums of self (the bias gradient of the layer
+        before), in one pass over gy"""
+        check(_lib.lib().zenu_hip_relu_backward_bias_grad(_dt(self.dtype), C.byref(self.desc()), C.byref(gbias.desc()),
+                                                          C.byref(gy.desc()), C.byref(x.desc()), float(alpha), _stream),
+              "relu_backward_bias_grad")
+
     # ---- clip (zenu-matrix/src/operation/clip.rs:289-318) -----------------------------------
     def clip(self, lo, hi):
         out = self.alloc_like()
@@ -538,6 +545,15 @@ def cross_entropy_backward(prob, ans, gloss=None):
     check(_lib.lib().zenu_hip_softmax_cross_entropy_backward(
         _dt(prob.dtype), C.byref(gpred.desc()), C.byref(prob.desc()), C.byref(ans.desc()),
         C.byref(gloss.desc()) if gloss is not None else None, _stream), "cross_entropy_backward")
+    return gpred
+
+
+def cross_entropy_backward_bias_grad(prob, ans, gbias, gloss=None):
+    """cross_entropy_backward() that also writes the column sums of the gradient to gbias"""
+    gpred = prob.alloc_like()
+    check(_lib.lib().zenu_hip_softmax_cross_entropy_backward_bias_grad(
+        _dt(prob.dtype), C.byref(gpred.desc()), C.byref(gbias.desc()), C.byref(prob.desc()), C.byref(ans.desc()),
+        C.byref(gloss.desc()) if gloss is not None else None, _stream), "cross_entropy_backward_bias_grad")
     return gpred
 
 
