@@ -698,6 +698,30 @@ public:
         }
     }
 
+    ~AdamW() { drop_schedule(); }
+    AdamW(const AdamW &) = delete;
+    AdamW &operator=(const AdamW &) = delete;
+
+    // For callers that record `update` into a HIP graph: take 1 - beta^t of the next n_steps updates from
+    // a table in device memory whose cursor every update advances, so that each replay of one recorded
+    // update is the next step (zenu_hip_adam_step_multi_scheduled; no counterpart in the reference).
+    void use_schedule(int n_steps)
+    {
+        drop_schedule();
+        check(zenu_hip_adam_schedule_create(&schedule_, DType<T>::value, (double)beta1, (double)beta2, step + 1, n_steps,
+                                            current_stream()), "adam_schedule_create");
+    }
+    void drop_schedule()
+    {
+        if (schedule_) zenu_hip_adam_schedule_destroy(schedule_, current_stream());
+        schedule_ = nullptr;
+    }
+    // next step of the schedule, steps left in it, updates refused because it had run out
+    void schedule_state(int64_t &next_step, int64_t &steps_left, int64_t &refused) const
+    {
+        check(zenu_hip_adam_schedule_query(schedule_, &next_step, &steps_left, &refused, current_stream()), "adam_schedule_query");
+    }
+
     // one launch for the whole model (zenu_hip_adam_step_multi)
     void update(const Parameters<T> &params)
     {
@@ -719,11 +743,21 @@ public:
             decay.push_back(weight_keys.count(kv.first) ? 1 : 0);
         }
         if (P.empty()) return;
+        if (schedule_) {
+            check(zenu_hip_adam_step_multi_scheduled(DType<T>::value, (int)P.size(), P.data(), G.data(), M.data(), V.data(),
+                                                     sizes.data(), (double)learning_rate, (double)epsilon, (double)weight_decay,
+                                                     decay.data(), schedule_, current_stream()),
+                  "adam_step_multi_scheduled");
+            return;
+        }
         check(zenu_hip_adam_step_multi(DType<T>::value, (int)P.size(), P.data(), G.data(), M.data(), V.data(), sizes.data(),
                                        (double)learning_rate, (double)beta1, (double)beta2, (double)epsilon,
                                        (double)weight_decay, decay.data(), (double)step, current_stream()),
               "adam_step_multi");
     }
+
+private:
+    void *schedule_ = nullptr;
 };
 
 template <typename T> class Adam : public AdamW<T> {   // zenu-optimizer/src/adam.rs:9-89

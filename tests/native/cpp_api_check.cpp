@@ -437,6 +437,30 @@ static void adam_w_net_test() // net_test.rs:191-232: one optimizer, two steps, 
                          0.1101, 0.1201, 0.1301, 0.1401}, {0.0800, 0.1800, 0.2801, 0.3800}, 2e-4));
 }
 
+static void adam_w_net_test_scheduled()   // the same two steps with the step-dependent scalars in device memory
+{
+    Net net;
+    AdamW<float> opt(0.01f, 0.9f, 0.999f, 1e-8f, 0.01f, net.p, {kW1, kW2});
+    opt.use_schedule(2);
+    for (int i = 0; i < 2; i++) {
+        net.backward();
+        opt.update(net.p);
+    }
+    REQUIRE(net.matches({0.0801, 0.1800, 0.2800, 0.3800, 0.4800, 0.5800, 0.0501, 0.0601}, {0.0801, 0.1800, 0.2800, 0.3800},
+                        {0.0801, 0.1800, 0.2800, 0.3800, 0.4800, 0.5800, 0.0501, 0.0601, 0.0702, 0.0801, 0.0901, 0.1001,
+                         0.1101, 0.1201, 0.1301, 0.1401}, {0.0800, 0.1800, 0.2801, 0.3800}, 2e-4));
+    int64_t next = 0, left = 0, refused = 0;
+    opt.schedule_state(next, left, refused);
+    REQUIRE(next == 3 && left == 0 && refused == 0);
+    net.backward();
+    opt.update(net.p);                        // past the end of the table: nothing changes, and it is counted
+    opt.schedule_state(next, left, refused);
+    REQUIRE(next == 3 && refused == 1);
+    REQUIRE(net.matches({0.0801, 0.1800, 0.2800, 0.3800, 0.4800, 0.5800, 0.0501, 0.0601}, {0.0801, 0.1800, 0.2800, 0.3800},
+                        {0.0801, 0.1800, 0.2800, 0.3800, 0.4800, 0.5800, 0.0501, 0.0601, 0.0702, 0.0801, 0.0901, 0.1001,
+                         0.1101, 0.1201, 0.1301, 0.1401}, {0.0800, 0.1800, 0.2801, 0.3800}, 2e-4));
+}
+
 int main(int argc, char **argv)
 {
     init(0);
@@ -452,6 +476,7 @@ int main(int argc, char **argv)
         {"softmax_cases", softmax_cases},
         {"cross_entropy_cases", cross_entropy_cases}, {"clip_cases", clip_cases}, {"sgd_net_test", sgd_net_test},
         {"adam_net_test", adam_net_test}, {"adam_w_net_test", adam_w_net_test},
+        {"adam_w_net_test_scheduled", adam_w_net_test_scheduled},
     };
     for (const Case &c : cases) {
         if (argc > 1 && std::string(argv[1]) != c.name) continue;

@@ -10,7 +10,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CASES = ["scalar_add_2d", "sliced_3d", "sliced_3d_assign", "matrix_add_sliced", "transposed", "broadcast_add",
          "broadcast_add_1x4x1x1_3x4x5x5", "sub_mul_div", "shape_errors", "unary_tables", "relu_cases", "sigmoid_cases",
          "sum_4d", "max_cases", "asum_cases", "copy_cases", "broadcast_cases", "conv_bias_cases", "mean_variance_cases", "stack_split_cases", "softmax_cases", "cross_entropy_cases",
-         "clip_cases", "sgd_net_test", "adam_net_test", "adam_w_net_test"]
+         "clip_cases", "sgd_net_test", "adam_net_test", "adam_w_net_test", "adam_w_net_test_scheduled"]
 
 
 def test_cpp_api_program_builds(tmp_path):
