@@ -758,7 +758,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, uin
 // stored and loaded as whole vectors' worth of device-scope words without a branch each.  The
 // accumulation order, the order of the LDS combine and the order of the fold are kernel B's, so
 // both give the same bits.
-template <typename T, typename Tr, int VEC, bool NT, bool PRE = false>
+template <typename T, typename Tr, int VEC, bool NT, bool PRE = false, int U = 4>
 __global__ __launch_bounds__(kBlock) void reduce_cols_regular_kernel(RedParams<T> p)
 {
     typedef typename Tr::Acc A;
@@ -766,7 +766,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_regular_kernel(RedParams<T
         A a[VEC];
     };
     __shared__ Cols lds[kBlock];
-    constexpr int TX = 32, TY = kBlock / TX, U = 4;
+    constexpr int TX = 32, TY = kBlock / TX;
     const int tx = threadIdx.x & (TX - 1), ty = threadIdx.x / TX;
     const int split = (int)blockIdx.y, splits = p.splits;
     const int64_t q = blockIdx.z;
