@@ -408,6 +408,16 @@ int zenu_hip_adam_step_multi_scheduled(int dtype, int n_tensors, void *const *p_
  * the first status other than ZENU_OK that any of them produced on this thread since the last
  * call, and clears it: a wrapper can poll it after a batch of calls (no counterpart in the
  * reference, whose kernels check nothing). */
+/* Self-check of the device math: f32 tanh, sigmoid, sinh, cosh, atan, asin and acos (fn = the
+ * zenu_unop_t value) use a 4-instruction division / square root that is exact only on the operands
+ * these functions produce.  The call evaluates the function on ALL 2^32 f32 bit patterns twice on
+ * the device -- as shipped, and with the IEEE division and square root in the same places -- and
+ * returns in *mismatches how many results differ (0 is the only acceptable answer) and in
+ * *example_bits (may be NULL) the bit pattern of one argument that differs.  fn = 1000 / 1001
+ * compare the bare division / square root on operands of every exponent, where they do differ
+ * (the short forms have no operand scaling): a check of the check.  Blocking; a few tens of milliseconds per function.  No counterpart in the reference. */
+int zenu_hip_selfcheck_short_division(int fn, uint64_t *mismatches, uint32_t *example_bits,
+                                      zenu_stream_t stream);
 int zenu_hip_last_status(void);
 
 #define ZENU_DECL_1D(T, S)                                                                        \

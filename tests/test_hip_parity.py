@@ -294,6 +294,37 @@ def test_tanh_sigmoid_dense_sweep(hip):
         assert max_ulp(got[ok], exp[ok]) == 0, (name, _libm_note(hip))
 
 
+@pytest.mark.parametrize("name", ["tanh", "sigmoid", "sinh", "cosh", "atan", "asin", "acos"])
+def test_short_division_equals_ieee_on_every_f32_argument(hip, name):
+    """The f32 tanh, sigmoid, sinh, cosh, atan, asin and acos use a 4-instruction division / square root
+    that is exact only on the operands these functions produce.  The library evaluates each function
+    on ALL 2^32 bit patterns twice on the device, as shipped and with the IEEE operations in the same
+    places, and counts the results that differ: none.  (The IEEE build is the one the host build of
+    the same source restates; its equality with the host libm is what the sweeps above sample and
+    tests/test_exhaustive_device.py exhausts.)"""
+    import ctypes as C
+    from zenu_amd import _lib
+    code = {"tanh": _lib.TANH, "sigmoid": _lib.SIGMOID, "sinh": _lib.SINH, "cosh": _lib.COSH, "atan": _lib.ATAN,
+            "asin": _lib.ASIN, "acos": _lib.ACOS}[name]
+    n, ex = C.c_uint64(), C.c_uint32()
+    _lib.check(hip.lib().zenu_hip_selfcheck_short_division(code, C.byref(n), C.byref(ex), hip.get_stream()), "selfcheck")
+    assert n.value == 0, f"{name}: {n.value} of 2^32 results differ, e.g. for the argument with bits {ex.value:#010x}"
+
+
+def test_short_division_selfcheck_can_fail(hip):
+    """a check of the check: on operands of every exponent the bare short division and square root do
+    differ from the IEEE operations (they have no operand scaling), and the same machinery counts it"""
+    import ctypes as C
+    from zenu_amd import _lib
+    for fn in (1000, 1001):
+        n, ex = C.c_uint64(), C.c_uint32()
+        _lib.check(hip.lib().zenu_hip_selfcheck_short_division(fn, C.byref(n), C.byref(ex), hip.get_stream()), "selfcheck")
+        print(f"[selfcheck] fn {fn}: {n.value} of 2^32 operand sets differ", flush=True)
+        assert 0 < n.value < (1 << 32)
+    n = C.c_uint64()
+    assert hip.lib().zenu_hip_selfcheck_short_division(_lib.EXP, C.byref(n), None, hip.get_stream()) == _lib.ERR_ARG
+
+
 def test_tanh_ulp2_variant(hip):
     """ZENU_TANH_ULP2 (no counterpart in the reference): never more than 2 ulp from the host tanhf,
     the tolerance the transcendental functions are allowed; checked on every 64th f32 bit pattern and

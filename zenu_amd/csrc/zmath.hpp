@@ -25,11 +25,27 @@
 // The host build of this header is compared with the host libm by tests/native/zmath_host_check.cpp
 // (tests/test_host_native.py runs it on a sample; on every f32 bit pattern and on 2e10 sampled
 // f64 inputs it was run during development, without a mismatch).
-#pragma once
+//
+// The header can be instantiated a second time under another namespace (define ZMATH_NAMESPACE
+// before including it again): selfcheck.hip does that with ZMATH_EXACT_DIVISION, which makes the
+// short division and square root below the IEEE operations, to compare the two builds of every
+// function on every f32 argument on the device.
 #include <math.h>
 #include <stdint.h>
 #include <string.h>
 
+#if defined(ZMATH_NAMESPACE)
+#define ZMATH_NS ZMATH_NAMESPACE
+#define ZMATH_EMIT 1
+#elif !defined(ZMATH_HPP_INCLUDED)
+#define ZMATH_HPP_INCLUDED
+#define ZMATH_NS zmath
+#define ZMATH_EMIT 1
+#endif
+#ifdef ZMATH_EMIT
+
+#undef ZM_HD
+#undef ZM_RARE
 #if defined(__HIPCC__)
 #define ZM_HD __host__ __device__ __forceinline__
 // a rarely taken path kept out of line: one copy per kernel instead of one per element of the
@@ -40,7 +56,7 @@
 #define ZM_RARE static
 #endif
 
-namespace zmath {
+namespace ZMATH_NS {
 
 ZM_HD uint32_t f2u(float f)
 {
@@ -184,7 +200,7 @@ ZM_HD float tanhf_fdlibm(float x)
 // divides; it checks everything but this sequence.
 ZM_HD float div_tanh(float a, float b)
 {
-#if defined(__HIP_DEVICE_COMPILE__)
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(ZMATH_EXACT_DIVISION)
     const float r = __builtin_amdgcn_rcpf(b);
     const float q = a * r;
     const float rem = __builtin_fmaf(-b, q, a);
@@ -201,7 +217,7 @@ ZM_HD float div_tanh(float a, float b)
 ZM_HD float div_fast(float a, float b) { return div_tanh(a, b); }
 ZM_HD float sqrt_fast(float t)
 {
-#if defined(__HIP_DEVICE_COMPILE__)
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(ZMATH_EXACT_DIVISION)
     const float y = __builtin_amdgcn_rsqf(t);
     const float s = t * y;
     const float h = 0.5f * y;
@@ -1766,4 +1782,8 @@ template <> struct Pow<float> {
 };
 #endif
 
-}  // namespace zmath
+}  // namespace ZMATH_NS
+
+#undef ZMATH_EMIT
+#undef ZMATH_NS
+#endif  // ZMATH_EMIT
