@@ -195,7 +195,7 @@ def test_softmax_special_rows(hip):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
-@pytest.mark.parametrize("n,c", [(256, 10), (1, 4), (1000, 64), (50, 1000), (70000, 3)])
+@pytest.mark.parametrize("n,c", [(256, 10), (1, 4), (255, 13), (7, 1), (128, 16), (3, 2), (1000, 64), (50, 1000), (70000, 3)])
 def test_cross_entropy(hip, dtype, n, c):
     print(f"[case] cross_entropy {n}x{c} {np.dtype(dtype).name}", flush=True)
     r = np.random.default_rng(n * 131 + c)
@@ -473,7 +473,7 @@ def test_relu_backward_bias_grad_views_and_errors(hip):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
-@pytest.mark.parametrize("n,c", [(256, 10), (1, 4), (200, 16), (257, 10), (64, 17), (1000, 64)])
+@pytest.mark.parametrize("n,c", [(256, 10), (1, 4), (200, 16), (255, 13), (9, 1), (257, 10), (64, 17), (1000, 64)])
 def test_cross_entropy_backward_bias_grad(hip, dtype, n, c):
     """gradient and its column sums from one call: the gradient is the bits of cross_entropy_backward,
     the column sums are within the bar of every sum of the oracle's sum_to and of the exact sums, and

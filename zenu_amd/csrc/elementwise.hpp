@@ -714,28 +714,64 @@ __global__ __launch_bounds__((TileThreads<T, F>::value)) void ew_tile_kernel(T *
             store_pack<T, VEC, NT>(obase + (int64_t)r * ldr0 + lane_v, apply_pack<T, VEC, F>(f, xa[k], y));
         }
     } else {
-        // edge tiles and unaligned operands: element-wise with bounds checks
-        if (trans_a || (F::NIN == 2 && trans_b)) {
-            for (int e = tid; e < kTile * kTile; e += kBlock) {
+        // Edge tiles and unaligned operands: element by element with bounds checks.  All loads of a
+        // phase are issued before the first use (an element outside the tile reads the tile's first
+        // one again and is dropped): with the loads inside the bounds check the compiler waits for each
+        // before it issues the next, and a small matrix made of edge tiles only (the [512,10] weights of a
+        // classifier head) took four memory round trips per phase instead of one.
+        constexpr int E = kTile * kTile / kBlock;
+        const bool ta = trans_a != 0;
+        const bool tb = (F::NIN == 2) && trans_b != 0;
+        if (ta || tb) {
+            T va[E], vb[E];
+#pragma unroll
+            for (int i = 0; i < E; i++) {
+                const int e = tid + i * kBlock;
                 const int r = e % kTile, c = e / kTile;
-                if (r < nr && c < nc) {
-                    if (trans_a) lds_a[r * kPitch + c] = abase[r + (int64_t)c * ldc1];
+                const bool ok = (r < nr) & (c < nc);
+                const int64_t off_r = ok ? r : 0, off_c = ok ? c : 0;
+                if (ta) va[i] = abase[off_r + off_c * ldc1];
+                if constexpr (F::NIN == 2) {
+                    if (tb) vb[i] = bbase[off_r + off_c * ldc2];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < E; i++) {
+                const int e = tid + i * kBlock;
+                const int r = e % kTile, c = e / kTile;
+                if ((r < nr) & (c < nc)) {
+                    if (ta) lds_a[r * kPitch + c] = va[i];
                     if constexpr (F::NIN == 2) {
-                        if (trans_b) lds_b[r * kPitch + c] = bbase[r + (int64_t)c * ldc2];
+                        if (tb) lds_b[r * kPitch + c] = vb[i];
                     }
                 }
             }
             __syncthreads();
         }
-        for (int e = tid; e < kTile * kTile; e += kBlock) {
+        T x[E], y[E];
+#pragma unroll
+        for (int i = 0; i < E; i++) {
+            const int e = tid + i * kBlock;
             const int c = e % kTile, r = e / kTile;
-            if (r < nr && c < nc) {
-                T x = trans_a ? lds_a[r * kPitch + c] : abase[(int64_t)r * ldr1 + (int64_t)c * ldc1];
-                T y = x;
-                if constexpr (F::NIN == 2)
-                    y = trans_b ? lds_b[r * kPitch + c]
-                                  : bbase[(int64_t)r * ldr2 + (int64_t)c * ldc2];
-                obase[(int64_t)r * ldr0 + c] = f(x, y);
+            const bool ok = (r < nr) & (c < nc);
+            const int64_t off_r = ok ? r : 0, off_c = ok ? c : 0;
+            if (!ta) x[i] = abase[off_r * ldr1 + off_c * ldc1];
+            if constexpr (F::NIN == 2) {
+                if (!tb) y[i] = bbase[off_r * ldr2 + off_c * ldc2];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < E; i++) {
+            const int e = tid + i * kBlock;
+            const int c = e % kTile, r = e / kTile;
+            if ((r < nr) & (c < nc)) {
+                if (ta) x[i] = lds_a[r * kPitch + c];
+                if constexpr (F::NIN == 2) {
+                    if (tb) y[i] = lds_b[r * kPitch + c];
+                } else {
+                    y[i] = x[i];
+                }
+                obase[(int64_t)r * ldr0 + c] = f(x[i], y[i]);
             }
         }
     }

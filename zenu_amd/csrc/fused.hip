@@ -334,7 +334,7 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_lines_kernel(const T *y, c
 {
     const int64_t line = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (colsum) {    // uniform; the host sends this only with R <= kLineRegs, inner == 1, one workgroup
-        __shared__ T lds[kWaves];
+        __shared__ T lds[kLineRegs * kWaves];
         const bool active = line < lines;
         const T g_total = CE ? (gout ? *gout : (T)1) / neg_n : (T)0;
         const int64_t base = (active ? line : 0) * R;
@@ -353,6 +353,8 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_lines_kernel(const T *y, c
                 sum = sum + t[r];
             }
         }
+        // the column sums in the order of block_red (butterfly inside a wavefront, then the wavefronts
+        // in index order), all columns behind ONE barrier instead of two per column
 #pragma unroll
         for (int r = 0; r < kLineRegs; r++) {
             if (r < R) {
@@ -360,9 +362,17 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_lines_kernel(const T *y, c
                 if (active) gx[base + r] = g;
                 T c = (T)0;
                 if (active) c = c + g;
-                c = block_red<T, false>(c, lds);
-                if (threadIdx.x == 0) colsum[r] = c;
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) c = c + __shfl_xor(c, o);
+                if ((threadIdx.x & 63) == 0) lds[r * kWaves + (threadIdx.x >> 6)] = c;
             }
+        }
+        __syncthreads();
+        if ((int64_t)threadIdx.x < R) {
+            T c = lds[threadIdx.x * kWaves];
+#pragma unroll
+            for (int w = 1; w < kWaves; w++) c = c + lds[threadIdx.x * kWaves + w];
+            colsum[threadIdx.x] = c;
         }
         return;
     }
@@ -480,6 +490,147 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_rows_kernel(const T *y, co
             for (int j = 0; j < VEC; j++) t.v[j] = t.v[j] - yv.v[j] * sum;
             store_pack<T, VEC, false>(gr + r, t);
         }
+    }
+}
+
+// ---- a classifier head's batch in ONE workgroup, four lanes per line -------------------------------------------
+// lines <= 256 of R <= 16 elements, contiguous (inner == 1).  One thread per line (the lines kernels
+// above) is a single wavefront per SIMD walking through 16 unrolled copies of exp / log / division:
+// 7-8 us for [256,10], most of it instruction fetch and dependent latencies that nothing overlaps.
+// Here a quad of lanes owns a line -- lane q holds elements q, q + 4, q + 8, q + 12 -- in a workgroup
+// of 1024 threads: four copies of the transcendental code, sixteen wavefronts.  Everything that the
+// one-thread form does in index order (the max scan, the sum of the exponentials, the sum of the
+// cross-entropy terms, the sum of t) is still done in index order, by every lane of the quad on
+// values gathered from its neighbours, so the bits are the same.
+constexpr int kHeadBlock = 1024;
+constexpr int kHeadLines = kHeadBlock / 4;
+constexpr int kHeadOwn = kLineRegs / 4;
+
+// full[r] for r = 4 i + q is own[i] of lane q of the quad
+template <typename T> __device__ __forceinline__ void quad_gather(const T (&own)[kHeadOwn], T (&full)[kLineRegs])
+{
+#pragma unroll
+    for (int i = 0; i < kHeadOwn; i++) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) full[4 * i + q] = __shfl(own[i], q, 4);
+    }
+}
+
+// Forward: y = softmax(x) per line, *loss = sum over lines of (sum_r target * log y) / neg_n, the row
+// terms folded as ce_finalize_kernel folds them (256 lanes: butterfly per wavefront, wavefronts in order).
+template <typename T>
+__global__ __launch_bounds__(kHeadBlock) void ce_head_forward_kernel(const T *x, T *y, int64_t lines, int64_t R,
+                                                                      const T *target, T *loss, T neg_n)
+{
+    __shared__ T terms[kHeadLines];
+    __shared__ T wave_sum[kHeadLines / 64];
+    const int q = threadIdx.x & 3;
+    const int64_t line = threadIdx.x >> 2;
+    const bool active = line < lines;
+    const int64_t base = (active ? line : 0) * R;
+    T v[kHeadOwn], tg[kHeadOwn];
+#pragma unroll
+    for (int i = 0; i < kHeadOwn; i++) {
+        const int r = 4 * i + q;
+        const int64_t off = base + (r < R ? r : 0);
+        v[i] = x[off];
+        tg[i] = target[off];
+    }
+    zmath::ExpLog<T> ml;
+    ml.init(true, true);
+    T full[kLineRegs];
+    quad_gather<T>(v, full);
+    T m = full[0];                       // max_axis: strict '>' from element 0 (max.rs:19-34)
+#pragma unroll
+    for (int r = 1; r < kLineRegs; r++)
+        if (r < R && full[r] > m) m = full[r];
+#pragma unroll
+    for (int i = 0; i < kHeadOwn; i++) v[i] = ml.exp(v[i] - m);
+    quad_gather<T>(v, full);
+    T sum = (T)0;                        // in index order from zero (sum.rs:20-25)
+#pragma unroll
+    for (int r = 0; r < kLineRegs; r++)
+        if (r < R) sum = sum + full[r];
+    T term[kHeadOwn];
+#pragma unroll
+    for (int i = 0; i < kHeadOwn; i++) {
+        const int r = 4 * i + q;
+        const T sm = v[i] / sum;
+        if (active && r < R) y[base + r] = sm;
+        term[i] = r < R ? tg[i] * ml.log(sm) : (T)0;
+    }
+    quad_gather<T>(term, full);
+    T acc = (T)0;
+#pragma unroll
+    for (int r = 0; r < kLineRegs; r++)
+        if (r < R) acc = acc + full[r];
+    if (q == 0) terms[line] = active ? (T)0 + acc : (T)0;
+    __syncthreads();
+    if (threadIdx.x < kHeadLines) {      // uniform per wavefront
+        T a = terms[threadIdx.x];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) a = a + __shfl_xor(a, o);
+        if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = a;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        T a = wave_sum[0];
+#pragma unroll
+        for (int w = 1; w < kHeadLines / 64; w++) a = a + wave_sum[w];
+        *loss = a / neg_n;
+    }
+}
+
+// Backward: gx = t - y * sum(t) with t = y * ((target * g_total) / y), and colsum[r] = the sum of gx over
+// the lines (when set), each column folded as block_red folds 256 lanes.
+template <typename T>
+__global__ __launch_bounds__(kHeadBlock) void ce_head_backward_kernel(const T *y, const T *target, T *gx, int64_t lines,
+                                                                       int64_t R, const T *gout, T neg_n, T *colsum)
+{
+    __shared__ T cols[kLineRegs][kHeadLines];      // gx by column, for the column sums
+    const int q = threadIdx.x & 3;
+    const int64_t line = threadIdx.x >> 2;
+    const bool active = line < lines;
+    const int64_t base = (active ? line : 0) * R;
+    const T g_total = (gout ? *gout : (T)1) / neg_n;
+    T yv[kHeadOwn], t[kHeadOwn];
+#pragma unroll
+    for (int i = 0; i < kHeadOwn; i++) {
+        const int r = 4 * i + q;
+        const int64_t off = base + (r < R ? r : 0);
+        yv[i] = y[off];
+        t[i] = target[off];
+    }
+#pragma unroll
+    for (int i = 0; i < kHeadOwn; i++) t[i] = yv[i] * ((t[i] * g_total) / yv[i]);
+    T full[kLineRegs];
+    quad_gather<T>(t, full);
+    T sum = (T)0;
+#pragma unroll
+    for (int r = 0; r < kLineRegs; r++)
+        if (r < R) sum = sum + full[r];
+#pragma unroll
+    for (int i = 0; i < kHeadOwn; i++) {
+        const int r = 4 * i + q;
+        const T g = t[i] - yv[i] * sum;
+        if (active && r < R) gx[base + r] = g;
+        if (colsum && r < R) cols[r][line] = active ? (T)0 + g : (T)0;
+    }
+    if (!colsum) return;                 // uniform
+    __syncthreads();
+    // wavefront w folds column w: four runs of 64 lines, each with the butterfly, then the runs in order
+    const int64_t col = threadIdx.x >> 6;
+    if (col < R) {
+        const int lane = threadIdx.x & 63;
+        T total = (T)0;
+#pragma unroll
+        for (int w = 0; w < kHeadLines / 64; w++) {
+            T c = cols[col][w * 64 + lane];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) c = c + __shfl_xor(c, o);
+            total = w == 0 ? c : total + c;
+        }
+        if (lane == 0) colsum[col] = total;
     }
 }
 
@@ -602,6 +753,13 @@ int softmax_forward_launch(const T *x, T *y, Geometry g, const T *target, T *row
 {
     constexpr int VEC = VecOf<T>::N;
     const int64_t lines = g.outer * g.inner;
+    if constexpr (CE) {
+        if (loss && g.inner == 1 && g.R <= kLineRegs && lines <= kHeadLines) {   // a classifier head: four lanes per line
+            ce_head_forward_kernel<T><<<1, kHeadBlock, 0, s>>>(x, y, lines, g.R, target, loss, neg_n);
+            ZENU_LAUNCH_CHECK();
+            return ZENU_OK;
+        }
+    }
     if (g.inner != 1 || g.R <= kLineMaxR) {
         const int64_t blocks = (lines + kBlock - 1) / kBlock;
         if (!grid_ok(blocks)) return ZENU_ERR_UNSUPPORTED;
@@ -630,6 +788,13 @@ int softmax_backward_launch(const T *y, const T *gy_or_target, T *gx, Geometry g
 {
     const int64_t lines = g.outer * g.inner;
     if (colsum && !(g.inner == 1 && g.R <= kLineRegs && lines <= kBlock)) return ZENU_ERR_UNSUPPORTED;
+    if constexpr (CE) {
+        if (g.inner == 1 && g.R <= kLineRegs && lines <= kHeadLines) {           // a classifier head: four lanes per line
+            ce_head_backward_kernel<T><<<1, kHeadBlock, 0, s>>>(y, gy_or_target, gx, lines, g.R, gout, neg_n, colsum);
+            ZENU_LAUNCH_CHECK();
+            return ZENU_OK;
+        }
+    }
     if (g.inner != 1 || g.R <= kLineMaxR) {
         const int64_t blocks = (lines + kBlock - 1) / kBlock;
         if (!grid_ok(blocks)) return ZENU_ERR_UNSUPPORTED;

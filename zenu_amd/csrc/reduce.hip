@@ -232,6 +232,7 @@ template <typename T> struct RedParams {
     int64_t outer_stride;
     int64_t elem_stride;
     int splits;              // workgroups along R
+    int cols_shift;          // column kernels: log2 of the lanes along the columns (chosen by the host)
     // results
     T *out_val;              // final value (may be null)
     int64_t *out_idx;        // final index (may be null)
@@ -664,8 +665,27 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(RedParams<T> p, uin
 #pragma unroll
             for (int j = 0; j < VEC; j++) lds[j * kBlock + threadIdx.x] = acc[j];   // [vector element][thread]: consecutive lanes, consecutive banks
             __syncthreads();
-            if (ty == 0) {   // row lane by row lane, the VEC columns side by side: ty_n - 1 dependent LDS round trips, not VEC times that
-                for (int w = 1; w < ty_n; w++) {
+            int left = ty_n;
+            if (ty_n > 8) {
+                // more than eight row lanes (narrow column tiles): row lanes 0..7 first take every
+                // eighth lane each, so that the chain of dependent LDS round trips is ty_n / 8 + 6 long
+                // instead of ty_n - 1
+                if (ty < 8) {
+                    for (int w = ty + 8; w < ty_n; w += 8) {
+#pragma unroll
+                        for (int j = 0; j < VEC; j++) acc[j] = Tr::merge(acc[j], lds[j * kBlock + w * tx_n + tx]);
+                    }
+                }
+                __syncthreads();
+                if (ty < 8) {
+#pragma unroll
+                    for (int j = 0; j < VEC; j++) lds[j * kBlock + threadIdx.x] = acc[j];
+                }
+                __syncthreads();
+                left = 8;
+            }
+            if (ty == 0) {   // row lane by row lane, the VEC columns side by side: dependent LDS round trips, but not VEC times as many
+                for (int w = 1; w < left; w++) {
 #pragma unroll
                     for (int j = 0; j < VEC; j++) acc[j] = Tr::merge(acc[j], lds[j * kBlock + w * tx_n + tx]);
                 }
@@ -903,6 +923,7 @@ int launch_rows(const RedParams<T> &p, hipStream_t s)
 }
 
 // threads along the columns for a cols launch: a power of two covering the row, at most kColsTx
+constexpr int64_t kSmallColsRows = 512, kSmallColsBytes = 4 << 20;   // see reduce_strided
 constexpr int kColsTx = 32;  // 32 lanes x 16 B = 512 B of a source row per wavefront half (measured best of 8..256)
 inline int cols_tx_shift(int64_t inner, int v)
 {
@@ -925,7 +946,7 @@ int launch_cols(const RedParams<T> &p, hipStream_t s)
     const bool vec = cols_vec_ok(p);
     const bool nt = vec && stream_source(p);
     const int v = vec ? VEC : 1;
-    const int shift = cols_tx_shift(p.inner, v);
+    const int shift = p.cols_shift;
     const int64_t per_tile = ((int64_t)1 << shift) * v;
     const int64_t col_tiles = (p.inner + per_tile - 1) / per_tile;
     const int64_t outer = p.nout / p.inner;
@@ -1014,11 +1035,19 @@ int reduce_strided(const T *src, int64_t outer, int64_t R, int64_t inner, int64_
     const bool use_cols = inner >= 16;
     if (pre_x && (!use_cols || !cols_vec_ok(p))) return ZENU_ERR_UNSUPPORTED;   // the caller falls back to two launches
     int64_t splits = 1, groups = nout;
+    p.cols_shift = 0;
     if (use_cols) {
         const int v = cols_vec_ok(p) ? VEC : 1;
-        const int shift = cols_tx_shift(inner, v);
-        const int64_t per_tile = ((int64_t)1 << shift) * v;
-        const int64_t col_tiles = (inner + per_tile - 1) / per_tile;
+        int shift = cols_tx_shift(inner, v);
+        auto tiles_at = [&](int sh) { return (inner + (((int64_t)1 << sh) * v) - 1) / (((int64_t)1 << sh) * v); };
+        // A small source with a short reduced axis is bound by latencies, and the hand-off of a split
+        // (about 3 us) is the longest of them: narrower column tiles (down to 128-byte row pieces, which
+        // stream at half the rate but there is little to stream) give more workgroups without one.
+        // Sum over axis 0 of [256,512] f32: 7.7 us as 4 tiles x 4 splits, 3.4 us as 16 tiles.
+        if (v > 1 && R <= kSmallColsRows && outer * R * inner * (int64_t)sizeof(T) <= kSmallColsBytes)
+            while (shift > 3 && outer * tiles_at(shift) < target_blocks) shift--;
+        p.cols_shift = shift;
+        const int64_t col_tiles = tiles_at(shift);
         const int64_t ty_n = kBlock >> shift;
         groups = outer * col_tiles;
         if (groups < target_blocks) {
