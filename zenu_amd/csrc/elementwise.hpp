@@ -532,12 +532,16 @@ __global__ __launch_bounds__(kBlock) void ew_rows_kernel(T *out, const T *a, con
 // a stand-alone probe, tiles walked along diagonals: 23.9 us, against 25.2 us with 256 threads and
 // four vectors each; 32x32 tiles with 256 threads copy as fast (24.1 us) but leave operands that
 // are not transposed with 128-byte row pieces.
-template <typename T> struct TileOf { static constexpr int N = sizeof(T) == 4 ? 64 : 32; };
+// SMALL halves the edge (32 / 16): few tiles of a small matrix leave most CUs idle and make each workgroup a
+// long chain; with a quarter of the tile per workgroup a transposed copy of [256,512] f32 takes 2.8 us
+// against 3.3 us, of [784,512] 3.4 against 3.6 (the MLP step of a 512-wide layer issues eleven of them).
+template <typename T, bool SMALL = false> struct TileOf { static constexpr int N = (sizeof(T) == 4 ? 64 : 32) / (SMALL ? 2 : 1); };
 // With two inputs (three streams, a + b^T) two vectors per thread and operand at 512 threads are the
 // fastest (stand-alone probe: 36.2 us with four at 256 threads, 35.5 us with two at 512, 35.7 us with
 // one at 1024).
-template <typename T, typename F> struct TileThreads {
-    static constexpr int value = F::NIN == 1 ? TileOf<T>::N * TileOf<T>::N / VecOf<T>::N : 512;
+template <typename T, typename F, bool SMALL = false> struct TileThreads {
+    static constexpr int kVecs = TileOf<T, SMALL>::N * TileOf<T, SMALL>::N / VecOf<T>::N;   // vectors per tile and operand
+    static constexpr int value = (F::NIN == 1 || kVecs < 512) ? kVecs : 512;
 };
 
 enum { kWalkRows = 0, kWalkCols = 1, kWalkDiagonal = 2 };
@@ -556,13 +560,13 @@ struct TileParams {
     uint32_t tiles_r_magic;     // min(floor(2^32 / tiles_r), 2^32 - 1): x mod tiles_r from one high multiply and a fix-up
 };
 
-template <typename T, bool NT, typename F>
-__global__ __launch_bounds__((TileThreads<T, F>::value)) void ew_tile_kernel(T *out, const T *a, const T *b,
-                                                                           TileParams p, F f)
+template <typename T, bool NT, typename F, bool SMALL = false>
+__global__ __launch_bounds__((TileThreads<T, F, SMALL>::value)) void ew_tile_kernel(T *out, const T *a, const T *b,
+                                                                                  TileParams p, F f)
 {
     constexpr int VEC = VecOf<T>::N;
-    constexpr int kTile = TileOf<T>::N;
-    constexpr int kBlock = TileThreads<T, F>::value;   // shadows the engine-wide 256
+    constexpr int kTile = TileOf<T, SMALL>::N;
+    constexpr int kBlock = TileThreads<T, F, SMALL>::value;   // shadows the engine-wide 256
     constexpr int kPitch = kTile + 1;
     // Eight lanes cover one 128-byte segment of a tile row; 32 segments per pass.  With eight (not
     // sixteen) lanes along the vector dim the 32 lanes that the LDS serves together -- eight
@@ -1086,36 +1090,47 @@ template <typename T, typename F> int launch_ew(EwProblem &p, F f, hipStream_t s
             for (int o = 1; o <= nin; o++)
                 if (!trans[o] && tp.ldc[o] == 0) vec = false;
             tp.vec_ok = vec ? 1 : 0;
-            constexpr int kTile = TileOf<T>::N;
-            tp.tiles_r = (tp.R + kTile - 1) / kTile;
-            tp.tiles_c = (tp.C + kTile - 1) / kTile;
-            {
-                const uint64_t m = (1ull << 32) / (uint64_t)tp.tiles_r;
-                tp.tiles_r_magic = m > 0xffffffffull ? 0xffffffffu : (uint32_t)m;
-            }
-            int64_t grid = tp.nbatch * tp.tiles_r * tp.tiles_c;
-            if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
-            tp.grid3d = (tp.tiles_r <= 65535 && tp.nbatch <= 65535) ? 1 : 0;
-            // Row by row unless a transposed input's pitch is within one row piece of a multiple of
-            // 4 KiB; then column by column if no other operand's pitch is, else along diagonals.
-            auto near_4k = [](int64_t elems) {
-                const int64_t r = ((elems < 0 ? -elems : elems) * (int64_t)sizeof(T)) % 4096;
-                return (r < 4096 - r ? r : 4096 - r) < kTile * (int64_t)sizeof(T);
+            // tile edge: halved when the full-size tiles would not give every CU two workgroups
+            auto launch_tiles = [&](auto small_c) -> int {
+                constexpr bool SMALL = decltype(small_c)::value;
+                constexpr int kTile = TileOf<T, SMALL>::N;
+                tp.tiles_r = (tp.R + kTile - 1) / kTile;
+                tp.tiles_c = (tp.C + kTile - 1) / kTile;
+                {
+                    const uint64_t m = (1ull << 32) / (uint64_t)tp.tiles_r;
+                    tp.tiles_r_magic = m > 0xffffffffull ? 0xffffffffu : (uint32_t)m;
+                }
+                int64_t grid = tp.nbatch * tp.tiles_r * tp.tiles_c;
+                if (grid > 0x7fffffffLL) return ZENU_ERR_UNSUPPORTED;
+                tp.grid3d = (tp.tiles_r <= 65535 && tp.nbatch <= 65535) ? 1 : 0;
+                // Row by row unless a transposed input's pitch is within one row piece of a multiple of
+                // 4 KiB; then column by column if no other operand's pitch is, else along diagonals.
+                auto near_4k = [](int64_t elems) {
+                    const int64_t r = ((elems < 0 ? -elems : elems) * (int64_t)sizeof(T)) % 4096;
+                    return (r < 4096 - r ? r : 4096 - r) < kTile * (int64_t)sizeof(T);
+                };
+                bool trans_near = false, direct_near = near_4k(tp.ldr[0]);
+                for (int o = 1; o <= nin; o++) {
+                    if (trans[o]) trans_near = trans_near || near_4k(tp.ldc[o]);
+                    else if (tp.ldc[o] == 1) direct_near = direct_near || near_4k(tp.ldr[o]);
+                }
+                tp.walk = !trans_near ? kWalkRows
+                          : (!direct_near && tp.grid3d && tp.tiles_c <= 65535) ? kWalkCols : kWalkDiagonal;
+                const bool by_cols = tp.walk == kWalkCols;
+                const dim3 g = !tp.grid3d ? dim3((unsigned)grid)
+                               : by_cols ? dim3((unsigned)tp.tiles_r, (unsigned)tp.tiles_c, (unsigned)tp.nbatch)
+                                         : dim3((unsigned)tp.tiles_c, (unsigned)tp.tiles_r, (unsigned)tp.nbatch);
+                const size_t lds = (size_t)(tp.trans_a + tp.trans_b) * kTile * (kTile + 1) * sizeof(T);
+                constexpr int kThreads = TileThreads<T, F, SMALL>::value;
+                if (nt) ew_tile_kernel<T, true, F, SMALL><<<g, kThreads, lds, stream>>>(out, a, b, tp, f);
+                else    ew_tile_kernel<T, false, F, SMALL><<<g, kThreads, lds, stream>>>(out, a, b, tp, f);
+                return ZENU_OK;
             };
-            bool trans_near = false, direct_near = near_4k(tp.ldr[0]);
-            for (int o = 1; o <= nin; o++) {
-                if (trans[o]) trans_near = trans_near || near_4k(tp.ldc[o]);
-                else if (tp.ldc[o] == 1) direct_near = direct_near || near_4k(tp.ldr[o]);
-            }
-            tp.walk = !trans_near ? kWalkRows
-                      : (!direct_near && tp.grid3d && tp.tiles_c <= 65535) ? kWalkCols : kWalkDiagonal;
-            const bool by_cols = tp.walk == kWalkCols;
-            const dim3 g = !tp.grid3d ? dim3((unsigned)grid)
-                           : by_cols ? dim3((unsigned)tp.tiles_r, (unsigned)tp.tiles_c, (unsigned)tp.nbatch)
-                                     : dim3((unsigned)tp.tiles_c, (unsigned)tp.tiles_r, (unsigned)tp.nbatch);
-            const size_t lds = (size_t)(tp.trans_a + tp.trans_b) * kTile * (kTile + 1) * sizeof(T);
-            if (nt) ew_tile_kernel<T, true, F><<<g, TileThreads<T, F>::value, lds, stream>>>(out, a, b, tp, f);
-            else    ew_tile_kernel<T, false, F><<<g, TileThreads<T, F>::value, lds, stream>>>(out, a, b, tp, f);
+            constexpr int kFullTile = TileOf<T>::N;
+            const int64_t full_tiles = tp.nbatch * ((tp.R + kFullTile - 1) / kFullTile) * ((tp.C + kFullTile - 1) / kFullTile);
+            const int rc_tiles = full_tiles < 2 * (int64_t)device_info().num_cus ? launch_tiles(std::true_type())
+                                                                                  : launch_tiles(std::false_type());
+            if (rc_tiles) return rc_tiles;
             ZENU_LAUNCH_CHECK();
             return ZENU_OK;
         }

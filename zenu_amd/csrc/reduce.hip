@@ -1041,11 +1041,12 @@ int reduce_strided(const T *src, int64_t outer, int64_t R, int64_t inner, int64_
         int shift = cols_tx_shift(inner, v);
         auto tiles_at = [&](int sh) { return (inner + (((int64_t)1 << sh) * v) - 1) / (((int64_t)1 << sh) * v); };
         // A small source with a short reduced axis is bound by latencies, and the hand-off of a split
-        // (about 3 us) is the longest of them: narrower column tiles (down to 128-byte row pieces, which
-        // stream at half the rate but there is little to stream) give more workgroups without one.
-        // Sum over axis 0 of [256,512] f32: 7.7 us as 4 tiles x 4 splits, 3.4 us as 16 tiles.
+        // (about 3 us) is the longest of them: narrower column tiles (down to 64-byte row pieces, which
+        // stream at less than half the rate, but there is little to stream) give more workgroups
+        // without one.  Column sums of [256,512] f32 with the ReLU-gradient transform: 7.7 us as
+        // 4 tiles x 4 splits, 5.8 us as 16 tiles of 32 columns, 5.0 us as 32 tiles of 16 columns.
         if (v > 1 && R <= kSmallColsRows && outer * R * inner * (int64_t)sizeof(T) <= kSmallColsBytes)
-            while (shift > 3 && outer * tiles_at(shift) < target_blocks) shift--;
+            while (shift > 2 && outer * tiles_at(shift) < target_blocks) shift--;
         p.cols_shift = shift;
         const int64_t col_tiles = tiles_at(shift);
         const int64_t ty_n = kBlock >> shift;
