@@ -213,7 +213,7 @@ def build_ops(z, workload, stream):
             return [fn(X.desc(), o0.desc(), o1.desc(), oi.as_ptr(), oa.as_ptr()) for X, o0, o1, oi, oa in sets]
         ops.append(Op(f"sum axis0 {dname}", "c2", dname, inb + 4096 * isz, x.size,
                       mk(lambda dx, d0, d1, pi, pa: (lambda: check(l.zenu_hip_sum_axis(dcode, ref(d0), ref(dx), 0, stream), "sum0"))),
-                      lambda: zo.sum_axis(x, 0), kernel=f"reduce_cols_kernel<{'float' if dname == 'f32' else 'double'}, SumTr, {16 // isz}, true>"))
+                      lambda: zo.sum_axis(x, 0), kernel=f"reduce_cols_regular_kernel<{'float' if dname == 'f32' else 'double'}, SumTr, {16 // isz}, true>"))
         ops.append(Op(f"sum axis1 {dname}", "c2", dname, inb + 8192 * isz, x.size,
                       mk(lambda dx, d0, d1, pi, pa: (lambda: check(l.zenu_hip_sum_axis(dcode, ref(d1), ref(dx), 1, stream), "sum1"))),
                       lambda: zo.sum_axis(x, 1)))
@@ -651,7 +651,7 @@ def capture_and_replay_c4(z, st, args, sync):
 TRAFFIC_PROFILES = {
     "adamw 25M": ("adam_kernel_c3_adamw25M_pmc_traffic.txt",
                   ("zenu_amd/csrc/optim.hip", "zenu_amd/csrc/vecmem.hpp", "zenu_amd/csrc/common.hpp")),
-    "sum axis0 f64": ("reduce_cols_kernel_c2_sum_axis0_f64_pmc_traffic.txt",
+    "sum axis0 f64": ("reduce_cols_regular_kernel_c2_sum_axis0_f64_pmc_traffic.txt",
                       ("zenu_amd/csrc/reduce.hip", "zenu_amd/csrc/vecmem.hpp", "zenu_amd/csrc/common.hpp")),
 }
 
