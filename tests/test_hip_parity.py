@@ -1047,7 +1047,11 @@ def test_sum_determinism(hip):
 
 RED_SHAPES = [(1,), (5,), (1000,), (100000,), (3, 4), (4, 3), (1, 7), (7, 1), (2, 3, 4, 5), (17, 1, 33),
               (64, 1025), (1025, 64), (3, 1000, 7), (300, 17, 40), (2, 2, 2, 2, 2, 3), (4096, 10), (10, 4096),
-              (256, 10), (9, 100003)]
+              (256, 10), (9, 100003),
+              # small sources reduced without a split on narrow column tiles; narrow inner runs whose row
+              # lanes (16, 32, 64 of them) are combined in two levels, with and without a split
+              (256, 512), (512, 2048), (300, 516), (17, 4096), (500, 24), (5000, 20), (700, 72), (2000, 100),
+              (3, 300, 40), (511, 16)]
 
 
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
