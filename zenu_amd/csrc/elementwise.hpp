@@ -131,7 +131,7 @@ template <typename T, int FN> struct UnaryF {
     {
         if constexpr (FN == ZENU_EXP) return m.exp(a);
         else if constexpr (FN == ZENU_LOG) return m.log(a);
-        else if constexpr (FN == ZENU_TANH) return dev_tanh(a, tr);
+        else if constexpr (FN == ZENU_TANH) return m.tanh(a, tr);
         else if constexpr (FN == ZENU_SQRT) return sqrt(a);
         else if constexpr (FN == ZENU_ABS) return fabs(a);
         else if constexpr (FN == ZENU_SIN) return dev_sin(a, sc.k);
@@ -148,7 +148,7 @@ template <typename T, int FN> struct UnaryF {
         }
         else if constexpr (FN == ZENU_SINH) return m.sinh(a, tr);
         else if constexpr (FN == ZENU_COSH) return m.cosh(a, tr);
-        else return dev_sigmoid(a, tr);
+        else return m.sigmoid(a, tr);
     }
 };
 

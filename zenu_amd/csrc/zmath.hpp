@@ -473,6 +473,26 @@ ZM_HD float expf_glibc(float x, const uint64_t *tab, const ExpfCoef &k = ExpfCoe
     return (float)y;
 }
 
+// The main path alone, for callers whose argument cannot overflow or underflow (|x| < 87): the
+// operations of expf_glibc on such an argument, nothing else.
+ZM_HD float expf_glibc_core(float x, const uint64_t *tab, const ExpfCoef &k = ExpfCoef())
+{
+    const double xd = (double)x;
+    const double z = k.inv_ln2n * xd;
+    double kd = z + k.shift;
+    const uint64_t ki = d2u(kd);
+    kd -= k.shift;
+    const double r = __builtin_fma(k.inv_ln2n, xd, -kd);
+    const uint64_t t = tab[ki % 32] + (ki << (52 - 5));
+    const double s = u2d(t);
+    const double p = __builtin_fma(k.c0, r, k.c1);
+    const double r2 = r * r;
+    double y = __builtin_fma(k.c2, r, 1.0);
+    y = __builtin_fma(p, r2, y);
+    y = y * s;
+    return (float)y;
+}
+
 // The same expf without a branch, for kernels whose scalar unit is the busy one (a branch per element
 // is half a dozen scalar instructions): the main path runs on any bit pattern (the table index is
 // taken modulo the table size; a NaN stays a NaN), overflow and underflow are two selects.  Same
@@ -1136,12 +1156,25 @@ ZM_HD const uint64_t *exp_table()
 #endif
 }
 
-ZM_HD double exp_glibc(double x, const uint64_t *tab)
+// The constants of the f64 routines as data: handed to a kernel as part of its argument they sit in
+// scalar registers and feed the f64 operations directly; written as literals each one is moved into
+// a register pair before every use, two scalar instructions per constant and element, and the one
+// scalar unit of a CU serves all four SIMDs.
+struct ExpCoef64 {
+    double inv_ln2n = 0x1.71547652b82fep0 * 128, neg_ln2hi_n = -0x1.62e42fefa0000p-8, neg_ln2lo_n = -0x1.cf79abc9e3b3ap-47,
+           shift = 0x1.8p52;
+    double c2 = 0x1.ffffffffffdbdp-2, c3 = 0x1.555555555543cp-3, c4 = 0x1.55555cf172b91p-5, c5 = 0x1.1111167a4d017p-7;
+};
+struct Expm1Coef64 {   // fdlibm's expm1: ln2 in two parts, 1/ln2, Q1..Q5
+    double ln2_hi = 0x1.62e42feep-1, ln2_lo = 0x1.a39ef35793c76p-33, invln2 = 0x1.71547652b82fep+0;
+    double q1 = -0x1.11111111110f4p-5, q2 = 0x1.a01a019fe5585p-10, q3 = -0x1.4ce199eaadbb7p-14, q4 = 0x1.0cfca86e65239p-18,
+           q5 = -0x1.afdb76e09c32dp-23;
+};
+
+ZM_HD double exp_glibc(double x, const uint64_t *tab, const ExpCoef64 &k = ExpCoef64())
 {
-    const double InvLn2N = 0x1.71547652b82fep0 * 128, NegLn2hiN = -0x1.62e42fefa0000p-8,
-                 NegLn2loN = -0x1.cf79abc9e3b3ap-47, Shift = 0x1.8p52;
-    const double C2 = 0x1.ffffffffffdbdp-2, C3 = 0x1.555555555543cp-3, C4 = 0x1.55555cf172b91p-5,
-                 C5 = 0x1.1111167a4d017p-7;
+    const double InvLn2N = k.inv_ln2n, NegLn2hiN = k.neg_ln2hi_n, NegLn2loN = k.neg_ln2lo_n, Shift = k.shift;
+    const double C2 = k.c2, C3 = k.c3, C4 = k.c4, C5 = k.c5;
     uint32_t abstop = (uint32_t)(d2u(x) >> 52) & 0x7ffu;
     if (abstop - 0x3c9u >= 0x408u - 0x3c9u) {            // |x| < 2^-54, |x| >= 512, inf or NaN
         if (abstop - 0x3c9u >= 0x80000000u) return 1.0 + x;
@@ -1185,6 +1218,23 @@ ZM_HD double exp_glibc(double x, const uint64_t *tab)
     return __builtin_fma(scale, tmp, scale);
 }
 ZM_HD double exp_glibc(double x) { return exp_glibc(x, exp_table()); }
+// the main path alone, for callers whose argument needs none of the special cases (2^-54 <= |x| < 512)
+ZM_HD double exp_glibc_core(double x, const uint64_t *tab, const ExpCoef64 &k = ExpCoef64())
+{
+    const double z = k.inv_ln2n * x;
+    double kd = z + k.shift;
+    const uint64_t ki = d2u(kd);
+    kd -= k.shift;
+    const double r = __builtin_fma(kd, k.neg_ln2lo_n, __builtin_fma(kd, k.neg_ln2hi_n, x));
+    const uint64_t idx = 2 * (ki % 128);
+    const uint64_t top = ki << (52 - 7);
+    const double tail = u2d(tab[idx]);
+    const uint64_t sbits = tab[idx + 1] + top;
+    const double r2 = r * r;
+    const double tmp = __builtin_fma(r2 * r2, __builtin_fma(r, k.c5, k.c4), __builtin_fma(r2, __builtin_fma(r, k.c3, k.c2), tail + r));
+    const double scale = u2d(sbits);
+    return __builtin_fma(scale, tmp, scale);
+}
 
 // ---- double precision: fdlibm s_expm1.c / s_tanh.c as shipped by glibc 2.35 (generic dbl-64) ----------
 
@@ -1337,12 +1387,11 @@ ZM_HD double tanh_fdlibm(double x)
 //     A = 1 - 2^-k, whose bit pattern comes out as 1 for the negative k; |x| >= 1 decides which;
 //   * |x| >= 6.5 (k could reach 20), infinities and NaN go to tanh_fdlibm.
 // The core works on a2 = 2|x|; the sigmoid passes |x| (see sigmoidf_zenu).
-ZM_HD double tanh_simd_core(double a2, double x)
+ZM_HD double tanh_simd_core(double a2, double x, const Expm1Coef64 &ck = Expm1Coef64())
 {
     const double one = 1.0, two = 2.0;
-    const double ln2_hi = u2d(0x3fe62e42fee00000ull), ln2_lo = u2d(0x3dea39ef35793c76ull), invln2 = u2d(0x3ff71547652b82feull);
-    const double Q1 = u2d(0xBFA11111111110F4ull), Q2 = u2d(0x3F5A01A019FE5585ull), Q3 = u2d(0xBF14CE199EAADBB7ull),
-                 Q4 = u2d(0x3ED0CFCA86E65239ull), Q5 = u2d(0xBE8AFDB76E09C32Dull);
+    const double ln2_hi = ck.ln2_hi, ln2_lo = ck.ln2_lo, invln2 = ck.invln2;
+    const double Q1 = ck.q1, Q2 = ck.q2, Q3 = ck.q3, Q4 = ck.q4, Q5 = ck.q5;
     const bool big = a2 >= two;              // |x| >= 1: expm1(+2|x|), else expm1(-2|x|)
     const double a = big ? a2 : -a2;
     int32_t k = (int32_t)(invln2 * a + (big ? 0.5 : -0.5));
@@ -1379,24 +1428,24 @@ ZM_HD double tanh_simd_core(double a2, double x)
 
 ZM_RARE double tanh_rare(double x) { return tanh_fdlibm(x); }
 
-ZM_HD double tanh_simd(double x)
+ZM_HD double tanh_simd(double x, const Expm1Coef64 &ck = Expm1Coef64())
 {
     const double ax = u2d(d2u(x) & 0x7fffffffffffffffull);
     if (__builtin_expect(!(ax < 6.5), 0)) return tanh_rare(x);
-    return tanh_simd_core(ax + ax, x);
+    return tanh_simd_core(ax + ax, x, ck);
 }
 
 // ZeNu's sigmoid composite in f64: tanh(x/2) needs 2|x/2| = |x| (where x/2 underflows and rounds,
 // tanh is below 2^-1022 either way and vanishes against 0.5); 0.5 tanh is exact or vanishes, so
 // the last two steps are one fused multiply-add
-ZM_HD double sigmoid_zenu(double x)
+ZM_HD double sigmoid_zenu(double x, const Expm1Coef64 &ck = Expm1Coef64())
 {
     const double ax = u2d(d2u(x) & 0x7fffffffffffffffull);
     if (__builtin_expect(!(ax < 13.0), 0)) {
         const double th = tanh_rare(x * 0.5);
         return 0.5 + 0.5 * th;
     }
-    return __builtin_fma(0.5, tanh_simd_core(ax, x), 0.5);
+    return __builtin_fma(0.5, tanh_simd_core(ax, x, ck), 0.5);
 }
 
 // sinh / cosh in f64 (fdlibm e_sinh.c / e_cosh.c as glibc 2.35 ships them) over the expm1 and exp above
@@ -1430,12 +1479,11 @@ ZM_HD double sinh_fdlibm(double x, const uint64_t *etab)
 // (k could reach 20), infinities and NaN go to sinh_fdlibm; |x| < 2^-28 returns x as in the sources.
 ZM_RARE double sinh_rare(double x, const uint64_t *etab) { return sinh_fdlibm(x, etab); }
 
-ZM_HD double sinh_simd(double x, const uint64_t *etab)
+ZM_HD double sinh_simd(double x, const uint64_t *etab, const Expm1Coef64 &ck = Expm1Coef64())
 {
     const double one = 1.0;
-    const double ln2_hi = u2d(0x3fe62e42fee00000ull), ln2_lo = u2d(0x3dea39ef35793c76ull), invln2 = u2d(0x3ff71547652b82feull);
-    const double Q1 = u2d(0xBFA11111111110F4ull), Q2 = u2d(0x3F5A01A019FE5585ull), Q3 = u2d(0xBF14CE199EAADBB7ull),
-                 Q4 = u2d(0x3ED0CFCA86E65239ull), Q5 = u2d(0xBE8AFDB76E09C32Dull);
+    const double ln2_hi = ck.ln2_hi, ln2_lo = ck.ln2_lo, invln2 = ck.invln2;
+    const double Q1 = ck.q1, Q2 = ck.q2, Q3 = ck.q3, Q4 = ck.q4, Q5 = ck.q5;
     const double a = u2d(d2u(x) & 0x7fffffffffffffffull);
     if (__builtin_expect(!(a < 13.0), 0)) return sinh_rare(x, etab);
     const uint32_t ix = hi_word(a);
@@ -1503,14 +1551,13 @@ ZM_HD double cosh_fdlibm(double x, const uint64_t *etab)
 // expm1 brings all of its branches along; below 2^-54, where it returns its argument, and below 2^-55,
 // where cosh returns 1, the k = 0 formula gives the same), exp above, |x| >= 22 out of line.
 ZM_RARE double cosh_rare(double x, const uint64_t *etab) { return cosh_fdlibm(x, etab); }
-ZM_HD double cosh_simd(double x, const uint64_t *etab)
+ZM_HD double cosh_simd(double x, const uint64_t *etab, const Expm1Coef64 &ck = Expm1Coef64(), const ExpCoef64 &ek = ExpCoef64())
 {
     const double one = 1.0, half = 0.5;
     const double a = u2d(d2u(x) & 0x7fffffffffffffffull);
     if (__builtin_expect(!(a < 22.0), 0)) return cosh_rare(x, etab);
     if (hi_word(a) < 0x3fd62e43u) {                      // |x| < 0.5 ln2
-        const double Q1 = u2d(0xBFA11111111110F4ull), Q2 = u2d(0x3F5A01A019FE5585ull), Q3 = u2d(0xBF14CE199EAADBB7ull),
-                     Q4 = u2d(0x3ED0CFCA86E65239ull), Q5 = u2d(0xBE8AFDB76E09C32Dull);
+        const double Q1 = ck.q1, Q2 = ck.q2, Q3 = ck.q3, Q4 = ck.q4, Q5 = ck.q5;
         const double hfx = half * a;
         const double hxs = a * hfx;
         const double R1 = one + hxs * Q1;
@@ -1525,7 +1572,7 @@ ZM_HD double cosh_simd(double x, const uint64_t *etab)
         const double w = one + t;
         return one + (t * t) / (w + w);
     }
-    const double t = exp_glibc(a, etab);
+    const double t = exp_glibc_core(a, etab, ek);        // 0.34 <= a < 22: none of exp's special cases
     return half * t + half / t;
 }
 
@@ -1666,7 +1713,7 @@ ZM_HD float sinhf_simd(float x, const uint64_t *etab, const TanhRegs &rg = TanhR
 
 // coshf with the same means: below 0.5 ln2 expm1's k = 0 path (no argument reduction), from there to
 // 22 expf; the quotients are div_tanh's.  |x| >= 22, infinities and NaN go to coshf_fdlibm.
-ZM_HD float coshf_simd(float x, const uint64_t *etab, const TanhRegs &rg = TanhRegs())
+ZM_HD float coshf_simd(float x, const uint64_t *etab, const TanhRegs &rg = TanhRegs(), const ExpfCoef &ek = ExpfCoef())
 {
     const float one = 1.0f, half = 0.5f;
     const float a = u2f(f2u(x) & 0x7fffffffu);
@@ -1686,7 +1733,9 @@ ZM_HD float coshf_simd(float x, const uint64_t *etab, const TanhRegs &rg = TanhR
         const float w = one + t;
         return one + div_tanh(t * t, w + w);
     }
-    const float t = expf_glibc(a, etab);
+    // 0.34 <= a < 22: expf's main path without its range checks, its f64 constants from the caller
+    // (a kernel holds them in scalar registers; as literals each costs two scalar moves per use)
+    const float t = expf_glibc_core(a, etab, ek);
     return half * t + div_tanh(half, t);
 }
 
@@ -1700,6 +1749,8 @@ ZM_HD float coshf_fdlibm(float x) { return coshf_fdlibm(x, exp2f_table()); }
 template <typename T> struct ExpLog;
 template <> struct ExpLog<double> {
     const uint64_t *etab;
+    ExpCoef64 ek;
+    Expm1Coef64 mk;
     __device__ __forceinline__ void init(bool need_exp, bool)
     {
         __shared__ uint64_t lds_exp64[256];
@@ -1710,13 +1761,16 @@ template <> struct ExpLog<double> {
         __syncthreads();
         etab = lds_exp64;
     }
-    __device__ __forceinline__ double exp(double x) const { return exp_glibc(x, etab); }
-    __device__ __forceinline__ double exp_flat(double x) const { return exp_glibc(x, etab); }
+    __device__ __forceinline__ double exp(double x) const { return exp_glibc(x, etab, ek); }
+    __device__ __forceinline__ double exp_flat(double x) const { return exp_glibc(x, etab, ek); }
     __device__ __forceinline__ double log(double x) const { return ::log(x); }
-    __device__ __forceinline__ double sinh(double x) const { return sinh_simd(x, etab); }
-    __device__ __forceinline__ double cosh(double x) const { return cosh_simd(x, etab); }
-    __device__ __forceinline__ double sinh(double x, const TanhRegs &) const { return sinh_simd(x, etab); }
-    __device__ __forceinline__ double cosh(double x, const TanhRegs &) const { return cosh_simd(x, etab); }
+    __device__ __forceinline__ double sinh(double x) const { return sinh_simd(x, etab, mk); }
+    __device__ __forceinline__ double cosh(double x) const { return cosh_simd(x, etab, mk, ek); }
+    __device__ __forceinline__ double sinh(double x, const TanhRegs &) const { return sinh_simd(x, etab, mk); }
+    __device__ __forceinline__ double cosh(double x, const TanhRegs &) const { return cosh_simd(x, etab, mk, ek); }
+    // no table: usable without init()
+    __device__ __forceinline__ double tanh(double x, const TanhRegs &) const { return tanh_simd(x, mk); }
+    __device__ __forceinline__ double sigmoid(double x, const TanhRegs &) const { return sigmoid_zenu(x, mk); }
 };
 template <> struct ExpLog<float> {
     const uint64_t *etab;
@@ -1739,10 +1793,13 @@ template <> struct ExpLog<float> {
     __device__ __forceinline__ float exp_flat(float x) const { return expf_glibc_flat(x, etab, ek); }
     __device__ __forceinline__ float log(float x) const { return logf_glibc(x, ltab, lk); }
     __device__ __forceinline__ float sinh(float x) const { return sinhf_simd(x, etab); }
-    __device__ __forceinline__ float cosh(float x) const { return coshf_simd(x, etab); }
+    __device__ __forceinline__ float cosh(float x) const { return coshf_simd(x, etab, TanhRegs(), ek); }
     // with the two register-held constants of the expm1 core pinned by the caller
     __device__ __forceinline__ float sinh(float x, const TanhRegs &rg) const { return sinhf_simd(x, etab, rg); }
-    __device__ __forceinline__ float cosh(float x, const TanhRegs &rg) const { return coshf_simd(x, etab, rg); }
+    __device__ __forceinline__ float cosh(float x, const TanhRegs &rg) const { return coshf_simd(x, etab, rg, ek); }
+    // no table: usable without init()
+    __device__ __forceinline__ float tanh(float x, const TanhRegs &rg) const { return tanhf_simd(x, rg); }
+    __device__ __forceinline__ float sigmoid(float x, const TanhRegs &rg) const { return sigmoidf_zenu(x, rg); }
 };
 
 // atanf's range table in LDS, same arrangement (init() by every thread of the workgroup, once)
