@@ -1121,6 +1121,50 @@ def test_reduction_views_reduced_in_place(hip, dt):
             assert_bits(V.max_axis(axis, True).to_numpy(), zo.max_axis(v, axis, True), what)
 
 
+@pytest.mark.parametrize("seed", range(int(os.environ.get("ZENU_FUZZ_SEEDS", "6"))))
+def test_reduction_geometry_fuzz(hip, seed):
+    """seeded random reduction geometries: 1-4 dims drawn from small, medium and large sizes (up to
+    about 2 M elements), a random axis, contiguous or transposed or row-sliced sources, f32 and f64 --
+    which kernel, tile width, split count and hand-off a reduction takes is decided from these.
+    Integer-valued data: the sums are exact whatever the order, ties are common; sum, max and arg-max
+    must be the oracle's bits."""
+    r = rng(7000 + seed)
+    for case in range(30):
+        nd = int(r.integers(1, 5))
+        budget = 2_000_000
+        shape = []
+        for d in range(nd):
+            kind = r.random()
+            hi = 9 if kind < 0.35 else (600 if kind < 0.8 else 70000)
+            n = int(r.integers(1, max(2, min(hi, budget) + 1)))
+            shape.append(n)
+            budget = max(1, budget // n)
+        shape = tuple(shape)
+        dt = np.float32 if r.random() < 0.6 else np.float64
+        base = r.integers(-8, 9, size=shape).astype(dt)
+        kind = r.random()
+        if nd >= 2 and kind < 0.3:
+            p = list(range(nd))
+            i, j = r.choice(nd, 2, replace=False)
+            p[i], p[j] = p[j], p[i]
+            v = base.transpose(p)
+        elif kind < 0.5 and shape[0] >= 4:
+            v = base[1::2]
+        else:
+            v = base
+        V = dev_view(hip, base, v)
+        axis = int(r.integers(0, v.ndim))
+        what = f"seed {seed} case {case}: {v.shape} strides {v.strides} axis {axis} {np.dtype(dt).name}"
+        print(what, flush=True)
+        assert_bits(V.sum(axis).to_numpy(), zo.sum_axis(v, axis), what)
+        assert_bits(V.sum(axis, True).to_numpy(), zo.sum_axis(v, axis, True), what + " keep_dim")
+        assert np.array_equal(np.array(V.max_axis_idx_ravel(axis)), zo.max_axis_idx_ravel(v, axis)), what
+        assert_bits(V.max_axis(axis).to_numpy(), zo.max_axis(v, axis), what)
+        if case % 5 == 0:
+            assert tuple(V.max_idx()) == tuple(zo.max_idx(v)), what
+            assert float(V.sum_all().to_numpy()) == float(v.astype(np.float64).sum()), what + " sum_all"
+
+
 def dev_view_on(hip, M, base, view):
     off = (view.__array_interface__["data"][0] - base.__array_interface__["data"][0]) // base.itemsize
     return hip.Matrix(M.buf, off, view.shape, tuple(s // base.itemsize for s in view.strides), base.dtype)
