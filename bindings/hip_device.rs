@@ -978,3 +978,31 @@ pub fn download<T: Num>(host: *mut T, dev: *const T, len: usize) {
 pub fn init(device: i32) {
     ok(unsafe { zenu_hip_init(device) });
 }
+
+/// Optional start-up check of the one thing the bit-exact f32 functions take on trust from the GPU
+/// they run on: `tanh`, the sigmoid, `sinh`, `cosh`, `atan`, `asin` and `acos` divide (and take square
+/// roots) with a short device sequence that is only correct on their own operand ranges.  The library
+/// evaluates each function with that sequence and with the IEEE operations on all 2^32 arguments
+/// (10-80 ms per function) and counts the arguments whose results differ; anything but zero is an error.
+pub fn self_check() -> Result<(), String> {
+    const FUNCTIONS: [(c_int, &str); 7] = [
+        (ZENU_TANH, "tanh"),
+        (ZENU_SIGMOID, "sigmoid"),
+        (ZENU_SINH, "sinh"),
+        (ZENU_COSH, "cosh"),
+        (ZENU_ATAN, "atan"),
+        (ZENU_ASIN, "asin"),
+        (ZENU_ACOS, "acos"),
+    ];
+    for (function, name) in FUNCTIONS {
+        let mut mismatches: u64 = 0;
+        let mut example: u32 = 0;
+        ok(unsafe { zenu_hip_selfcheck_short_division(function, &mut mismatches, &mut example, current_stream()) });
+        if mismatches != 0 {
+            return Err(format!(
+                "{name}: {mismatches} of 2^32 f32 arguments differ between the short and the IEEE division, e.g. bits {example:#010x}"
+            ));
+        }
+    }
+    Ok(())
+}
