@@ -529,7 +529,7 @@ ZM_HD float logf_glibc_full(float x, const double *tab)
     if (ix - 0x00800000u >= 0x7f800000u - 0x00800000u) { // x < 2^-126, inf or NaN
         if (ix * 2 == 0) return u2f(0xff800000u);        // log(+-0) = -inf
         if (ix == 0x7f800000u) return x;                 // log(inf) = inf
-        if ((ix & 0x80000000u) || ix * 2 >= 0xff000000u) return (x - x) / (x - x);   // NaN
+        if ((ix & 0x80000000u) || ix * 2 >= 0xff000000u) return (x - x) * u2f(0x7f800000u);   // NaN: the sources' (x - x) / (x - x) without the division
         ix = f2u(x * 0x1p23f);                           // subnormal: normalise
         ix -= 23u << 23;
     }
@@ -612,7 +612,7 @@ ZM_HD float powf_glibc_full(float x, float y, const uint64_t *etab, const double
         }
         if (ix & 0x80000000u) {                          // finite x < 0
             const int yint = powf_checkint(iy);
-            if (yint == 0) return (x - x) / (x - x);
+            if (yint == 0) return (x - x) * u2f(0x7f800000u);   // NaN: the sources' (x - x) / (x - x) without the division
             if (yint == 1) sign_bias = 1u << (5 + 11);
             ix &= 0x7fffffffu;
         }
@@ -1013,7 +1013,9 @@ ZM_HD float asinf_fdlibm(float x)
     const uint32_t hx = f2u(x);
     const uint32_t ix = hx & 0x7fffffffu;
     if (ix == 0x3f800000u) return x * pio2_hi + x * pio2_lo;     // asin(+-1) = +-pi/2
-    if (ix > 0x3f800000u) return (x - x) / (x - x);              // |x| > 1, NaN
+    // |x| > 1, NaN: the sources' (x - x) / (x - x); a NaN either way, without the division (a third of
+    // normally distributed arguments end here, and a division is eleven instructions for the whole wavefront)
+    if (ix > 0x3f800000u) return (x - x) * u2f(0x7f800000u);
     // both ranges evaluate the same polynomial, of x^2 below 0.5 and of (1 - |x|) / 2 above: once here
     const bool small = ix < 0x3f000000u;                 // |x| < 0.5
     if (small && ix < 0x32000000u) return x;             // |x| < 2^-27
@@ -1045,7 +1047,7 @@ ZM_HD float acosf_fdlibm(float x)
     const uint32_t ix = hx & 0x7fffffffu;
     const bool neg = (hx >> 31) != 0;
     if (ix == 0x3f800000u) return neg ? pi + 2.0f * pio2_lo : 0.0f;   // acos(-1) = pi, acos(1) = 0
-    if (ix > 0x3f800000u) return (x - x) / (x - x);                   // |x| > 1, NaN
+    if (ix > 0x3f800000u) return (x - x) * u2f(0x7f800000u);          // |x| > 1, NaN: the sources' (x - x) / (x - x) without the division
     // the three ranges evaluate the same rational function p(z) / q(z), of x^2, (1 + x) / 2 or
     // (1 - x) / 2: once here, whatever mix of ranges a wavefront holds
     const bool small = ix < 0x3f000000u;                 // |x| < 0.5
