@@ -418,6 +418,18 @@ int zenu_hip_adam_step_multi_scheduled(int dtype, int n_tensors, void *const *p_
  * (the short forms have no operand scaling): a check of the check.  Blocking; a few tens of milliseconds per function.  No counterpart in the reference. */
 int zenu_hip_selfcheck_short_division(int fn, uint64_t *mismatches, uint32_t *example_bits,
                                       zenu_stream_t stream);
+/* Every f32 bit pattern of [first, first + count) through unary function fn (a zenu_unop_t value:
+ * exp, log, tanh, sigmoid, sin, cos, asin, acos, atan, sinh, cosh -- the functions whose results are
+ * meant to be a host libm's bits), folded on the device into one 64-bit sum per block of
+ * 2^block_log2 patterns (8 <= block_log2 <= 32; count a multiple of the block size):
+ * sums_dev[b] = sum over the block of T(argument bits, result bits) mod 2^64, T = the finalizer of
+ * splitmix64 applied to (argument << 32 | result), every NaN result counted as 0x7fc00000.  A
+ * caller that folds the results of ITS libm the same way learns, without copying a result, whether
+ * the device returns that libm's bits on every argument (the whole range takes the device 0.1-0.2 s
+ * per function; 16 host threads need 10-20 s).  Asynchronous on `stream`.  No counterpart in the
+ * reference. */
+int zenu_hip_unary_range_hash(int fn, uint64_t first, uint64_t count, int block_log2,
+                              uint64_t *sums_dev, zenu_stream_t stream);
 int zenu_hip_last_status(void);
 
 #define ZENU_DECL_1D(T, S)                                                                        \

@@ -188,3 +188,93 @@ int zo_larger_shape(int nx, const int64_t *x, int ny, const int64_t *y)
 #define ZO_COSH_FN cosh
 #define ZO_POW_FN pow
 #include "zenu_oracle_impl.inc"
+
+/* ------------------------------------------------------------------ */
+/* Every f32 bit pattern of a range through one unary function, folded   */
+/* into a 64-bit sum per block of patterns.  The library computes the    */
+/* same sums on the device (zenu_hip_unary_range_hash); equal sums mean  */
+/* equal results on every argument of the block, with nothing copied.    */
+/* The functions are the libm calls of zo_unary_fn_f32 and the sigmoid   */
+/* composite of zo_sigmoid_f32 (x*half, tanh, half*t, half+u, each        */
+/* rounded to f32).  Threads only split the range.                       */
+/* ------------------------------------------------------------------ */
+#include <pthread.h>
+
+/* one term: the argument's and the result's bits through the finalizer of splitmix64; every NaN counts as one value */
+uint64_t zo_range_hash_term(uint32_t arg_bits, uint32_t res_bits)
+{
+    if ((res_bits & 0x7fffffffu) > 0x7f800000u) res_bits = 0x7fc00000u;
+    uint64_t z = ((uint64_t)arg_bits << 32) | res_bits;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+}
+
+static inline float zo_range_fn(int fn, float x)
+{
+    if (fn == ZO_SIGMOID_COMPOSITE) {
+        const float half = 1.0f / (1.0f + 1.0f);
+        const float t1 = x * half;
+        const float t2 = tanhf(t1);
+        const float t3 = half * t2;
+        return half + t3;
+    }
+    return zo_unary_fn_f32(fn, x);
+}
+
+typedef struct {
+    int fn, block_log2;
+    uint64_t first_block, n_blocks, first;
+    uint64_t *sums;
+} zo_range_job;
+
+static void *zo_range_worker(void *arg)
+{
+    const zo_range_job *j = (const zo_range_job *)arg;
+    const uint64_t per = 1ull << j->block_log2;
+    for (uint64_t b = j->first_block; b < j->first_block + j->n_blocks; b++) {
+        uint64_t sum = 0;
+        const uint64_t start = j->first + b * per;
+        for (uint64_t i = 0; i < per; i++) {
+            const uint32_t bits = (uint32_t)(start + i);
+            float x, y;
+            uint32_t rb;
+            memcpy(&x, &bits, 4);
+            y = zo_range_fn(j->fn, x);
+            memcpy(&rb, &y, 4);
+            sum += zo_range_hash_term(bits, rb);
+        }
+        j->sums[b] = sum;
+    }
+    return NULL;
+}
+
+/* sums[b] for the patterns first + b * 2^block_log2 ... of `count` patterns (a multiple of the block size) */
+int zo_unary_range_hash_f32(int fn, uint64_t first, uint64_t count, int block_log2, uint64_t *sums, int nthreads)
+{
+    if (block_log2 < 0 || block_log2 > 32 || (count & ((1ull << block_log2) - 1)) || first + count > (1ull << 32))
+        return ZO_ERR_ARG;
+    if (fn < ZO_EXP || fn > ZO_SIGMOID_COMPOSITE) return ZO_ERR_ARG;
+    const uint64_t blocks = count >> block_log2;
+    if (nthreads < 1) nthreads = 1;
+    if (nthreads > 64) nthreads = 64;
+    if ((uint64_t)nthreads > blocks) nthreads = (int)(blocks ? blocks : 1);
+    pthread_t th[64];
+    zo_range_job jobs[64];
+    uint64_t next = 0;
+    for (int t = 0; t < nthreads; t++) {
+        const uint64_t share = blocks / (uint64_t)nthreads + ((uint64_t)t < blocks % (uint64_t)nthreads ? 1 : 0);
+        jobs[t].fn = fn;
+        jobs[t].block_log2 = block_log2;
+        jobs[t].first = first;
+        jobs[t].first_block = next;
+        jobs[t].n_blocks = share;
+        jobs[t].sums = sums;
+        next += share;
+    }
+    for (int t = 1; t < nthreads; t++)
+        if (pthread_create(&th[t], NULL, zo_range_worker, &jobs[t])) return ZO_ERR_ARG;
+    zo_range_worker(&jobs[0]);
+    for (int t = 1; t < nthreads; t++) pthread_join(th[t], NULL);
+    return ZO_OK;
+}

@@ -71,6 +71,8 @@ enum {
     ZO_SIN = 5, ZO_COS = 6, ZO_TAN = 7, ZO_ASIN = 8, ZO_ACOS = 9, ZO_ATAN = 10,
     ZO_SINH = 11, ZO_COSH = 12
 };
+/* for zo_unary_range_hash_f32 only: the sigmoid composite of zo_sigmoid_f32 as a function of one argument */
+enum { ZO_SIGMOID_COMPOSITE = 13 };
 
 /* number of leaf (device-trait) calls issued since the last reset: mirrors the
  * call-counting tests of zenu-matrix/src/with_clousers.rs:356-379 */
@@ -143,6 +145,15 @@ int  zo_larger_shape(int nx, const int64_t *x, int ny, const int64_t *y);
 
 ZO_DECLARE(float, f32)
 ZO_DECLARE(double, f64)
+
+/* Every f32 bit pattern of [first, first + count) through unary function `fn` (ZO_EXP ... ZO_COSH, or
+ * ZO_SIGMOID_COMPOSITE), folded into one 64-bit sum per block of 2^block_log2 patterns:
+ * sums[b] = sum over the block of zo_range_hash_term(argument bits, result bits) mod 2^64.  The HIP
+ * library computes the same sums on the device, so that every argument can be compared without
+ * copying results.  `nthreads` threads split the blocks (the functions themselves stay the plain
+ * libm calls of the one-thread path). */
+uint64_t zo_range_hash_term(uint32_t arg_bits, uint32_t res_bits);
+int zo_unary_range_hash_f32(int fn, uint64_t first, uint64_t count, int block_log2, uint64_t *sums, int nthreads);
 
 #ifdef __cplusplus
 }

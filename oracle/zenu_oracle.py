@@ -153,6 +153,27 @@ def sigmoid(to, x):
     _chk(getattr(lib(), f"zo_sigmoid_{s}")(C.byref(view(to)), C.byref(view(x))), "sigmoid")
 
 
+SIGMOID_COMPOSITE = 13
+
+
+def unary_range_hash(fn, first, count, block_log2, nthreads=1):
+    """one 64-bit sum per block of 2^block_log2 f32 bit patterns of [first, first + count): every
+    pattern through unary function `fn` (or SIGMOID_COMPOSITE), argument and result bits hashed and added"""
+    sums = np.zeros(count >> block_log2, dtype=np.uint64)
+    f = lib().zo_unary_range_hash_f32
+    f.argtypes = [C.c_int, C.c_uint64, C.c_uint64, C.c_int, C.c_void_p, C.c_int]
+    f.restype = C.c_int
+    _chk(f(fn, first, count, block_log2, sums.ctypes.data, nthreads), "unary_range_hash")
+    return sums
+
+
+def range_hash_term(arg_bits, res_bits):
+    f = lib().zo_range_hash_term
+    f.argtypes = [C.c_uint32, C.c_uint32]
+    f.restype = C.c_uint64
+    return int(f(arg_bits, res_bits))
+
+
 def copy_from(to, src):
     s, _ = _sfx(to.dtype)
     _chk(getattr(lib(), f"zo_copy_from_{s}")(C.byref(view(to)), C.byref(view(src))), "copy_from")

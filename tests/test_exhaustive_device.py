@@ -1,9 +1,13 @@
-"""Every f32 bit pattern through the kernels whose results are meant to be the host libm's bits.
+"""Every f32 bit pattern through the elementwise kernels, results copied back and compared element by
+element: the eleven functions whose results are meant to be the host libm's bits, the two that are
+allowed a distance (tan: 1 ulp, tanh_ulp2: 2 ulp), powf for seven exponents, f64 sweeps and tensors
+beyond 2^31 / 2^32 elements.
 
-Opt-in (ZENU_EXHAUSTIVE=1): 2^32 arguments per function take a few minutes of host time for the
-oracle even on 16 threads, too long for the default suite, which checks every 64th pattern on the
-device (test_hip_parity.py) and every 31st in the host build of the same source
-(test_host_native.py).  Run as
+Opt-in (ZENU_EXHAUSTIVE=1): moving 2^32 results to the host and comparing them there takes half a minute
+per function.  The default suite compares the eleven bit-exact functions on all 2^32 arguments too, but
+through sums folded on the device and on the host (test_hip_parity.py::
+test_every_f32_argument_equals_the_host_libm, two seconds per function), and every 16th pattern element by
+element; the host build of the same source is compared on every 31st pattern (test_host_native.py).  Run as
     ZENU_EXHAUSTIVE=1 python -u -m pytest tests/test_exhaustive_device.py -m gpu -x -s --timeout 3000
 """
 import os

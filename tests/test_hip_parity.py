@@ -14,6 +14,7 @@ Bars (written where they are used):
       the sequential CPU sum itself cannot meet.
 """
 import os
+import time
 import subprocess
 
 import numpy as np
@@ -262,6 +263,75 @@ def test_validated_libm_is_named(hip):
         return
     # another host libm: the 0-ulp tests below compare against it and may legitimately differ
     print("note:", note)
+
+
+RANGE_HASH_DEFAULT = [("tanh", zo.TANH, "TANH"), ("sigmoid", zo.SIGMOID_COMPOSITE, "SIGMOID"), ("exp", zo.EXP, "EXP")]
+RANGE_HASH_MORE = [("log", zo.LOG, "LOG"), ("sinh", zo.SINH, "SINH"), ("cosh", zo.COSH, "COSH"), ("sin", zo.SIN, "SIN"),
+                   ("cos", zo.COS, "COS"), ("asin", zo.ASIN, "ASIN"), ("acos", zo.ACOS, "ACOS"), ("atan", zo.ATAN, "ATAN")]
+
+
+def _range_hash_case(hip, name, zo_fn, hip_fn):
+    """all 2^32 f32 arguments of one function: the device folds its results into one 64-bit sum per
+    2^20 arguments, the host folds the host libm's results the same way on its cores, and the 4096
+    sums must be equal -- every argument is compared and no result crosses the bus.  A block that
+    differs is then evaluated element by element to name the first argument."""
+    import ctypes as C
+    from zenu_amd import _lib
+    block_log2 = 20
+    blocks = 1 << (32 - block_log2)
+    sums = hip.Matrix.alloc((2 * blocks,), dtype=np.float32)       # 4096 x 8 bytes of device memory
+    fn = getattr(_lib, hip_fn)
+    _lib.check(hip.lib().zenu_hip_unary_range_hash(fn, 0, 1 << 32, block_log2, sums.as_ptr(), hip.get_stream()),
+               "unary_range_hash")
+    threads = max(1, min(16, os.cpu_count() or 1))
+    t0 = time.time()
+    host = zo.unary_range_hash(zo_fn, 0, 1 << 32, block_log2, threads)
+    dev = sums.to_numpy().view(np.uint64)
+    print(f"[range hash] {name}: 2^32 arguments, host libm on {threads} threads {time.time() - t0:.1f} s", flush=True)
+    bad = np.flatnonzero(dev != host)
+    if bad.size:
+        b = int(bad[0])
+        bits = np.arange(b << block_log2, (b + 1) << block_log2, dtype=np.uint64).astype(np.uint32)
+        x = bits.view(np.float32)
+        got = getattr(hip.Matrix.from_numpy(x), name)().to_numpy()
+        exp = np.empty_like(x)
+        with np.errstate(all="ignore"):
+            zo.sigmoid(exp, x) if zo_fn == zo.SIGMOID_COMPOSITE else zo.unary(zo_fn, exp, x)
+        d = np.flatnonzero((got.view(np.uint32) != exp.view(np.uint32)) & ~(np.isnan(got) & np.isnan(exp)))
+        first = f"first: x bits {int(bits[d[0]]):#010x}, device {got[d[0]]!r}, libm {exp[d[0]]!r}" if d.size else "(the element-wise path agrees)"
+        raise AssertionError(f"{name}: {bad.size} of {blocks} blocks differ, the first is block {b}; {first}; {_libm_note(hip)}")
+
+
+@pytest.mark.parametrize("name,zo_fn,hip_fn", RANGE_HASH_DEFAULT + RANGE_HASH_MORE)
+def test_every_f32_argument_equals_the_host_libm(hip, name, zo_fn, hip_fn):
+    """tanh, the sigmoid composite and exp -- the transcendental functions of the benchmark configs -- and
+    the other eight f32 functions whose results are meant to be the host libm's bits, each on ALL 2^32 f32
+    bit patterns against the host libm, in every run of the suite (a few seconds of host time per
+    function on 16 threads)"""
+    _range_hash_case(hip, name, zo_fn, hip_fn)
+
+
+def test_range_hash_sees_one_differing_result(hip):
+    """the sums are a comparison, not a formality: the device's sums of exp over one block against the
+    host's sums of the same block of ANOTHER function differ, and a host-side recomputation of one
+    block's sum from element-wise device results equals the device's sum"""
+    from zenu_amd import _lib
+    sums = hip.Matrix.alloc((2 * 16,), dtype=np.float32)
+    first, block_log2 = 0x3f000000, 16
+    _lib.check(hip.lib().zenu_hip_unary_range_hash(_lib.EXP, first, 16 << block_log2, block_log2, sums.as_ptr(), hip.get_stream()), "hash")
+    dev = sums.to_numpy().view(np.uint64)
+    assert np.array_equal(dev, zo.unary_range_hash(zo.EXP, first, 16 << block_log2, block_log2, 2))
+    assert not np.any(dev == zo.unary_range_hash(zo.TANH, first, 16 << block_log2, block_log2, 2))
+    bits = np.arange(first, first + (1 << block_log2), dtype=np.uint64).astype(np.uint32)
+    got = hip.Matrix.from_numpy(bits.view(np.float32)).exp().to_numpy().view(np.uint32)
+    total = sum(zo.range_hash_term(int(a), int(r)) for a, r in zip(bits[:4096], got[:4096])) % (1 << 64)
+    sums2 = hip.Matrix.alloc((2,), dtype=np.float32)
+    _lib.check(hip.lib().zenu_hip_unary_range_hash(_lib.EXP, first, 4096, 12, sums2.as_ptr(), hip.get_stream()), "hash")
+    assert int(sums2.to_numpy().view(np.uint64)[0]) == total
+    # refusals
+    assert hip.lib().zenu_hip_unary_range_hash(_lib.SQRT, 0, 1 << 20, 20, sums.as_ptr(), hip.get_stream()) == _lib.ERR_ARG
+    assert hip.lib().zenu_hip_unary_range_hash(_lib.EXP, 0, (1 << 20) + 1, 20, sums.as_ptr(), hip.get_stream()) == _lib.ERR_ARG
+    assert hip.lib().zenu_hip_unary_range_hash(_lib.EXP, 1 << 31, 1 << 32, 20, sums.as_ptr(), hip.get_stream()) == _lib.ERR_ARG
 
 
 def test_tanh_sigmoid_dense_sweep(hip):

@@ -44,3 +44,33 @@ def test_leaf_call_counts():
     zo.reset_leaf_calls()
     zo.sum_axis(x, 0)         # shape[axis] slice adds (sum.rs:20-25)
     assert zo.leaf_calls() == 64
+
+
+def test_unary_range_hash_is_the_fold_of_the_element_wise_results():
+    """zo.unary_range_hash (the host side of the every-argument comparison with the device): a block's sum
+    is the sum of the documented term over the element-wise results of the same function, NaN results
+    count as one value, threads only split the blocks, and the sigmoid composite is zo.sigmoid"""
+    def fold(bits, res):
+        rb = res.view(np.uint32).astype(np.uint64)
+        rb = np.where(np.isnan(res), np.uint64(0x7fc00000), rb)
+        z = (bits.astype(np.uint64) << np.uint64(32)) | rb
+        with np.errstate(over="ignore"):
+            z = (z ^ (z >> np.uint64(30))) * np.uint64(0xbf58476d1ce4e5b9)
+            z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94d049bb133111eb)
+            z = z ^ (z >> np.uint64(31))
+            return int(z.sum(dtype=np.uint64))
+    for fn, first in ((zo.TANH, 0x3f000000), (zo.EXP, 0xc2000000), (zo.LOG, 0xbf7f0000), (zo.SIGMOID_COMPOSITE, 0x7f7f0000),
+                      (zo.ASIN, 0x3f7f0000)):
+        sums = zo.unary_range_hash(fn, first, 4 << 16, 16, 3)
+        assert np.array_equal(sums, zo.unary_range_hash(fn, first, 4 << 16, 16, 1))
+        for b in range(4):
+            bits = np.arange(first + (b << 16), first + ((b + 1) << 16), dtype=np.uint64).astype(np.uint32)
+            x = bits.view(np.float32)
+            out = np.empty_like(x)
+            with np.errstate(all="ignore"):
+                zo.sigmoid(out, x) if fn == zo.SIGMOID_COMPOSITE else zo.unary(fn, out, x)
+            assert fold(bits, out) == int(sums[b]), (fn, b)
+    assert zo.range_hash_term(1, 0x7fc00001) == zo.range_hash_term(1, 0xffc12345)     # any NaN
+    assert zo.range_hash_term(1, 2) != zo.range_hash_term(2, 1)
+    with pytest.raises(zo.OracleError):
+        zo.unary_range_hash(zo.TANH, 0, (1 << 16) + 5, 16, 1)

@@ -1,0 +1,84 @@
+// rangehash.hip -- every f32 bit pattern of a range through a unary function of the library, folded
+// into one 64-bit sum per block of patterns.  A host that folds its own libm's results the same way
+// (one term per argument: argument and result bits through the finalizer of splitmix64, every NaN
+// counted as one value) can compare every argument of the function with the device without copying
+// a single result: equal sums, equal bits.  The functor is the one the elementwise kernels apply
+// (elementwise.hpp), so what is checked is the arithmetic that ships.
+#include "elementwise.hpp"
+
+namespace zenu {
+namespace {
+
+__device__ __forceinline__ uint64_t range_hash_term(uint32_t arg_bits, uint32_t res_bits)
+{
+    if ((res_bits & 0x7fffffffu) > 0x7f800000u) res_bits = 0x7fc00000u;
+    uint64_t z = ((uint64_t)arg_bits << 32) | res_bits;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+}
+
+constexpr int kHashBlock = 256;
+
+// one workgroup per block of 2^block_log2 patterns
+template <int FN>
+__global__ __launch_bounds__(kHashBlock) void range_hash_kernel(uint64_t first, int block_log2, uint64_t *sums,
+                                                                UnaryF<float, FN> f)
+{
+    __shared__ uint64_t part[kHashBlock / 64];
+    f.init();
+    const uint64_t per = 1ull << block_log2;
+    const uint64_t start = first + (uint64_t)blockIdx.x * per;
+    uint64_t sum = 0;
+    for (uint64_t i = threadIdx.x; i < per; i += kHashBlock) {
+        const uint32_t bits = (uint32_t)(start + i);
+        const float x = __uint_as_float(bits);
+        sum += range_hash_term(bits, __float_as_uint(f(x, x)));
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint64_t total = 0;
+#pragma unroll
+        for (int w = 0; w < kHashBlock / 64; w++) total += part[w];
+        sums[blockIdx.x] = total;
+    }
+}
+
+template <int FN> int launch_range_hash(uint64_t first, uint64_t blocks, int block_log2, uint64_t *sums, hipStream_t s)
+{
+    range_hash_kernel<FN><<<(unsigned)blocks, kHashBlock, 0, s>>>(first, block_log2, sums, UnaryF<float, FN>());
+    ZENU_LAUNCH_CHECK();
+    return ZENU_OK;
+}
+
+}  // namespace
+}  // namespace zenu
+
+using namespace zenu;
+
+extern "C" int zenu_hip_unary_range_hash(int fn, uint64_t first, uint64_t count, int block_log2, uint64_t *sums_dev,
+                                         zenu_stream_t stream)
+{
+    if (!sums_dev || block_log2 < 8 || block_log2 > 32) return ZENU_ERR_ARG;
+    if ((count & ((1ull << block_log2) - 1)) || count == 0 || first + count > (1ull << 32)) return ZENU_ERR_ARG;
+    const uint64_t blocks = count >> block_log2;
+    if (blocks > 0x7fffffffull) return ZENU_ERR_UNSUPPORTED;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    switch (fn) {
+    case ZENU_EXP: return launch_range_hash<ZENU_EXP>(first, blocks, block_log2, sums_dev, s);
+    case ZENU_LOG: return launch_range_hash<ZENU_LOG>(first, blocks, block_log2, sums_dev, s);
+    case ZENU_TANH: return launch_range_hash<ZENU_TANH>(first, blocks, block_log2, sums_dev, s);
+    case ZENU_SIGMOID: return launch_range_hash<ZENU_SIGMOID>(first, blocks, block_log2, sums_dev, s);
+    case ZENU_SIN: return launch_range_hash<ZENU_SIN>(first, blocks, block_log2, sums_dev, s);
+    case ZENU_COS: return launch_range_hash<ZENU_COS>(first, blocks, block_log2, sums_dev, s);
+    case ZENU_ASIN: return launch_range_hash<ZENU_ASIN>(first, blocks, block_log2, sums_dev, s);
+    case ZENU_ACOS: return launch_range_hash<ZENU_ACOS>(first, blocks, block_log2, sums_dev, s);
+    case ZENU_ATAN: return launch_range_hash<ZENU_ATAN>(first, blocks, block_log2, sums_dev, s);
+    case ZENU_SINH: return launch_range_hash<ZENU_SINH>(first, blocks, block_log2, sums_dev, s);
+    case ZENU_COSH: return launch_range_hash<ZENU_COSH>(first, blocks, block_log2, sums_dev, s);
+    default: return ZENU_ERR_ARG;
+    }
+}
