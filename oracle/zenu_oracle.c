@@ -222,8 +222,39 @@ static inline float zo_range_fn(int fn, float x)
     return zo_unary_fn_f32(fn, x);
 }
 
+static inline uint64_t zo_mix64(uint64_t z)
+{
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+}
+
+/* f64 argument number i: high word i * step + offset, a pseudo-random low word from i and salt */
+uint64_t zo_range_arg_f64(uint64_t i, uint32_t step, uint32_t offset, uint64_t salt)
+{
+    const uint64_t hi = (uint32_t)(i * step + offset);
+    const uint64_t lo = (uint32_t)(((i + salt) * 0x9E3779B97F4A7C15ull) >> 29);
+    return (hi << 32) | lo;
+}
+
+static inline double zo_range_fn_f64(int fn, double x)
+{
+    if (fn == ZO_SIGMOID_COMPOSITE) {
+        const double half = 1.0 / (1.0 + 1.0);
+        const double t1 = x * half;
+        const double t2 = tanh(t1);
+        const double t3 = half * t2;
+        return half + t3;
+    }
+    return zo_unary_fn_f64(fn, x);
+}
+
+/* kind 0: f32 unary (fn); kind 1: f32 powf with `exponent`; kind 2: f64 unary (fn) on zo_range_arg_f64 */
 typedef struct {
-    int fn, block_log2;
+    int kind, fn, block_log2;
+    float exponent;
+    uint32_t step, offset;
+    uint64_t salt;
     uint64_t first_block, n_blocks, first;
     uint64_t *sums;
 } zo_range_job;
@@ -235,14 +266,27 @@ static void *zo_range_worker(void *arg)
     for (uint64_t b = j->first_block; b < j->first_block + j->n_blocks; b++) {
         uint64_t sum = 0;
         const uint64_t start = j->first + b * per;
-        for (uint64_t i = 0; i < per; i++) {
-            const uint32_t bits = (uint32_t)(start + i);
-            float x, y;
-            uint32_t rb;
-            memcpy(&x, &bits, 4);
-            y = zo_range_fn(j->fn, x);
-            memcpy(&rb, &y, 4);
-            sum += zo_range_hash_term(bits, rb);
+        if (j->kind == 2) {
+            for (uint64_t i = 0; i < per; i++) {
+                const uint64_t bits = zo_range_arg_f64(start + i, j->step, j->offset, j->salt);
+                double x, y;
+                uint64_t rb;
+                memcpy(&x, &bits, 8);
+                y = zo_range_fn_f64(j->fn, x);
+                memcpy(&rb, &y, 8);
+                if ((rb & 0x7fffffffffffffffull) > 0x7ff0000000000000ull) rb = 0x7ff8000000000000ull;
+                sum += zo_mix64(zo_mix64(bits) + rb);
+            }
+        } else {
+            for (uint64_t i = 0; i < per; i++) {
+                const uint32_t bits = (uint32_t)(start + i);
+                float x, y;
+                uint32_t rb;
+                memcpy(&x, &bits, 4);
+                y = j->kind == 1 ? powf(x, j->exponent) : zo_range_fn(j->fn, x);
+                memcpy(&rb, &y, 4);
+                sum += zo_range_hash_term(bits, rb);
+            }
         }
         j->sums[b] = sum;
     }
@@ -250,11 +294,11 @@ static void *zo_range_worker(void *arg)
 }
 
 /* sums[b] for the patterns first + b * 2^block_log2 ... of `count` patterns (a multiple of the block size) */
-int zo_unary_range_hash_f32(int fn, uint64_t first, uint64_t count, int block_log2, uint64_t *sums, int nthreads)
+static int zo_range_hash_run(zo_range_job proto, uint64_t first, uint64_t count, int block_log2, uint64_t *sums, int nthreads)
 {
     if (block_log2 < 0 || block_log2 > 32 || (count & ((1ull << block_log2) - 1)) || first + count > (1ull << 32))
         return ZO_ERR_ARG;
-    if (fn < ZO_EXP || fn > ZO_SIGMOID_COMPOSITE) return ZO_ERR_ARG;
+    if (proto.kind != 1 && (proto.fn < ZO_EXP || proto.fn > ZO_SIGMOID_COMPOSITE)) return ZO_ERR_ARG;
     const uint64_t blocks = count >> block_log2;
     if (nthreads < 1) nthreads = 1;
     if (nthreads > 64) nthreads = 64;
@@ -264,7 +308,7 @@ int zo_unary_range_hash_f32(int fn, uint64_t first, uint64_t count, int block_lo
     uint64_t next = 0;
     for (int t = 0; t < nthreads; t++) {
         const uint64_t share = blocks / (uint64_t)nthreads + ((uint64_t)t < blocks % (uint64_t)nthreads ? 1 : 0);
-        jobs[t].fn = fn;
+        jobs[t] = proto;
         jobs[t].block_log2 = block_log2;
         jobs[t].first = first;
         jobs[t].first_block = next;
@@ -278,3 +322,39 @@ int zo_unary_range_hash_f32(int fn, uint64_t first, uint64_t count, int block_lo
     for (int t = 1; t < nthreads; t++) pthread_join(th[t], NULL);
     return ZO_OK;
 }
+
+int zo_unary_range_hash_f32(int fn, uint64_t first, uint64_t count, int block_log2, uint64_t *sums, int nthreads)
+{
+    zo_range_job j;
+    memset(&j, 0, sizeof j);
+    j.kind = 0;
+    j.fn = fn;
+    return zo_range_hash_run(j, first, count, block_log2, sums, nthreads);
+}
+
+/* the same for powf(x, exponent) over the f32 bases x */
+int zo_powf_range_hash_f32(float exponent, uint64_t first, uint64_t count, int block_log2, uint64_t *sums, int nthreads)
+{
+    zo_range_job j;
+    memset(&j, 0, sizeof j);
+    j.kind = 1;
+    j.exponent = exponent;
+    return zo_range_hash_run(j, first, count, block_log2, sums, nthreads);
+}
+
+/* f64: argument number i of [first, first + count) is zo_range_arg_f64(i, step, offset, salt); the term is
+ * mix64(mix64(argument bits) + result bits), every NaN result counted as 0x7ff8000000000000 */
+int zo_unary_range_hash_f64(int fn, uint64_t first, uint64_t count, int block_log2, uint32_t step, uint32_t offset,
+                            uint64_t salt, uint64_t *sums, int nthreads)
+{
+    zo_range_job j;
+    memset(&j, 0, sizeof j);
+    if (step == 0) return ZO_ERR_ARG;
+    j.kind = 2;
+    j.fn = fn;
+    j.step = step;
+    j.offset = offset;
+    j.salt = salt;
+    return zo_range_hash_run(j, first, count, block_log2, sums, nthreads);
+}
+

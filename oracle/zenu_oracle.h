@@ -154,6 +154,14 @@ ZO_DECLARE(double, f64)
  * libm calls of the one-thread path). */
 uint64_t zo_range_hash_term(uint32_t arg_bits, uint32_t res_bits);
 int zo_unary_range_hash_f32(int fn, uint64_t first, uint64_t count, int block_log2, uint64_t *sums, int nthreads);
+/* the same for powf(x, exponent) over the f32 bases, and for the f64 functions on sampled arguments:
+ * argument number i is zo_range_arg_f64(i, step, offset, salt) (high word i * step + offset, a
+ * pseudo-random low word), the term mix64(mix64(argument bits) + result bits) with mix64 the finalizer of
+ * splitmix64 and every NaN result counted as 0x7ff8000000000000 */
+int zo_powf_range_hash_f32(float exponent, uint64_t first, uint64_t count, int block_log2, uint64_t *sums, int nthreads);
+uint64_t zo_range_arg_f64(uint64_t i, uint32_t step, uint32_t offset, uint64_t salt);
+int zo_unary_range_hash_f64(int fn, uint64_t first, uint64_t count, int block_log2, uint32_t step, uint32_t offset,
+                            uint64_t salt, uint64_t *sums, int nthreads);
 
 #ifdef __cplusplus
 }

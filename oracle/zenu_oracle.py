@@ -167,6 +167,32 @@ def unary_range_hash(fn, first, count, block_log2, nthreads=1):
     return sums
 
 
+def powf_range_hash(exponent, first, count, block_log2, nthreads=1):
+    sums = np.zeros(count >> block_log2, dtype=np.uint64)
+    f = lib().zo_powf_range_hash_f32
+    f.argtypes = [C.c_float, C.c_uint64, C.c_uint64, C.c_int, C.c_void_p, C.c_int]
+    f.restype = C.c_int
+    _chk(f(exponent, first, count, block_log2, sums.ctypes.data, nthreads), "powf_range_hash")
+    return sums
+
+
+def unary_range_hash_f64(fn, first, count, block_log2, step, offset, salt, nthreads=1):
+    """f64: argument number i has the high word i * step + offset and a pseudo-random low word (range_arg_f64)"""
+    sums = np.zeros(count >> block_log2, dtype=np.uint64)
+    f = lib().zo_unary_range_hash_f64
+    f.argtypes = [C.c_int, C.c_uint64, C.c_uint64, C.c_int, C.c_uint32, C.c_uint32, C.c_uint64, C.c_void_p, C.c_int]
+    f.restype = C.c_int
+    _chk(f(fn, first, count, block_log2, step, offset, salt, sums.ctypes.data, nthreads), "unary_range_hash_f64")
+    return sums
+
+
+def range_arg_f64(i, step, offset, salt):
+    f = lib().zo_range_arg_f64
+    f.argtypes = [C.c_uint64, C.c_uint32, C.c_uint32, C.c_uint64]
+    f.restype = C.c_uint64
+    return int(f(i, step, offset, salt))
+
+
 def range_hash_term(arg_bits, res_bits):
     f = lib().zo_range_hash_term
     f.argtypes = [C.c_uint32, C.c_uint32]

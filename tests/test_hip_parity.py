@@ -311,6 +311,57 @@ def test_every_f32_argument_equals_the_host_libm(hip, name, zo_fn, hip_fn):
     _range_hash_case(hip, name, zo_fn, hip_fn)
 
 
+@pytest.mark.parametrize("exponent", [2.0, 0.5, 2.5, -1.0, 3.0, -0.5, 1.0 / 3.0])
+def test_powf_every_f32_base_equals_the_host_libm(hip, exponent):
+    """powf(x, exponent) for ALL 2^32 f32 bases (negative bases, zeros, subnormals, infinities and NaN
+    included) against the host libm, through the folded sums"""
+    block_log2 = 20
+    blocks = 1 << (32 - block_log2)
+    from zenu_amd import _lib
+    sums = hip.Matrix.alloc((2 * blocks,), dtype=np.float32)
+    _lib.check(hip.lib().zenu_hip_powf_range_hash(exponent, 0, 1 << 32, block_log2, sums.as_ptr(), hip.get_stream()), "powf_range_hash")
+    threads = max(1, min(16, os.cpu_count() or 1))
+    t0 = time.time()
+    host = zo.powf_range_hash(np.float32(exponent), 0, 1 << 32, block_log2, threads)
+    dev = sums.to_numpy().view(np.uint64)
+    print(f"[range hash] powf(x, {exponent}): 2^32 bases, host libm on {threads} threads {time.time() - t0:.1f} s", flush=True)
+    bad = np.flatnonzero(dev != host)
+    assert bad.size == 0, f"powf(x, {exponent}): {bad.size} of {blocks} blocks differ, the first is block {int(bad[0])} (bases from bits {int(bad[0]) << block_log2:#010x}); {_libm_note(hip)}"
+
+
+@pytest.mark.parametrize("name,zo_fn,hip_fn", [("tanh", zo.TANH, "TANH"), ("sigmoid", zo.SIGMOID_COMPOSITE, "SIGMOID"),
+                                               ("exp", zo.EXP, "EXP"), ("sinh", zo.SINH, "SINH"), ("cosh", zo.COSH, "COSH")])
+def test_f64_sampled_arguments_equal_the_host_libm(hip, name, zo_fn, hip_fn):
+    """f64 cannot be exhausted: every value of the high word (sign, exponent, 20 mantissa bits) with a
+    pseudo-random low word -- 2^32 arguments per function, other low words with every ZENU_F64_HASH_SALT --
+    against the host libm through the folded sums"""
+    from zenu_amd import _lib
+    block_log2 = 20
+    count = 1 << 32
+    salt = int(os.environ.get("ZENU_F64_HASH_SALT", "0"))
+    step, offset = 1, 0
+    sums = hip.Matrix.alloc((2 * (count >> block_log2),), dtype=np.float32)
+    _lib.check(hip.lib().zenu_hip_unary_range_hash_f64(getattr(_lib, hip_fn), 0, count, block_log2, step, offset, salt,
+                                                       sums.as_ptr(), hip.get_stream()), "unary_range_hash_f64")
+    threads = max(1, min(16, os.cpu_count() or 1))
+    t0 = time.time()
+    host = zo.unary_range_hash_f64(zo_fn, 0, count, block_log2, step, offset, salt, threads)
+    dev = sums.to_numpy().view(np.uint64)
+    print(f"[range hash] {name} f64: 2^32 arguments, host libm on {threads} threads {time.time() - t0:.1f} s", flush=True)
+    bad = np.flatnonzero(dev != host)
+    if bad.size:
+        b = int(bad[0])
+        bits = np.array([zo.range_arg_f64(i, step, offset, salt) for i in range(b << block_log2, (b << block_log2) + 4096)], dtype=np.uint64)
+        x = bits.view(np.float64)
+        got = getattr(hip.Matrix.from_numpy(x), name)().to_numpy()
+        exp = np.empty_like(x)
+        with np.errstate(all="ignore"):
+            zo.sigmoid(exp, x) if zo_fn == zo.SIGMOID_COMPOSITE else zo.unary(zo_fn, exp, x)
+        d = np.flatnonzero((got.view(np.uint64) != exp.view(np.uint64)) & ~(np.isnan(got) & np.isnan(exp)))
+        first = f"x = {x[d[0]]!r}: device {got[d[0]]!r}, libm {exp[d[0]]!r}" if d.size else "(its first 4096 arguments agree element-wise)"
+        raise AssertionError(f"{name} f64: {bad.size} blocks differ, the first is block {b}; {first}; {_libm_note(hip)}")
+
+
 def test_range_hash_sees_one_differing_result(hip):
     """the sums are a comparison, not a formality: the device's sums of exp over one block against the
     host's sums of the same block of ANOTHER function differ, and a host-side recomputation of one

@@ -74,3 +74,42 @@ def test_unary_range_hash_is_the_fold_of_the_element_wise_results():
     assert zo.range_hash_term(1, 2) != zo.range_hash_term(2, 1)
     with pytest.raises(zo.OracleError):
         zo.unary_range_hash(zo.TANH, 0, (1 << 16) + 5, 16, 1)
+
+
+def test_powf_and_f64_range_hashes_are_folds_of_the_element_wise_results():
+    """the powf and f64 forms of the host-side fold: a block's sum equals the sum of the documented terms over
+    element-wise results, the f64 arguments are the documented (high word, pseudo-random low word) pairs"""
+    def mix(z):
+        with np.errstate(over="ignore"):
+            z = (z ^ (z >> np.uint64(30))) * np.uint64(0xbf58476d1ce4e5b9)
+            z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94d049bb133111eb)
+            return z ^ (z >> np.uint64(31))
+    first = 0xbf000000            # negative bases: NaN results
+    sums = zo.powf_range_hash(np.float32(2.5), first, 2 << 16, 16, 2)
+    for b in range(2):
+        bits = np.arange(first + (b << 16), first + ((b + 1) << 16), dtype=np.uint64).astype(np.uint32)
+        x = bits.view(np.float32)
+        out = np.empty_like(x)
+        with np.errstate(all="ignore"):
+            zo.powf(out, x, 2.5)
+        rb = np.where(np.isnan(out), np.uint64(0x7fc00000), out.view(np.uint32).astype(np.uint64))
+        with np.errstate(over="ignore"):
+            assert int(mix((bits.astype(np.uint64) << np.uint64(32)) | rb).sum(dtype=np.uint64)) == int(sums[b])
+    step, offset, salt = 4, 3, 7
+    i0 = 0x0ff00000               # high words around 0x3fc00000: arguments near 0.125 .. 
+    sums = zo.unary_range_hash_f64(zo.TANH, i0, 2 << 12, 12, step, offset, salt, 2)
+    for b in range(2):
+        idx = np.arange(i0 + (b << 12), i0 + ((b + 1) << 12), dtype=np.uint64)
+        with np.errstate(over="ignore"):
+            hi = (idx * np.uint64(step) + np.uint64(offset)) & np.uint64(0xffffffff)
+            lo = (((idx + np.uint64(salt)) * np.uint64(0x9E3779B97F4A7C15)) >> np.uint64(29)) & np.uint64(0xffffffff)
+        bits = (hi << np.uint64(32)) | lo
+        assert int(bits[5]) == zo.range_arg_f64(int(idx[5]), step, offset, salt)
+        x = bits.view(np.float64)
+        out = np.empty_like(x)
+        zo.unary(zo.TANH, out, x)
+        rb = np.where(np.isnan(out), np.uint64(0x7ff8000000000000), out.view(np.uint64))
+        with np.errstate(over="ignore"):
+            assert int(mix(mix(bits) + rb).sum(dtype=np.uint64)) == int(sums[b])
+    with pytest.raises(zo.OracleError):
+        zo.unary_range_hash_f64(zo.TANH, 0, 1 << 12, 12, 0, 0, 0, 1)

@@ -40,7 +40,7 @@ def test_every_declared_symbol_is_bound_with_matching_arity_and_types():
     assert sorted(fns) == sorted(declared)                     # nothing missing, nothing extra
     # zenu_hip_* entry points: the ctypes table is a second, hand-written reading of the header
     # (on LP64, ctypes' c_size_t and c_uint64 are one class: a size_t parameter reads usize, a uint64_t one u64)
-    ctypes_to_rust = {C.c_int: {"c_int"}, C.c_int64: {"i64"}, C.c_double: {"f64"}, C.c_size_t: {"usize", "u64"}}
+    ctypes_to_rust = {C.c_int: {"c_int"}, C.c_int64: {"i64"}, C.c_double: {"f64"}, C.c_size_t: {"usize", "u64"}, C.c_uint32: {"u32"}}
     for name, argtypes in _lib.SIGNATURES.items():
         rargs, ret = fns[name]
         assert len(rargs) == len(argtypes), name
