@@ -1006,3 +1006,44 @@ pub fn self_check() -> Result<(), String> {
     }
     Ok(())
 }
+
+/// Does the host libm behind the `Cpu` device give, for `function` (a `ZENU_*` unary id), the bits this device
+/// gives?  Both sides fold their results over the f32 bit patterns `first .. first + count` (count a
+/// multiple of 2^20) into one 64-bit sum per 2^20 arguments -- the device in `zenu_hip_unary_range_hash`,
+/// the host here with `host` (e.g. `f32::tanh`; for `ZENU_SIGMOID` the composite
+/// `|x| 0.5 + 0.5 * (x * 0.5).tanh()`) -- and the sums are compared: equal sums, equal bits on every
+/// argument, and no result crosses the bus.  All 2^32 arguments take the device 0.1 s and one host
+/// thread about half a minute; split the range over threads for less.
+pub fn agrees_with_host_libm(function: c_int, host: fn(f32) -> f32, first: u64, count: u64) -> bool {
+    const BLOCK_LOG2: c_int = 20;
+    let blocks = (count >> BLOCK_LOG2) as usize;
+    let bytes = blocks * std::mem::size_of::<u64>();
+    let dev = Hip::alloc(bytes).unwrap();
+    ok(unsafe { zenu_hip_unary_range_hash(function, first, count, BLOCK_LOG2, dev.cast::<u64>(), current_stream()) });
+    let mut device_sums = vec![0u64; blocks];
+    ok(unsafe { zenu_hip_memcpy_d2h(device_sums.as_mut_ptr().cast::<c_void>(), dev.cast::<c_void>(), bytes, current_stream()) });
+    Hip::drop_ptr(dev);
+    let mix = |mut z: u64| {
+        z = (z ^ (z >> 30)).wrapping_mul(0xbf58_476d_1ce4_e5b9);
+        z = (z ^ (z >> 27)).wrapping_mul(0x94d0_49bb_1331_11eb);
+        z ^ (z >> 31)
+    };
+    for (b, device_sum) in device_sums.iter().enumerate() {
+        let start = first + ((b as u64) << BLOCK_LOG2);
+        let mut sum = 0u64;
+        let mut offset = 0u64;
+        while offset < (1u64 << BLOCK_LOG2) {
+            let bits = (start + offset) as u32;
+            offset += 1;
+            let mut result = host(f32::from_bits(bits)).to_bits();
+            if result & 0x7fff_ffff > 0x7f80_0000 {
+                result = 0x7fc0_0000; // every NaN counts as one value
+            }
+            sum = sum.wrapping_add(mix((u64::from(bits) << 32) | u64::from(result)));
+        }
+        if sum != *device_sum {
+            return false;
+        }
+    }
+    true
+}
