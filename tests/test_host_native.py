@@ -20,11 +20,29 @@ def test_allocator_bookkeeping(tmp_path):
     size classes, same-stream and cross-stream reuse, split/merge, OOM -> trim -> retry, foreign
     pointers, blocks taken during a stream capture staying out of ordinary requests until released,
     and a randomized stress run against a shadow model"""
-    exe = build("allocator_host_check.cpp", str(tmp_path / "alloc_check"))
+    exe = build("allocator_host_check.cpp", str(tmp_path / "alloc_check"),
+                ("-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined"))   # the bookkeeping under the sanitizers
     out = subprocess.run([exe], capture_output=True, text=True)
     assert out.returncode == 0, out.stdout + out.stderr
     for name in ("size_classes", "same_stream_reuse", "cross_stream_reuse", "retire_stream", "split_merge_trim", "oom_retry",
                  "injected_failure", "not_owned", "capture_blocks", "stress"):
+        assert f"ok {name}" in out.stdout
+
+
+def test_shape_algebra_against_brute_force(tmp_path):
+    """zenu_amd/csrc/shape.cpp compiled for the host (address and undefined-behaviour sanitizers on): 20 000
+    seeded random elementwise problems -- up to six dims, three operands, permuted / sliced / broadcast
+    strides -- must visit exactly the original (output, input, input) offsets after ew_collapse, with no
+    size-1 dim left and the output's strides in decreasing order; the alias rule must refuse every pair of
+    views that share an element without being the same view, accept the output's own view and every pair of
+    disjoint ranges (60 000 random pairs against an element-by-element model); the shape rules on the
+    reference's own cases (dim_dyn.rs:24-58, broadcast.rs:13-44)"""
+    exe = build("shape_host_check.cpp", str(tmp_path / "shape_check"),
+                ("-g", "-O1", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", "-fsanitize=address,undefined",
+                 "-fno-sanitize-recover=undefined"))
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0, out.stdout + out.stderr
+    for name in ("collapse", "alias", "rules"):
         assert f"ok {name}" in out.stdout
 
 
