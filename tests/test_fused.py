@@ -508,6 +508,37 @@ def test_cross_entropy_backward_bias_grad(hip, dtype, n, c):
         assert bits_equal(gb2.to_numpy(), gb.to_numpy())
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+def test_cross_entropy_head_every_small_geometry(hip, dtype):
+    """every batch of 1..256 rows (at the wavefront and workgroup edges) with every class count 1..16 -- the
+    geometries that the four-lanes-per-line kernels take: probabilities and gradients are the oracle's bits,
+    the loss and the bias gradient within the bar of a sum"""
+    M = hip.Matrix
+    r = np.random.default_rng(77)
+    tol = 1e-5 if dtype == np.float32 else 1e-12
+    for n in (1, 2, 3, 4, 5, 63, 64, 65, 127, 128, 129, 191, 255, 256):
+        for c in range(1, 17):
+            pred = r.standard_normal((n, c)).astype(dtype) * 3
+            ans = np.zeros((n, c), dtype=dtype)
+            ans[np.arange(n), r.integers(0, c, n)] = 1
+            loss_ref, prob_ref = cpu_matrix.cross_entropy(CpuMatrix.from_numpy(pred), CpuMatrix.from_numpy(ans))
+            loss, prob = hip.cross_entropy(M.from_numpy(pred), M.from_numpy(ans))
+            p = prob.to_numpy()
+            if dtype == np.float32:
+                assert bits_equal(p, prob_ref.a), (n, c)
+            else:
+                assert rel_err(p, prob_ref.a) <= 1e-14, (n, c)
+            lr = float(loss_ref.a)
+            assert abs(float(loss.to_numpy()) - lr) <= 4 * tol * max(abs(lr), 1e-30) + 1e-30, (n, c)
+            gb = M.from_numpy(np.full(c, 9.0, dtype=dtype))
+            g = hip.cross_entropy_backward_bias_grad(prob, M.from_numpy(ans), gb, None).to_numpy()
+            gref = cpu_matrix.cross_entropy_backward(CpuMatrix.from_numpy(p), CpuMatrix.from_numpy(ans)).a
+            assert bits_equal(g, gref), (n, c)
+            g64 = gref.astype(np.float64)
+            scale = np.maximum(np.abs(g64.sum(0)), np.abs(g64).sum(0) / np.sqrt(n))
+            assert np.all(np.abs(gb.to_numpy() - g64.sum(0)) <= tol * scale + 1e-300), (n, c)
+
+
 def test_cross_entropy_single_launch_equals_two_launches(hip):
     """up to 256 rows the cross-entropy forward folds its row terms in the workgroup that computed them;
     257 rows take the two-launch road: on the first 256 rows of the same data both give the same
