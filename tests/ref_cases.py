@@ -602,6 +602,50 @@ def clip_cases(dev):  # zenu-matrix/src/operation/clip.rs:321-372; zenu-cuda/src
 
 
 @case
+def view_cases(dev):  # zenu-matrix/src/operation/transpose.rs:70-206, reshape.rs:108-176, add_axis.rs:25-33
+    M = dev.M
+    # transpose_2d: [[1,2,3],[4,5,6]] transposed, read element by element
+    a = M.from_numpy(np.array([1., 2., 3., 4., 5., 6.], dtype=np.float32).reshape(2, 3)).transpose()
+    got = a.to_default_stride().to_numpy()
+    assert got.shape == (3, 2)
+    for (i, j), v in {(0, 0): 1., (0, 1): 4., (1, 0): 2., (1, 1): 5., (2, 0): 3., (2, 1): 6.}.items():
+        assert got[i, j] == v
+    # inplace_transpose_4d: element (i, j, k, l) = 1000 i + 100 j + 10 k + l on [3,4,5,6]; transpose_by_index
+    # [1,0,2,3] into a new matrix.  The reference's literal lists the result row by row: [4,3,5,6] with
+    # element (j, i, k, l) = 1000 i + 100 j + 10 k + l (its first rows: 0..5, 10..15, ..., 40..45, 1000..1005).
+    i, j, k, l = np.meshgrid(np.arange(3), np.arange(4), np.arange(5), np.arange(6), indexing="ij")
+    x = (1000 * i + 100 * j + 10 * k + l).astype(np.float32)
+    out = M.from_numpy(x).transpose_by_index([1, 0, 2, 3]).to_default_stride()
+    ans = np.empty((4, 3, 5, 6), dtype=np.float32)
+    for jj in range(4):
+        for ii in range(3):
+            for kk in range(5):
+                for ll in range(6):
+                    ans[jj, ii, kk, ll] = 1000 * ii + 100 * jj + 10 * kk + ll
+    assert list(ans.reshape(-1)[:12]) == [0., 1., 2., 3., 4., 5., 10., 11., 12., 13., 14., 15.]     # the literal's first entries
+    assert list(ans.reshape(-1)[30:36]) == [1000., 1001., 1002., 1003., 1004., 1005.]
+    eq(out, ans)
+    # swap_axis (2-d) and swap_axis_3d: transpose_swap_index_new_matrix(0, 1)
+    eq(M.from_numpy(np.array([1., 2., 3., 4., 5., 6.], dtype=np.float32).reshape(2, 3)).transpose_by_index([1, 0]).to_default_stride(),
+       [1., 4., 2., 5., 3., 6.], (3, 2))
+    x3 = np.arange(1, 25, dtype=np.float32).reshape(2, 3, 4)
+    eq(M.from_numpy(x3).transpose_by_index([1, 0, 2]).to_default_stride(),
+       [1., 2., 3., 4., 13., 14., 15., 16., 5., 6., 7., 8., 17., 18., 19., 20., 9., 10., 11., 12., 21., 22., 23., 24.], (3, 2, 4))
+    # reshape_3d_1d, reshape_1d_3d: views of the same data
+    r18 = np.arange(1, 19, dtype=np.float32)
+    eq(M.from_numpy(r18.reshape(2, 3, 3)).reshape([18]), r18, (18,))
+    eq(M.from_numpy(np.arange(1, 7, dtype=np.float32)).reshape([2, 3, 1]), [1., 2., 3., 4., 5., 6.], (2, 3, 1))
+    # reshape_new_matrix_3d_1d: transpose_by_index [2,1,0], then a new default-stride matrix reshaped to [18]
+    eq(M.from_numpy(r18.reshape(2, 3, 3)).transpose_by_index([2, 1, 0]).to_default_stride().reshape([18]),
+       [1., 10., 4., 13., 7., 16., 2., 11., 5., 14., 8., 17., 3., 12., 6., 15., 9., 18.], (18,))
+    # add_axis: [2,2] -> [1,2,2], same data; a - ans has asum 0
+    a = M.from_numpy(np.array([1., 2., 3., 4.], dtype=np.float32).reshape(2, 2)).add_axis(0)
+    assert tuple(a.shape) == (1, 2, 2)
+    ans = M.from_numpy(np.array([1., 2., 3., 4.], dtype=np.float32).reshape(1, 2, 2))
+    assert float((a - ans).asum()) == 0.0
+
+
+@case
 def broadcast_cases(dev):  # zenu-matrix/src/operation/broadcast.rs:53-165
     for src, sshape, dshape in (([1.], [], [3]), ([1.], [], [2, 3]), ([1., 2., 3.], [3], [2, 3]),
                                 ([1., 2.], [1, 2], [2, 3, 1, 2]), ([1., 2., 3., 4.], [1, 1, 1, 4], [2, 3, 4, 4])):
