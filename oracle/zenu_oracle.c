@@ -316,10 +316,12 @@ static int zo_range_hash_run(zo_range_job proto, uint64_t first, uint64_t count,
         jobs[t].sums = sums;
         next += share;
     }
-    for (int t = 1; t < nthreads; t++)
-        if (pthread_create(&th[t], NULL, zo_range_worker, &jobs[t])) return ZO_ERR_ARG;
+    int started = 1;
+    for (; started < nthreads; started++)
+        if (pthread_create(&th[started], NULL, zo_range_worker, &jobs[started])) break;
     zo_range_worker(&jobs[0]);
-    for (int t = 1; t < nthreads; t++) pthread_join(th[t], NULL);
+    for (int t = started; t < nthreads; t++) zo_range_worker(&jobs[t]);   /* threads that could not be started: done here */
+    for (int t = 1; t < started; t++) pthread_join(th[t], NULL);
     return ZO_OK;
 }
 

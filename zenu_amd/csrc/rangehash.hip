@@ -20,21 +20,10 @@ __device__ __forceinline__ uint64_t range_hash_term(uint32_t arg_bits, uint32_t 
 
 constexpr int kHashBlock = 256;
 
-// one workgroup per block of 2^block_log2 patterns
-template <int FN>
-__global__ __launch_bounds__(kHashBlock) void range_hash_kernel(uint64_t first, int block_log2, uint64_t *sums,
-                                                                UnaryF<float, FN> f)
+// the workgroup's terms added up (mod 2^64, so the order does not matter) and stored as the sum of its block
+__device__ __forceinline__ void store_block_sum(uint64_t sum, uint64_t *sums)
 {
     __shared__ uint64_t part[kHashBlock / 64];
-    f.init();
-    const uint64_t per = 1ull << block_log2;
-    const uint64_t start = first + (uint64_t)blockIdx.x * per;
-    uint64_t sum = 0;
-    for (uint64_t i = threadIdx.x; i < per; i += kHashBlock) {
-        const uint32_t bits = (uint32_t)(start + i);
-        const float x = __uint_as_float(bits);
-        sum += range_hash_term(bits, __float_as_uint(f(x, x)));
-    }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = sum;
@@ -45,39 +34,30 @@ __global__ __launch_bounds__(kHashBlock) void range_hash_kernel(uint64_t first, 
         for (int w = 0; w < kHashBlock / 64; w++) total += part[w];
         sums[blockIdx.x] = total;
     }
+}
+
+// one workgroup per block of 2^block_log2 f32 patterns, any functor over f32 (a unary function, powf with its exponent)
+template <typename F>
+__global__ __launch_bounds__(kHashBlock) void range_hash_functor_kernel(uint64_t first, int block_log2, uint64_t *sums, F f)
+{
+    f.init();
+    const uint64_t per = 1ull << block_log2;
+    const uint64_t start = first + (uint64_t)blockIdx.x * per;
+    uint64_t sum = 0;
+    for (uint64_t i = threadIdx.x; i < per; i += kHashBlock) {
+        const uint32_t bits = (uint32_t)(start + i);
+        const float x = __uint_as_float(bits);
+        sum += range_hash_term(bits, __float_as_uint(f(x, x)));
+    }
+    store_block_sum(sum, sums);
 }
 
 template <int FN> int launch_range_hash(uint64_t first, uint64_t blocks, int block_log2, uint64_t *sums, hipStream_t s)
 {
-    range_hash_kernel<FN><<<(unsigned)blocks, kHashBlock, 0, s>>>(first, block_log2, sums, UnaryF<float, FN>());
+    range_hash_functor_kernel<UnaryF<float, FN>><<<(unsigned)blocks, kHashBlock, 0, s>>>(first, block_log2, sums,
+                                                                                         UnaryF<float, FN>());
     ZENU_LAUNCH_CHECK();
     return ZENU_OK;
-}
-
-// the same with any functor over f32 (powf with its exponent)
-template <typename F>
-__global__ __launch_bounds__(kHashBlock) void range_hash_functor_kernel(uint64_t first, int block_log2, uint64_t *sums, F f)
-{
-    __shared__ uint64_t part[kHashBlock / 64];
-    f.init();
-    const uint64_t per = 1ull << block_log2;
-    const uint64_t start = first + (uint64_t)blockIdx.x * per;
-    uint64_t sum = 0;
-    for (uint64_t i = threadIdx.x; i < per; i += kHashBlock) {
-        const uint32_t bits = (uint32_t)(start + i);
-        const float x = __uint_as_float(bits);
-        sum += range_hash_term(bits, __float_as_uint(f(x, x)));
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = sum;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint64_t total = 0;
-#pragma unroll
-        for (int w = 0; w < kHashBlock / 64; w++) total += part[w];
-        sums[blockIdx.x] = total;
-    }
 }
 
 // f64: the arguments cannot be exhausted.  Argument number i has the high word i * step + offset (sign,
@@ -102,7 +82,6 @@ __global__ __launch_bounds__(kHashBlock) void range_hash_f64_kernel(uint64_t fir
                                                                     uint32_t offset, uint64_t salt, uint64_t *sums,
                                                                     UnaryF<double, FN> f)
 {
-    __shared__ uint64_t part[kHashBlock / 64];
     f.init();
     const uint64_t per = 1ull << block_log2;
     const uint64_t start = first + (uint64_t)blockIdx.x * per;
@@ -114,16 +93,7 @@ __global__ __launch_bounds__(kHashBlock) void range_hash_f64_kernel(uint64_t fir
         if ((rb & 0x7fffffffffffffffull) > 0x7ff0000000000000ull) rb = 0x7ff8000000000000ull;
         sum += mix64(mix64(bits) + rb);
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = sum;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint64_t total = 0;
-#pragma unroll
-        for (int w = 0; w < kHashBlock / 64; w++) total += part[w];
-        sums[blockIdx.x] = total;
-    }
+    store_block_sum(sum, sums);
 }
 
 template <int FN>
