@@ -980,16 +980,17 @@ pub fn init(device: i32) {
 }
 
 /// Optional start-up check of the one thing the bit-exact f32 functions take on trust from the GPU
-/// they run on: `tanh`, the sigmoid, `sinh`, `cosh`, `atan`, `asin` and `acos` divide (and take square
+/// they run on: `tanh`, the sigmoid, `sinh`, `cosh`, `tan`, `atan`, `asin` and `acos` divide (and take square
 /// roots) with a short device sequence that is only correct on their own operand ranges.  The library
 /// evaluates each function with that sequence and with the IEEE operations on all 2^32 arguments
 /// (10-80 ms per function) and counts the arguments whose results differ; anything but zero is an error.
 pub fn self_check() -> Result<(), String> {
-    const FUNCTIONS: [(c_int, &str); 7] = [
+    const FUNCTIONS: [(c_int, &str); 8] = [
         (ZENU_TANH, "tanh"),
         (ZENU_SIGMOID, "sigmoid"),
         (ZENU_SINH, "sinh"),
         (ZENU_COSH, "cosh"),
+        (ZENU_TAN, "tan"),
         (ZENU_ATAN, "atan"),
         (ZENU_ASIN, "asin"),
         (ZENU_ACOS, "acos"),

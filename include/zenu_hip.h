@@ -408,7 +408,7 @@ int zenu_hip_adam_step_multi_scheduled(int dtype, int n_tensors, void *const *p_
  * the first status other than ZENU_OK that any of them produced on this thread since the last
  * call, and clears it: a wrapper can poll it after a batch of calls (no counterpart in the
  * reference, whose kernels check nothing). */
-/* Self-check of the device math: f32 tanh, sigmoid, sinh, cosh, atan, asin and acos (fn = the
+/* Self-check of the device math: f32 tanh, sigmoid, sinh, cosh, tan, atan, asin and acos (fn = the
  * zenu_unop_t value) use a 4-instruction division / square root that is exact only on the operands
  * these functions produce.  The call evaluates the function on ALL 2^32 f32 bit patterns twice on
  * the device -- as shipped, and with the IEEE division and square root in the same places -- and
@@ -419,7 +419,7 @@ int zenu_hip_adam_step_multi_scheduled(int dtype, int n_tensors, void *const *p_
 int zenu_hip_selfcheck_short_division(int fn, uint64_t *mismatches, uint32_t *example_bits,
                                       zenu_stream_t stream);
 /* Every f32 bit pattern of [first, first + count) through unary function fn (a zenu_unop_t value:
- * exp, log, tanh, sigmoid, sin, cos, asin, acos, atan, sinh, cosh -- the functions whose results are
+ * exp, log, tanh, sigmoid, sin, cos, tan, asin, acos, atan, sinh, cosh -- the functions whose results are
  * meant to be a host libm's bits), folded on the device into one 64-bit sum per block of
  * 2^block_log2 patterns (8 <= block_log2 <= 32; count a multiple of the block size):
  * sums_dev[b] = sum over the block of T(argument bits, result bits) mod 2^64, T = the finalizer of

@@ -107,7 +107,7 @@ template <typename T> struct UnaryExtra<T, ZENU_COS> {
     __device__ __forceinline__ void init() {}
 };
 template <> struct UnaryExtra<float, ZENU_TAN> {
-    zmath::SinCosCoef k;
+    zmath::TanfCoef tk;
     __device__ __forceinline__ void init() {}
 };
 template <> struct UnaryExtra<float, ZENU_ATAN> {
@@ -137,7 +137,7 @@ template <typename T, int FN> struct UnaryF {
         else if constexpr (FN == ZENU_SIN) return dev_sin(a, sc.k);
         else if constexpr (FN == ZENU_COS) return dev_cos(a, sc.k);
         else if constexpr (FN == ZENU_TAN) {
-            if constexpr (sizeof(T) == 4) return zmath::tanf_ulp1(a, sc.k);
+            if constexpr (sizeof(T) == 4) return zmath::tanf_glibc(a, sc.tk);
             else return tan(a);
         }
         else if constexpr (FN == ZENU_ASIN) return dev_asin(a);

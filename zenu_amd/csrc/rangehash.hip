@@ -126,6 +126,7 @@ extern "C" int zenu_hip_unary_range_hash(int fn, uint64_t first, uint64_t count,
     case ZENU_SIGMOID: return launch_range_hash<ZENU_SIGMOID>(first, blocks, block_log2, sums_dev, s);
     case ZENU_SIN: return launch_range_hash<ZENU_SIN>(first, blocks, block_log2, sums_dev, s);
     case ZENU_COS: return launch_range_hash<ZENU_COS>(first, blocks, block_log2, sums_dev, s);
+    case ZENU_TAN: return launch_range_hash<ZENU_TAN>(first, blocks, block_log2, sums_dev, s);
     case ZENU_ASIN: return launch_range_hash<ZENU_ASIN>(first, blocks, block_log2, sums_dev, s);
     case ZENU_ACOS: return launch_range_hash<ZENU_ACOS>(first, blocks, block_log2, sums_dev, s);
     case ZENU_ATAN: return launch_range_hash<ZENU_ATAN>(first, blocks, block_log2, sums_dev, s);

@@ -1,7 +1,7 @@
 // selfcheck.hip -- the short division and square root of zmath.hpp against the IEEE operations,
 // on the device, on every f32 argument of every function that uses them.
 //
-// tanh, the sigmoid, sinh, cosh, atan, asin and acos replace the compiler's 11-instruction IEEE
+// tanh, the sigmoid, sinh, cosh, tan, atan, asin and acos replace the compiler's 11-instruction IEEE
 // division (and the square root) by a reciprocal estimate and one correction by the exact
 // remainder.  That sequence is not correctly rounded for every operand pair, only for the pairs
 // these functions feed it, and the only proof of that is exhaustive.  Here the header is
@@ -45,6 +45,7 @@ enum { kDivPairs = 1000, kSqrtArgs = 1001 };
             else if constexpr (FN == ZENU_ATAN) return NS::atanf_fdlibm(x, at.tab);                    \
             else if constexpr (FN == ZENU_ASIN) return NS::asinf_fdlibm(x);                            \
             else if constexpr (FN == ZENU_ACOS) return NS::acosf_fdlibm(x);                            \
+            else if constexpr (FN == ZENU_TAN) return NS::tanf_glibc(x);                               \
             else if constexpr (FN == kDivPairs) {                                                      \
                 /* arbitrary operands, every exponent: the short sequence has no operand scaling, */   \
                 /* so quotients of very large or very small operands come out wrong               */   \
@@ -121,6 +122,7 @@ extern "C" int zenu_hip_selfcheck_short_division(int fn, uint64_t *mismatches, u
         case ZENU_ATAN: rc = run_check<ZENU_ATAN>(d, s); break;
         case ZENU_ASIN: rc = run_check<ZENU_ASIN>(d, s); break;
         case ZENU_ACOS: rc = run_check<ZENU_ACOS>(d, s); break;
+        case ZENU_TAN: rc = run_check<ZENU_TAN>(d, s); break;
         case kDivPairs: rc = run_check<kDivPairs>(d, s); break;
         case kSqrtArgs: rc = run_check<kSqrtArgs>(d, s); break;
         default: rc = ZENU_ERR_ARG;

@@ -875,61 +875,114 @@ ZM_HD float sincosf_glibc(float y, int cosine, const SinCosCoef &k = SinCosCoef(
     }
     return (y - y) / (y - y);                            // inf, NaN
 }
-// tanf evaluated in double: sincosf's argument reduction, its sine and cosine polynomials, and
-// their quotient (sin / cos in the even quadrants, -cos / sin in the odd ones), rounded once.  NOT
-// the host library's bits (its tanf is fdlibm's float code, whose argument reduction could not be
-// reproduced), but never more than 1 unit in the last place away from them: over all 2^32
-// arguments 97.5 % are equal and 2.5 % one apart.  IEEE operations only: host and device agree.
-ZM_HD float tanf_ulp1(float y, const SinCosCoef &k = SinCosCoef())
+// tanf (glibc 2.35: s_tanf.c and k_tanf.c are fdlibm's float code; e_rem_pio2f.c hands them sincosf's
+// argument reduction: the reduced argument in double, split into a float and the float remainder,
+// and the quadrant).  These files have no FMA build: every product rounds, also the one of the
+// reduction that sinf / cosf fuse.  Equal to the host libm on all 2^32 arguments.
+//
+// Restructured for 64-wide execution: one path through the reduction, the polynomial and ONE
+// division for every lane (the sources branch three ways after the polynomial, and two of the
+// branches divide).  What the sources decide beforehand folds into that path:
+//   * |x| <= pi/4 (their call of the kernel on x itself): the reduction finds quadrant 0 there and
+//     leaves x alone, with remainder 0;
+//   * a reduced argument below 2^-13 in an even quadrant (they return it): the general formula does
+//     too, x + (y + ...) with everything in the bracket below a quarter unit of x -- except that y can
+//     be exactly half a unit, so the case keeps its select;
+//   * x = 0 in an odd quadrant (1 / |x|) cannot occur: no float but 0 reduces to 0.
+// |x| >= 120: |x| times 4/pi as a 32 x 96 bit fixed-point product.  Returns the remainder after the
+// nearest multiple of pi/2 (in units of pi/2 2^-62, below 2^61 in magnitude) shifted left by one, with
+// the parity of that multiple in bit 0.  Out of line: few tensors hold such arguments.
+ZM_RARE int64_t tanf_reduce_large(uint32_t xi)
 {
-    const double Pi63 = 0x1.921FB54442D18p-62;
-    const uint32_t top = (f2u(y) >> 20) & 0x7ffu;
-    double x;
+    const uint32_t *arr = inv_pio4_table() + ((xi >> 26) & 15u);
+    const int shift = (int)((xi >> 23) & 7u);
+    xi = (xi & 0xffffffu) | 0x800000u;
+    xi <<= shift;
+    uint64_t res0 = (uint64_t)(uint32_t)(xi * arr[0]);
+    const uint64_t res1 = (uint64_t)xi * arr[4];
+    const uint64_t res2 = (uint64_t)xi * arr[8];
+    res0 = (res2 >> 32) | (res0 << 32);
+    res0 += res1;
+    const uint64_t q = (res0 + (1ull << 61)) >> 62;
+    res0 -= q << 62;
+    return (int64_t)(res0 << 1) | (int64_t)(q & 1u);
+}
+struct TanfCoef {
+    double hpi_inv = 0x1.45F306DC9C883p+23, hpi = 0x1.921FB54442D18p0;
+};
+ZM_HD float tanf_glibc(float xf, const TanfCoef &k = TanfCoef())
+{
+    const float pio4 = 7.8539812565e-01f, pio4lo = 3.7748947079e-08f;
+    const float T0 = 3.3333334327e-01f, T1 = 1.3333334029e-01f, T2 = 5.3968254477e-02f, T3 = 2.1869488060e-02f,
+                T4 = 8.8632395491e-03f, T5 = 3.5920790397e-03f, T6 = 1.4562094584e-03f, T7 = 5.8804126456e-04f,
+                T8 = 2.4646313977e-04f, T9 = 7.8179444245e-05f, T10 = 7.1407252108e-05f, T11 = -1.8558637748e-05f,
+                T12 = 2.5907305826e-05f;
+    const uint32_t top = (f2u(xf) >> 20) & 0x7ffu;
+    double dx = (double)xf;
     int n;
-    if (__builtin_expect(top < (0x42f00000u >> 20), 1)) {        // |y| < 120
-        x = (double)y;
-        const double r = x * k.hpi_inv;
+    if (__builtin_expect(top < (0x42f00000u >> 20), 1)) {        // |x| < 120
+        const double r = dx * k.hpi_inv;
         n = ((int32_t)r + 0x800000) >> 24;
-        x = __builtin_fma(-(double)n, k.hpi, x);
+        dx = dx - (double)n * k.hpi;
     } else if (top < (0x7f800000u >> 20)) {
-        uint32_t xi = f2u(y);
-        const int sign = (int)(xi >> 31);
-        const uint32_t *arr = inv_pio4_table() + ((xi >> 26) & 15u);
-        const int shift = (int)((xi >> 23) & 7u);
-        xi = (xi & 0xffffffu) | 0x800000u;
-        xi <<= shift;
-        uint64_t res0 = (uint64_t)(uint32_t)(xi * arr[0]);
-        const uint64_t res1 = (uint64_t)xi * arr[4];
-        const uint64_t res2 = (uint64_t)xi * arr[8];
-        res0 = (res2 >> 32) | (res0 << 32);
-        res0 += res1;
-        const uint64_t q = (res0 + (1ull << 61)) >> 62;
-        res0 -= q << 62;
-        x = (double)(int64_t)res0 * Pi63;
-        if (sign) x = -x;
-        n = (int)q;                                      // only its parity matters, and -q has q's
+        const int64_t packed = tanf_reduce_large(f2u(xf));
+        dx = (double)(packed >> 1) * 0x1.921FB54442D18p-62;
+        if (f2u(xf) >> 31) dx = -dx;
+        n = (int)(packed & 1);                           // only the quadrant's parity matters, and -q has q's
     } else {
-        return (y - y) / (y - y);                        // inf, NaN
+        return (xf - xf) * u2f(0x7f800000u);             // inf, NaN: the sources' x - x
     }
-    // on |x| (every step is odd resp. even in x): the quotient is then non-negative, a zero included,
-    // and takes the sign of x in the even quadrants, the opposite one in the odd ones
-    const double ax = __builtin_fabs(x);
-    const double x2 = x * x;
-    const double x3 = ax * x2;
-    const double s1 = __builtin_fma(x2, k.s3, k.s2);
-    const double x7 = x3 * x2;
-    const double sv = __builtin_fma(x3, k.s1, ax);
-    const double sn = __builtin_fma(x7, s1, sv);
-    const double x4 = x2 * x2;
-    const double c2 = __builtin_fma(x2, k.c4, k.c3);
-    const double c1 = __builtin_fma(x2, k.c1, 1.0);
-    const double x6 = x4 * x2;
-    const double c = __builtin_fma(x4, k.c2, c1);
-    const double cs = __builtin_fma(x6, c2, c);
+    const float y0 = (float)dx;
+    const float y1 = (float)(dx - (double)y0);
     const bool odd = (n & 1) != 0;
-    const float q = (float)((odd ? cs : sn) / (odd ? sn : cs));
-    const uint32_t neg = (uint32_t)(d2u(x) >> 63) ^ (uint32_t)odd;
-    return u2f(f2u(q) | (neg << 31));
+    const float fiy = odd ? -1.0f : 1.0f;                // the sources' iy
+
+    const uint32_t hx = f2u(y0);
+    const uint32_t ix = hx & 0x7fffffffu;
+    const bool big = ix >= 0x3f2ca140u;                  // |y0| >= 0.6744: tan(pi/4 - |y0|) and the angle sum
+    const bool tiny = ix < 0x39000000u;                  // |y0| < 2^-13
+    const uint32_t sgn = hx & 0x80000000u;
+    float x = y0, y = y1;
+    if (big) {
+        const float z0 = pio4 - u2f(ix);
+        const float w0 = pio4lo - u2f(f2u(y1) ^ sgn);
+        x = z0 + w0;
+        y = 0.0f;
+    }
+    const float z = x * x;
+    const float w2 = z * z;
+    // the two innermost Horner steps of the first polynomial and the three innermost of the second are
+    // fused: that changes none of the 2^32 results (each was tried alone, then all five together;
+    // fusing any other step changes between 36 and 22 535 338 of them)
+    float r = __builtin_fmaf(w2, __builtin_fmaf(w2, T11, T9), T7);
+    r = T1 + w2 * (T3 + w2 * (T5 + w2 * r));
+    float v = __builtin_fmaf(w2, __builtin_fmaf(w2, __builtin_fmaf(w2, T12, T10), T8), T6);
+    v = z * (T2 + w2 * (T4 + w2 * v));
+    const float s = z * x;
+    r = y + z * (s * (r + v) + y);
+    r += T0 * s;
+    const float w = x + r;
+    // the one quotient: w w / (w + iy) of the first branch, -1 / w of an odd quadrant (-1 / y0 below 2^-13)
+    const float num = big ? w * w : -1.0f;
+    const float den = big ? w + fiy : (tiny ? y0 : w);
+    const float q = div_fast(num, den);
+    float res;
+    if (big) {
+        // (products with 2 are exact: fusing them changes no rounding)
+        res = __builtin_fmaf(-2.0f, x - (q - r), fiy);
+        if (__builtin_fabsf(x) < 0x1p-13f) res = fiy * __builtin_fmaf(-2.0f * fiy, x, 1.0f);
+        res = u2f(f2u(res) ^ sgn);
+    } else if (!odd) {
+        res = tiny ? y0 : w;
+    } else {
+        // -1 / (x + r) to more than a float: the quotient and w cut to 12 bits, corrected by the products' remainders
+        const float zc = u2f(f2u(w) & 0xfffff000u);
+        const float vc = r - (zc - x);
+        const float tc = u2f(f2u(q) & 0xfffff000u);
+        const float sc = __builtin_fmaf(tc, zc, 1.0f);   // 12 x 12 bits: the product is exact
+        res = tiny ? q : tc + q * (sc + tc * vc);
+    }
+    return res;
 }
 
 ZM_HD float sinf_glibc(float x, const SinCosCoef &k = SinCosCoef()) { return sincosf_glibc(x, 0, k); }
