@@ -368,7 +368,7 @@ def build_ops(z, workload, stream):
         out64_h = np.empty_like(a64)
         sets64 = [(M.from_numpy(a64), M.alloc((n, n), dtype=np.float64)) for _ in range(nsets(4 * nb))]
         for name, fn in (("exp f64", _lib.EXP), ("tanh f64", _lib.TANH), ("sigmoid f64", _lib.SIGMOID), ("sinh f64", _lib.SINH),
-                         ("cosh f64", _lib.COSH)):
+                         ("cosh f64", _lib.COSH), ("sin f64", _lib.SIN), ("cos f64", _lib.COS)):
             ls = [(lambda d=O.desc(), s_=A.desc(), fn=fn: check(l.zenu_hip_unary(fn, _lib.F64, ref(d), ref(s_), stream), "unary f64"))
                   for A, O in sets64]
             cpu = (lambda: zo.sigmoid(out64_h, a64)) if fn == _lib.SIGMOID else (lambda fn=fn: zo.unary(fn, out64_h, a64))

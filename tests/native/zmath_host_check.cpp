@@ -11,6 +11,12 @@
 
 #include "../../zenu_amd/csrc/zmath.hpp"
 
+// sin and cos through pointers the compiler cannot see through: called on the same argument side by side
+// they would be merged into one sincos call, which is another function of the library (it reduces
+// |x| < 2.426265 differently and differs from sin / cos in the last bit on 1 in 1000 of such arguments)
+static double (*volatile libm_sin)(double) = sin;
+static double (*volatile libm_cos)(double) = cos;
+
 int main(int argc, char **argv)
 {
     const uint64_t stride = argc > 1 ? strtoull(argv[1], nullptr, 10) : 1;
@@ -66,14 +72,16 @@ int main(int argc, char **argv)
     for (auto &t : th) t.join();
     // double precision: every stride-th value of the HIGH word (sign, exponent, 20 mantissa bits) with
     // a pseudo-random low word, plus low words 0 and all-ones
-    std::atomic<uint64_t> bad_tanh64{0}, bad_expm164{0}, bad_sig64{0}, bad_exp64{0}, bad_sinh64{0}, bad_cosh64{0};
+    std::atomic<uint64_t> bad_tanh64{0}, bad_expm164{0}, bad_sig64{0}, bad_exp64{0}, bad_sinh64{0}, bad_cosh64{0}, bad_sin64{0}, bad_cos64{0};
     th.clear();
     for (int w = 0; w < nt; w++)
         th.emplace_back([&, w]() {
-            uint64_t b0 = 0, b1 = 0, b2 = 0, b3 = 0, b4 = 0, b5 = 0, rng = 0x9E3779B97F4A7C15ull * (w + 1);
+            uint64_t b0 = 0, b1 = 0, b2 = 0, b3 = 0, b4 = 0, b5 = 0, b6 = 0, b7 = 0, rng = 0x9E3779B97F4A7C15ull * (w + 1);
+            uint64_t round = 0;
             for (uint64_t u = (uint64_t)w * stride; u < (1ull << 32); u += stride * nt) {
                 rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17;
                 const uint32_t lows[3] = {(uint32_t)rng, 0u, 0xffffffffu};
+                const bool trig = (round++ & 7) == 0;     // sin / cos on every eighth high word (the host libm takes 100 ns on large arguments)
                 for (uint32_t lo : lows) {
                     const double x = zmath::u2d((u << 32) | lo);
                     const double ref = tanh(x), got = zmath::tanh_fdlibm(x), got2 = zmath::tanh_simd(x);
@@ -90,6 +98,11 @@ int main(int argc, char **argv)
                     const double chr = cosh(x), chg = zmath::cosh_fdlibm(x), chs = zmath::cosh_simd(x, zmath::exp_table());
                     if ((chr != chr) ? !(chg != chg) : zmath::d2u(chg) != zmath::d2u(chr)) b5++;
                     if ((chr != chr) ? !(chs != chs) : zmath::d2u(chs) != zmath::d2u(chr)) b5++;   // the form the kernels use
+                    if (trig) {
+                        const double snr = libm_sin(x), sng = zmath::sin_glibc(x), csr = libm_cos(x), csg = zmath::cos_glibc(x);
+                        if ((snr != snr) ? !(sng != sng) : zmath::d2u(sng) != zmath::d2u(snr)) b6++;
+                        if ((csr != csr) ? !(csg != csg) : zmath::d2u(csg) != zmath::d2u(csr)) b7++;
+                    }
                 }
                 // arguments where exp is finite and not 1: uniform in +-745 and in +-4
                 const double m = (double)(int64_t)rng / 9.2233720368547758e18;
@@ -101,6 +114,12 @@ int main(int argc, char **argv)
                     if (zmath::d2u(zmath::tanh_fdlibm(x)) != zmath::d2u(ref) || zmath::d2u(zmath::tanh_simd(x)) != zmath::d2u(ref)) b0++;
                     if (zmath::d2u(zmath::sigmoid_zenu(x)) != zmath::d2u(0.5 + 0.5 * tanh(0.5 * x))) b2++;
                 }
+                // sin / cos in each of their argument ranges: +-0.855, +-2.43, +-10, +-1000, +-1e6, +-1.05e8
+                if (trig)
+                    for (double x : {m * 0.855, m * 2.43, m * 10.0, m * 1000.0, m * 1e6, m * 1.05e8}) {
+                        if (zmath::d2u(zmath::sin_glibc(x)) != zmath::d2u(libm_sin(x))) b6++;
+                        if (zmath::d2u(zmath::cos_glibc(x)) != zmath::d2u(libm_cos(x))) b7++;
+                    }
                 for (double x : {m * 745.0, m * 4.0}) {
                     const double er = exp(x), eg = zmath::exp_glibc(x);
                     if (zmath::d2u(eg) != zmath::d2u(er)) b3++;
@@ -110,7 +129,7 @@ int main(int argc, char **argv)
                     if (zmath::d2u(chg) != zmath::d2u(chr)) b5++;
                 }
             }
-            bad_tanh64 += b0; bad_expm164 += b1; bad_sig64 += b2; bad_exp64 += b3; bad_sinh64 += b4; bad_cosh64 += b5;
+            bad_tanh64 += b0; bad_expm164 += b1; bad_sig64 += b2; bad_exp64 += b3; bad_sinh64 += b4; bad_cosh64 += b5; bad_sin64 += b6; bad_cos64 += b7;
         });
     for (auto &t : th) t.join();
     // powf(x, y)
@@ -152,5 +171,6 @@ int main(int argc, char **argv)
     printf("atanf_fdlibm %llu asinf_fdlibm %llu acosf_fdlibm %llu\n", (unsigned long long)bad_atan.load(),
            (unsigned long long)bad_asin.load(), (unsigned long long)bad_acos.load());
     printf("tanhf_ulp2_beyond_2ulp %llu tanf_glibc %llu\n", (unsigned long long)far_ulp2.load(), (unsigned long long)bad_tan.load());
-    return (bad_tan + bad_sinh_simd + bad_cosh_simd + far_ulp2 + bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64 + bad_exp64 + bad_sinh64 + bad_cosh64 + bad_exp + bad_log + bad_pow + bad_sinh + bad_cosh + bad_sin + bad_cos + bad_atan + bad_asin + bad_acos) ? 1 : 0;
+    printf("sin_glibc %llu cos_glibc %llu\n", (unsigned long long)bad_sin64.load(), (unsigned long long)bad_cos64.load());
+    return (bad_sin64 + bad_cos64 + bad_tan + bad_sinh_simd + bad_cosh_simd + far_ulp2 + bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64 + bad_exp64 + bad_sinh64 + bad_cosh64 + bad_exp + bad_log + bad_pow + bad_sinh + bad_cosh + bad_sin + bad_cos + bad_atan + bad_asin + bad_acos) ? 1 : 0;
 }

@@ -53,7 +53,8 @@ def test_zmath_matches_host_libm(tmp_path):
     each; stride 1, all 2^32, was run during development with the same result); powf on every 31st
     base for 19 fixed exponents and on two pseudo-random (base, exponent) pairs per base; f64 tanh,
     expm1, exp, sinh, cosh and the sigmoid composite on every 31st high word with three low words
-    each plus uniform samples in +-745 and +-4 (about 700 M points); f64 tanh in both of its forms
+    each plus uniform samples in +-745 and +-4 (about 700 M points); f64 sin and cos on every 248th high
+    word with three low words each plus uniform samples in each of their six argument ranges (150 M points each); f64 tanh in both of its forms
     (fdlibm's branches and the single path the kernels use) and the sigmoid also on 400 M uniform
     samples in +-1, +-4 and +-20.  tanhf_ulp2, the variant that
     is not meant to give libm's bits, must stay within 2 units in the last place of tanhf on the
@@ -67,4 +68,4 @@ def test_zmath_matches_host_libm(tmp_path):
                                   "expf_glibc", "0", "logf_glibc", "0", "powf_glibc", "0",
                                   "sinhf_fdlibm", "0", "coshf_fdlibm", "0", "sinhf_simd", "0", "coshf_simd", "0", "sinf_glibc", "0", "cosf_glibc", "0",
                                   "atanf_fdlibm", "0", "asinf_fdlibm", "0", "acosf_fdlibm", "0",
-                                  "tanhf_ulp2_beyond_2ulp", "0", "tanf_glibc", "0"]
+                                  "tanhf_ulp2_beyond_2ulp", "0", "tanf_glibc", "0", "sin_glibc", "0", "cos_glibc", "0"]

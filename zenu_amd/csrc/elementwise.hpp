@@ -80,10 +80,6 @@ template <typename T, int OP> struct ScalarF {
 
 __device__ __forceinline__ float dev_tanh(float x, const zmath::TanhRegs &rg) { return zmath::tanhf_simd(x, rg); }
 __device__ __forceinline__ double dev_tanh(double x, const zmath::TanhRegs &) { return zmath::tanh_simd(x); }
-__device__ __forceinline__ float dev_sin(float x, const zmath::SinCosCoef &k) { return zmath::sinf_glibc(x, k); }
-__device__ __forceinline__ double dev_sin(double x, const zmath::SinCosCoef &) { return sin(x); }
-__device__ __forceinline__ float dev_cos(float x, const zmath::SinCosCoef &k) { return zmath::cosf_glibc(x, k); }
-__device__ __forceinline__ double dev_cos(double x, const zmath::SinCosCoef &) { return cos(x); }
 __device__ __forceinline__ float dev_asin(float x) { return zmath::asinf_fdlibm(x); }
 __device__ __forceinline__ double dev_asin(double x) { return asin(x); }
 __device__ __forceinline__ float dev_acos(float x) { return zmath::acosf_fdlibm(x); }
@@ -93,18 +89,32 @@ __device__ __forceinline__ double dev_atan(double x) { return atan(x); }
 __device__ __forceinline__ float dev_sigmoid(float x, const zmath::TanhRegs &rg) { return zmath::sigmoidf_zenu(x, rg); }
 __device__ __forceinline__ double dev_sigmoid(double x, const zmath::TanhRegs &) { return zmath::sigmoid_zenu(x); }
 
-// what single functions carry besides: the f64 constants of the f32 sine / cosine / tangent (in the
-// functor, a kernel argument), the range table of the f32 arc tangent (in LDS); every other function nothing
+// what single functions carry besides: the f64 constants of the sine / cosine / tangent (in the functor, a
+// kernel argument), the tables of the f64 sine / cosine and of the f32 arc tangent (in LDS); every other function nothing
 template <typename T, int FN> struct UnaryExtra {
     __device__ __forceinline__ void init() {}
 };
-template <typename T> struct UnaryExtra<T, ZENU_SIN> {
+template <> struct UnaryExtra<float, ZENU_SIN> {
     zmath::SinCosCoef k;
     __device__ __forceinline__ void init() {}
+    __device__ __forceinline__ float sin(float x) const { return zmath::sinf_glibc(x, k); }
 };
-template <typename T> struct UnaryExtra<T, ZENU_COS> {
+template <> struct UnaryExtra<float, ZENU_COS> {
     zmath::SinCosCoef k;
     __device__ __forceinline__ void init() {}
+    __device__ __forceinline__ float cos(float x) const { return zmath::cosf_glibc(x, k); }
+};
+template <> struct UnaryExtra<double, ZENU_SIN> {
+    zmath::SinCos64Coef k;
+    zmath::SinCos64Lds t;
+    __device__ __forceinline__ void init() { t.init(); }
+    __device__ __forceinline__ double sin(double x) const { return zmath::sin_glibc(x, t.tab, k); }
+};
+template <> struct UnaryExtra<double, ZENU_COS> {
+    zmath::SinCos64Coef k;
+    zmath::SinCos64Lds t;
+    __device__ __forceinline__ void init() { t.init(); }
+    __device__ __forceinline__ double cos(double x) const { return zmath::cos_glibc(x, t.tab, k); }
 };
 template <> struct UnaryExtra<float, ZENU_TAN> {
     zmath::TanfCoef tk;
@@ -134,8 +144,8 @@ template <typename T, int FN> struct UnaryF {
         else if constexpr (FN == ZENU_TANH) return m.tanh(a, tr);
         else if constexpr (FN == ZENU_SQRT) return sqrt(a);
         else if constexpr (FN == ZENU_ABS) return fabs(a);
-        else if constexpr (FN == ZENU_SIN) return dev_sin(a, sc.k);
-        else if constexpr (FN == ZENU_COS) return dev_cos(a, sc.k);
+        else if constexpr (FN == ZENU_SIN) return sc.sin(a);
+        else if constexpr (FN == ZENU_COS) return sc.cos(a);
         else if constexpr (FN == ZENU_TAN) {
             if constexpr (sizeof(T) == 4) return zmath::tanf_glibc(a, sc.tk);
             else return tan(a);
@@ -259,6 +269,17 @@ template <typename F> struct IsValuBound { static constexpr bool value = false; 
 template <typename T> struct IsValuBound<UnaryF<T, ZENU_TANH>> { static constexpr bool value = true; };
 template <typename T> struct IsValuBound<UnaryF<T, ZENU_SIGMOID>> { static constexpr bool value = true; };
 template <> struct IsValuBound<TanhUlp2F> { static constexpr bool value = true; };   // 24.4 us against 27.1 at 64 x 1
+// f64 sine / cosine: a 3.5 KiB table per workgroup, and 60 f64 operations per element
+template <> struct IsValuBound<UnaryF<double, ZENU_SIN>> { static constexpr bool value = true; };
+template <> struct IsValuBound<UnaryF<double, ZENU_COS>> { static constexpr bool value = true; };
+// measured on 2^24 elements (us at 64 x 1 -> at 256 x 2): f32 sin 25.6 -> 23.8, cos 25.9 -> 23.8, asin 25.4 -> 24.0,
+// sinh 25.7 -> 25.2, cosh 26.4 -> 25.0; f64 sinh 63.9 -> 61.6, cosh 62.4 -> 55.4, sin 88.4 -> 53.0, cos 86.4 -> 51.4.
+// (f32 acos 25.0 -> 26.3 and atan 23.5 -> 24.7 prefer the small shape, tan does not care.)
+template <typename T> struct IsValuBound<UnaryF<T, ZENU_SINH>> { static constexpr bool value = true; };
+template <typename T> struct IsValuBound<UnaryF<T, ZENU_COSH>> { static constexpr bool value = true; };
+template <> struct IsValuBound<UnaryF<float, ZENU_SIN>> { static constexpr bool value = true; };
+template <> struct IsValuBound<UnaryF<float, ZENU_COS>> { static constexpr bool value = true; };
+template <> struct IsValuBound<UnaryF<float, ZENU_ASIN>> { static constexpr bool value = true; };
 template <typename T> struct IsValuBound<TanhBwdF<T>> { static constexpr bool value = true; };
 template <typename T> struct IsValuBound<SigmoidBwdF<T>> { static constexpr bool value = true; };
 

@@ -1797,6 +1797,352 @@ ZM_HD float coshf_simd(float x, const uint64_t *etab, const TanhRegs &rg = TanhR
 ZM_HD float sinhf_fdlibm(float x) { return sinhf_fdlibm(x, exp2f_table()); }
 ZM_HD float coshf_fdlibm(float x) { return coshf_fdlibm(x, exp2f_table()); }
 
+// ---- double precision sin / cos: s_sin.c and branred.c as glibc 2.35 ships them (the IBM Accurate
+// Mathematical Library without its multi-precision fall-backs) ------------------------------------------
+// |x| < 2^-26: x resp. 1.  The argument is brought to a in [-pi/4, pi/4] plus a small da and a quadrant n:
+//   * |x| < 0.855469: a = x;
+//   * |x| < 2.426265: a = pi/2 - |x| (sin: da = the low part of pi/2; cos: a and da renormalised);
+//   * |x| < 105414350: x - n pi/2 in three pieces of pi/2 (27, 26 and 52 + bits), n from a round-to-integer add;
+//   * above: 2/pi in 24-bit pieces times the two 27-bit halves of x, six pieces each from the one that
+//     reaches the binary point, the integer parts dropped (branred.c).
+// sine (even n) on |a| < 0.126 is a degree-11 Taylor form; otherwise sine and cosine (odd n) come from
+// sin(xi), cos(xi) at xi = k/128 (the nearest multiple, read off a + 1.5 2^45), each as a double and the
+// double of the remainder, and short polynomials in a - xi, combined by the angle-sum formulas with the
+// small terms first.  The table is regenerated here from that definition (exact rational arithmetic).
+// Fused multiply-adds where the compiler fuses them in the x86-64 build that CPUs with FMA select
+// (s_sin.c has one; branred.c has none, and its products are exact anyway).  Equal to the host libm's
+// sin and cos on 6.4e8 sampled arguments each: uniform in +-0.855, +-2.43, +-10, +-1000, +-1e6, +-1.05e8,
+// +-1e-3, +-1e-9, and random mantissas under every exponent from 2^26 to 2^1023.
+// (The library's sincos is another function: it reduces |x| < 2.426265 like the larger arguments and
+// differs from sin / cos in the last bit on 1 in 1000 of them.)
+#define ZM_SINCOS64_TAB                                                                                     \
+    {                                                                                                       \
+      0x0000000000000000ull, 0x0000000000000000ull, 0x3ff0000000000000ull, 0x0000000000000000ull,           \
+      0x3f7fffeaaaaeeeefull, 0xbc1e45e2ec67b77cull, 0x3fefffc000155552ull, 0x3c8f4a01a0196daeull,           \
+      0x3f8fffaaaaeeeed5ull, 0xbc02ab639a9f0776ull, 0x3fefff000155549full, 0x3c828a28a03a5ef3ull,           \
+      0x3f97ff7001033255ull, 0x3bfefe2b51527336ull, 0x3feffdc006bff7e6ull, 0x3c8ae6dae86977bdull,           \
+      0x3f9ffeaaaeeee86full, 0xbc3cd406fb224ae2ull, 0x3feffc00155527d3ull, 0xbc83b54492d89b5bull,           \
+      0x3fa3feb2b12d45d5ull, 0x3c34ec54203d1c11ull, 0x3feff9c03414a7baull, 0x3c6991f4be6c59bfull,           \
+      0x3fa7fdc01032fba9ull, 0xbc4599bdf46e997aull, 0x3feff7006bfdf99full, 0xbc78b3b560648d5full,           \
+      0x3fabfc6d78586dacull, 0x3c18e4fd03dbf236ull, 0x3feff3c0c8103a31ull, 0x3c74856dbddc0e66ull,           \
+      0x3faffaaaeeed4edbull, 0xbc42d16d32684b69ull, 0x3feff0015549f4d3ull, 0x3c8328387b99426full,           \
+      0x3fb1fc343d808befull, 0xbc5f3d32e6f3be4full, 0x3fefebc222a8ef9full, 0x3c57934934f54c77ull,           \
+      0x3fb3facb12d1755bull, 0xbc5921915299468bull, 0x3fefe7034129ef6full, 0xbc6cbf4337c96f97ull,           \
+      0x3fb5f911fd10b737ull, 0xbc50184f02be9102ull, 0x3fefe1c4c3c873ebull, 0xbc35a9c9057c4a02ull,           \
+      0x3fb7f701032550e4ull, 0x3c3afc2d1800501aull, 0x3fefdc06bf7e6b9bull, 0x3c831902b535f8dbull,           \
+      0x3fb9f4902d55d1f9ull, 0x3c52696d7eac1dc1ull, 0x3fefd5c94b43e000ull, 0xbc62e768cb4f92f9ull,           \
+      0x3fbbf1b78568391dull, 0x3c5e91841dea4cc8ull, 0x3fefcf0c800e99b1ull, 0x3c6ea3d786d186acull,           \
+      0x3fbdee6f16c1cce6ull, 0xbc450f8e2fb71673ull, 0x3fefc7d078d1bc88ull, 0x3c8075d2447db685ull,           \
+      0x3fbfeaaeee86ee36ull, 0xbc4afcb2bcc6f03bull, 0x3fefc015527d5bd3ull, 0x3c8b68f35094efb8ull,           \
+      0x3fc0f3378ddd71d1ull, 0x3c6d8468724f0f9eull, 0x3fefb7db2bfe0695ull, 0x3c821dadf4f65ab1ull,           \
+      0x3fc1f0d3d7afceafull, 0xbc66ef95099769a5ull, 0x3fefaf22263c4bd3ull, 0xbc552ace133a2769ull,           \
+      0x3fc2ee285e4ab88full, 0xbc6e4d0f05dee058ull, 0x3fefa5ea641c36f2ull, 0x3c404da6ed17cc7cull,           \
+      0x3fc3eb312c5d66cbull, 0x3c647d666b66cb91ull, 0x3fef9c340a7cc428ull, 0x3c8c5b6b063b7462ull,           \
+      0x3fc4e7ea4dc5f27bull, 0x3c5949db2ac072fcull, 0x3fef91ff40374d01ull, 0xbc67d03f4d3a9e4cull,           \
+      0x3fc5e44fcfa126f3ull, 0xbc66f443063f89b6ull, 0x3fef874c2e1eecf6ull, 0xbc8c6514e1332b16ull,           \
+      0x3fc6e05dc05a4d4cull, 0xbbd32c5c8b81c919ull, 0x3fef7c1afeffde24ull, 0xbc78f55bc47540b1ull,           \
+      0x3fc7dc102fbaf2b5ull, 0x3c45ab50e23c97c3ull, 0x3fef706bdf9ece1cull, 0xbc8698c80c36dcb4ull,           \
+      0x3fc8d7632efaa944ull, 0xbc620fa262cbb953ull, 0x3fef643efeb82acdull, 0x3c76b00ac1fe28acull,           \
+      0x3fc9d252d0cec312ull, 0x3c59c43d80b1137dull, 0x3fef57948cff6797ull, 0x3c6e3a0d3e03b1d4ull,           \
+      0x3fcaccdb297a0765ull, 0xbc59883b57d6cdeaull, 0x3fef4a6cbd1e3a79ull, 0x3c813df0edaebb57ull,           \
+      0x3fcbc6f84edc6199ull, 0x3c69c1a56a7b0cabull, 0x3fef3cc7c3b3d16eull, 0xbc621a3ad28a3494ull,           \
+      0x3fccc0a6588289a3ull, 0xbc6868d09bc87c6bull, 0x3fef2ea5d753ffedull, 0x3c8cc4215f56d583ull,           \
+      0x3fcdb9e15fb5a5d0ull, 0xbc632e20d6cc6fc2ull, 0x3fef20073086649full, 0x3c7b940416c1984bull,           \
+      0x3fceb2a57f8ae5a3ull, 0xbc60be06af572cebull, 0x3fef10ec09c5873bull, 0x3c8d9072762c1283ull,           \
+      0x3fcfaaeed4f31577ull, 0xbc615d88508e32b8ull, 0x3fef01549f7deea1ull, 0x3c8d3c1e99e5cafdull,           \
+      0x3fd0515cbf65155cull, 0xbc79b8c29dfd8ec7ull, 0x3feef141300d2f26ull, 0xbc82aa1b08ded372ull,           \
+      0x3fd0cd00cef36436ull, 0xbc79fb0a0c93e2b4ull, 0x3feee0b1fbc0f11cull, 0xbc4bfd2380bbc3b1ull,           \
+      0x3fd14861aa94ddebull, 0xbc6be881b5b615a4ull, 0x3feecfa744d5efa1ull, 0xbc556d0a4af541d0ull,           \
+      0x3fd1c37d64c6b876ull, 0x3c746076fe0dcff4ull, 0x3feebe214f76efa8ull, 0xbc802f9f12ba543eull,           \
+      0x3fd23e52111aaf36ull, 0xbc74f080334eff18ull, 0x3feeac2061bbaf4full, 0x3c62c1d53e94658dull,           \
+      0x3fd2b8ddc43eb49full, 0x3c61553899f2d807ull, 0x3fee99a4c3a7cd83ull, 0xbc82264b1bc53ce8ull,           \
+      0x3fd3331e94049f87ull, 0x3c7e0cb6b40c302cull, 0x3fee86aebf29a9edull, 0x3c89397afdbb58a7ull,           \
+      0x3fd3ad129769d3d8ull, 0x3c003d550487839aull, 0x3fee733ea0193d40ull, 0xbc86428b3546ce13ull,           \
+      0x3fd426b7e69ee697ull, 0xbc7f09c75705c59full, 0x3fee5f54b436e9d0ull, 0x3c87eb0fd02fc8bcull,           \
+      0x3fd4a00c9b0f3d20ull, 0x3c7823ba6bb08eadull, 0x3fee4af14b2a449cull, 0xbc868ca02e8a6833ull,           \
+      0x3fd5190ecf68a77aull, 0x3c7b357155eef0f3ull, 0x3fee3614b680d6a5ull, 0xbc727793aa015237ull,           \
+      0x3fd591bc9fa2f597ull, 0x3c67c74bac3fe0cbull, 0x3fee20bf49acd6c1ull, 0xbc5660aec7ef636bull,           \
+      0x3fd60a1429078775ull, 0x3c5b1fd80ba89133ull, 0x3fee0af15a03dbceull, 0x3c5fe8e702771ae6ull,           \
+      0x3fd682138a38d7f7ull, 0xbc7d889202444aadull, 0x3fedf4ab3ebd875eull, 0xbc8e2d8a7e6736c4ull,           \
+      0x3fd6f9b8e33a0255ull, 0x3c742bc14ee9da0dull, 0x3feddded50f228d6ull, 0xbc6e80c8d42ba2bfull,           \
+      0x3fd7710255764214ull, 0xbc66ead7314bb6ceull, 0x3fedc6b7eb995912ull, 0x3c54b364776dcd35ull,           \
+      0x3fd7e7ee03c86d4eull, 0xbc7b63bcdabf5af2ull, 0x3fedaf0b6b888e83ull, 0x3c8a249e2b5e5ceaull,           \
+      0x3fd85e7a12826949ull, 0x3c78a40e9b5face0ull, 0x3fed96e82f71a9dcull, 0x3c8ff61bd5d2039dull,           \
+      0x3fd8d4a4a774992full, 0x3c744a02ea766326ull, 0x3fed7e4e97e17b4aull, 0xbc63b770352bed94ull,           \
+      0x3fd94a6be9f546c5ull, 0xbc769ce13e683f58ull, 0x3fed653f073e4040ull, 0xbc876236434bec37ull,           \
+      0x3fd9bfce02e80510ull, 0x3c709e39a320b0a4ull, 0x3fed4bb9e1c619e0ull, 0x3c8f34bb77858f61ull,           \
+      0x3fda34c91cc50ccaull, 0xbc5a310e3b50cecdull, 0x3fed31bf8d8d7c06ull, 0x3c7e60dd3089cbddull,           \
+      0x3fdaa95b63a09277ull, 0xbc66293eb13c0381ull, 0x3fed1750727d94f0ull, 0x3c80d52b1ec1a48eull,           \
+      0x3fdb1d8305321617ull, 0xbc7ae242cb99f519ull, 0x3fecfc6cfa52ad9full, 0x3c88b5b5508f2a0dull,           \
+      0x3fdb913e30dbac43ull, 0xbc7e38ad2f6c3ff1ull, 0x3fece115909a82e5ull, 0x3c81f139bb31109aull,           \
+      0x3fdc048b17b140a3ull, 0x3c619fe6757e9fa7ull, 0x3fecc54aa2b2972eull, 0x3c64ee162ba83a98ull,           \
+      0x3fdc7767ec7fd19eull, 0xbc5eb14d1a3d5826ull, 0x3feca90c9fc67d0bull, 0xbc646a81485e3462ull,           \
+      0x3fdce9d2e3d4a51full, 0xbc62fc8a12dae298ull, 0x3fec8c5bf8ce1a84ull, 0x3c7ab3d1a1590123ull,           \
+      0x3fdd5bca34047661ull, 0x3c728a44a75fc29cull, 0x3fec6f39208be53bull, 0xbc8741dbfbaadb42ull,           \
+      0x3fddcd4c15329c9aull, 0x3c70d4c6e171fd9aull, 0x3fec51a48b8b175eull, 0xbc61bbb43b9aa880ull,           \
+      0x3fde3e56c1582a69ull, 0xbc50a4821099f88full, 0x3fec339eb01ddd81ull, 0xbc8caaf5ee82c5c0ull,           \
+      0x3fdeaee8744b05f0ull, 0xbc5789b43c9b027dull, 0x3fec1528065b7d50ull, 0xbc8892111312e828ull,           \
+      0x3fdf1eff6bc4f97bull, 0x3c717212f8a7525cull, 0x3febf641081e7536ull, 0x3c8b7bd71628a9a1ull,           \
+      0x3fdf8e99e76abc97ull, 0x3c59d950af2d00a3ull, 0x3febd6ea310294f5ull, 0x3c731bbcc88c109dull,           \
+      0x3fdffdb628d2f57aull, 0x3c6f4a992e905b6aull, 0x3febb723fe630f32ull, 0x3c772bd2452d0a39ull,           \
+      0x3fe0362939c69955ull, 0xbc82d8cd78397b01ull, 0x3feb96eeef58840eull, 0x3c545a3cc78fade0ull,           \
+      0x3fe06d3686946e5bull, 0x3c83f5ae4538ff1bull, 0x3feb764b84b704c2ull, 0xbc8f5848c21b389bull,           \
+      0x3fe0a4021e9e1001ull, 0xbc86f643a13914f6ull, 0x3feb553a410c104eull, 0x3c58ff7947027a15ull,           \
+      0x3fe0da8b26b5672eull, 0xbc8a58def0bee909ull, 0x3feb33bba89c8948ull, 0x3c8ea6a51d1f6ca9ull,           \
+      0x3fe110d0c4b69c3bull, 0x3c8d918998809981ull, 0x3feb11d04162a4c6ull, 0x3c71dd561efbc0c2ull,           \
+      0x3fe146d21f8b7f82ull, 0x3c7bf9535e2739a8ull, 0x3feaef78930bd275ull, 0xbc7f836279746f94ull,           \
+      0x3fe17c8e5f2eedb0ull, 0x3c635e57102e2488ull, 0x3feaccb526f69de5ull, 0x3c88fb6a8dd6b6ccull,           \
+      0x3fe1b204acb02fddull, 0xbc5f190c70cbb5feull, 0x3feaa98688308913ull, 0xbc0b83d607cd5072ull,           \
+      0x3fe1e7343236574cull, 0x3c722a3fa4f41d5aull, 0x3fea85ed4373e02dull, 0x3c69be06385ec792ull,           \
+      0x3fe21c1c1b0394cfull, 0x3c5e5b324b23aa31ull, 0x3fea61e9e72586afull, 0x3c858330e2fd453full,           \
+      0x3fe250bb93788bbbull, 0x3c7ea3d02457bcceull, 0x3fea3d7d0352bdcfull, 0xbc868dbaeca19669ull,           \
+      0x3fe28511c917a067ull, 0xbc801df1d9a16b70ull, 0x3fea18a729aee445ull, 0x3c395e25736c0357ull,           \
+      0x3fe2b91dea88421eull, 0xbc8fa371db216ab0ull, 0x3fe9f368ed912f85ull, 0xbc81d200c5791606ull,           \
+      0x3fe2ecdf279a3082ull, 0x3c8d3557e0e7e37eull, 0x3fe9cdc2e3f25e5cull, 0x3c83f99112993f62ull,           \
+      0x3fe32054b148bc4full, 0x3c8f6b42095a135bull, 0x3fe9a7b5a36a6514ull, 0x3c8722cfcc9fa7a9ull,           \
+      0x3fe3537db9be0367ull, 0x3c6b327e7af040f0ull, 0x3fe98141c42e1310ull, 0x3c8d1ff80488f08dull,           \
+      0x3fe386597456282bull, 0xbc710fada93b07a8ull, 0x3fe95a67e00cb1fdull, 0xbc80befda21f862dull,           \
+      0x3fe3b8e715a2840aull, 0xbc797653a7d2f07aull, 0x3fe93328926d9e92ull, 0xbc8bb77003600cdaull,           \
+      0x3fe3eb25d36cd53aull, 0xbc5be570e1570fc0ull, 0x3fe90b84784ddaf7ull, 0xbc70feb10ab93b87ull,           \
+      0x3fe41d14e4ba6790ull, 0x3c84608fd287ecf5ull, 0x3fe8e37c303d9ad1ull, 0xbc6463a4b53d4bf8ull,           \
+      0x3fe44eb381cf386bull, 0xbc83ed6c1e6a5505ull, 0x3fe8bb105a5dc900ull, 0x3c8863e03e9474c1ull,           \
+      0x3fe48000e431159full, 0xbc8b194a7463ed10ull, 0x3fe89241985d871full, 0x3c8c48d9c413ed84ull,           \
+      0x3fe4b0fc46aab761ull, 0x3c20da05738cc59cull, 0x3fe869108d77a6c6ull, 0x3c7338ffe2bfe9ddull,           \
+      0x3fe4e1a4e54ed51bull, 0xbc8a492f89b7c76aull, 0x3fe83f7dde701ca0ull, 0xbc4152cf609bc6e8ull,           \
+      0x3fe511f9fd7b351cull, 0xbc85c0e861c48831ull, 0x3fe8158a31916d5dull, 0xbc6de8b90b8228deull,           \
+      0x3fe541facddbb724ull, 0x3c7232c28520d391ull, 0x3fe7eb362eaa1488ull, 0x3c5a1d65a4a5959full,           \
+      0x3fe571a6966d59b3ull, 0x3c5c843b4d0fb197ull, 0x3fe7c0827f09e54full, 0xbc6c73d6d72aee68ull,           \
+      0x3fe5a0fc98813a12ull, 0xbc8d82e2b7d4227bull, 0x3fe7956fcd7f6543ull, 0xbc8ab276e9d45ae4ull,           \
+      0x3fe5cffc16bf8f0dull, 0x3c896cb370eb578aull, 0x3fe769fec655211full, 0xbc6827d5cf8c68c5ull,           \
+      0x3fe5fea4552a9e57ull, 0x3c80b6cef7ee20b7ull, 0x3fe73e30174efba1ull, 0xbc65d3ae3d94ad5full,           \
+      0x3fe62cf49921ac79ull, 0xbc8edd9855b6241aull, 0x3fe712046fa77678ull, 0x3c8425b0a5029c81ull,           \
+      0x3fe65aec2963e755ull, 0x3c8126f96b71053cull, 0x3fe6e57c800cf55eull, 0x3c860286dedbd0a6ull,           \
+      0x3fe6888a4e134b2full, 0xbc86b7d37644d5e6ull, 0x3fe6b898fa9efb5dull, 0x3c715ac786ccf4b2ull,           \
+      0x3fe6b5ce50b7821aull, 0xbc65d5158f702e0full, 0x3fe68b5a92eb6253ull, 0xbc89a91ad985f89cull,           \
+      0x3fe6e2b77c40bde1ull, 0xbc70e729857fad53ull, 0x3fe65dc1fdeb8cbaull, 0xbc597c1b47337c77ull,           \
+      0x3fe70f451d0a8c40ull, 0x3c697ede3885770dull, 0x3fe62fcff20191c7ull, 0x3c6d9143895756efull,           \
+      0x3fe73b7680dea578ull, 0xbc72248306dc12a2ull, 0x3fe6018526f563dfull, 0x3c846ca5e0e432d0ull,           \
+      0x3fe7674af6f7b524ull, 0x3c7e9d3f94ac84a8ull, 0x3fe5d2e255f1f17aull, 0x3c80314104c8892bull,           \
+      0x3fe792c1d0041d52ull, 0xbc8abf05eeb354ebull, 0x3fe5a3e839824077ull, 0x3c8428aa2759be62ull,           \
+      0x3fe7bdda5e28b3c2ull, 0x3c4ad1197ccd0392ull, 0x3fe574978d8e83f2ull, 0x3c8f4714af282d23ull,           \
+      0x3fe7e893f5037959ull, 0x3c80eefbaa650c4cull, 0x3fe544f10f592ca5ull, 0xbc8e7ae8e6c7a62full,           \
+      0x3fe812ede9ae4ba4ull, 0xbc87830adf402ddaull, 0x3fe514f57d7bf3daull, 0x3c747a108073c259ull,           \
+      0x3fe83ce792c1906eull, 0xbc7f3899682b4a7dull, 0x3fe4e4a597e4e10eull, 0x3c7ccd992849f6c8ull            \
+    }
+#define ZM_TOVERP_TAB                                                                                       \
+    {                                                                                                       \
+      10680707.0, 7228996.0, 1387004.0, 2578385.0, 16069853.0, 12639074.0, 9804092.0, 4427841.0,            \
+      16666979.0, 11263675.0, 12935607.0, 2387514.0, 4345298.0, 14681673.0, 3074569.0, 13734428.0,          \
+      16653803.0, 1880361.0, 10960616.0, 8533493.0, 3062596.0, 8710556.0, 7349940.0, 6258241.0,             \
+      3772886.0, 3769171.0, 3798172.0, 8675211.0, 12450088.0, 3874808.0, 9961438.0, 366607.0,               \
+      15675153.0, 9132554.0, 7151469.0, 3571407.0, 2607881.0, 12013382.0, 4155038.0, 6285869.0,             \
+      7677882.0, 13102053.0, 15825725.0, 473591.0, 9065106.0, 15363067.0, 6271263.0, 9264392.0,             \
+      5636912.0, 4652155.0, 7056368.0, 13614112.0, 10155062.0, 1944035.0, 9527646.0, 15080200.0,            \
+      6658437.0, 6231200.0, 6832269.0, 16767104.0, 5075751.0, 3212806.0, 1398474.0, 7579849.0,              \
+      6349435.0, 12618859.0, 4703257.0, 12806093.0, 14477321.0, 2786137.0, 12875403.0, 9837734.0,           \
+      14528324.0, 13719321.0, 343717.0                                                                      \
+    }
+static const uint64_t kSinCos64TabHost[444] = ZM_SINCOS64_TAB;
+static const double kToverpHost[75] = ZM_TOVERP_TAB;
+#if defined(__HIPCC__)
+static __device__ const uint64_t kSinCos64TabDev[444] = ZM_SINCOS64_TAB;
+static __device__ const double kToverpDev[75] = ZM_TOVERP_TAB;
+#endif
+ZM_HD const double *sincos64_table()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return reinterpret_cast<const double *>(kSinCos64TabDev);
+#else
+    return reinterpret_cast<const double *>(kSinCos64TabHost);
+#endif
+}
+ZM_HD const double *toverp_table()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return kToverpDev;
+#else
+    return kToverpHost;
+#endif
+}
+
+// the constants as data (a kernel argument: scalar registers feed the f64 operations directly)
+struct SinCos64Coef {
+    double big = 0x1.8p45, toint = 0x1.8p52, hpinv = 0x1.45f306dc9c883p-1;
+    double hp0 = 0x1.921fb54442d18p0, hp1 = 0x1.1a62633145c07p-54;
+    double mp1 = 0x1.921FB58000000p0, mp2 = -0x1.DDE973C000000p-27, pp3 = -0x1.CB3B398000000p-55, pp4 = -0x1.d747f23e32ed7p-83;
+    double sn3 = -1.66666666666664880952546298448555E-01, sn5 = 8.33333214285722277379541354343671E-03;
+    double cs2 = 4.99999999999999999999950396842453E-01, cs4 = -4.16666666666664434524222570944589E-02,
+           cs6 = 1.38888874007937613028114285595617E-03;
+    double s1 = -0x1.5555555555555p-3, s2 = 0x1.1111111110ECEp-7, s3 = -0x1.A01A019DB08B8p-13, s4 = 0x1.71DE27B9A7ED9p-19,
+           s5 = -0x1.ADDFFC2FCDF59p-26;
+};
+
+// sin (n even) or cos (n odd) of a + da, negated for n = 2, 3 (the sources' do_sincos with do_sin, do_cos,
+// TAYLOR_SIN).  do_sin and do_cos are one path here: a wavefront usually holds both parities.  With
+// (M, m) = (sin xi, its low part) and (P, p) = (cos xi, its low part) for the sine, and (cos xi, low) and
+// (-sin xi, -low) for the cosine, both corrections read P s + (-M c + (s p + m)) and both results M + cor;
+// what differs is where da enters s and c.
+ZM_HD double sincos64_eval(double a, double da, int n, const double *tab, const SinCos64Coef &k)
+{
+    const double aa = __builtin_fabs(a);
+    const bool cosine = (n & 1) != 0;
+    double r;
+    if (!cosine && aa < 0.126) {
+        const double xx = a * a;
+        double p = __builtin_fma(k.s5, xx, k.s4);
+        p = __builtin_fma(p, xx, k.s3);
+        p = __builtin_fma(p, xx, k.s2);
+        p = __builtin_fma(p, xx, k.s1);
+        const double t = __builtin_fma(__builtin_fma(p, a, -0.5 * da), xx, da);
+        r = a + t;
+    } else {
+        const double u = k.big + aa;                     // its low mantissa bits: the nearest multiple of 1/128
+        const double *e = tab + 4 * (int)(uint32_t)d2u(u);
+        const uint64_t flip = cosine ? 0x8000000000000000ull : 0ull;
+        const double M = e[cosine ? 2 : 0], m = e[cosine ? 3 : 1];
+        const double P = u2d(d2u(e[cosine ? 0 : 2]) ^ flip), p = u2d(d2u(e[cosine ? 1 : 3]) ^ flip);
+        // da with the sign of a (the sine takes a = 0 as negative, which only matters to the sign of a zero)
+        const double dx = (cosine ? a < 0 : a <= 0) ? -da : da;
+        const double x0 = aa - (u - k.big);
+        const double x = cosine ? x0 + dx : x0;
+        const double xx = x * x;
+        const double t = __builtin_fma(x * xx, __builtin_fma(xx, k.sn5, k.sn3), cosine ? x : dx);
+        const double s = cosine ? t : x + t;
+        const double c = __builtin_fma(x, cosine ? 0.0 : dx, xx * __builtin_fma(xx, __builtin_fma(xx, k.cs6, k.cs4), k.cs2));
+        const double cor = __builtin_fma(P, s, __builtin_fma(-M, c, __builtin_fma(s, p, m)));
+        r = M + cor;
+        if (!cosine) r = __builtin_copysign(r, a);
+    }
+    return (n & 2) ? -r : r;
+}
+
+// |x| >= 105414350 (branred.c, then the evaluation above with quadrant n + nadd).  Out of line: few tensors hold
+// such arguments.  (It builds its own constants: a reference to the caller's would force them into memory there.)
+ZM_RARE double sincos64_huge(double x, int nadd, const double *tab)
+{
+    const SinCos64Coef k;
+    const double tm600 = 0x1p-600, split = 134217729.0, tm24 = 0x1p-24, big = 0x1.8p52, big1 = 0x1.8p54;
+    const double mp2 = -0x1.DDE9740000000p-27;           // branred.c's second piece of pi/2 is shorter than s_sin.c's
+    const double *toverp = toverp_table();
+    x *= tm600;
+    double t = x * split;
+    const double x1 = t - (t - x);
+    const double x2 = x - x1;
+    double b1 = 0, bb1 = 0, sum1 = 0, b2 = 0, bb2 = 0, sum2 = 0;
+    for (int h = 0; h < 2; h++) {
+        const double xp = h ? x2 : x1;
+        double r[6], s, sum = 0;
+        int j = (int)((d2u(xp) >> 52) & 2047u);
+        j = (j - 450) / 24;
+        if (j < 0) j = 0;
+        double gor = u2d(d2u(0x1p576) - ((uint64_t)(j * 24) << 52));
+        for (int i = 0; i < 6; i++) {
+            r[i] = xp * toverp[j + i] * gor;
+            gor *= tm24;
+        }
+        for (int i = 0; i < 3; i++) {
+            s = (r[i] + big) - big;
+            sum += s;
+            r[i] -= s;
+        }
+        t = 0;
+        for (int i = 0; i < 6; i++) t += r[5 - i];
+        double bb = (((((r[0] - t) + r[1]) + r[2]) + r[3]) + r[4]) + r[5];
+        s = (t + big) - big;
+        sum += s;
+        t -= s;
+        const double b = t + bb;
+        bb = (t - b) + bb;
+        s = (sum + big1) - big1;
+        sum -= s;
+        if (h) { b2 = b; bb2 = bb; sum2 = sum; }
+        else { b1 = b; bb1 = bb; sum1 = sum; }
+    }
+    double sum = sum1 + sum2;
+    double b = b1 + b2;
+    double bb = (__builtin_fabs(b1) > __builtin_fabs(b2)) ? (b1 - b) + b2 : (b2 - b) + b1;
+    if (b > 0.5) { b -= 1.0; sum += 1.0; }
+    else if (b < -0.5) { b += 1.0; sum -= 1.0; }
+    double s = b + (bb + bb1 + bb2);
+    t = ((b - s) + bb) + (bb1 + bb2);
+    b = s * split;
+    const double t1 = b - (b - s);
+    const double t2 = s - t1;
+    b = s * k.hp0;
+    bb = (((t1 * k.mp1 - b) + t1 * mp2) + t2 * k.mp1) + (t2 * mp2 + s * k.hp1 + t * k.hp0);
+    s = b + bb;
+    t = (b - s) + bb;
+    return sincos64_eval(s, t, (int)sum + nadd, tab, k);
+}
+
+// x - n pi/2 for |x| < 105414350 as a + da; returns n + nadd
+ZM_HD int sincos64_reduce(double x, int nadd, double &a, double &da, const SinCos64Coef &k)
+{
+    const double t = __builtin_fma(x, k.hpinv, k.toint);
+    const double xn = t - k.toint;
+    const double y = __builtin_fma(-xn, k.mp2, __builtin_fma(-xn, k.mp1, x));
+    double t1 = xn * k.pp3;
+    const double t2 = y - t1;
+    double db = (y - t2) - t1;
+    t1 = xn * k.pp4;
+    const double b = t2 - t1;
+    db += (t2 - b) - t1;
+    a = b;
+    da = db;
+    return (int)(uint32_t)d2u(t) + nadd;
+}
+
+ZM_HD double sin_glibc(double x, const double *tab, const SinCos64Coef &k = SinCos64Coef())
+{
+    const uint32_t hi = (uint32_t)(d2u(x) >> 32) & 0x7fffffffu;
+    if (hi < 0x3e500000u) return x;                      // |x| < 2^-26
+    double a, da;
+    int n;
+    if (hi < 0x3feb6000u) {                              // |x| < 0.855469
+        a = x;
+        da = 0.0;
+        n = 0;
+    } else if (hi < 0x400368fdu) {                       // |x| < 2.426265: cos(pi/2 - |x|) with the sign of x
+        a = k.hp0 - __builtin_fabs(x);
+        da = k.hp1;
+        n = (d2u(x) >> 63) ? 3 : 1;
+    } else if (hi < 0x419921FBu) {                       // |x| < 105414350
+        n = sincos64_reduce(x, 0, a, da, k);
+    } else if (hi < 0x7ff00000u) {
+        return sincos64_huge(x, 0, tab);
+    } else {
+        return x - x;                                    // inf, NaN (the sources' x / x)
+    }
+    return sincos64_eval(a, da, n, tab, k);
+}
+
+ZM_HD double cos_glibc(double x, const double *tab, const SinCos64Coef &k = SinCos64Coef())
+{
+    const uint32_t hi = (uint32_t)(d2u(x) >> 32) & 0x7fffffffu;
+    if (hi < 0x3e400000u) return 1.0;                    // |x| < 2^-27
+    double a, da;
+    int n;
+    if (hi < 0x3feb6000u) {
+        a = x;
+        da = 0.0;
+        n = 1;
+    } else if (hi < 0x400368fdu) {                       // sin(pi/2 - |x|), the difference renormalised
+        const double y = k.hp0 - __builtin_fabs(x);
+        a = y + k.hp1;
+        da = (y - a) + k.hp1;
+        n = 0;
+    } else if (hi < 0x419921FBu) {
+        n = sincos64_reduce(x, 1, a, da, k);
+    } else if (hi < 0x7ff00000u) {
+        return sincos64_huge(x, 1, tab);
+    } else {
+        return x - x;
+    }
+    return sincos64_eval(a, da, n, tab, k);
+}
+ZM_HD double sin_glibc(double x) { return sin_glibc(x, sincos64_table()); }
+ZM_HD double cos_glibc(double x) { return cos_glibc(x, sincos64_table()); }
+
 #if defined(__HIPCC__)
 // exp / log / sinh / cosh as the kernels call them: through tables copied to LDS by init(), which
 // every thread of the workgroup (at least 64 threads) calls once before anything else (it
@@ -1866,6 +2212,18 @@ struct AtanfLds {
         if (threadIdx.x < 40) lds_atan[threadIdx.x] = kAtanfTabDev[threadIdx.x];
         __syncthreads();
         tab = lds_atan;
+    }
+};
+
+// the f64 sine / cosine table in LDS, same arrangement
+struct SinCos64Lds {
+    const double *tab;
+    __device__ __forceinline__ void init()
+    {
+        __shared__ uint64_t lds_sincos[444];
+        for (int i = threadIdx.x; i < 444; i += blockDim.x) lds_sincos[i] = kSinCos64TabDev[i];
+        __syncthreads();
+        tab = reinterpret_cast<const double *>(lds_sincos);
     }
 };
 
