@@ -367,13 +367,16 @@ def build_ops(z, workload, stream):
         a64 = a.astype(np.float64)
         out64_h = np.empty_like(a64)
         sets64 = [(M.from_numpy(a64), M.alloc((n, n), dtype=np.float64)) for _ in range(nsets(4 * nb))]
+        pos64 = np.abs(a64) + 0.01
+        sets64p = [(M.from_numpy(pos64), O) for _, O in sets64]
         for name, fn in (("exp f64", _lib.EXP), ("tanh f64", _lib.TANH), ("sigmoid f64", _lib.SIGMOID), ("sinh f64", _lib.SINH),
-                         ("cosh f64", _lib.COSH), ("sin f64", _lib.SIN), ("cos f64", _lib.COS)):
+                         ("cosh f64", _lib.COSH), ("sin f64", _lib.SIN), ("cos f64", _lib.COS), ("log f64", _lib.LOG)):
+            src_sets, src_h = (sets64p, pos64) if fn == _lib.LOG else (sets64, a64)
             ls = [(lambda d=O.desc(), s_=A.desc(), fn=fn: check(l.zenu_hip_unary(fn, _lib.F64, ref(d), ref(s_), stream), "unary f64"))
-                  for A, O in sets64]
-            cpu = (lambda: zo.sigmoid(out64_h, a64)) if fn == _lib.SIGMOID else (lambda fn=fn: zo.unary(fn, out64_h, a64))
+                  for A, O in src_sets]
+            cpu = (lambda: zo.sigmoid(out64_h, a64)) if fn == _lib.SIGMOID else (lambda fn=fn, h=src_h: zo.unary(fn, out64_h, h))
             ops.append(Op(name, "next", "f64", 4 * nb, n * n, ls, cpu))
-        ops[-1].keep = (sets, sets64)
+        ops[-1].keep = (sets, sets64, sets64p)
 
     # ---- the same kernels on larger tensors: how much of the distance to the roofline is the fixed
     # cost of a launch at the BASELINE sizes (not a BASELINE config) --------------------------------------

@@ -433,8 +433,8 @@ int zenu_hip_unary_range_hash(int fn, uint64_t first, uint64_t count, int block_
 /* The same for powf(x, exponent) over the f32 bases x. */
 int zenu_hip_powf_range_hash(double exponent, uint64_t first, uint64_t count, int block_log2,
                              uint64_t *sums_dev, zenu_stream_t stream);
-/* The same for the f64 functions whose results are meant to be a host libm's bits (exp, tanh, sigmoid,
- * sinh, cosh, sin, cos) on SAMPLED arguments: argument number i of [first, first + count) has the high word
+/* The same for the f64 functions whose results are meant to be a host libm's bits (exp, log, tanh,
+ * sigmoid, sinh, cosh, sin, cos) on SAMPLED arguments: argument number i of [first, first + count) has the high word
  * (sign, exponent, 20 mantissa bits) (uint32_t)(i * step + offset) and the low word
  * (uint32_t)(((i + salt) * 0x9E3779B97F4A7C15) >> 29); the term is M(M(argument bits) + result bits)
  * with M the finalizer of splitmix64 and every NaN result counted as 0x7ff8000000000000. */

@@ -72,11 +72,11 @@ int main(int argc, char **argv)
     for (auto &t : th) t.join();
     // double precision: every stride-th value of the HIGH word (sign, exponent, 20 mantissa bits) with
     // a pseudo-random low word, plus low words 0 and all-ones
-    std::atomic<uint64_t> bad_tanh64{0}, bad_expm164{0}, bad_sig64{0}, bad_exp64{0}, bad_sinh64{0}, bad_cosh64{0}, bad_sin64{0}, bad_cos64{0};
+    std::atomic<uint64_t> bad_tanh64{0}, bad_expm164{0}, bad_sig64{0}, bad_exp64{0}, bad_sinh64{0}, bad_cosh64{0}, bad_sin64{0}, bad_cos64{0}, bad_log64{0};
     th.clear();
     for (int w = 0; w < nt; w++)
         th.emplace_back([&, w]() {
-            uint64_t b0 = 0, b1 = 0, b2 = 0, b3 = 0, b4 = 0, b5 = 0, b6 = 0, b7 = 0, rng = 0x9E3779B97F4A7C15ull * (w + 1);
+            uint64_t b0 = 0, b1 = 0, b2 = 0, b3 = 0, b4 = 0, b5 = 0, b6 = 0, b7 = 0, b8 = 0, rng = 0x9E3779B97F4A7C15ull * (w + 1);
             uint64_t round = 0;
             for (uint64_t u = (uint64_t)w * stride; u < (1ull << 32); u += stride * nt) {
                 rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17;
@@ -98,6 +98,8 @@ int main(int argc, char **argv)
                     const double chr = cosh(x), chg = zmath::cosh_fdlibm(x), chs = zmath::cosh_simd(x, zmath::exp_table());
                     if ((chr != chr) ? !(chg != chg) : zmath::d2u(chg) != zmath::d2u(chr)) b5++;
                     if ((chr != chr) ? !(chs != chs) : zmath::d2u(chs) != zmath::d2u(chr)) b5++;   // the form the kernels use
+                    const double lgr = log(x), lgg = zmath::log_glibc(x);
+                    if ((lgr != lgr) ? !(lgg != lgg) : zmath::d2u(lgg) != zmath::d2u(lgr)) b8++;
                     if (trig) {
                         const double snr = libm_sin(x), sng = zmath::sin_glibc(x), csr = libm_cos(x), csg = zmath::cos_glibc(x);
                         if ((snr != snr) ? !(sng != sng) : zmath::d2u(sng) != zmath::d2u(snr)) b6++;
@@ -120,6 +122,9 @@ int main(int argc, char **argv)
                         if (zmath::d2u(zmath::sin_glibc(x)) != zmath::d2u(libm_sin(x))) b6++;
                         if (zmath::d2u(zmath::cos_glibc(x)) != zmath::d2u(libm_cos(x))) b7++;
                     }
+                // log around 1 (both of its branches), on [0, 100) and log-uniform over the whole range
+                for (double x : {1.0 + m * 0.5, fabs(m) * 100.0, exp(m * 700.0)})
+                    if (zmath::d2u(zmath::log_glibc(x)) != zmath::d2u(log(x))) b8++;
                 for (double x : {m * 745.0, m * 4.0}) {
                     const double er = exp(x), eg = zmath::exp_glibc(x);
                     if (zmath::d2u(eg) != zmath::d2u(er)) b3++;
@@ -129,7 +134,7 @@ int main(int argc, char **argv)
                     if (zmath::d2u(chg) != zmath::d2u(chr)) b5++;
                 }
             }
-            bad_tanh64 += b0; bad_expm164 += b1; bad_sig64 += b2; bad_exp64 += b3; bad_sinh64 += b4; bad_cosh64 += b5; bad_sin64 += b6; bad_cos64 += b7;
+            bad_tanh64 += b0; bad_expm164 += b1; bad_sig64 += b2; bad_exp64 += b3; bad_sinh64 += b4; bad_cosh64 += b5; bad_sin64 += b6; bad_cos64 += b7; bad_log64 += b8;
         });
     for (auto &t : th) t.join();
     // powf(x, y)
@@ -171,6 +176,6 @@ int main(int argc, char **argv)
     printf("atanf_fdlibm %llu asinf_fdlibm %llu acosf_fdlibm %llu\n", (unsigned long long)bad_atan.load(),
            (unsigned long long)bad_asin.load(), (unsigned long long)bad_acos.load());
     printf("tanhf_ulp2_beyond_2ulp %llu tanf_glibc %llu\n", (unsigned long long)far_ulp2.load(), (unsigned long long)bad_tan.load());
-    printf("sin_glibc %llu cos_glibc %llu\n", (unsigned long long)bad_sin64.load(), (unsigned long long)bad_cos64.load());
-    return (bad_sin64 + bad_cos64 + bad_tan + bad_sinh_simd + bad_cosh_simd + far_ulp2 + bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64 + bad_exp64 + bad_sinh64 + bad_cosh64 + bad_exp + bad_log + bad_pow + bad_sinh + bad_cosh + bad_sin + bad_cos + bad_atan + bad_asin + bad_acos) ? 1 : 0;
+    printf("sin_glibc %llu cos_glibc %llu log_glibc %llu\n", (unsigned long long)bad_sin64.load(), (unsigned long long)bad_cos64.load(), (unsigned long long)bad_log64.load());
+    return (bad_log64 + bad_sin64 + bad_cos64 + bad_tan + bad_sinh_simd + bad_cosh_simd + far_ulp2 + bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64 + bad_exp64 + bad_sinh64 + bad_cosh64 + bad_exp + bad_log + bad_pow + bad_sinh + bad_cosh + bad_sin + bad_cos + bad_atan + bad_asin + bad_acos) ? 1 : 0;
 }

@@ -52,7 +52,7 @@ def test_zmath_matches_host_libm(tmp_path):
     cos, tan, atan, asin, acos and the sigmoid composite on every 31st f32 bit pattern (138 M points
     each; stride 1, all 2^32, was run during development with the same result); powf on every 31st
     base for 19 fixed exponents and on two pseudo-random (base, exponent) pairs per base; f64 tanh,
-    expm1, exp, sinh, cosh and the sigmoid composite on every 31st high word with three low words
+    expm1, exp, log, sinh, cosh and the sigmoid composite on every 31st high word with three low words
     each plus uniform samples in +-745 and +-4 (about 700 M points); f64 sin and cos on every 248th high
     word with three low words each plus uniform samples in each of their six argument ranges (150 M points each); f64 tanh in both of its forms
     (fdlibm's branches and the single path the kernels use) and the sigmoid also on 400 M uniform
@@ -68,4 +68,35 @@ def test_zmath_matches_host_libm(tmp_path):
                                   "expf_glibc", "0", "logf_glibc", "0", "powf_glibc", "0",
                                   "sinhf_fdlibm", "0", "coshf_fdlibm", "0", "sinhf_simd", "0", "coshf_simd", "0", "sinf_glibc", "0", "cosf_glibc", "0",
                                   "atanf_fdlibm", "0", "asinf_fdlibm", "0", "acosf_fdlibm", "0",
-                                  "tanhf_ulp2_beyond_2ulp", "0", "tanf_glibc", "0", "sin_glibc", "0", "cos_glibc", "0"]
+                                  "tanhf_ulp2_beyond_2ulp", "0", "tanf_glibc", "0", "sin_glibc", "0", "cos_glibc", "0", "log_glibc", "0"]
+
+
+def _macro_numbers(text, name, following, pattern):
+    import re
+    start = text.index("#define " + name)
+    return re.findall(pattern, text[start:text.index(following, start)])
+
+
+def test_generated_tables_are_what_their_generators_give(tmp_path):
+    """the tables of the f64 sine / cosine and the f64 log in zmath.hpp against the programs that make them:
+    sin(k/128), cos(k/128) and the pieces of 2/pi in full; of the log table (two and a half minutes of search
+    for all 128 subintervals) the first two subintervals and the last, where the host libm picks the entry
+    among the candidates of the published construction"""
+    import re
+    import sys
+    src = open(os.path.join(ROOT, "zenu_amd", "csrc", "zmath.hpp")).read()
+    gen_dir = os.path.join(ROOT, "zenu_amd", "csrc", "tablegen")
+    out = subprocess.run([sys.executable, os.path.join(gen_dir, "sincos64_tables.py")], capture_output=True, text=True, check=True).stdout
+    sincos, toverp = out.split("ZM_TOVERP_TAB")
+    hexes = r"0x[0-9a-f]{16}ull"
+    assert re.findall(hexes, sincos) == _macro_numbers(src, "ZM_SINCOS64_TAB", "#define ZM_TOVERP_TAB", hexes)
+    assert re.findall(r"\d+\.0", toverp) == _macro_numbers(src, "ZM_TOVERP_TAB", "static const uint64_t kSinCos64TabHost", r"\d+\.0")
+    exe = str(tmp_path / "log64_table")
+    subprocess.check_call(["g++", "-O2", "-std=gnu++17", "-fext-numeric-literals", "-ffp-contract=off", "-mfma", "-fopenmp",
+                           os.path.join(gen_dir, "log64_table.cpp"), "-lquadmath", "-o", exe])
+    table = _macro_numbers(src, "ZM_LOG64_TAB", "static const uint64_t kLog64TabHost", hexes)
+    assert len(table) == 256
+    for first, last in ((0, 2), (127, 128)):
+        got = subprocess.run([exe, str(first), str(last)], capture_output=True, text=True)
+        assert got.returncode == 0, got.stderr
+        assert re.findall(hexes, got.stdout) == table[2 * first:2 * last]

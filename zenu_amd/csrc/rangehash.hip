@@ -162,6 +162,7 @@ extern "C" int zenu_hip_unary_range_hash_f64(int fn, uint64_t first, uint64_t co
     switch (fn) {
     case ZENU_EXP: return launch_range_hash_f64<ZENU_EXP>(first, blocks, block_log2, step, offset, salt, sums_dev, s);
     case ZENU_TANH: return launch_range_hash_f64<ZENU_TANH>(first, blocks, block_log2, step, offset, salt, sums_dev, s);
+    case ZENU_LOG: return launch_range_hash_f64<ZENU_LOG>(first, blocks, block_log2, step, offset, salt, sums_dev, s);
     case ZENU_SIN: return launch_range_hash_f64<ZENU_SIN>(first, blocks, block_log2, step, offset, salt, sums_dev, s);
     case ZENU_COS: return launch_range_hash_f64<ZENU_COS>(first, blocks, block_log2, step, offset, salt, sums_dev, s);
     case ZENU_SIGMOID: return launch_range_hash_f64<ZENU_SIGMOID>(first, blocks, block_log2, step, offset, salt, sums_dev, s);

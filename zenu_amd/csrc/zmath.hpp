@@ -1797,6 +1797,156 @@ ZM_HD float coshf_simd(float x, const uint64_t *etab, const TanhRegs &rg = TanhR
 ZM_HD float sinhf_fdlibm(float x) { return sinhf_fdlibm(x, exp2f_table()); }
 ZM_HD float coshf_fdlibm(float x) { return coshf_fdlibm(x, exp2f_table()); }
 
+// ---- double precision log: the table-driven routine glibc ships since 2.28 (from ARM's optimized routines) ----
+// x = 2^k z, z in [0.6875, 1.375) in 128 subintervals (80 of 1/256 below 1, 48 of 1/128 above); with c near the
+// centre of z's subinterval, log(x) = k ln2 + log(c) + log1p(z/c - 1): r = z invc - 1 by one fused multiply-add,
+// k ln2_hi + logc exact (logc and ln2_hi are multiples of 2^-43), a degree-5 polynomial in r.  Arguments in
+// [1 - 2^-4, 1 + 0x1.09p-4) take a degree-11 polynomial in x - 1 instead, with r - r^2/2 carried in two parts.
+// The table {invc, logc} is not defined by a formula: its authors tried the 2^30 doubles around 1 / centre as
+// invc and kept one whose log(c), c = 1 / invc, lies within 2^-66 of a multiple of 2^-43 (and which meets
+// further conditions of the build without fused multiply-add).  It is rebuilt here along that construction
+// (tablegen/log64_table.cpp): every invc of that range whose log(c) is that close to the grid -- about 420
+// per subinterval -- is a candidate, and the candidate that gives the host libm's bits on 10^5 random
+// arguments of its subinterval is the entry; for every subinterval exactly one does.  The polynomial
+// coefficients and the split of ln2 are the sources' constants.  Fused multiply-adds as in the x86-64
+// build that CPUs with FMA select (every a + b c, including y = r^3 p + lo in the branch near 1).
+// Equal to the host libm's log on 8e8 sampled arguments (uniform bit patterns, [0.5, 1.5), [0, 100), and
+// log-uniform over +-700), zero, negative, infinite and subnormal arguments included.
+#define ZM_LOG64_TAB                                                                                        \
+    {                                                                                                       \
+      0x3ff734f0c3e0de9full, 0xbfd7cc7f79e69000ull, 0x3ff713786a2ce91full, 0xbfd76feec20d0000ull,           \
+      0x3ff6f26008fab5a0ull, 0xbfd713e31351e000ull, 0x3ff6d1a61f138c7dull, 0xbfd6b85b38287800ull,           \
+      0x3ff6b1490bc5b4d1ull, 0xbfd65d5590807800ull, 0x3ff69147332f0cbaull, 0xbfd602d076180000ull,           \
+      0x3ff6719f18224223ull, 0xbfd5a8ca86909000ull, 0x3ff6524f99a51ed9ull, 0xbfd54f4356035000ull,           \
+      0x3ff63356aa8f24c4ull, 0xbfd4f637c36b4000ull, 0x3ff614b36b9ddc14ull, 0xbfd49da7fda85000ull,           \
+      0x3ff5f66452c65c4cull, 0xbfd445923989a800ull, 0x3ff5d867b5912c4full, 0xbfd3edf439b0b800ull,           \
+      0x3ff5babccb5b90deull, 0xbfd396ce448f7000ull, 0x3ff59d61f2d91a78ull, 0xbfd3401e17bda000ull,           \
+      0x3ff5805612465687ull, 0xbfd2e9e2ef468000ull, 0x3ff56397cee76bd3ull, 0xbfd2941b3830e000ull,           \
+      0x3ff54725e2a77f93ull, 0xbfd23ec58cda8800ull, 0x3ff52aff42064583ull, 0xbfd1e9e129279000ull,           \
+      0x3ff50f22dbb2bddfull, 0xbfd1956d2b48f800ull, 0x3ff4f38f4734ded7ull, 0xbfd141679ab9f800ull,           \
+      0x3ff4d843cfde2840ull, 0xbfd0edd094ef9800ull, 0x3ff4bd3ec078a3c8ull, 0xbfd09aa518db1000ull,           \
+      0x3ff4a27fc3e0258aull, 0xbfd047e65263b800ull, 0x3ff4880524d48434ull, 0xbfcfeb224586f000ull,           \
+      0x3ff46dce1b192d0bull, 0xbfcf474a7517b000ull, 0x3ff453d9d3391854ull, 0xbfcea4443d103000ull,           \
+      0x3ff43a2744b4845aull, 0xbfce020d44e9b000ull, 0x3ff420b54115f8fbull, 0xbfcd60a22977f000ull,           \
+      0x3ff40782da3ef4b1ull, 0xbfccc00104959000ull, 0x3ff3ee8f5d57fe8full, 0xbfcc202956891000ull,           \
+      0x3ff3d5d9a00b4ce9ull, 0xbfcb81178d811000ull, 0x3ff3bd60c010c12bull, 0xbfcae2c9ccd3d000ull,           \
+      0x3ff3a5242b75dab8ull, 0xbfca45402e129000ull, 0x3ff38d22cd9fd002ull, 0xbfc9a877681df000ull,           \
+      0x3ff3755bc5847a1cull, 0xbfc90c6d69483000ull, 0x3ff35dce49ad36e2ull, 0xbfc87120a645c000ull,           \
+      0x3ff34679984dd440ull, 0xbfc7d68fb4143000ull, 0x3ff32f5cceffcb24ull, 0xbfc73cb83c627000ull,           \
+      0x3ff3187775a10d49ull, 0xbfc6a39a9b376000ull, 0x3ff301c8373e3990ull, 0xbfc60b3154b7a000ull,           \
+      0x3ff2eb4ebb95f841ull, 0xbfc5737d76243000ull, 0x3ff2d50a0219a9d1ull, 0xbfc4dc7b8fc23000ull,           \
+      0x3ff2bef9a8b7fd2aull, 0xbfc4462c51d20000ull, 0x3ff2a91c7a0c1babull, 0xbfc3b08abc830000ull,           \
+      0x3ff293726014b530ull, 0xbfc31b996b490000ull, 0x3ff27dfa5757a1f5ull, 0xbfc2875490a44000ull,           \
+      0x3ff268b39b1d3bbfull, 0xbfc1f3b9f879a000ull, 0x3ff2539d838ff5bdull, 0xbfc160c8252ca000ull,           \
+      0x3ff23eb7aac9083bull, 0xbfc0ce7f57f72000ull, 0x3ff22a012ba940b6ull, 0xbfc03cdc49fea000ull,           \
+      0x3ff2157996cc4132ull, 0xbfbf57bdbc4b8000ull, 0x3ff201201dd2fc9bull, 0xbfbe370896404000ull,           \
+      0x3ff1ecf4494d480bull, 0xbfbd17983ef94000ull, 0x3ff1d8f5528f6569ull, 0xbfbbf9674ed8a000ull,           \
+      0x3ff1c52311577e7cull, 0xbfbadc79202f6000ull, 0x3ff1b17c74cb26e9ull, 0xbfb9c0c3e7288000ull,           \
+      0x3ff19e010c2c1ab6ull, 0xbfb8a646b372c000ull, 0x3ff18ab07bb670bdull, 0xbfb78d01b3ac0000ull,           \
+      0x3ff1778a25efbcb6ull, 0xbfb674f145380000ull, 0x3ff1648d354c31daull, 0xbfb55e0e6d878000ull,           \
+      0x3ff151b990275fddull, 0xbfb4485cdea1e000ull, 0x3ff13f0ea432d24cull, 0xbfb333d94d6aa000ull,           \
+      0x3ff12c8b7210f9daull, 0xbfb22079f8c56000ull, 0x3ff11a3028ecb531ull, 0xbfb10e4698622000ull,           \
+      0x3ff107fbda8434afull, 0xbfaffa6c6ad20000ull, 0x3ff0f5ee0f4e6bb3ull, 0xbfadda8d4a774000ull,           \
+      0x3ff0e4065d2a9fceull, 0xbfabbcece4850000ull, 0x3ff0d244632ca521ull, 0xbfa9a1894012c000ull,           \
+      0x3ff0c0a77ce2981aull, 0xbfa788583302c000ull, 0x3ff0af2f83c636d1ull, 0xbfa5715e67d68000ull,           \
+      0x3ff09ddb98a01339ull, 0xbfa35c8a49658000ull, 0x3ff08cabaf52e7dfull, 0xbfa149e364154000ull,           \
+      0x3ff07b9f2f4e28fbull, 0xbf9e72c082eb8000ull, 0x3ff06ab58c358f19ull, 0xbf9a55f152528000ull,           \
+      0x3ff059eea5ecf92cull, 0xbf963d62cf818000ull, 0x3ff04949cdd12c90ull, 0xbf9228fb8caa0000ull,           \
+      0x3ff038c6c6f0ada9ull, 0xbf8c317b20f90000ull, 0x3ff02865137932a9ull, 0xbf8419355daa0000ull,           \
+      0x3ff0182427ea7348ull, 0xbf781203c2ec0000ull, 0x3ff008040614b195ull, 0xbf60040979240000ull,           \
+      0x3fefe01ff726fa1aull, 0x3f6feff384900000ull, 0x3fefa11cc261ea74ull, 0x3f87dc41353d0000ull,           \
+      0x3fef6310b081992eull, 0x3f93cea3c4c28000ull, 0x3fef25f63ceeadcdull, 0x3f9b9fc114890000ull,           \
+      0x3feee9c8039113e7ull, 0x3fa1b0d8ce110000ull, 0x3feeae8078cbb1abull, 0x3fa58a5bd001c000ull,           \
+      0x3fee741aa29d0c9bull, 0x3fa95c8340d88000ull, 0x3fee3a91830a99b5ull, 0x3fad276aef578000ull,           \
+      0x3fee01e009609a56ull, 0x3fb07598e598c000ull, 0x3fedca01e577bb98ull, 0x3fb253f5e30d2000ull,           \
+      0x3fed92f20b7c9103ull, 0x3fb42edd8b380000ull, 0x3fed5cac66fb5cceull, 0x3fb606598757c000ull,           \
+      0x3fed272caa5ede9dull, 0x3fb7da76356a0000ull, 0x3fecf26e3e6b2ccdull, 0x3fb9ab434e1c6000ull,           \
+      0x3fecbe6da2a77902ull, 0x3fbb78c7bb0d6000ull, 0x3fec8b266d37086dull, 0x3fbd431332e72000ull,           \
+      0x3fec5894bd5d5804ull, 0x3fbf0a3171de6000ull, 0x3fec26b533bb9f8cull, 0x3fc067152b914000ull,           \
+      0x3febf583eeece73full, 0x3fc147858292b000ull, 0x3febc4fd75db96c1ull, 0x3fc2266ecdca3000ull,           \
+      0x3feb951e0c864a28ull, 0x3fc303d7a6c55000ull, 0x3feb65e2c5ef3e2cull, 0x3fc3dfc33c331000ull,           \
+      0x3feb374867c9888bull, 0x3fc4ba366b7a8000ull, 0x3feb094b211d304aull, 0x3fc5933928d1f000ull,           \
+      0x3feadbe885f2ef7eull, 0x3fc66acd2418f000ull, 0x3feaaf1d31603da2ull, 0x3fc740f8ec669000ull,           \
+      0x3fea82e63fd358a7ull, 0x3fc815c0f51af000ull, 0x3fea5740ef09738bull, 0x3fc8e92954f68000ull,           \
+      0x3fea2c2a90ab4b27ull, 0x3fc9bb3602f84000ull, 0x3fea01a01393f2d1ull, 0x3fca8bed1c2c0000ull,           \
+      0x3fe9d79f24db3c1bull, 0x3fcb5b515c01d000ull, 0x3fe9ae2505c7b190ull, 0x3fcc2967ccbcc000ull,           \
+      0x3fe9852ef297ce2full, 0x3fccf635d5486000ull, 0x3fe95cbaeea44b75ull, 0x3fcdc1bd3446c000ull,           \
+      0x3fe934c69de74838ull, 0x3fce8c01b8cfe000ull, 0x3fe90d4f2f6752e6ull, 0x3fcf5509c0179000ull,           \
+      0x3fe8e6528effd79dull, 0x3fd00e6c121fb800ull, 0x3fe8bfce9fcc007cull, 0x3fd071b80e93d000ull,           \
+      0x3fe899c0dabec30eull, 0x3fd0d46b9e867000ull, 0x3fe87427aa2317fbull, 0x3fd13687334bd000ull,           \
+      0x3fe84f00acb39a08ull, 0x3fd1980d67234800ull, 0x3fe82a49e8653e55ull, 0x3fd1f8ffe0cc8000ull,           \
+      0x3fe8060195f40260ull, 0x3fd2595fd7636800ull, 0x3fe7e22563e0a329ull, 0x3fd2b9300914a800ull,           \
+      0x3fe7beb377dcb5adull, 0x3fd3187210436000ull, 0x3fe79baa679725c2ull, 0x3fd377266dec1800ull,           \
+      0x3fe77907f2170657ull, 0x3fd3d54ffbaf3000ull, 0x3fe756cadbd6130cull, 0x3fd432eee32fe000ull            \
+    }
+static const uint64_t kLog64TabHost[256] = ZM_LOG64_TAB;
+#if defined(__HIPCC__)
+static __device__ const uint64_t kLog64TabDev[256] = ZM_LOG64_TAB;
+#endif
+ZM_HD const double *log64_table()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return reinterpret_cast<const double *>(kLog64TabDev);
+#else
+    return reinterpret_cast<const double *>(kLog64TabHost);
+#endif
+}
+
+// the constants as data (a kernel argument: scalar registers feed the f64 operations directly)
+struct LogCoef64 {
+    double a0 = -0x1.0000000000001p-1, a1 = 0x1.555555551305bp-2, a2 = -0x1.fffffffeb459p-3, a3 = 0x1.999b324f10111p-3,
+           a4 = -0x1.55575e506c89fp-3;
+    double b1 = 0x1.5555555555577p-2, b2 = -0x1.ffffffffffdcbp-3, b3 = 0x1.999999995dd0cp-3, b4 = -0x1.55555556745a7p-3,
+           b5 = 0x1.24924a344de3p-3, b6 = -0x1.fffffa4423d65p-4, b7 = 0x1.c7184282ad6cap-4, b8 = -0x1.999eb43b068ffp-4,
+           b9 = 0x1.78182f7afd085p-4, b10 = -0x1.5521375d145cdp-4;
+    double ln2hi = 0x1.62e42fefa3800p-1, ln2lo = 0x1.ef35793c76730p-45;
+};
+
+ZM_HD double log_glibc(double x, const double *tab, const LogCoef64 &k = LogCoef64())
+{
+    uint64_t ix = d2u(x);
+    const uint64_t lo1 = 0x3fee000000000000ull, hi1 = 0x3ff1090000000000ull;   // 1 - 2^-4, 1 + 0x1.09p-4
+    if (ix - lo1 < hi1 - lo1) {
+        if (ix == 0x3ff0000000000000ull) return 0.0;
+        const double r = x - 1.0, r2 = r * r, r3 = r * r2;
+        const double p3 = __builtin_fma(r3, k.b10, __builtin_fma(r2, k.b9, __builtin_fma(r, k.b8, k.b7)));
+        const double p2 = __builtin_fma(r3, p3, __builtin_fma(r2, k.b6, __builtin_fma(r, k.b5, k.b4)));
+        const double p1 = __builtin_fma(r3, p2, __builtin_fma(r2, k.b3, __builtin_fma(r, k.b2, k.b1)));
+        // r - r^2 / 2 as hi + lo: r split at 2^-27 relative, so that the square of the high part is exact
+        double w = r * 0x1p27;
+        const double rhi = r + w - w, rlo = r - rhi;
+        w = rhi * rhi * -0.5;
+        const double hi = r + w;
+        double lo = r - hi + w;
+        lo = __builtin_fma(-0.5 * rlo, rhi + r, lo);
+        return __builtin_fma(r3, p1, lo) + hi;
+    }
+    const uint32_t top = (uint32_t)(ix >> 48);
+    if (__builtin_expect(top - 0x0010u >= 0x7ff0u - 0x0010u, 0)) {
+        if (ix * 2 == 0) return -u2d(0x7ff0000000000000ull);                  // log(+-0) = -inf
+        if (ix == 0x7ff0000000000000ull) return x;                             // log(inf) = inf
+        if ((top & 0x8000u) || (top & 0x7ff0u) == 0x7ff0u) return (x - x) * u2d(0x7ff0000000000000ull);   // negative, NaN
+        ix = d2u(x * 0x1p52);                                                  // subnormal: normalise
+        ix -= 52ull << 52;
+    }
+    const uint64_t tmp = ix - 0x3fe6000000000000ull;
+    const int i = (int)((tmp >> 45) & 127u);
+    const int64_t ke = (int64_t)tmp >> 52;
+    const double z = u2d(ix - (tmp & (0xfffull << 52)));
+    const double invc = tab[2 * i], logc = tab[2 * i + 1];
+    const double r = __builtin_fma(z, invc, -1.0);
+    const double kd = (double)ke;
+    const double w = __builtin_fma(kd, k.ln2hi, logc);
+    const double hi = w + r;
+    const double lo = __builtin_fma(kd, k.ln2lo, (w - hi) + r);
+    const double r2 = r * r;
+    const double p = __builtin_fma(r2, __builtin_fma(r, k.a4, k.a3), __builtin_fma(r, k.a2, k.a1));
+    double y = __builtin_fma(r2, k.a0, lo);
+    y = __builtin_fma(r * r2, p, y);
+    return y + hi;
+}
+ZM_HD double log_glibc(double x) { return log_glibc(x, log64_table()); }
+
 // ---- double precision sin / cos: s_sin.c and branred.c as glibc 2.35 ships them (the IBM Accurate
 // Mathematical Library without its multi-precision fall-backs) ------------------------------------------
 // |x| < 2^-26: x resp. 1.  The argument is brought to a in [-pi/4, pi/4] plus a small da and a quadrant n:
@@ -1808,7 +1958,8 @@ ZM_HD float coshf_fdlibm(float x) { return coshf_fdlibm(x, exp2f_table()); }
 // sine (even n) on |a| < 0.126 is a degree-11 Taylor form; otherwise sine and cosine (odd n) come from
 // sin(xi), cos(xi) at xi = k/128 (the nearest multiple, read off a + 1.5 2^45), each as a double and the
 // double of the remainder, and short polynomials in a - xi, combined by the angle-sum formulas with the
-// small terms first.  The table is regenerated here from that definition (exact rational arithmetic).
+// small terms first.  The table is regenerated here from that definition (exact rational arithmetic:
+// tablegen/sincos64_tables.py).
 // Fused multiply-adds where the compiler fuses them in the x86-64 build that CPUs with FMA select
 // (s_sin.c has one; branred.c has none, and its products are exact anyway).  Equal to the host libm's
 // sin and cos on 6.4e8 sampled arguments each: uniform in +-0.855, +-2.43, +-10, +-1000, +-1e6, +-1.05e8,
@@ -2152,19 +2303,26 @@ template <> struct ExpLog<double> {
     const uint64_t *etab;
     ExpCoef64 ek;
     Expm1Coef64 mk;
-    __device__ __forceinline__ void init(bool need_exp, bool)
+    const double *ltab;
+    LogCoef64 lk;
+    __device__ __forceinline__ void init(bool need_exp, bool need_log)
     {
         __shared__ uint64_t lds_exp64[256];
-        if (need_exp && threadIdx.x < 64) {
+        __shared__ uint64_t lds_log64[256];
+        if (threadIdx.x < 64) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) lds_exp64[threadIdx.x + 64 * i] = kExpTabDev[threadIdx.x + 64 * i];
+            for (int i = 0; i < 4; i++) {
+                if (need_exp) lds_exp64[threadIdx.x + 64 * i] = kExpTabDev[threadIdx.x + 64 * i];
+                if (need_log) lds_log64[threadIdx.x + 64 * i] = kLog64TabDev[threadIdx.x + 64 * i];
+            }
         }
         __syncthreads();
         etab = lds_exp64;
+        ltab = reinterpret_cast<const double *>(lds_log64);
     }
     __device__ __forceinline__ double exp(double x) const { return exp_glibc(x, etab, ek); }
     __device__ __forceinline__ double exp_flat(double x) const { return exp_glibc(x, etab, ek); }
-    __device__ __forceinline__ double log(double x) const { return ::log(x); }
+    __device__ __forceinline__ double log(double x) const { return log_glibc(x, ltab, lk); }
     __device__ __forceinline__ double sinh(double x) const { return sinh_simd(x, etab, mk); }
     __device__ __forceinline__ double cosh(double x) const { return cosh_simd(x, etab, mk, ek); }
     __device__ __forceinline__ double sinh(double x, const TanhRegs &) const { return sinh_simd(x, etab, mk); }
