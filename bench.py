@@ -376,6 +376,10 @@ def build_ops(z, workload, stream):
                   for A, O in src_sets]
             cpu = (lambda: zo.sigmoid(out64_h, a64)) if fn == _lib.SIGMOID else (lambda fn=fn, h=src_h: zo.unary(fn, out64_h, h))
             ops.append(Op(name, "next", "f64", 4 * nb, n * n, ls, cpu))
+        ops.append(Op("powf(x, 2.5) f64", "next", "f64", 4 * nb, n * n,
+                      [(lambda d=O.desc(), s_=A.desc(): check(l.zenu_hip_powf(_lib.F64, ref(d), ref(s_), 2.5, stream), "powf f64"))
+                       for A, O in sets64p],
+                      lambda: zo.powf(out64_h, pos64, 2.5)))
         ops[-1].keep = (sets, sets64, sets64p)
 
     # ---- the same kernels on larger tensors: how much of the distance to the roofline is the fixed

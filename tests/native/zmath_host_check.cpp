@@ -137,6 +137,33 @@ int main(int argc, char **argv)
             bad_tanh64 += b0; bad_expm164 += b1; bad_sig64 += b2; bad_exp64 += b3; bad_sinh64 += b4; bad_cosh64 += b5; bad_sin64 += b6; bad_cos64 += b7; bad_log64 += b8;
         });
     for (auto &t : th) t.join();
+    // pow(x, y) in double: both forms (the complete routine and the one the kernels inline) on uniform bit patterns
+    // for both arguments, on moderate pairs, and on negative / log-uniform bases under fixed exponents
+    std::atomic<uint64_t> bad_pow64{0};
+    th.clear();
+    for (int w = 0; w < nt; w++)
+        th.emplace_back([&, w]() {
+            uint64_t b = 0, rng = 0xA0761D6478BD642Full * (w + 1);
+            auto next = [&]() { rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17; return rng; };
+            auto one = [&](double x, double y) {
+                const double ref = pow(x, y), got = zmath::pow_glibc_full(x, y), got2 = zmath::pow_glibc(x, y);
+                if ((ref != ref) ? !(got != got) : zmath::d2u(got) != zmath::d2u(ref)) b++;
+                if ((ref != ref) ? !(got2 != got2) : zmath::d2u(got2) != zmath::d2u(ref)) b++;
+            };
+            const double ys[] = {2.0, 0.5, 2.5, -1.0, 3.0, -0.5, 1.0 / 3.0, 0.0, 1.0, -2.0, 10.25, 1e-3, 55.0, -3.0, 1e-20, 1e300,
+                                 INFINITY, -INFINITY, NAN, 0x1p-66, 0x1p63, 4503599627370497.0};
+            for (uint64_t u = (uint64_t)w * stride * 16; u < (1ull << 32); u += stride * nt * 16) {
+                one(zmath::u2d(next()), zmath::u2d(next()));
+                const double m1 = (double)(next() >> 11) * 0x1p-53, m2 = (double)(int64_t)next() / 9.2233720368547758e18;
+                one(m1 * 4.0, m2 * 40.0);
+                one(0.5 + m1, m2 * 1000.0);
+                one(exp(m2 * 300.0), ys[next() % 22]);
+                one(m2 * 10.0, ys[next() % 22]);
+                one(zmath::u2d(next()), ys[next() % 22]);
+            }
+            bad_pow64 += b;
+        });
+    for (auto &t : th) t.join();
     // powf(x, y)
     std::atomic<uint64_t> bad_pow{0};
     th.clear();
@@ -177,5 +204,6 @@ int main(int argc, char **argv)
            (unsigned long long)bad_asin.load(), (unsigned long long)bad_acos.load());
     printf("tanhf_ulp2_beyond_2ulp %llu tanf_glibc %llu\n", (unsigned long long)far_ulp2.load(), (unsigned long long)bad_tan.load());
     printf("sin_glibc %llu cos_glibc %llu log_glibc %llu\n", (unsigned long long)bad_sin64.load(), (unsigned long long)bad_cos64.load(), (unsigned long long)bad_log64.load());
-    return (bad_log64 + bad_sin64 + bad_cos64 + bad_tan + bad_sinh_simd + bad_cosh_simd + far_ulp2 + bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64 + bad_exp64 + bad_sinh64 + bad_cosh64 + bad_exp + bad_log + bad_pow + bad_sinh + bad_cosh + bad_sin + bad_cos + bad_atan + bad_asin + bad_acos) ? 1 : 0;
+    printf("pow_glibc %llu\n", (unsigned long long)bad_pow64.load());
+    return (bad_pow64 + bad_log64 + bad_sin64 + bad_cos64 + bad_tan + bad_sinh_simd + bad_cosh_simd + far_ulp2 + bad_fdlibm + bad_simd + bad_expm1 + bad_sig + bad_tanh64 + bad_expm164 + bad_sig64 + bad_exp64 + bad_sinh64 + bad_cosh64 + bad_exp + bad_log + bad_pow + bad_sinh + bad_cosh + bad_sin + bad_cos + bad_atan + bad_asin + bad_acos) ? 1 : 0;
 }

@@ -53,7 +53,9 @@ def test_zmath_matches_host_libm(tmp_path):
     each; stride 1, all 2^32, was run during development with the same result); powf on every 31st
     base for 19 fixed exponents and on two pseudo-random (base, exponent) pairs per base; f64 tanh,
     expm1, exp, log, sinh, cosh and the sigmoid composite on every 31st high word with three low words
-    each plus uniform samples in +-745 and +-4 (about 700 M points); f64 sin and cos on every 248th high
+    each plus uniform samples in +-745 and +-4 (about 700 M points); f64 pow in both of its forms on 5 * 10^7 pairs
+    (uniform bit patterns for both arguments, moderate pairs, negative and log-uniform bases under 22 fixed
+    exponents); f64 sin and cos on every 248th high
     word with three low words each plus uniform samples in each of their six argument ranges (150 M points each); f64 tanh in both of its forms
     (fdlibm's branches and the single path the kernels use) and the sigmoid also on 400 M uniform
     samples in +-1, +-4 and +-20.  tanhf_ulp2, the variant that
@@ -68,7 +70,7 @@ def test_zmath_matches_host_libm(tmp_path):
                                   "expf_glibc", "0", "logf_glibc", "0", "powf_glibc", "0",
                                   "sinhf_fdlibm", "0", "coshf_fdlibm", "0", "sinhf_simd", "0", "coshf_simd", "0", "sinf_glibc", "0", "cosf_glibc", "0",
                                   "atanf_fdlibm", "0", "asinf_fdlibm", "0", "acosf_fdlibm", "0",
-                                  "tanhf_ulp2_beyond_2ulp", "0", "tanf_glibc", "0", "sin_glibc", "0", "cos_glibc", "0", "log_glibc", "0"]
+                                  "tanhf_ulp2_beyond_2ulp", "0", "tanf_glibc", "0", "sin_glibc", "0", "cos_glibc", "0", "log_glibc", "0", "pow_glibc", "0"]
 
 
 def _macro_numbers(text, name, following, pattern):
@@ -81,7 +83,7 @@ def test_generated_tables_are_what_their_generators_give(tmp_path):
     """the tables of the f64 sine / cosine and the f64 log in zmath.hpp against the programs that make them:
     sin(k/128), cos(k/128) and the pieces of 2/pi in full; of the log table (two and a half minutes of search
     for all 128 subintervals) the first two subintervals and the last, where the host libm picks the entry
-    among the candidates of the published construction"""
+    among the candidates of the published construction; the log table of the f64 pow in full"""
     import re
     import sys
     src = open(os.path.join(ROOT, "zenu_amd", "csrc", "zmath.hpp")).read()
@@ -91,6 +93,8 @@ def test_generated_tables_are_what_their_generators_give(tmp_path):
     hexes = r"0x[0-9a-f]{16}ull"
     assert re.findall(hexes, sincos) == _macro_numbers(src, "ZM_SINCOS64_TAB", "#define ZM_TOVERP_TAB", hexes)
     assert re.findall(r"\d+\.0", toverp) == _macro_numbers(src, "ZM_TOVERP_TAB", "static const uint64_t kSinCos64TabHost", r"\d+\.0")
+    out = subprocess.run([sys.executable, os.path.join(gen_dir, "pow64_table.py")], capture_output=True, text=True, check=True).stdout
+    assert re.findall(hexes, out) == _macro_numbers(src, "ZM_POW64_LOG_TAB", "static const uint64_t kPow64LogTabHost", hexes)
     exe = str(tmp_path / "log64_table")
     subprocess.check_call(["g++", "-O2", "-std=gnu++17", "-fext-numeric-literals", "-ffp-contract=off", "-mfma", "-fopenmp",
                            os.path.join(gen_dir, "log64_table.cpp"), "-lquadmath", "-o", exe])

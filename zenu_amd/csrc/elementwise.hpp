@@ -280,6 +280,8 @@ template <typename T> struct IsValuBound<UnaryF<T, ZENU_COSH>> { static constexp
 template <> struct IsValuBound<UnaryF<float, ZENU_SIN>> { static constexpr bool value = true; };
 template <> struct IsValuBound<UnaryF<float, ZENU_COS>> { static constexpr bool value = true; };
 template <> struct IsValuBound<UnaryF<float, ZENU_ASIN>> { static constexpr bool value = true; };
+// f64 powf: 5 KiB of tables per workgroup (89 us at 64 x 1)
+template <> struct IsValuBound<PowF<double>> { static constexpr bool value = true; };
 template <typename T> struct IsValuBound<TanhBwdF<T>> { static constexpr bool value = true; };
 template <typename T> struct IsValuBound<SigmoidBwdF<T>> { static constexpr bool value = true; };
 

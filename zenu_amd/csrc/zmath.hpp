@@ -1947,6 +1947,340 @@ ZM_HD double log_glibc(double x, const double *tab, const LogCoef64 &k = LogCoef
 }
 ZM_HD double log_glibc(double x) { return log_glibc(x, log64_table()); }
 
+// ---- double precision pow: the routine glibc ships since 2.28 (from ARM's optimized routines) -----------
+// log(x) as hi + lo to about 68 bits -- x = 2^k z, z in [0x1.69555p-1, 0x1.69555p0) in 128 subintervals, 1 / c a
+// multiple of 1/128 resp. 1/256 so that r = z / c - 1 is exact, k ln2 + log(c) + r - r^2 / 2 carried in two
+// doubles, a degree-7 polynomial for the rest -- then y log(x) as ehi + elo and exp of that through exp's
+// table with the tail added to the reduced argument and the sign of a negative base (odd integer y) carried
+// in the scale.  The log table IS defined by a formula (tablegen/pow64_table.py rebuilds it with exact
+// rational arithmetic: invc = the nearest multiple, logc = log(c) rounded to a multiple of 2^-43, logctail =
+// the nearest double of the rest); the polynomial and the split of ln2 are the sources' constants.  Fused
+// multiply-adds as in the x86-64 build that CPUs with FMA select: every a + b c, including the polynomial's
+// last product into the sum of the low parts.  Equal to the host libm's pow on 1.6e8 sampled pairs: uniform bit
+// patterns for both arguments, bases in [0, 4) with exponents in +-40, bases in [0.5, 1.5) with exponents in
+// +-1000, log-uniform and negative bases under sixteen fixed exponents.
+#define ZM_POW64_LOG_TAB                                                                                    \
+    {                                                                                                       \
+      0x3ff6a00000000000ull, 0xbfd62c82f2b9c800ull, 0x3cfab42428375680ull,                                  \
+      0x3ff6800000000000ull, 0xbfd5d1bdbf580800ull, 0xbd1ca508d8e0f720ull,                                  \
+      0x3ff6600000000000ull, 0xbfd5767717455800ull, 0xbd2362a4d5b6506dull,                                  \
+      0x3ff6400000000000ull, 0xbfd51aad872df800ull, 0xbce684e49eb067d5ull,                                  \
+      0x3ff6200000000000ull, 0xbfd4be5f95777800ull, 0xbd041b6993293ee0ull,                                  \
+      0x3ff6000000000000ull, 0xbfd4618bc21c6000ull, 0x3d13d82f484c84ccull,                                  \
+      0x3ff5e00000000000ull, 0xbfd404308686a800ull, 0x3cdc42f3ed820b3aull,                                  \
+      0x3ff5c00000000000ull, 0xbfd3a64c55694800ull, 0x3d20b1c686519460ull,                                  \
+      0x3ff5a00000000000ull, 0xbfd347dd9a988000ull, 0x3d25594dd4c58092ull,                                  \
+      0x3ff5800000000000ull, 0xbfd2e8e2bae12000ull, 0x3d267b1e99b72bd8ull,                                  \
+      0x3ff5600000000000ull, 0xbfd2895a13de8800ull, 0x3d15ca14b6cfb03full,                                  \
+      0x3ff5600000000000ull, 0xbfd2895a13de8800ull, 0x3d15ca14b6cfb03full,                                  \
+      0x3ff5400000000000ull, 0xbfd22941fbcf7800ull, 0xbd165a242853da76ull,                                  \
+      0x3ff5200000000000ull, 0xbfd1c898c1699800ull, 0xbd1fafbc68e75404ull,                                  \
+      0x3ff5000000000000ull, 0xbfd1675cababa800ull, 0x3d1f1fc63382a8f0ull,                                  \
+      0x3ff4e00000000000ull, 0xbfd1058bf9ae4800ull, 0xbd26a8c4fd055a66ull,                                  \
+      0x3ff4c00000000000ull, 0xbfd0a324e2739000ull, 0xbd0c6bee7ef4030eull,                                  \
+      0x3ff4a00000000000ull, 0xbfd0402594b4d000ull, 0xbcf036b89ef42d7full,                                  \
+      0x3ff4a00000000000ull, 0xbfd0402594b4d000ull, 0xbcf036b89ef42d7full,                                  \
+      0x3ff4800000000000ull, 0xbfcfb9186d5e4000ull, 0x3d0d572aab993c87ull,                                  \
+      0x3ff4600000000000ull, 0xbfcef0adcbdc6000ull, 0x3d2b26b79c86af24ull,                                  \
+      0x3ff4400000000000ull, 0xbfce27076e2af000ull, 0xbd172f4f543fff10ull,                                  \
+      0x3ff4200000000000ull, 0xbfcd5c216b4fc000ull, 0x3d21ba91bbca681bull,                                  \
+      0x3ff4000000000000ull, 0xbfcc8ff7c79aa000ull, 0x3d27794f689f8434ull,                                  \
+      0x3ff4000000000000ull, 0xbfcc8ff7c79aa000ull, 0x3d27794f689f8434ull,                                  \
+      0x3ff3e00000000000ull, 0xbfcbc286742d9000ull, 0x3d194eb0318bb78full,                                  \
+      0x3ff3c00000000000ull, 0xbfcaf3c94e80c000ull, 0x3cba4e633fcd9066ull,                                  \
+      0x3ff3a00000000000ull, 0xbfca23bc1fe2b000ull, 0xbd258c64dc46c1eaull,                                  \
+      0x3ff3a00000000000ull, 0xbfca23bc1fe2b000ull, 0xbd258c64dc46c1eaull,                                  \
+      0x3ff3800000000000ull, 0xbfc9525a9cf45000ull, 0xbd2ad1d904c1d4e3ull,                                  \
+      0x3ff3600000000000ull, 0xbfc87fa06520d000ull, 0x3d2bbdbf7fdbfa09ull,                                  \
+      0x3ff3400000000000ull, 0xbfc7ab890210e000ull, 0x3d2bdb9072534a58ull,                                  \
+      0x3ff3400000000000ull, 0xbfc7ab890210e000ull, 0x3d2bdb9072534a58ull,                                  \
+      0x3ff3200000000000ull, 0xbfc6d60fe719d000ull, 0xbd10e46aa3b2e266ull,                                  \
+      0x3ff3000000000000ull, 0xbfc5ff3070a79000ull, 0xbd1e9e439f105039ull,                                  \
+      0x3ff3000000000000ull, 0xbfc5ff3070a79000ull, 0xbd1e9e439f105039ull,                                  \
+      0x3ff2e00000000000ull, 0xbfc526e5e3a1b000ull, 0xbd20de8b90075b8full,                                  \
+      0x3ff2c00000000000ull, 0xbfc44d2b6ccb8000ull, 0x3d170cc16135783cull,                                  \
+      0x3ff2c00000000000ull, 0xbfc44d2b6ccb8000ull, 0x3d170cc16135783cull,                                  \
+      0x3ff2a00000000000ull, 0xbfc371fc201e9000ull, 0x3cf178864d27543aull,                                  \
+      0x3ff2800000000000ull, 0xbfc29552f81ff000ull, 0xbd248d301771c408ull,                                  \
+      0x3ff2600000000000ull, 0xbfc1b72ad52f6000ull, 0xbd2e80a41811a396ull,                                  \
+      0x3ff2600000000000ull, 0xbfc1b72ad52f6000ull, 0xbd2e80a41811a396ull,                                  \
+      0x3ff2400000000000ull, 0xbfc0d77e7cd09000ull, 0x3d0a699688e85bf4ull,                                  \
+      0x3ff2400000000000ull, 0xbfc0d77e7cd09000ull, 0x3d0a699688e85bf4ull,                                  \
+      0x3ff2200000000000ull, 0xbfbfec9131dbe000ull, 0xbd2575545ca333f2ull,                                  \
+      0x3ff2000000000000ull, 0xbfbe27076e2b0000ull, 0x3d2a342c2af0003cull,                                  \
+      0x3ff2000000000000ull, 0xbfbe27076e2b0000ull, 0x3d2a342c2af0003cull,                                  \
+      0x3ff1e00000000000ull, 0xbfbc5e548f5bc000ull, 0xbd1d0c57585fbe06ull,                                  \
+      0x3ff1c00000000000ull, 0xbfba926d3a4ae000ull, 0x3d253935e85baac8ull,                                  \
+      0x3ff1c00000000000ull, 0xbfba926d3a4ae000ull, 0x3d253935e85baac8ull,                                  \
+      0x3ff1a00000000000ull, 0xbfb8c345d631a000ull, 0x3d137c294d2f5668ull,                                  \
+      0x3ff1a00000000000ull, 0xbfb8c345d631a000ull, 0x3d137c294d2f5668ull,                                  \
+      0x3ff1800000000000ull, 0xbfb6f0d28ae56000ull, 0xbd269737c93373daull,                                  \
+      0x3ff1600000000000ull, 0xbfb51b073f062000ull, 0x3d1f025b61c65e57ull,                                  \
+      0x3ff1600000000000ull, 0xbfb51b073f062000ull, 0x3d1f025b61c65e57ull,                                  \
+      0x3ff1400000000000ull, 0xbfb341d7961be000ull, 0x3d2c5edaccf913dfull,                                  \
+      0x3ff1400000000000ull, 0xbfb341d7961be000ull, 0x3d2c5edaccf913dfull,                                  \
+      0x3ff1200000000000ull, 0xbfb16536eea38000ull, 0x3d147c5e768fa309ull,                                  \
+      0x3ff1000000000000ull, 0xbfaf0a30c0118000ull, 0x3d2d599e83368e91ull,                                  \
+      0x3ff1000000000000ull, 0xbfaf0a30c0118000ull, 0x3d2d599e83368e91ull,                                  \
+      0x3ff0e00000000000ull, 0xbfab42dd71198000ull, 0x3d1c827ae5d6704cull,                                  \
+      0x3ff0e00000000000ull, 0xbfab42dd71198000ull, 0x3d1c827ae5d6704cull,                                  \
+      0x3ff0c00000000000ull, 0xbfa77458f632c000ull, 0xbd2cfc4634f2a1eeull,                                  \
+      0x3ff0c00000000000ull, 0xbfa77458f632c000ull, 0xbd2cfc4634f2a1eeull,                                  \
+      0x3ff0a00000000000ull, 0xbfa39e87b9fec000ull, 0x3cf502b7f526feaaull,                                  \
+      0x3ff0a00000000000ull, 0xbfa39e87b9fec000ull, 0x3cf502b7f526feaaull,                                  \
+      0x3ff0800000000000ull, 0xbf9f829b0e780000ull, 0xbd2980267c7e09e4ull,                                  \
+      0x3ff0800000000000ull, 0xbf9f829b0e780000ull, 0xbd2980267c7e09e4ull,                                  \
+      0x3ff0600000000000ull, 0xbf97b91b07d58000ull, 0xbd288d5493faa639ull,                                  \
+      0x3ff0400000000000ull, 0xbf8fc0a8b0fc0000ull, 0xbcdf1e7cf6d3a69cull,                                  \
+      0x3ff0400000000000ull, 0xbf8fc0a8b0fc0000ull, 0xbcdf1e7cf6d3a69cull,                                  \
+      0x3ff0200000000000ull, 0xbf7fe02a6b100000ull, 0xbd19e23f0dda40e4ull,                                  \
+      0x3ff0200000000000ull, 0xbf7fe02a6b100000ull, 0xbd19e23f0dda40e4ull,                                  \
+      0x3ff0000000000000ull, 0x0000000000000000ull, 0x0000000000000000ull,                                  \
+      0x3ff0000000000000ull, 0x0000000000000000ull, 0x0000000000000000ull,                                  \
+      0x3fefc00000000000ull, 0x3f80101575890000ull, 0xbd10c76b999d2be8ull,                                  \
+      0x3fef800000000000ull, 0x3f90205658938000ull, 0xbd23dc5b06e2f7d2ull,                                  \
+      0x3fef400000000000ull, 0x3f98492528c90000ull, 0xbd2aa0ba325a0c34ull,                                  \
+      0x3fef000000000000ull, 0x3fa0415d89e74000ull, 0x3d0111c05cf1d753ull,                                  \
+      0x3feec00000000000ull, 0x3fa466aed42e0000ull, 0xbd2c167375bdfd28ull,                                  \
+      0x3fee800000000000ull, 0x3fa894aa149fc000ull, 0xbd197995d05a267dull,                                  \
+      0x3fee400000000000ull, 0x3faccb73cdddc000ull, 0xbd1a68f247d82807ull,                                  \
+      0x3fee200000000000ull, 0x3faeea31c006c000ull, 0xbd0e113e4fc93b7bull,                                  \
+      0x3fede00000000000ull, 0x3fb1973bd1466000ull, 0xbd25325d560d9e9bull,                                  \
+      0x3feda00000000000ull, 0x3fb3bdf5a7d1e000ull, 0x3d2cc85ea5db4ed7ull,                                  \
+      0x3fed600000000000ull, 0x3fb5e95a4d97a000ull, 0xbd2c69063c5d1d1eull,                                  \
+      0x3fed400000000000ull, 0x3fb700d30aeac000ull, 0x3cec1e8da99ded32ull,                                  \
+      0x3fed000000000000ull, 0x3fb9335e5d594000ull, 0x3d23115c3abd47daull,                                  \
+      0x3fecc00000000000ull, 0x3fbb6ac88dad6000ull, 0xbd1390802bf768e5ull,                                  \
+      0x3feca00000000000ull, 0x3fbc885801bc4000ull, 0x3d2646d1c65aacd3ull,                                  \
+      0x3fec600000000000ull, 0x3fbec739830a2000ull, 0xbd2dc068afe645e0ull,                                  \
+      0x3fec400000000000ull, 0x3fbfe89139dbe000ull, 0xbd2534d64fa10afdull,                                  \
+      0x3fec000000000000ull, 0x3fc1178e8227e000ull, 0x3d21ef78ce2d07f2ull,                                  \
+      0x3febe00000000000ull, 0x3fc1aa2b7e23f000ull, 0x3d2ca78e44389934ull,                                  \
+      0x3feba00000000000ull, 0x3fc2d1610c868000ull, 0x3d039d6ccb81b4a1ull,                                  \
+      0x3feb800000000000ull, 0x3fc365fcb0159000ull, 0x3cc62fa8234b7289ull,                                  \
+      0x3feb400000000000ull, 0x3fc4913d8333b000ull, 0x3d25837954fdb678ull,                                  \
+      0x3feb200000000000ull, 0x3fc527e5e4a1b000ull, 0x3d2633e8e5697dc7ull,                                  \
+      0x3feae00000000000ull, 0x3fc6574ebe8c1000ull, 0x3d19cf8b2c3c2e78ull,                                  \
+      0x3feac00000000000ull, 0x3fc6f0128b757000ull, 0xbd25118de59c21e1ull,                                  \
+      0x3feaa00000000000ull, 0x3fc7898d85445000ull, 0xbd1c661070914305ull,                                  \
+      0x3fea600000000000ull, 0x3fc8beafeb390000ull, 0xbd073d54aae92cd1ull,                                  \
+      0x3fea400000000000ull, 0x3fc95a5adcf70000ull, 0x3d07f22858a0ff6full,                                  \
+      0x3fea000000000000ull, 0x3fca93ed3c8ae000ull, 0xbd28724350562169ull,                                  \
+      0x3fe9e00000000000ull, 0x3fcb31d8575bd000ull, 0xbd0c358d4eace1aaull,                                  \
+      0x3fe9c00000000000ull, 0x3fcbd087383be000ull, 0xbd2d4bc4595412b6ull,                                  \
+      0x3fe9a00000000000ull, 0x3fcc6ffbc6f01000ull, 0xbcf1ec72c5962bd2ull,                                  \
+      0x3fe9600000000000ull, 0x3fcdb13db0d49000ull, 0xbd2aff2af715b035ull,                                  \
+      0x3fe9400000000000ull, 0x3fce530effe71000ull, 0x3cc212276041f430ull,                                  \
+      0x3fe9200000000000ull, 0x3fcef5ade4dd0000ull, 0xbcca211565bb8e11ull,                                  \
+      0x3fe9000000000000ull, 0x3fcf991c6cb3b000ull, 0x3d1bcbecca0cdf30ull,                                  \
+      0x3fe8c00000000000ull, 0x3fd07138604d5800ull, 0x3cf89cdb16ed4e91ull,                                  \
+      0x3fe8a00000000000ull, 0x3fd0c42d67616000ull, 0x3d27188b163ceae9ull,                                  \
+      0x3fe8800000000000ull, 0x3fd1178e8227e800ull, 0xbd2c210e63a5f01cull,                                  \
+      0x3fe8600000000000ull, 0x3fd16b5ccbacf800ull, 0x3d2b9acdf7a51681ull,                                  \
+      0x3fe8400000000000ull, 0x3fd1bf99635a6800ull, 0x3d2ca6ed5147bdb7ull,                                  \
+      0x3fe8200000000000ull, 0x3fd214456d0eb800ull, 0x3d0a87deba46baeaull,                                  \
+      0x3fe7e00000000000ull, 0x3fd2bef07cdc9000ull, 0x3d2a9cfa4a5004f4ull,                                  \
+      0x3fe7c00000000000ull, 0x3fd314f1e1d36000ull, 0xbd28e27ad3213cb8ull,                                  \
+      0x3fe7a00000000000ull, 0x3fd36b6776be1000ull, 0x3d116ecdb0f177c8ull,                                  \
+      0x3fe7800000000000ull, 0x3fd3c25277333000ull, 0x3d183b54b606bd5cull,                                  \
+      0x3fe7600000000000ull, 0x3fd419b423d5e800ull, 0x3d08e436ec90e09dull,                                  \
+      0x3fe7400000000000ull, 0x3fd4718dc271c800ull, 0xbd2f27ce0967d675ull,                                  \
+      0x3fe7200000000000ull, 0x3fd4c9e09e173000ull, 0xbd2e20891b0ad8a4ull,                                  \
+      0x3fe7000000000000ull, 0x3fd522ae0738a000ull, 0x3d2ebe708164c759ull,                                  \
+      0x3fe6e00000000000ull, 0x3fd57bf753c8d000ull, 0x3d1fadedee5d40efull,                                  \
+      0x3fe6c00000000000ull, 0x3fd5d5bddf596000ull, 0xbd0a0b2a08a465dcull                                   \
+    }
+static const uint64_t kPow64LogTabHost[384] = ZM_POW64_LOG_TAB;
+#if defined(__HIPCC__)
+static __device__ const uint64_t kPow64LogTabDev[384] = ZM_POW64_LOG_TAB;
+#endif
+ZM_HD const double *pow64_log_table()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return reinterpret_cast<const double *>(kPow64LogTabDev);
+#else
+    return reinterpret_cast<const double *>(kPow64LogTabHost);
+#endif
+}
+
+// the constants as data (a kernel argument: scalar registers feed the f64 operations directly)
+struct PowCoef64 {
+    double a1 = 0x1.555555555556p-2 * -2, a2 = -0x1.0000000000006p-2 * -2, a3 = 0x1.999999959554ep-3 * 4,
+           a4 = -0x1.555555529a47ap-3 * 4, a5 = 0x1.2495b9b4845e9p-3 * -8, a6 = -0x1.0002b8b263fc3p-3 * -8;
+    double ln2hi = 0x1.62e42fefa3800p-1, ln2lo = 0x1.ef35793c76730p-45;
+    ExpCoef64 e;
+};
+
+// log(x) of a positive normal x given by its bits, as the returned high part plus *tail
+ZM_HD double pow_log_inline(uint64_t ix, double *tail, const double *ltab, const PowCoef64 &k)
+{
+    const uint64_t tmp = ix - 0x3fe6955500000000ull;
+    const int i = (int)((tmp >> 45) & 127u);
+    const int64_t ke = (int64_t)tmp >> 52;
+    const double z = u2d(ix - (tmp & (0xfffull << 52)));
+    const double kd = (double)ke;
+    const double invc = ltab[3 * i], logc = ltab[3 * i + 1], logctail = ltab[3 * i + 2];
+    const double r = __builtin_fma(z, invc, -1.0);
+    const double t1 = __builtin_fma(kd, k.ln2hi, logc);
+    const double t2 = t1 + r;
+    const double lo1 = __builtin_fma(kd, k.ln2lo, logctail);
+    const double lo2 = t1 - t2 + r;
+    const double ar = -0.5 * r, ar2 = r * ar, ar3 = r * ar2;
+    const double hi = t2 + ar2;
+    const double lo3 = __builtin_fma(ar, r, -ar2);
+    const double lo4 = t2 - hi + ar2;
+    const double p = __builtin_fma(ar2, __builtin_fma(ar2, __builtin_fma(r, k.a6, k.a5), __builtin_fma(r, k.a4, k.a3)),
+                                   __builtin_fma(r, k.a2, k.a1));
+    const double lo = __builtin_fma(ar3, p, lo1 + lo2 + lo3 + lo4);
+    const double y = hi + lo;
+    *tail = hi - y + lo;
+    return y;
+}
+
+// exp(x + xtail), negated when sign_bias is set (it is added to the scale's exponent field, where it lands on the sign)
+ZM_HD double pow_exp_inline(double x, double xtail, uint32_t sign_bias, const uint64_t *etab, const ExpCoef64 &k)
+{
+    uint32_t abstop = (uint32_t)(d2u(x) >> 52) & 0x7ffu;
+    if (abstop - 0x3c9u >= 0x408u - 0x3c9u) {            // |x| < 2^-54 or |x| >= 512
+        if (abstop - 0x3c9u >= 0x80000000u) {
+            const double one = 1.0 + x;
+            return sign_bias ? -one : one;
+        }
+        if (abstop >= 0x409u) {                          // |x| >= 1024: under- or overflow
+            if (d2u(x) >> 63) return sign_bias ? -0.0 : 0.0;
+            return u2d(sign_bias ? 0xfff0000000000000ull : 0x7ff0000000000000ull);
+        }
+        abstop = 0;                                      // large |x|: the special case below
+    }
+    const double z = k.inv_ln2n * x;
+    double kd = z + k.shift;
+    const uint64_t ki = d2u(kd);
+    kd -= k.shift;
+    double r = __builtin_fma(kd, k.neg_ln2lo_n, __builtin_fma(kd, k.neg_ln2hi_n, x));
+    r += xtail;
+    const uint64_t idx = 2 * (ki % 128);
+    const uint64_t top = (ki + sign_bias) << (52 - 7);
+    const double tail = u2d(etab[idx]);
+    uint64_t sbits = etab[idx + 1] + top;
+    const double r2 = r * r;
+    const double tmp = __builtin_fma(r2 * r2, __builtin_fma(r, k.c5, k.c4), __builtin_fma(r2, __builtin_fma(r, k.c3, k.c2), tail + r));
+    if (abstop == 0) {
+        if ((ki & 0x80000000u) == 0) {                   // k > 0: the exponent of scale may have overflowed
+            sbits -= 1009ull << 52;
+            const double scale = u2d(sbits);
+            return 0x1p1009 * __builtin_fma(scale, tmp, scale);
+        }
+        sbits += 1022ull << 52;                          // k < 0: care in the subnormal range
+        const double scale = u2d(sbits);
+        double y = scale + scale * tmp;
+        if (__builtin_fabs(y) < 1.0) {
+            const double one = y < 0.0 ? -1.0 : 1.0;
+            double lo = scale - y + scale * tmp;
+            const double hi = one + y;
+            lo = one - hi + y + lo;
+            y = (hi + lo) - one;
+            if (y == 0.0) y = u2d(sbits & 0x8000000000000000ull);
+        }
+        return 0x1p-1022 * y;
+    }
+    const double scale = u2d(sbits);
+    return __builtin_fma(scale, tmp, scale);
+}
+
+// 0: y is not an integer, 1: odd, 2: even
+ZM_HD int pow_checkint(uint64_t iy)
+{
+    const int e = (int)(iy >> 52) & 0x7ff;
+    if (e < 0x3ff) return 0;
+    if (e > 0x3ff + 52) return 2;
+    if (iy & ((1ull << (0x3ff + 52 - e)) - 1)) return 0;
+    if (iy & (1ull << (0x3ff + 52 - e))) return 1;
+    return 2;
+}
+ZM_HD bool pow_zeroinfnan(uint64_t i) { return 2 * i - 1 >= 2 * 0x7ff0000000000000ull - 1; }
+ZM_HD bool pow_issignaling(uint64_t i) { return 2 * (i ^ 0x0008000000000000ull) > 2 * 0x7ff8000000000000ull; }
+
+ZM_HD double pow_glibc_full(double x, double y, const double *ltab, const uint64_t *etab, const PowCoef64 &k = PowCoef64())
+{
+    const uint64_t one = 0x3ff0000000000000ull, inf = 0x7ff0000000000000ull;
+    uint32_t sign_bias = 0;
+    uint64_t ix = d2u(x);
+    const uint64_t iy = d2u(y);
+    uint32_t topx = (uint32_t)(ix >> 52);
+    const uint32_t topy = (uint32_t)(iy >> 52);
+    if (topx - 0x001u >= 0x7ffu - 0x001u || (topy & 0x7ffu) - 0x3beu >= 0x43eu - 0x3beu) {
+        // x subnormal, zero, negative, infinite or NaN; or |y| < 2^-65, |y| >= 2^63 or NaN
+        if (pow_zeroinfnan(iy)) {
+            if (2 * iy == 0) return pow_issignaling(ix) ? x + y : 1.0;
+            if (ix == one) return pow_issignaling(iy) ? x + y : 1.0;
+            if (2 * ix > 2 * inf || 2 * iy > 2 * inf) return x + y;
+            if (2 * ix == 2 * one) return 1.0;
+            if ((2 * ix < 2 * one) == !(iy >> 63)) return 0.0;   // |x| < 1 && y == inf, or |x| > 1 && y == -inf
+            return y * y;
+        }
+        if (pow_zeroinfnan(ix)) {
+            double x2 = x * x;
+            if ((ix >> 63) && pow_checkint(iy) == 1) x2 = -x2;
+            return (iy >> 63) ? 1 / x2 : x2;
+        }
+        if (ix >> 63) {                                  // finite x < 0
+            const int yint = pow_checkint(iy);
+            if (yint == 0) return (x - x) * u2d(inf);    // the sources' (x - x) / (x - x): a NaN
+            if (yint == 1) sign_bias = 0x800u << 7;
+            ix &= 0x7fffffffffffffffull;
+            topx &= 0x7ffu;
+        }
+        if ((topy & 0x7ffu) - 0x3beu >= 0x43eu - 0x3beu) {
+            if (ix == one) return 1.0;
+            if ((topy & 0x7ffu) < 0x3beu) return ix > one ? 1.0 + y : 1.0 - y;   // |y| < 2^-65
+            return (ix > one) == (topy < 0x800u) ? u2d(inf) : 0.0;
+        }
+        if (topx == 0) {                                 // subnormal x: normalise
+            ix = d2u(x * 0x1p52);
+            ix &= 0x7fffffffffffffffull;
+            ix -= 52ull << 52;
+        }
+    }
+    double lo;
+    const double hi = pow_log_inline(ix, &lo, ltab, k);
+    const double ehi = y * hi;
+    const double elo = __builtin_fma(y, lo, __builtin_fma(y, hi, -ehi));
+    return pow_exp_inline(ehi, elo, sign_bias, etab, k.e);
+}
+ZM_HD double pow_glibc_full(double x, double y) { return pow_glibc_full(x, y, pow64_log_table(), exp_table()); }
+// (builds its own constants: a reference to the caller's would force them into memory there)
+ZM_RARE double pow_rare(double x, double y, const double *ltab, const uint64_t *etab) { return pow_glibc_full(x, y, ltab, etab); }
+
+// pow as the kernels call it: the main path as straight-line code (positive normal x, 2^-65 <= |y| < 2^63,
+// 2^-54 <= |y log x| < 512: no special case applies, no sign to carry), everything else out of line
+ZM_HD double pow_glibc(double x, double y, const double *ltab, const uint64_t *etab, const PowCoef64 &k = PowCoef64())
+{
+    const uint64_t ix = d2u(x), iy = d2u(y);
+    const uint32_t topx = (uint32_t)(ix >> 52), topy = (uint32_t)(iy >> 52);
+    if (__builtin_expect(topx - 0x001u >= 0x7ffu - 0x001u || (topy & 0x7ffu) - 0x3beu >= 0x43eu - 0x3beu, 0))
+        return pow_rare(x, y, ltab, etab);
+    double lo;
+    const double hi = pow_log_inline(ix, &lo, ltab, k);
+    const double ehi = y * hi;
+    const double elo = __builtin_fma(y, lo, __builtin_fma(y, hi, -ehi));
+    const uint32_t abstop = (uint32_t)(d2u(ehi) >> 52) & 0x7ffu;
+    if (__builtin_expect(abstop - 0x3c9u >= 0x408u - 0x3c9u, 0)) return pow_rare(x, y, ltab, etab);
+    const ExpCoef64 &e = k.e;
+    const double z = e.inv_ln2n * ehi;
+    double kd = z + e.shift;
+    const uint64_t ki = d2u(kd);
+    kd -= e.shift;
+    double r = __builtin_fma(kd, e.neg_ln2lo_n, __builtin_fma(kd, e.neg_ln2hi_n, ehi));
+    r += elo;
+    const uint64_t idx = 2 * (ki % 128);
+    const double tail = u2d(etab[idx]);
+    const double scale = u2d(etab[idx + 1] + (ki << (52 - 7)));
+    const double r2 = r * r;
+    const double tmp = __builtin_fma(r2 * r2, __builtin_fma(r, e.c5, e.c4), __builtin_fma(r2, __builtin_fma(r, e.c3, e.c2), tail + r));
+    return __builtin_fma(scale, tmp, scale);
+}
+ZM_HD double pow_glibc(double x, double y) { return pow_glibc(x, y, pow64_log_table(), exp_table()); }
+
 // ---- double precision sin / cos: s_sin.c and branred.c as glibc 2.35 ships them (the IBM Accurate
 // Mathematical Library without its multi-precision fall-backs) ------------------------------------------
 // |x| < 2^-26: x resp. 1.  The argument is brought to a in [-pi/4, pi/4] plus a small da and a quadrant n:
@@ -2385,10 +2719,23 @@ struct SinCos64Lds {
     }
 };
 
-// pow with the same arrangement: f32 through powf's two tables in LDS, f64 from the math library
-template <typename T> struct Pow {
-    __device__ __forceinline__ void init() {}
-    __device__ __forceinline__ T pow(T x, T y) const { return ::pow(x, y); }
+// pow with the same arrangement: its log and exp tables in LDS
+template <typename T> struct Pow;
+template <> struct Pow<double> {
+    const double *ltab;
+    const uint64_t *etab;
+    __device__ __forceinline__ void init()
+    {
+        __shared__ uint64_t lds_powlog[384];
+        __shared__ uint64_t lds_powexp[256];
+        for (int i = threadIdx.x; i < 384; i += blockDim.x) lds_powlog[i] = kPow64LogTabDev[i];
+        for (int i = threadIdx.x; i < 256; i += blockDim.x) lds_powexp[i] = kExpTabDev[i];
+        __syncthreads();
+        ltab = reinterpret_cast<const double *>(lds_powlog);
+        etab = lds_powexp;
+    }
+    PowCoef64 k;
+    __device__ __forceinline__ double pow(double x, double y) const { return pow_glibc(x, y, ltab, etab, k); }
 };
 template <> struct Pow<float> {
     const uint64_t *etab;
