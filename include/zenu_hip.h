@@ -86,9 +86,9 @@ int zenu_hip_init(int device);
 int zenu_hip_shutdown(void);
 const char *zenu_hip_status_string(int status);
 /* hipError_t of the last failed runtime call on this thread, and its text. */
-/* The host math library whose results the device's exp, log, tanh, sigmoid, powf, sinh, cosh, sin,
- * cos, asin, acos and atan reproduce bit for bit (the routines are restated from it and compared
- * with it on every f32 argument).  ZeNu's CPU device calls whatever libm the host has: on a host
+/* The host math library whose results the device's exp, log, tanh, sigmoid, powf, sinh, cosh, sin and
+ * cos (f32 and f64) and its f32 tan, asin, acos and atan reproduce bit for bit (the routines are
+ * restated from it and compared with it on every f32 argument and on 10^8 to 10^10 sampled f64 ones).  ZeNu's CPU device calls whatever libm the host has: on a host
  * whose libm rounds some of these functions differently (glibc 2.41 and later return correctly
  * rounded results from several f32 functions), CPU and device results differ by the difference between
  * the two libms -- at most 1 ulp for the functions themselves, more for the sigmoid, whose last
