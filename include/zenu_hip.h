@@ -441,6 +441,10 @@ int zenu_hip_powf_range_hash(double exponent, uint64_t first, uint64_t count, in
 int zenu_hip_unary_range_hash_f64(int fn, uint64_t first, uint64_t count, int block_log2, uint32_t step,
                                   uint32_t offset, uint64_t salt, uint64_t *sums_dev,
                                   zenu_stream_t stream);
+/* The same for the f64 powf(x, exponent) over sampled bases x. */
+int zenu_hip_powf_range_hash_f64(double exponent, uint64_t first, uint64_t count, int block_log2,
+                                 uint32_t step, uint32_t offset, uint64_t salt, uint64_t *sums_dev,
+                                 zenu_stream_t stream);
 int zenu_hip_last_status(void);
 
 #define ZENU_DECL_1D(T, S)                                                                        \

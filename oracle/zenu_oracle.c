@@ -249,10 +249,11 @@ static inline double zo_range_fn_f64(int fn, double x)
     return zo_unary_fn_f64(fn, x);
 }
 
-/* kind 0: f32 unary (fn); kind 1: f32 powf with `exponent`; kind 2: f64 unary (fn) on zo_range_arg_f64 */
+/* kind 0: f32 unary (fn); kind 1: f32 powf with `exponent`; kind 2: f64 unary (fn) on zo_range_arg_f64; kind 3: f64 pow with `exponent64` */
 typedef struct {
     int kind, fn, block_log2;
     float exponent;
+    double exponent64;
     uint32_t step, offset;
     uint64_t salt;
     uint64_t first_block, n_blocks, first;
@@ -266,13 +267,13 @@ static void *zo_range_worker(void *arg)
     for (uint64_t b = j->first_block; b < j->first_block + j->n_blocks; b++) {
         uint64_t sum = 0;
         const uint64_t start = j->first + b * per;
-        if (j->kind == 2) {
+        if (j->kind == 2 || j->kind == 3) {
             for (uint64_t i = 0; i < per; i++) {
                 const uint64_t bits = zo_range_arg_f64(start + i, j->step, j->offset, j->salt);
                 double x, y;
                 uint64_t rb;
                 memcpy(&x, &bits, 8);
-                y = zo_range_fn_f64(j->fn, x);
+                y = j->kind == 3 ? pow(x, j->exponent64) : zo_range_fn_f64(j->fn, x);
                 memcpy(&rb, &y, 8);
                 if ((rb & 0x7fffffffffffffffull) > 0x7ff0000000000000ull) rb = 0x7ff8000000000000ull;
                 sum += zo_mix64(zo_mix64(bits) + rb);
@@ -354,6 +355,21 @@ int zo_unary_range_hash_f64(int fn, uint64_t first, uint64_t count, int block_lo
     if (step == 0) return ZO_ERR_ARG;
     j.kind = 2;
     j.fn = fn;
+    j.step = step;
+    j.offset = offset;
+    j.salt = salt;
+    return zo_range_hash_run(j, first, count, block_log2, sums, nthreads);
+}
+
+/* the same for pow(x, exponent) over the sampled f64 bases x */
+int zo_powf_range_hash_f64(double exponent, uint64_t first, uint64_t count, int block_log2, uint32_t step, uint32_t offset,
+                           uint64_t salt, uint64_t *sums, int nthreads)
+{
+    zo_range_job j;
+    memset(&j, 0, sizeof j);
+    if (step == 0) return ZO_ERR_ARG;
+    j.kind = 3;
+    j.exponent64 = exponent;
     j.step = step;
     j.offset = offset;
     j.salt = salt;

@@ -162,6 +162,8 @@ int zo_powf_range_hash_f32(float exponent, uint64_t first, uint64_t count, int b
 uint64_t zo_range_arg_f64(uint64_t i, uint32_t step, uint32_t offset, uint64_t salt);
 int zo_unary_range_hash_f64(int fn, uint64_t first, uint64_t count, int block_log2, uint32_t step, uint32_t offset,
                             uint64_t salt, uint64_t *sums, int nthreads);
+int zo_powf_range_hash_f64(double exponent, uint64_t first, uint64_t count, int block_log2, uint32_t step, uint32_t offset,
+                           uint64_t salt, uint64_t *sums, int nthreads);
 
 #ifdef __cplusplus
 }

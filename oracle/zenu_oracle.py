@@ -186,6 +186,16 @@ def unary_range_hash_f64(fn, first, count, block_log2, step, offset, salt, nthre
     return sums
 
 
+def powf_range_hash_f64(exponent, first, count, block_log2, step, offset, salt, nthreads=1):
+    """the same for pow(x, exponent) over the sampled f64 bases"""
+    sums = np.zeros(count >> block_log2, dtype=np.uint64)
+    f = lib().zo_powf_range_hash_f64
+    f.argtypes = [C.c_double, C.c_uint64, C.c_uint64, C.c_int, C.c_uint32, C.c_uint32, C.c_uint64, C.c_void_p, C.c_int]
+    f.restype = C.c_int
+    _chk(f(exponent, first, count, block_log2, step, offset, salt, sums.ctypes.data, nthreads), "powf_range_hash_f64")
+    return sums
+
+
 def range_arg_f64(i, step, offset, salt):
     f = lib().zo_range_arg_f64
     f.argtypes = [C.c_uint64, C.c_uint32, C.c_uint32, C.c_uint64]

@@ -363,6 +363,28 @@ def test_f64_sampled_arguments_equal_the_host_libm(hip, name, zo_fn, hip_fn):
         raise AssertionError(f"{name} f64: {bad.size} blocks differ, the first is block {b}; {first}; {_libm_note(hip)}")
 
 
+@pytest.mark.parametrize("exponent", [2.5, -3.0, 0.3])
+def test_powf_f64_sampled_bases_equal_the_host_libm(hip, exponent):
+    """f64 powf(x, exponent): every fourth value of the base's high word (sign, exponent, 20 mantissa bits) with a
+    pseudo-random low word -- 2^30 bases per exponent, zeros, negative, subnormal, infinite and NaN bases
+    among them -- against the host libm through the folded sums"""
+    from zenu_amd import _lib
+    block_log2 = 20
+    count = 1 << 30
+    salt = int(os.environ.get("ZENU_F64_HASH_SALT", "0"))
+    step, offset = 4, 1
+    sums = hip.Matrix.alloc((2 * (count >> block_log2),), dtype=np.float32)
+    _lib.check(hip.lib().zenu_hip_powf_range_hash_f64(exponent, 0, count, block_log2, step, offset, salt, sums.as_ptr(),
+                                                      hip.get_stream()), "powf_range_hash_f64")
+    threads = max(1, min(16, os.cpu_count() or 1))
+    t0 = time.time()
+    host = zo.powf_range_hash_f64(exponent, 0, count, block_log2, step, offset, salt, threads)
+    dev = sums.to_numpy().view(np.uint64)
+    print(f"[range hash] powf(x, {exponent}) f64: 2^30 bases, host libm on {threads} threads {time.time() - t0:.1f} s", flush=True)
+    bad = np.flatnonzero(dev != host)
+    assert bad.size == 0, f"powf(x, {exponent}) f64: {bad.size} blocks differ, the first is block {int(bad[0])}; {_libm_note(hip)}"
+
+
 def test_range_hash_sees_one_differing_result(hip):
     """the sums are a comparison, not a formality: the device's sums of exp over one block against the
     host's sums of the same block of ANOTHER function differ, and a host-side recomputation of one

@@ -111,5 +111,22 @@ def test_powf_and_f64_range_hashes_are_folds_of_the_element_wise_results():
         rb = np.where(np.isnan(out), np.uint64(0x7ff8000000000000), out.view(np.uint64))
         with np.errstate(over="ignore"):
             assert int(mix(mix(bits) + rb).sum(dtype=np.uint64)) == int(sums[b])
+    # the f64 powf over the same arguments
+    sums = zo.powf_range_hash_f64(-1.5, i0, 2 << 12, 12, step, offset, salt, 2)
+    for b in range(2):
+        idx = np.arange(i0 + (b << 12), i0 + ((b + 1) << 12), dtype=np.uint64)
+        with np.errstate(over="ignore"):
+            hi = (idx * np.uint64(step) + np.uint64(offset)) & np.uint64(0xffffffff)
+            lo = (((idx + np.uint64(salt)) * np.uint64(0x9E3779B97F4A7C15)) >> np.uint64(29)) & np.uint64(0xffffffff)
+        bits = (hi << np.uint64(32)) | lo
+        x = bits.view(np.float64)
+        out = np.empty_like(x)
+        with np.errstate(all="ignore"):
+            zo.powf(out, x, -1.5)
+        rb = np.where(np.isnan(out), np.uint64(0x7ff8000000000000), out.view(np.uint64))
+        with np.errstate(over="ignore"):
+            assert int(mix(mix(bits) + rb).sum(dtype=np.uint64)) == int(sums[b])
     with pytest.raises(zo.OracleError):
         zo.unary_range_hash_f64(zo.TANH, 0, 1 << 12, 12, 0, 0, 0, 1)
+    with pytest.raises(zo.OracleError):
+        zo.powf_range_hash_f64(2.0, 0, 1 << 12, 12, 0, 0, 0, 1)

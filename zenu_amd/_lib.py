@@ -96,6 +96,7 @@ SIGNATURES = {
     "zenu_hip_unary_range_hash": [_i, C.c_uint64, C.c_uint64, _i, _vp, _vp],
     "zenu_hip_powf_range_hash": [C.c_double, C.c_uint64, C.c_uint64, _i, _vp, _vp],
     "zenu_hip_unary_range_hash_f64": [_i, C.c_uint64, C.c_uint64, _i, C.c_uint32, C.c_uint32, C.c_uint64, _vp, _vp],
+    "zenu_hip_powf_range_hash_f64": [C.c_double, C.c_uint64, C.c_uint64, _i, C.c_uint32, C.c_uint32, C.c_uint64, _vp, _vp],
     "zenu_hip_sum_all": [_i, _vp, _TP, _vp],
     "zenu_hip_sum_to": [_i, _TP, _TP, _vp],
     "zenu_hip_max_axis": [_i, _TP, _TP, _i, _vp],

@@ -77,10 +77,9 @@ __device__ __forceinline__ uint64_t range_arg_f64(uint64_t i, uint32_t step, uin
     return (hi << 32) | lo;
 }
 
-template <int FN>
+template <typename F>
 __global__ __launch_bounds__(kHashBlock) void range_hash_f64_kernel(uint64_t first, int block_log2, uint32_t step,
-                                                                    uint32_t offset, uint64_t salt, uint64_t *sums,
-                                                                    UnaryF<double, FN> f)
+                                                                    uint32_t offset, uint64_t salt, uint64_t *sums, F f)
 {
     f.init();
     const uint64_t per = 1ull << block_log2;
@@ -100,8 +99,8 @@ template <int FN>
 int launch_range_hash_f64(uint64_t first, uint64_t blocks, int block_log2, uint32_t step, uint32_t offset, uint64_t salt,
                           uint64_t *sums, hipStream_t s)
 {
-    range_hash_f64_kernel<FN><<<(unsigned)blocks, kHashBlock, 0, s>>>(first, block_log2, step, offset, salt, sums,
-                                                                      UnaryF<double, FN>());
+    range_hash_f64_kernel<UnaryF<double, FN>><<<(unsigned)blocks, kHashBlock, 0, s>>>(first, block_log2, step, offset, salt,
+                                                                                      sums, UnaryF<double, FN>());
     ZENU_LAUNCH_CHECK();
     return ZENU_OK;
 }
@@ -172,3 +171,18 @@ extern "C" int zenu_hip_unary_range_hash_f64(int fn, uint64_t first, uint64_t co
     }
 }
 
+
+extern "C" int zenu_hip_powf_range_hash_f64(double exponent, uint64_t first, uint64_t count, int block_log2, uint32_t step,
+                                            uint32_t offset, uint64_t salt, uint64_t *sums_dev, zenu_stream_t stream)
+{
+    if (!sums_dev || block_log2 < 8 || block_log2 > 32 || step == 0) return ZENU_ERR_ARG;
+    if ((count & ((1ull << block_log2) - 1)) || count == 0 || first + count > (1ull << 32)) return ZENU_ERR_ARG;
+    const uint64_t blocks = count >> block_log2;
+    if (blocks > 0x7fffffffull) return ZENU_ERR_UNSUPPORTED;
+    PowF<double> f;
+    f.s = exponent;
+    range_hash_f64_kernel<PowF<double>><<<(unsigned)blocks, kHashBlock, 0, reinterpret_cast<hipStream_t>(stream)>>>(
+        first, block_log2, step, offset, salt, sums_dev, f);
+    ZENU_LAUNCH_CHECK();
+    return ZENU_OK;
+}
