@@ -523,10 +523,7 @@ def test_cross_entropy_head_every_small_geometry(hip, dtype):
             loss_ref, prob_ref = cpu_matrix.cross_entropy(CpuMatrix.from_numpy(pred), CpuMatrix.from_numpy(ans))
             loss, prob = hip.cross_entropy(M.from_numpy(pred), M.from_numpy(ans))
             p = prob.to_numpy()
-            if dtype == np.float32:
-                assert bits_equal(p, prob_ref.a), (n, c)
-            else:
-                assert rel_err(p, prob_ref.a) <= 1e-14, (n, c)
+            assert bits_equal(p, prob_ref.a), (n, c)
             lr = float(loss_ref.a)
             assert abs(float(loss.to_numpy()) - lr) <= 4 * tol * max(abs(lr), 1e-30) + 1e-30, (n, c)
             gb = M.from_numpy(np.full(c, 9.0, dtype=dtype))
