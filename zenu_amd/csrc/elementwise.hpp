@@ -273,7 +273,7 @@ template <> struct IsValuBound<TanhUlp2F> { static constexpr bool value = true; 
 template <> struct IsValuBound<UnaryF<double, ZENU_SIN>> { static constexpr bool value = true; };
 template <> struct IsValuBound<UnaryF<double, ZENU_COS>> { static constexpr bool value = true; };
 // measured on 2^24 elements (us at 64 x 1 -> at 256 x 2): f32 sin 25.6 -> 23.8, cos 25.9 -> 23.8, asin 25.4 -> 24.0,
-// sinh 25.7 -> 25.2, cosh 26.4 -> 25.0; f64 sinh 63.9 -> 61.6, cosh 62.4 -> 55.4, sin 88.4 -> 53.0, cos 86.4 -> 51.4.
+// sinh 25.7 -> 25.2, cosh 26.4 -> 25.0; f64 sinh 63.9 -> 61.6, cosh 62.4 -> 55.4, sin 88.4 -> 49.8, cos 86.4 -> 49.6.
 // (f32 acos 25.0 -> 26.3 and atan 23.5 -> 24.7 prefer the small shape, tan does not care.)
 template <typename T> struct IsValuBound<UnaryF<T, ZENU_SINH>> { static constexpr bool value = true; };
 template <typename T> struct IsValuBound<UnaryF<T, ZENU_COSH>> { static constexpr bool value = true; };

@@ -2462,17 +2462,14 @@ struct SinCos64Coef {
            s5 = -0x1.ADDFFC2FCDF59p-26;
 };
 
-// sin (n even) or cos (n odd) of a + da, negated for n = 2, 3 (the sources' do_sincos with do_sin, do_cos,
-// TAYLOR_SIN).  do_sin and do_cos are one path here: a wavefront usually holds both parities.  With
-// (M, m) = (sin xi, its low part) and (P, p) = (cos xi, its low part) for the sine, and (cos xi, low) and
-// (-sin xi, -low) for the cosine, both corrections read P s + (-M c + (s p + m)) and both results M + cor;
-// what differs is where da enters s and c.
+// sin (n even) or cos (n odd) of a + da, negated for n = 2, 3 (the sources' do_sincos with do_sin, do_cos, TAYLOR_SIN).
+// The two table paths are kept apart as in the sources: merged into one path with selected operands (both
+// corrections read P s + (-M c + (s p + m)) for suitable M, m, P, p) the kernels measured 2 to 10 % slower.
 ZM_HD double sincos64_eval(double a, double da, int n, const double *tab, const SinCos64Coef &k)
 {
     const double aa = __builtin_fabs(a);
-    const bool cosine = (n & 1) != 0;
     double r;
-    if (!cosine && aa < 0.126) {
+    if ((n & 1) == 0 && aa < 0.126) {
         const double xx = a * a;
         double p = __builtin_fma(k.s5, xx, k.s4);
         p = __builtin_fma(p, xx, k.s3);
@@ -2483,20 +2480,24 @@ ZM_HD double sincos64_eval(double a, double da, int n, const double *tab, const 
     } else {
         const double u = k.big + aa;                     // its low mantissa bits: the nearest multiple of 1/128
         const double *e = tab + 4 * (int)(uint32_t)d2u(u);
-        const uint64_t flip = cosine ? 0x8000000000000000ull : 0ull;
-        const double M = e[cosine ? 2 : 0], m = e[cosine ? 3 : 1];
-        const double P = u2d(d2u(e[cosine ? 0 : 2]) ^ flip), p = u2d(d2u(e[cosine ? 1 : 3]) ^ flip);
-        // da with the sign of a (the sine takes a = 0 as negative, which only matters to the sign of a zero)
-        const double dx = (cosine ? a < 0 : a <= 0) ? -da : da;
-        const double x0 = aa - (u - k.big);
-        const double x = cosine ? x0 + dx : x0;
-        const double xx = x * x;
-        const double t = __builtin_fma(x * xx, __builtin_fma(xx, k.sn5, k.sn3), cosine ? x : dx);
-        const double s = cosine ? t : x + t;
-        const double c = __builtin_fma(x, cosine ? 0.0 : dx, xx * __builtin_fma(xx, __builtin_fma(xx, k.cs6, k.cs4), k.cs2));
-        const double cor = __builtin_fma(P, s, __builtin_fma(-M, c, __builtin_fma(s, p, m)));
-        r = M + cor;
-        if (!cosine) r = __builtin_copysign(r, a);
+        const double sn = e[0], ssn = e[1], cs = e[2], ccs = e[3];
+        if (n & 1) {
+            const double dx = a < 0 ? -da : da;
+            const double x = aa - (u - k.big) + dx;
+            const double xx = x * x;
+            const double s = __builtin_fma(x * xx, __builtin_fma(xx, k.sn5, k.sn3), x);
+            const double c = xx * __builtin_fma(xx, __builtin_fma(xx, k.cs6, k.cs4), k.cs2);
+            const double cor = __builtin_fma(-sn, s, __builtin_fma(-cs, c, __builtin_fma(-s, ssn, ccs)));
+            r = cs + cor;
+        } else {
+            const double dx = a <= 0 ? -da : da;
+            const double x = aa - (u - k.big);
+            const double xx = x * x;
+            const double s = x + __builtin_fma(x * xx, __builtin_fma(xx, k.sn5, k.sn3), dx);
+            const double c = __builtin_fma(x, dx, xx * __builtin_fma(xx, __builtin_fma(xx, k.cs6, k.cs4), k.cs2));
+            const double cor = __builtin_fma(cs, s, __builtin_fma(-sn, c, __builtin_fma(s, ccs, ssn)));
+            r = __builtin_copysign(sn + cor, a);
+        }
     }
     return (n & 2) ? -r : r;
 }
