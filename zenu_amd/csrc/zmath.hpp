@@ -2,15 +2,18 @@
 // the reference's CPU path calls (Rust f32::tanh / exp / ln / powf ... -> libm tanhf / expf / logf /
 // powf ...; glibc 2.35 is what this image ships).
 //
-//   f32: tanh, expm1, exp, log, powf, sinh, cosh, sin, cos, atan, asin, acos, the sigmoid composite
-//   f64: tanh, expm1, exp, sinh, cosh, the sigmoid composite
+//   f32: tanh, expm1, exp, log, powf, sinh, cosh, sin, cos, tan, atan, asin, acos, the sigmoid composite
+//   f64: tanh, expm1, exp, log, pow, sinh, cosh, sin, cos, the sigmoid composite
+//   (f64 tan, asin, acos, atan are not here: the host's routines rest on tables and fitted coefficients
+//   that their sources give only as literals; the kernels call the device math library for them)
 //
 // Why not the device math library: ZeNu's sigmoid is the composite 0.5 + 0.5*tanh(0.5*x)
 // (zenu-autograd/src/activation/sigmoid.rs:7-15).  For negative x the final add cancels, so a
 // 1-ulp difference in tanh becomes tens of ulps in the sigmoid; parity therefore needs the
 // same tanh bits as the CPU path, not merely an accurate tanh.  The other functions follow the
 // same idea: each restates the algorithm the host libm uses (fdlibm's float and double routines,
-// ARM's table-driven expf / logf / powf / sinf / cosf / exp as glibc carries them), with the fused
+// ARM's table-driven expf / logf / powf / sinf / cosf / exp / log / pow and IBM's double sin / cos as
+// glibc carries them; tables rebuilt from their definitions, see tablegen/), with the fused
 // multiply-adds exactly where the x86-64 build that CPUs with FMA select has them, so host and
 // device produce identical bits.
 //
@@ -1698,7 +1701,7 @@ ZM_HD float tanhf_ulp2(float x, const TanhUlp2Coef &q)
 }
 ZM_HD float tanhf_ulp2(float x) { return tanhf_ulp2(x, TanhUlp2Coef()); }
 
-// what the kernels call: f32 from the restatements above, f64 exp / log from the math library
+// the f32 restatements above with their tables at hand
 ZM_HD float expf_glibc(float x) { return expf_glibc(x, exp2f_table()); }
 ZM_HD float logf_glibc(float x) { return logf_glibc(x, logf_table()); }
 ZM_HD float powf_glibc(float x, float y) { return powf_glibc(x, y, exp2f_table(), powf_log2_table()); }
@@ -2632,7 +2635,7 @@ ZM_HD double cos_glibc(double x) { return cos_glibc(x, sincos64_table()); }
 #if defined(__HIPCC__)
 // exp / log / sinh / cosh as the kernels call them: through tables copied to LDS by init(), which
 // every thread of the workgroup (at least 64 threads) calls once before anything else (it
-// synchronises).  Only the f64 log comes from the math library.
+// synchronises).
 template <typename T> struct ExpLog;
 template <> struct ExpLog<double> {
     const uint64_t *etab;
